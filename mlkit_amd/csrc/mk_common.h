@@ -1,0 +1,90 @@
+// Shared host/device helpers of libmlkit_amd (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/mlkit_amd.h"
+
+// Records the message returned by mk_last_error() and returns `code`.
+int mk_fail(int code, const char *format, ...);
+
+#define MK_REQUIRE(condition, code, ...)                 \
+    do {                                                 \
+        if (!(condition)) return mk_fail((code), __VA_ARGS__); \
+    } while (0)
+
+// Launch errors surface here: nothing is synchronised, only the launch status is read.
+#define MK_LAUNCH_CHECK(name)                                                        \
+    do {                                                                             \
+        hipError_t status_ = hipGetLastError();                                      \
+        if (status_ != hipSuccess)                                                   \
+            return mk_fail(MK_ERR_HIP, "%s: %s", (name), hipGetErrorString(status_)); \
+    } while (0)
+
+static inline int mk_dtype_bytes(int dtype) { return dtype == MK_F32 ? 4 : 2; }
+static inline bool mk_dtype_valid(int dtype) { return dtype >= MK_F32 && dtype <= MK_BF16; }
+static inline int mk_cdiv(int a, int b) { return (a + b - 1) / b; }
+static inline int mk_gcd(int a, int b) {
+    while (b) {
+        int t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
+}
+
+#ifdef __HIPCC__
+
+typedef uint32_t mk_u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t mk_u32x3 __attribute__((ext_vector_type(3)));
+typedef uint32_t mk_u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 mk_h2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float mk_bf16_to_float(uint16_t bits) {
+    return __uint_as_float(static_cast<uint32_t>(bits) << 16);
+}
+
+// Round-to-nearest-even fp32 -> bf16 bit pattern (NaN kept quiet).
+__device__ __forceinline__ uint16_t mk_float_to_bf16(float value) {
+    uint32_t bits = __float_as_uint(value);
+    if ((bits & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((bits >> 16) | 0x40u);
+    bits += 0x7fffu + ((bits >> 16) & 1u);
+    return static_cast<uint16_t>(bits >> 16);
+}
+
+// Element `index` of a buffer of MK_F32 / MK_F16 / MK_BF16 values, as fp32.
+__device__ __forceinline__ float mk_load_as_float(const void *base, size_t index, int dtype) {
+    if (dtype == MK_F32) return static_cast<const float *>(base)[index];
+    const uint16_t raw = static_cast<const uint16_t *>(base)[index];
+    if (dtype == MK_F16) return static_cast<float>(__builtin_bit_cast(_Float16, raw));
+    return mk_bf16_to_float(raw);
+}
+
+__device__ __forceinline__ void mk_store_from_float(void *base, size_t index, int dtype, float value) {
+    if (dtype == MK_F32) {
+        static_cast<float *>(base)[index] = value;
+    } else if (dtype == MK_F16) {
+        static_cast<uint16_t *>(base)[index] =
+            __builtin_bit_cast(uint16_t, static_cast<_Float16>(value));
+    } else {
+        static_cast<uint16_t *>(base)[index] = mk_float_to_bf16(value);
+    }
+}
+
+// Sum over aligned groups of `SEG` lanes (a power of two up to 64); every lane of a
+// group receives the group's sum.  Lanes of a 64-wide wavefront exchange values with
+// DPP inside rows of 16 and with ds_bpermute across rows.
+template <int SEG>
+__device__ __forceinline__ float mk_segment_sum(float value) {
+    if (SEG >= 2) value += __shfl_xor(value, 1, 64);
+    if (SEG >= 4) value += __shfl_xor(value, 2, 64);
+    if (SEG >= 8) value += __shfl_xor(value, 4, 64);
+    if (SEG >= 16) value += __shfl_xor(value, 8, 64);
+    if (SEG >= 32) value += __shfl_xor(value, 16, 64);
+    if (SEG >= 64) value += __shfl_xor(value, 32, 64);
+    return value;
+}
+
+#endif  // __HIPCC__

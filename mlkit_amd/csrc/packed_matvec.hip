@@ -1,0 +1,225 @@
+// Packed scalar-codec matrix-vector product: planning, the word-at-a-time kernel for
+// layouts the chunked kernel does not take, and the C entry points.
+//
+// Replaces the reference's `matrix_vector` wrapper and direct launch
+// (kernels/packed_linear.py:181-226, inference/packed_linear.py:181-245 in
+// /root/reference/src/mlkit).
+
+#include <cstdlib>
+
+#include "packed_matvec_impl.h"
+
+#define MK_DECLARE_WIDTH(n)                                                                  \
+    bool mk_matvec_launch_b##n(const mk_matvec::MatvecArgs &, const mk_matvec::Plan &, int, \
+                               bool, hipStream_t);
+MK_DECLARE_WIDTH(2) MK_DECLARE_WIDTH(3) MK_DECLARE_WIDTH(4) MK_DECLARE_WIDTH(5)
+MK_DECLARE_WIDTH(6) MK_DECLARE_WIDTH(7) MK_DECLARE_WIDTH(8)
+#undef MK_DECLARE_WIDTH
+
+namespace {
+
+using mk_matvec::kChunkCodes;
+using mk_matvec::kMaxTableEntries;
+using mk_matvec::MatvecArgs;
+using mk_matvec::Plan;
+
+int next_pow2(int v) {
+    int p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+// ---------------------------------------------------------------------------------
+// Word-at-a-time kernel for every layout the chunked kernel does not take: one
+// wavefront per row, lanes stride over packing words assembled from bytes.
+// ---------------------------------------------------------------------------------
+struct WordArgs {
+    const void *x;
+    const uint8_t *packed;
+    const void *scales;
+    const void *zeros;
+    const float *values;
+    const void *bias;
+    void *y;
+    int samples, rows, width, group, groups;
+    int x_dtype, scale_dtype, bias_dtype;
+    int bits, bytes_per_word, codes_per_word, uniform;
+    float grid_min, grid_step;
+};
+
+__global__ void packed_matvec_words_kernel(const WordArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int sample_base = blockIdx.y * 8;
+    if (row >= a.rows) return;
+    const int row_words = a.width / a.codes_per_word;
+    const uint8_t *row_ptr = a.packed + static_cast<size_t>(row) * row_words * a.bytes_per_word;
+    const uint64_t mask = (1ull << a.bits) - 1ull;
+    float acc[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) acc[m] = 0.0f;
+    for (int word = lane; word < row_words; word += 64) {
+        uint64_t bits = 0;
+        for (int b = 0; b < a.bytes_per_word; ++b)
+            bits |= static_cast<uint64_t>(row_ptr[static_cast<size_t>(word) * a.bytes_per_word + b]) << (8 * b);
+        for (int i = 0; i < a.codes_per_word; ++i) {
+            const int k = word * a.codes_per_word + i;
+            const uint32_t code = static_cast<uint32_t>((bits >> (i * a.bits)) & mask);
+            const size_t slot = static_cast<size_t>(row) * a.groups + k / a.group;
+            float weight = a.uniform ? a.grid_min + static_cast<float>(code) * a.grid_step
+                                     : a.values[code];
+            weight *= mk_load_as_float(a.scales, slot, a.scale_dtype);
+            if (a.zeros) weight += mk_load_as_float(a.zeros, slot, a.scale_dtype);
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                const int sample = sample_base + m;
+                if (sample < a.samples)
+                    acc[m] = __builtin_fmaf(
+                        weight, mk_load_as_float(a.x, static_cast<size_t>(sample) * a.width + k, a.x_dtype),
+                        acc[m]);
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        const float total = mk_segment_sum<64>(acc[m]);
+        const int sample = sample_base + m;
+        if (lane == 0 && sample < a.samples) {
+            float result = total;
+            if (a.bias) result += mk_load_as_float(a.bias, row, a.bias_dtype);
+            mk_store_from_float(a.y, static_cast<size_t>(sample) * a.rows + row, a.x_dtype, result);
+        }
+    }
+}
+
+// Chooses the lane/row decomposition of the chunked kernel; returns false when the
+// layer needs the word kernel (widths or groups that are not multiples of 32 codes,
+// or a scale tile that does not fit in LDS).
+bool plan_chunked(int samples, int rows, int width, int group, int groups, int bits, int x_dtype,
+                  bool uniform, bool has_zero, Plan &p) {
+    if (bits < 2 || width % kChunkCodes != 0) return false;
+    if (group % kChunkCodes != 0 && group < width) return false;
+    const int chunks_per_row = width / kChunkCodes;
+    const int max_tile = x_dtype == MK_F32 ? 4 : 8;
+    int mt = 1;
+    while (mt < samples && mt < max_tile) mt <<= 1;
+    const int budget = (x_dtype == MK_F32 ? 4 : 8) / mt;  // chunks whose activations fit in registers
+    int c = 1;
+    while (c < budget && c * 64 < chunks_per_row) c <<= 1;
+    int seg;
+    if (chunks_per_row <= 64) {
+        seg = next_pow2(chunks_per_row);
+        c = 1;
+    } else {
+        seg = 64 * mk_cdiv(chunks_per_row, 64 * c);
+    }
+    if (seg > 1024) return false;
+    const int target_threads = 256;
+    int rows_parallel = seg >= target_threads ? 1 : target_threads / seg;
+    if (seg < 64 && rows_parallel % (64 / seg) != 0) rows_parallel = 64 / seg;
+    const int threads = seg * rows_parallel;
+    if (threads % 64 != 0 || threads > 1024) return false;
+    int u = 32 / (c * bits);
+    u = u < 1 ? 1 : (u > 8 ? 8 : u);
+    // Rows per workgroup: enough passes to amortise the activation load, few enough
+    // that every compute unit gets several workgroups.
+    int rows_per_thread = u;
+    const int waves_per_row = seg > 64 ? seg / 64 : 1;
+    while (true) {
+        const long workgroups = mk_cdiv(rows, rows_parallel * rows_per_thread * 2);
+        if (workgroups < 1024 || rows_per_thread * 2 > 64) break;
+        rows_per_thread *= 2;
+    }
+    auto lds_for = [&](int rpt) {
+        const size_t tile_rows = static_cast<size_t>(rows_parallel) * rpt;
+        size_t floats = (uniform ? 0 : kMaxTableEntries) + tile_rows * groups * (has_zero ? 2 : 1);
+        if (waves_per_row > 1) floats += tile_rows * mt * waves_per_row;
+        return floats * sizeof(float);
+    };
+    while (lds_for(rows_per_thread) > 60 * 1024 && rows_per_thread > u) rows_per_thread /= 2;
+    if (lds_for(rows_per_thread) > 60 * 1024) return false;
+    p.sample_tile = mt;
+    p.chunks = c;
+    p.seg_lanes = seg;
+    p.rows_parallel = rows_parallel;
+    p.rows_per_thread = rows_per_thread;
+    p.threads = threads;
+    p.grid_x = mk_cdiv(rows, rows_parallel * rows_per_thread);
+    p.lds_bytes = lds_for(rows_per_thread);
+    return true;
+}
+
+}  // namespace
+
+extern "C" int mk_packed_layout_supported(int bits, int input_width, int group) {
+    if (bits < 1 || bits > 8 || input_width < 1 || group < 1) return 0;
+    const int divisor = mk_gcd(bits, 8);
+    const int codes_per_word = 8 / divisor;
+    if (input_width % codes_per_word || group % codes_per_word) return 0;
+    const int group_words = group / codes_per_word;
+    int tile_words = group_words & -group_words;
+    if (tile_words > 128 / codes_per_word) tile_words = 128 / codes_per_word;
+    return tile_words * codes_per_word >= 16 ? 1 : 0;
+}
+
+extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packed, const void *scales,
+                                int scale_dtype, const float *values, int n_values, const void *zeros,
+                                const void *bias, int bias_dtype, void *y, int samples,
+                                int output_width, int input_width, int group, int bits, int uniform,
+                                float grid_min, float grid_step, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(x && packed && scales && y, MK_ERR_INVALID, "mk_packed_matvec: null tensor pointer");
+    MK_REQUIRE(mk_dtype_valid(x_dtype) && mk_dtype_valid(scale_dtype), MK_ERR_INVALID,
+               "mk_packed_matvec: unknown dtype code");
+    MK_REQUIRE(!bias || mk_dtype_valid(bias_dtype), MK_ERR_INVALID, "mk_packed_matvec: unknown bias dtype");
+    MK_REQUIRE(samples >= 1 && output_width >= 1 && input_width >= 1 && group >= 1, MK_ERR_INVALID,
+               "mk_packed_matvec: sizes must be positive");
+    MK_REQUIRE(bits >= 1 && bits <= 8, MK_ERR_INVALID, "mk_packed_matvec: code width must be 1..8 bits");
+    MK_REQUIRE(uniform || (values && n_values >= 1 && n_values <= (1 << bits)), MK_ERR_INVALID,
+               "mk_packed_matvec: a value table of at most 2^bits entries is required");
+    MK_REQUIRE(mk_packed_layout_supported(bits, input_width, group), MK_ERR_UNSUPPORTED,
+               "mk_packed_matvec: rows or scale groups split a packing word (bits=%d width=%d group=%d)",
+               bits, input_width, group);
+    const int groups = mk_cdiv(input_width, group);
+    const bool aligned = (reinterpret_cast<uintptr_t>(packed) & 3u) == 0 &&
+                         (reinterpret_cast<uintptr_t>(x) & 15u) == 0 &&
+                         (static_cast<size_t>(input_width) * mk_dtype_bytes(x_dtype)) % 16 == 0;
+    Plan plan;
+    if (aligned && plan_chunked(samples, output_width, input_width, group, groups, bits, x_dtype,
+                                uniform != 0, zeros != nullptr, plan)) {
+        MatvecArgs a;
+        a.x = x; a.packed = packed; a.scales = scales; a.zeros = zeros; a.values = values;
+        a.bias = bias; a.y = y;
+        a.samples = samples; a.rows = output_width; a.width = input_width; a.group = group;
+        a.groups = groups; a.n_values = n_values; a.scale_dtype = scale_dtype; a.bias_dtype = bias_dtype;
+        a.seg_lanes = plan.seg_lanes; a.rows_parallel = plan.rows_parallel;
+        a.rows_per_thread = plan.rows_per_thread; a.chunks_per_row = input_width / kChunkCodes;
+        a.grid_min = grid_min; a.grid_step = grid_step;
+        bool launched = false;
+        switch (bits) {
+            case 2: launched = mk_matvec_launch_b2(a, plan, x_dtype, uniform != 0, stream); break;
+            case 3: launched = mk_matvec_launch_b3(a, plan, x_dtype, uniform != 0, stream); break;
+            case 4: launched = mk_matvec_launch_b4(a, plan, x_dtype, uniform != 0, stream); break;
+            case 5: launched = mk_matvec_launch_b5(a, plan, x_dtype, uniform != 0, stream); break;
+            case 6: launched = mk_matvec_launch_b6(a, plan, x_dtype, uniform != 0, stream); break;
+            case 7: launched = mk_matvec_launch_b7(a, plan, x_dtype, uniform != 0, stream); break;
+            case 8: launched = mk_matvec_launch_b8(a, plan, x_dtype, uniform != 0, stream); break;
+        }
+        if (launched) {
+            MK_LAUNCH_CHECK("mk_packed_matvec");
+            return MK_OK;
+        }
+    }
+    WordArgs w;
+    w.x = x; w.packed = packed; w.scales = scales; w.zeros = zeros; w.values = values; w.bias = bias;
+    w.y = y; w.samples = samples; w.rows = output_width; w.width = input_width; w.group = group;
+    w.groups = groups; w.x_dtype = x_dtype; w.scale_dtype = scale_dtype; w.bias_dtype = bias_dtype;
+    w.bits = bits;
+    const int divisor = mk_gcd(bits, 8);
+    w.bytes_per_word = bits / divisor; w.codes_per_word = 8 / divisor; w.uniform = uniform;
+    w.grid_min = grid_min; w.grid_step = grid_step;
+    dim3 grid(mk_cdiv(output_width, 4), mk_cdiv(samples, 8));
+    hipLaunchKernelGGL(packed_matvec_words_kernel, grid, dim3(256), 0, stream, w);
+    MK_LAUNCH_CHECK("mk_packed_matvec");
+    return MK_OK;
+}

@@ -1,0 +1,61 @@
+"""Shared builders for the parity tests: seeded synthetic layers quantised by the oracle."""
+
+import numpy as np
+import torch
+
+from oracle import bitstream, scaling
+
+F32 = np.float32
+
+
+def normal_weight(rows, width, seed, scale=0.02, outlier_fraction=0.0, student_t=False):
+    """fp16-rounded weights: N(0, scale^2), optional x20 outlier columns or Student-t(5)."""
+    generator = torch.Generator().manual_seed(seed)
+    weight = torch.randn(rows, width, generator=generator)
+    if student_t:
+        chi = torch.randn(5, rows, width, generator=generator).square().sum(0) / 5
+        weight = weight / chi.sqrt()
+    weight = weight * scale
+    if outlier_fraction:
+        count = max(1, round(outlier_fraction * width))
+        columns = torch.randperm(width, generator=generator)[:count]
+        weight[:, columns] *= 20
+    return weight.half().float().numpy()
+
+
+def activations(samples, width, seed, dtype=torch.float16):
+    generator = torch.Generator().manual_seed(seed)
+    return torch.randn(samples, width, generator=generator).to(dtype)
+
+
+def quantised_layer(weight, values, *, bits, group, integer, asym=False, scale="absmax", fmt="fp16"):
+    """Oracle quantisation + packing.  Returns a dict of numpy arrays."""
+    result = scaling.quantize(weight, values, group=group, integer=integer, asym=asym,
+                              scale=scale, fmt=fmt)
+    result["packed"] = bitstream.pack(result["codes"], bits)
+    result["bits"] = bits
+    result["shape"] = weight.shape
+    result["dense"] = scaling.decode_grouped(result["codes"], result["scales"], result["values"],
+                                             result["group"], result["zero"])
+    return result
+
+
+def to_device(layer, scale_dtype=torch.float16, device="cuda"):
+    """Device tensors of a quantised layer in the dtypes PackedLinear keeps them in."""
+    out = {
+        "packed": torch.from_numpy(layer["packed"]).to(device),
+        "scales": torch.from_numpy(layer["scales"]).to(device=device, dtype=scale_dtype),
+        "values": torch.from_numpy(np.asarray(layer["values"], dtype=F32)).to(device),
+        "zeros": None,
+    }
+    if layer["zero"] is not None:
+        out["zeros"] = torch.from_numpy(layer["zero"]).to(device=device, dtype=scale_dtype)
+    return out
+
+
+def uniform_grid(values):
+    """(is_uniform, minimum, step) the way PackedLinear derives it (inference/packed_linear.py:90-97)."""
+    values = torch.as_tensor(np.asarray(values, dtype=F32))
+    steps = values.diff()
+    uniform = bool(len(steps) and torch.allclose(steps, steps[0].expand_as(steps)))
+    return uniform, float(values[0]), float(steps[0]) if len(steps) else 1.0

@@ -1,0 +1,162 @@
+"""GPU parity of the packed matvec (through the C ABI) against the oracle's
+reconstruct-then-matmul.  Tolerances: fp16/bf16 activations, max |y - y_ref| <= 1e-3 * max |y_ref|
+(fp32 accumulate) against a float64 yardstick, plus the reference's own allclose bounds
+(tests/inference/test_packed_linear.py:13-24,91-98,162-186)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import matvec as oracle_matvec, scaling
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+
+def run_matvec(layer, x, bias=None, scale_dtype=torch.float16):
+    from mlkit_amd.kernels import packed_linear
+
+    tensors = helpers.to_device(layer, scale_dtype)
+    rows, width = layer["shape"]
+    layout = packed_linear.layout_for(layer["bits"], width, layer["group"])
+    assert layout is not None
+    uniform, minimum, step = helpers.uniform_grid(layer["values"])
+    inputs = x.cuda().contiguous()
+    output = torch.empty((inputs.shape[0], rows), dtype=inputs.dtype, device="cuda")
+    packed_linear.matrix_vector(
+        inputs, tensors["packed"], tensors["scales"], tensors["values"], tensors["zeros"],
+        None if bias is None else bias.cuda(), output, layer["group"], layout,
+        uniform_grid=uniform, grid_minimum=minimum, grid_step=step)
+    torch.cuda.synchronize()
+    return output.float().cpu().numpy()
+
+
+def check(y, layer, x, bias=None, relative=1e-3):
+    reference = oracle_matvec.reconstruct_then_matmul_f64(
+        x.float().numpy(), layer["dense"], None if bias is None else bias.float().numpy())
+    scale = np.abs(reference).max()
+    error = np.abs(y - reference).max() / scale
+    assert error <= relative, f"max error {error:.3e} of the output range"
+    return error
+
+
+INT4 = scaling.int_values(4)
+
+
+def test_config1_int4_asym_g128_4096x4096():
+    weight = helpers.normal_weight(4096, 4096, seed=1)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True, asym=True)
+    x = helpers.activations(1, 4096, seed=2)
+    y = run_matvec(layer, x)
+    check(y, layer, x)
+    fp32_reference = oracle_matvec.reconstruct_then_matmul(
+        x.float().numpy(), layer["packed"], 4, layer["shape"], layer["scales"], layer["values"],
+        128, layer["zero"])
+    np.testing.assert_allclose(y, fp32_reference, rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("shape", [(896, 896), (128, 896), (4864, 896), (896, 4864)])
+@pytest.mark.parametrize("samples", [1, 2, 4, 8])
+def test_config2_decoder_shapes_int4_g128(shape, samples):
+    weight = helpers.normal_weight(*shape, seed=3, outlier_fraction=0.001)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
+    x = helpers.activations(samples, shape[1], seed=4)
+    check(run_matvec(layer, x), layer, x)
+
+
+@pytest.mark.parametrize("samples", [1, 8])
+def test_config2_tied_output_head(samples):
+    weight = helpers.normal_weight(151936, 896, seed=5, outlier_fraction=0.001)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
+    x = helpers.activations(samples, 896, seed=6)
+    check(run_matvec(layer, x), layer, x)
+
+
+CODECS = {
+    "int2-g64": dict(values=scaling.int_values(2), bits=2, group=64, integer=True),
+    "int3-g64": dict(values=scaling.int_values(3), bits=3, group=64, integer=True),
+    "nf4-g64": dict(values=scaling.NF4_VALUES, bits=4, group=64, integer=False),
+    "cb3-g64-mse": dict(values=np.array([-1, -.5, -.25, 0, .25, .5, 1], dtype=np.float32), bits=3,
+                        group=64, integer=False, scale="mse"),
+}
+
+
+@pytest.mark.parametrize("name", CODECS)
+@pytest.mark.parametrize("shape", [(4096, 4096), (1024, 4096), (4096, 14336)])
+@pytest.mark.parametrize("samples", [1, 8])
+def test_config3_sub_byte_and_codebook_codecs(name, shape, samples):
+    options = dict(CODECS[name])
+    values = options.pop("values")
+    rows = shape[0] if shape[1] == 4096 else 512  # full width, a row slice of the widest layer
+    weight = helpers.normal_weight(rows, shape[1], seed=7, student_t=True)
+    layer = helpers.quantised_layer(weight, values, **options)
+    x = helpers.activations(samples, shape[1], seed=8)
+    check(run_matvec(layer, x), layer, x)
+
+
+def test_metric_shape_int4_g128_4096x14336_all_row_counts():
+    weight = helpers.normal_weight(4096, 14336, seed=9)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
+    for samples in (1, 2, 4, 8):
+        x = helpers.activations(samples, 14336, seed=10 + samples)
+        check(run_matvec(layer, x), layer, x)
+
+
+def test_down_projection_14336x4096():
+    weight = helpers.normal_weight(14336, 4096, seed=11)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
+    for samples in (1, 8):
+        x = helpers.activations(samples, 4096, seed=12)
+        check(run_matvec(layer, x), layer, x)
+
+
+WIDTHS = {
+    "int2": (scaling.int_values(2), 2, 64, True),
+    "int3": (scaling.int_values(3), 3, 64, True),
+    "int5": (scaling.int_values(5), 5, 64, True),
+    "int6": (scaling.int_values(6), 6, 32, True),
+    "int7": (scaling.int_values(7), 7, 64, True),
+    "int8": (scaling.int_values(8), 8, 128, True),
+    "codebook3": (np.linspace(-1, 1, 7, dtype=np.float32) ** 3, 3, 32, False),
+    "int4-g16": (scaling.int_values(4), 4, 16, True),
+    "int3-g48": (scaling.int_values(3), 3, 48, True),
+}
+
+
+@pytest.mark.parametrize("name", WIDTHS)
+@pytest.mark.parametrize("samples", [1, 3, 8, 20])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_every_code_width_and_activation_dtype(name, samples, dtype):
+    values, bits, group, integer = WIDTHS[name]
+    width = 288 if group == 48 else 256
+    weight = helpers.normal_weight(37, width, seed=13, scale=1.0)
+    for asym in (False, True):
+        layer = helpers.quantised_layer(weight, values, bits=bits, group=group, integer=integer,
+                                        asym=asym, fmt="fp32")
+        assert layer["packed"].size == 37 * width * bits // 8
+        x = helpers.activations(samples, width, seed=14, dtype=dtype)
+        bias = helpers.activations(1, 37, seed=15, dtype=dtype)[0]
+        y = run_matvec(layer, x, bias=bias, scale_dtype=torch.float32)
+        if dtype == torch.float32:
+            reference = oracle_matvec.reconstruct_then_matmul(
+                x.numpy(), layer["packed"], bits, layer["shape"], layer["scales"], layer["values"],
+                group, layer["zero"], bias.numpy())
+            np.testing.assert_allclose(y, reference, rtol=1e-4, atol=1e-4)
+        else:
+            check(y, layer, x, bias, relative=1e-3 if dtype == torch.float16 else 8e-3)
+
+
+def test_rejects_layouts_that_split_a_word():
+    from mlkit_amd import native
+
+    lib = native.library()
+    assert lib.mk_packed_layout_supported(4, 255, 64) == 0
+    assert lib.mk_packed_layout_supported(3, 250, 50) == 0
+    assert lib.mk_packed_layout_supported(4, 4096, 128) == 1
+    x = torch.zeros(1, 250, device="cuda")
+    status = lib.mk_packed_matvec(
+        x.data_ptr(), 0, x.data_ptr(), x.data_ptr(), 0, x.data_ptr(), 8, None, None, 0, x.data_ptr(),
+        1, 16, 250, 50, 3, 1, 0.0, 1.0, None)
+    assert status == native.MK_ERR_UNSUPPORTED
+    assert "packing word" in native.last_error()
