@@ -62,6 +62,29 @@ __device__ __forceinline__ float mk_load_as_float(const void *base, size_t index
     return mk_bf16_to_float(raw);
 }
 
+// The same load split in two, branch-free, so that many can be in flight before any is
+// used: the aligned dword holding the element is fetched from a 4-byte aligned buffer
+// and the element is shifted out of it only when it is converted.
+struct MkRaw {
+    uint32_t word;
+    uint32_t shift;
+};
+
+__device__ __forceinline__ MkRaw mk_load_raw(const void *aligned_base, size_t index, int dtype) {
+    const size_t byte = index << (dtype == MK_F32 ? 2 : 1);
+    MkRaw raw;
+    raw.word = static_cast<const uint32_t *>(aligned_base)[byte >> 2];
+    raw.shift = (static_cast<uint32_t>(byte) & 3u) * 8u;
+    return raw;
+}
+
+__device__ __forceinline__ float mk_raw_to_float(MkRaw raw, int dtype) {
+    const uint32_t bits = raw.word >> raw.shift;
+    const float from_half = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits)));
+    const float from_bits = __uint_as_float(dtype == MK_F32 ? bits : bits << 16);
+    return dtype == MK_F16 ? from_half : from_bits;
+}
+
 __device__ __forceinline__ void mk_store_from_float(void *base, size_t index, int dtype, float value) {
     if (dtype == MK_F32) {
         static_cast<float *>(base)[index] = value;

@@ -42,6 +42,7 @@ struct WordArgs {
     const void *bias;
     void *y;
     int samples, rows, width, group, groups;
+    int first_row;  // rows [first_row, rows) are multiplied
     int x_dtype, scale_dtype, bias_dtype;
     int bits, bytes_per_word, codes_per_word, uniform;
     float grid_min, grid_step;
@@ -49,7 +50,7 @@ struct WordArgs {
 
 __global__ void packed_matvec_words_kernel(const WordArgs a) {
     const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int row = a.first_row + blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int sample_base = blockIdx.y * 8;
     if (row >= a.rows) return;
     const int row_words = a.width / a.codes_per_word;
@@ -92,60 +93,63 @@ __global__ void packed_matvec_words_kernel(const WordArgs a) {
     }
 }
 
+// Dynamic LDS of one workgroup: value table, fp32 scale (and zero) tile, per-wave row sums.
+size_t lds_bytes_for(const Plan &p, int groups, bool uniform, bool has_zero) {
+    (void)has_zero;
+    const size_t tile_rows = static_cast<size_t>(p.rows_parallel) * p.rows_per_thread;
+    size_t tile_slots = tile_rows * groups;
+    if (tile_slots < 4u * p.threads) tile_slots = 4u * p.threads;  // kStaged * threads
+    size_t floats = (uniform ? 0 : kMaxTableEntries) + 2 * tile_slots;
+    floats += tile_rows > static_cast<size_t>(p.threads) ? tile_rows : p.threads;  // bias tile
+    const int group_rows = p.sample_tile >= 8 ? 1 : (p.sample_tile == 4 ? 2 : 4);
+    floats += 2 * static_cast<size_t>(group_rows) * p.sample_tile * p.threads;  // per-lane sums, two buffers
+    return floats * sizeof(float);
+}
+
+int tuning(const char *name, int fallback) {
+    const char *text = std::getenv(name);
+    return text && *text ? std::atoi(text) : fallback;
+}
+
 // Chooses the lane/row decomposition of the chunked kernel; returns false when the
 // layer needs the word kernel (widths or groups that are not multiples of 32 codes,
 // or a scale tile that does not fit in LDS).
+//
+// A row's chunks are spread over `seg` lanes (a power of two up to 64, or whole
+// wavefronts), one chunk per lane, two when a row has more than 512 chunks.  Every
+// thread owns 2U rows, so a workgroup multiplies a tile of rows_parallel * 2U adjacent
+// rows; rows_parallel grows (up to 256 threads) only while the grid keeps at least two
+// workgroups per compute unit.
 bool plan_chunked(int samples, int rows, int width, int group, int groups, int bits, int x_dtype,
                   bool uniform, bool has_zero, Plan &p) {
     if (bits < 2 || width % kChunkCodes != 0) return false;
     if (group % kChunkCodes != 0 && group < width) return false;
     const int chunks_per_row = width / kChunkCodes;
-    const int max_tile = x_dtype == MK_F32 ? 4 : 8;
+    int c = chunks_per_row > 512 ? 2 : 1;
+    if (chunks_per_row > 1024) return false;
+    const int max_tile = (x_dtype == MK_F32 ? 4 : 8) / c;
     int mt = 1;
     while (mt < samples && mt < max_tile) mt <<= 1;
-    const int budget = (x_dtype == MK_F32 ? 4 : 8) / mt;  // chunks whose activations fit in registers
-    int c = 1;
-    while (c < budget && c * 64 < chunks_per_row) c <<= 1;
-    int seg;
-    if (chunks_per_row <= 64) {
-        seg = next_pow2(chunks_per_row);
-        c = 1;
-    } else {
-        seg = 64 * mk_cdiv(chunks_per_row, 64 * c);
-    }
-    if (seg > 1024) return false;
-    const int target_threads = 256;
-    int rows_parallel = seg >= target_threads ? 1 : target_threads / seg;
-    if (seg < 64 && rows_parallel % (64 / seg) != 0) rows_parallel = 64 / seg;
+    const int lanes = mk_cdiv(chunks_per_row, c);
+    const int seg = lanes <= 64 ? next_pow2(lanes) : 64 * mk_cdiv(lanes, 64);
+    const int rows_per_thread = mk_matvec::kThreadRows;
+    int rows_parallel = seg < 64 ? 64 / seg : 1;
+    const int wanted_workgroups = tuning("MK_MATVEC_WORKGROUPS", 512);
+    while (seg * rows_parallel * 2 <= 256 &&
+           rows / (rows_parallel * 2 * rows_per_thread) >= wanted_workgroups)
+        rows_parallel *= 2;
+    rows_parallel = tuning("MK_MATVEC_ROWS_PARALLEL", rows_parallel);
     const int threads = seg * rows_parallel;
-    if (threads % 64 != 0 || threads > 1024) return false;
-    int u = 32 / (c * bits);
-    u = u < 1 ? 1 : (u > 8 ? 8 : u);
-    // Rows per workgroup: enough passes to amortise the activation load, few enough
-    // that every compute unit gets several workgroups.
-    int rows_per_thread = u;
-    const int waves_per_row = seg > 64 ? seg / 64 : 1;
-    while (true) {
-        const long workgroups = mk_cdiv(rows, rows_parallel * rows_per_thread * 2);
-        if (workgroups < 1024 || rows_per_thread * 2 > 64) break;
-        rows_per_thread *= 2;
-    }
-    auto lds_for = [&](int rpt) {
-        const size_t tile_rows = static_cast<size_t>(rows_parallel) * rpt;
-        size_t floats = (uniform ? 0 : kMaxTableEntries) + tile_rows * groups * (has_zero ? 2 : 1);
-        if (waves_per_row > 1) floats += tile_rows * mt * waves_per_row;
-        return floats * sizeof(float);
-    };
-    while (lds_for(rows_per_thread) > 60 * 1024 && rows_per_thread > u) rows_per_thread /= 2;
-    if (lds_for(rows_per_thread) > 60 * 1024) return false;
+    if (threads % 64 != 0 || threads > 512) return false;
     p.sample_tile = mt;
     p.chunks = c;
     p.seg_lanes = seg;
     p.rows_parallel = rows_parallel;
-    p.rows_per_thread = rows_per_thread;
     p.threads = threads;
-    p.grid_x = mk_cdiv(rows, rows_parallel * rows_per_thread);
-    p.lds_bytes = lds_for(rows_per_thread);
+    p.rows_per_thread = rows_per_thread;
+    p.lds_bytes = lds_bytes_for(p, groups, uniform, has_zero);
+    if (p.lds_bytes > 60 * 1024) return false;
+    p.grid_x = 0;
     return true;
 }
 
@@ -182,44 +186,66 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
                bits, input_width, group);
     const int groups = mk_cdiv(input_width, group);
     const bool aligned = (reinterpret_cast<uintptr_t>(packed) & 3u) == 0 &&
+                         (reinterpret_cast<uintptr_t>(scales) & 3u) == 0 &&
+                         (reinterpret_cast<uintptr_t>(zeros) & 3u) == 0 &&
+                         (reinterpret_cast<uintptr_t>(bias) & 3u) == 0 &&
                          (reinterpret_cast<uintptr_t>(x) & 15u) == 0 &&
                          (static_cast<size_t>(input_width) * mk_dtype_bytes(x_dtype)) % 16 == 0;
+    const int divisor = mk_gcd(bits, 8);
+    int done_rows = 0;  // rows [0, done_rows) are covered by a chunked kernel
     Plan plan;
-    if (aligned && plan_chunked(samples, output_width, input_width, group, groups, bits, x_dtype,
+    if (aligned && !tuning("MK_MATVEC_NO_STREAM4", 0) &&
+        mk_matvec::stream4_accepts(input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
+        (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
+        mk_matvec::Stream4Args s4;
+        s4.x = x; s4.packed = packed; s4.scales = scales; s4.zeros = zeros; s4.bias = bias; s4.y = y;
+        s4.samples = samples; s4.rows = output_width; s4.width = input_width; s4.group = group;
+        s4.groups = groups; s4.bias_dtype = bias_dtype; s4.grid_min = grid_min; s4.grid_step = grid_step;
+        done_rows = mk_matvec::stream4_launch(s4, stream);
+        if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
+    } else if (aligned && plan_chunked(samples, output_width, input_width, group, groups, bits, x_dtype,
                                 uniform != 0, zeros != nullptr, plan)) {
-        MatvecArgs a;
-        a.x = x; a.packed = packed; a.scales = scales; a.zeros = zeros; a.values = values;
-        a.bias = bias; a.y = y;
-        a.samples = samples; a.rows = output_width; a.width = input_width; a.group = group;
-        a.groups = groups; a.n_values = n_values; a.scale_dtype = scale_dtype; a.bias_dtype = bias_dtype;
-        a.seg_lanes = plan.seg_lanes; a.rows_parallel = plan.rows_parallel;
-        a.rows_per_thread = plan.rows_per_thread; a.chunks_per_row = input_width / kChunkCodes;
-        a.grid_min = grid_min; a.grid_step = grid_step;
-        bool launched = false;
-        switch (bits) {
-            case 2: launched = mk_matvec_launch_b2(a, plan, x_dtype, uniform != 0, stream); break;
-            case 3: launched = mk_matvec_launch_b3(a, plan, x_dtype, uniform != 0, stream); break;
-            case 4: launched = mk_matvec_launch_b4(a, plan, x_dtype, uniform != 0, stream); break;
-            case 5: launched = mk_matvec_launch_b5(a, plan, x_dtype, uniform != 0, stream); break;
-            case 6: launched = mk_matvec_launch_b6(a, plan, x_dtype, uniform != 0, stream); break;
-            case 7: launched = mk_matvec_launch_b7(a, plan, x_dtype, uniform != 0, stream); break;
-            case 8: launched = mk_matvec_launch_b8(a, plan, x_dtype, uniform != 0, stream); break;
-        }
-        if (launched) {
-            MK_LAUNCH_CHECK("mk_packed_matvec");
-            return MK_OK;
+        const int tile_rows = plan.rows_parallel * plan.rows_per_thread;
+        const int tiles = output_width / tile_rows;
+        if (tiles > 0) {
+            MatvecArgs a;
+            a.x = x; a.packed = packed; a.scales = scales; a.zeros = zeros; a.values = values;
+            a.bias = bias; a.y = y;
+            a.scale_row_offset = 0;
+            a.samples = samples; a.rows = output_width; a.width = input_width; a.group = group;
+            a.groups = groups; a.n_values = n_values; a.scale_dtype = scale_dtype; a.bias_dtype = bias_dtype;
+            a.seg_lanes = plan.seg_lanes; a.rows_parallel = plan.rows_parallel;
+            a.chunks_per_row = input_width / kChunkCodes;
+            a.grid_min = grid_min; a.grid_step = grid_step;
+            plan.grid_x = tiles;
+            bool launched = false;
+            switch (bits) {
+                case 2: launched = mk_matvec_launch_b2(a, plan, x_dtype, uniform != 0, stream); break;
+                case 3: launched = mk_matvec_launch_b3(a, plan, x_dtype, uniform != 0, stream); break;
+                case 4: launched = mk_matvec_launch_b4(a, plan, x_dtype, uniform != 0, stream); break;
+                case 5: launched = mk_matvec_launch_b5(a, plan, x_dtype, uniform != 0, stream); break;
+                case 6: launched = mk_matvec_launch_b6(a, plan, x_dtype, uniform != 0, stream); break;
+                case 7: launched = mk_matvec_launch_b7(a, plan, x_dtype, uniform != 0, stream); break;
+                case 8: launched = mk_matvec_launch_b8(a, plan, x_dtype, uniform != 0, stream); break;
+            }
+            if (launched) {
+                MK_LAUNCH_CHECK("mk_packed_matvec");
+                done_rows = tiles * tile_rows;
+            }
         }
     }
-    WordArgs w;
-    w.x = x; w.packed = packed; w.scales = scales; w.zeros = zeros; w.values = values; w.bias = bias;
-    w.y = y; w.samples = samples; w.rows = output_width; w.width = input_width; w.group = group;
-    w.groups = groups; w.x_dtype = x_dtype; w.scale_dtype = scale_dtype; w.bias_dtype = bias_dtype;
-    w.bits = bits;
-    const int divisor = mk_gcd(bits, 8);
-    w.bytes_per_word = bits / divisor; w.codes_per_word = 8 / divisor; w.uniform = uniform;
-    w.grid_min = grid_min; w.grid_step = grid_step;
-    dim3 grid(mk_cdiv(output_width, 4), mk_cdiv(samples, 8));
-    hipLaunchKernelGGL(packed_matvec_words_kernel, grid, dim3(256), 0, stream, w);
-    MK_LAUNCH_CHECK("mk_packed_matvec");
+    if (done_rows < output_width) {
+        WordArgs w;
+        w.x = x; w.packed = packed; w.scales = scales; w.zeros = zeros; w.values = values; w.bias = bias;
+        w.y = y; w.samples = samples; w.rows = output_width; w.width = input_width; w.group = group;
+        w.groups = groups; w.first_row = done_rows;
+        w.x_dtype = x_dtype; w.scale_dtype = scale_dtype; w.bias_dtype = bias_dtype;
+        w.bits = bits;
+        w.bytes_per_word = bits / divisor; w.codes_per_word = 8 / divisor; w.uniform = uniform;
+        w.grid_min = grid_min; w.grid_step = grid_step;
+        dim3 grid(mk_cdiv(output_width - done_rows, 4), mk_cdiv(samples, 8));
+        hipLaunchKernelGGL(packed_matvec_words_kernel, grid, dim3(256), 0, stream, w);
+        MK_LAUNCH_CHECK("mk_packed_matvec");
+    }
     return MK_OK;
 }

@@ -25,6 +25,9 @@ namespace mk_matvec {
 
 constexpr int kChunkCodes = 32;
 constexpr int kMaxTableEntries = 256;
+#ifndef MK_MATVEC_AHEAD
+#define MK_MATVEC_AHEAD 8
+#endif
 
 struct MatvecArgs {
     const void *x;
@@ -44,11 +47,25 @@ struct MatvecArgs {
     int bias_dtype;
     int seg_lanes;        // lanes (incl. idle ones) that share one row
     int rows_parallel;    // rows in flight per workgroup pass
-    int rows_per_thread;  // passes per workgroup
     int chunks_per_row;   // width / 32
+    int scale_row_offset; // row of `scales`/`zeros` that row 0 of this launch uses
     float grid_min;
     float grid_step;
 };
+
+// Arguments of the 4-bit streaming kernel (packed_matvec_stream4.hip).
+struct Stream4Args {
+    const void *x;        // fp16 [samples, width]
+    const uint8_t *packed;
+    const void *scales;   // fp16 [rows, groups]
+    const void *zeros;    // fp16 [rows, groups] or null
+    const void *bias;     // [rows] of bias_dtype, or null
+    void *y;              // fp16 [samples, rows]
+    int samples, rows, width, group, groups, bias_dtype;
+    float grid_min, grid_step;
+};
+bool stream4_accepts(int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
+int stream4_launch(const Stream4Args &a, hipStream_t stream);
 
 // ---------------------------------------------------------------------------------
 // Activation registers.  XT: MK_F32 keeps 32 floats per chunk; MK_F16 / MK_BF16 keep
@@ -74,41 +91,59 @@ __device__ __forceinline__ float x_element(const XChunk<XT> &x, int k) {
 }
 
 template <int XT>
-__device__ __forceinline__ void load_x_chunk(XChunk<XT> &x, const void *base, size_t element,
-                                             bool active, float &sum) {
+__device__ __forceinline__ void load_x_chunk(XChunk<XT> &x, const void *base, size_t element) {
     constexpr int kWords = XT == MK_F32 ? 32 : 16;
-    if (active) {
-        const mk_u32x4 *src = reinterpret_cast<const mk_u32x4 *>(
-            static_cast<const uint8_t *>(base) + element * (XT == MK_F32 ? 4 : 2));
+    const mk_u32x4 *src = reinterpret_cast<const mk_u32x4 *>(
+        static_cast<const uint8_t *>(base) + element * (XT == MK_F32 ? 4 : 2));
 #pragma unroll
-        for (int i = 0; i < kWords / 4; ++i) {
-            const mk_u32x4 v = src[i];
-            x.r[4 * i + 0] = v.x;
-            x.r[4 * i + 1] = v.y;
-            x.r[4 * i + 2] = v.z;
-            x.r[4 * i + 3] = v.w;
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < kWords; ++i) x.r[i] = 0u;
+    for (int i = 0; i < kWords / 4; ++i) {
+        const mk_u32x4 v = src[i];
+        x.r[4 * i + 0] = v.x;
+        x.r[4 * i + 1] = v.y;
+        x.r[4 * i + 2] = v.z;
+        x.r[4 * i + 3] = v.w;
     }
-    float total = 0.0f;
-#pragma unroll
-    for (int k = 0; k < 32; ++k) total += x_element<XT>(x, k);
-    sum = total;
 }
 
-// (x0,x1)(x2,x3)(x4,x5)(x6,x7) -> (x0,x4)(x1,x5)(x2,x6)(x3,x7) for every eight codes.
-__device__ __forceinline__ void pair_for_nibbles(XChunk<MK_F16> &x) {
+// Sum of the 32 activations of a chunk in fp32.
+template <int XT>
+__device__ __forceinline__ float chunk_sum(const XChunk<XT> &x) {
+    float total = 0.0f;
+    if constexpr (XT == MK_F16) {
+        const mk_h2 ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            total = __builtin_amdgcn_fdot2(ones, __builtin_bit_cast(mk_h2, x.r[j]), total, false);
+    } else {
+#pragma unroll
+        for (int k = 0; k < 32; ++k) total += x_element<XT>(x, k);
+    }
+    return total;
+}
+
+// (x0,x1)(x2,x3)(x4,x5)(x6,x7) -> (x0,x4) (x1,x5)/16 (x2,x6) (x3,x7)/16 for every eight
+// codes: the pair order and scaling the 4-bit extraction of chunk_dot expects.  Returns
+// what that extraction accumulates for all-zero codes, 1024 * sum(stored values).
+__device__ __forceinline__ float pair_for_nibbles(XChunk<MK_F16> &x) {
+    const mk_h2 sixteenth = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
+    const mk_h2 base = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+    auto scaled = [&](uint32_t pair) __attribute__((always_inline)) {
+        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(mk_h2, pair) * sixteenth);
+    };
+    float offset = 0.0f;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         const uint32_t p0 = x.r[4 * g + 0], p1 = x.r[4 * g + 1];
         const uint32_t p2 = x.r[4 * g + 2], p3 = x.r[4 * g + 3];
         x.r[4 * g + 0] = __builtin_amdgcn_perm(p2, p0, 0x05040100u);
-        x.r[4 * g + 1] = __builtin_amdgcn_perm(p2, p0, 0x07060302u);
+        x.r[4 * g + 1] = scaled(__builtin_amdgcn_perm(p2, p0, 0x07060302u));
         x.r[4 * g + 2] = __builtin_amdgcn_perm(p3, p1, 0x05040100u);
-        x.r[4 * g + 3] = __builtin_amdgcn_perm(p3, p1, 0x07060302u);
+        x.r[4 * g + 3] = scaled(__builtin_amdgcn_perm(p3, p1, 0x07060302u));
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            offset = __builtin_amdgcn_fdot2(base, __builtin_bit_cast(mk_h2, x.r[4 * g + j]), offset, false);
     }
+    return offset;
 }
 
 // ---------------------------------------------------------------------------------
@@ -171,24 +206,26 @@ __device__ __forceinline__ void chunk_dot(const CodeChunk<BITS> &codes, const XC
 #pragma unroll
     for (int m = 0; m < MT; ++m) dot[m] = 0.0f;
     if constexpr (BITS == 4 && XT == MK_F16 && UNIFORM) {
-        // Two codes at a time: a nibble OR-ed into the mantissa of fp16 1024.0 is
-        // 1024 + c (or 1024 + 16 c one nibble up), which one packed op turns into c
-        // exactly; v_dot2_f32_f16 then accumulates both products in fp32.
-        const mk_h2 bias_low = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
-        const mk_h2 sixteenth = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
-        const mk_h2 bias_high = {static_cast<_Float16>(-64.0f), static_cast<_Float16>(-64.0f)};
+        // Two codes at a time.  v_bfi_b32 drops a nibble into the mantissa of both halves
+        // of the fp16 pair (1024, 1024): bits 0..3 give 1024 + c, bits 4..7 give
+        // 1024 + 16 c (those activations were pre-scaled by 1/16).  Each product is exact
+        // in fp32 and v_dot2_f32_f16 accumulates in fp32; the caller subtracts the
+        // code-independent part, 1024 * sum(stored activations), once per chunk.
+        // (word & mask) | (magic & ~mask) is one v_bfi_b32; `magic` is kept opaque so the
+        // second term is not folded into a constant.
+        uint32_t magic = 0x64006400u;
+        asm volatile("" : "+v"(magic));
+        auto insert = [&](uint32_t mask, uint32_t word) __attribute__((always_inline)) {
+            return __builtin_bit_cast(mk_h2, (word & mask) | (magic & ~mask));
+        };
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t w = codes.w[i];
             const uint32_t w8 = w >> 8;
-            const mk_h2 t0 = __builtin_bit_cast(mk_h2, (w & 0x000f000fu) | 0x64006400u);
-            const mk_h2 t1 = __builtin_bit_cast(mk_h2, (w & 0x00f000f0u) | 0x64006400u);
-            const mk_h2 t2 = __builtin_bit_cast(mk_h2, (w8 & 0x000f000fu) | 0x64006400u);
-            const mk_h2 t3 = __builtin_bit_cast(mk_h2, (w8 & 0x00f000f0u) | 0x64006400u);
-            const mk_h2 h0 = t0 - bias_low;
-            const mk_h2 h1 = t1 * sixteenth + bias_high;
-            const mk_h2 h2 = t2 - bias_low;
-            const mk_h2 h3 = t3 * sixteenth + bias_high;
+            const mk_h2 h0 = insert(0x000f000fu, w);   // codes 0 and 4
+            const mk_h2 h1 = insert(0x00f000f0u, w);   // codes 1 and 5 (x16)
+            const mk_h2 h2 = insert(0x000f000fu, w8);  // codes 2 and 6
+            const mk_h2 h3 = insert(0x00f000f0u, w8);  // codes 3 and 7 (x16)
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 float d = dot[m];
@@ -215,191 +252,350 @@ __device__ __forceinline__ void chunk_dot(const CodeChunk<BITS> &codes, const XC
     }
 }
 
-template <int BITS, int C>
-constexpr int rows_in_flight() {
-    int u = 32 / (C * BITS);
-    return u < 1 ? 1 : (u > 8 ? 8 : u);
+// A thread owns kThreadRows rows of its workgroup's tile; they are finished in groups of
+// group_rows<MT>() rows (at most 8 row sums per thread and group) while the code stream
+// runs rows_ahead() rows in front.
+constexpr int kThreadRows = 16;
+
+template <int MT>
+constexpr int group_rows() {
+    return MT >= 8 ? 1 : (MT == 4 ? 2 : 4);
 }
 
-template <int BITS, int XT, int MT, int C, bool UNIFORM>
-struct RowBatch {
-    static constexpr int U = rows_in_flight<BITS, C>();
-    CodeChunk<BITS> codes[U][C];
+template <int BITS, int C>
+constexpr int rows_ahead() {
+    return 64 / (C * BITS) >= 8 ? 8 : 4;
+}
 
-    // Issues the code loads of rows `pass .. pass+U-1` of this thread.
-    __device__ __forceinline__ void load(const MatvecArgs &a, int pass, int row_base, int row_phase,
-                                         int lane_in_row, const bool (&chunk_active)[C]) {
-        const size_t row_bytes = static_cast<size_t>(a.chunks_per_row) * (4 * BITS);
+// Element `index` (counted from `base`, a uniform address) of a 2- or 4-byte typed
+// buffer, fetched as the aligned dword that holds it; convert with mk_raw_to_float.
+__device__ __forceinline__ MkRaw load_raw_near(const uint8_t *base, uint32_t index, int dtype) {
+    const uint32_t misalignment = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(base)) & 3u;
+    const uint32_t byte = misalignment + (index << (dtype == MK_F32 ? 2 : 1));
+    MkRaw raw;
+    raw.word = reinterpret_cast<const uint32_t *>(base - misalignment)[byte >> 2];
+    raw.shift = (byte & 3u) * 8u;
+    return raw;
+}
+
+// The value lane `lane ^ (1 << STAGE)` holds, by vector-ALU lane moves only (DPP inside
+// rows of 16 lanes, v_permlane16_swap / v_permlane32_swap across rows).
+template <int STAGE>
+__device__ __forceinline__ float lane_exchange(float value, int lane) {
+    const int bits = __builtin_bit_cast(int, value);
+    int moved;
+    if constexpr (STAGE == 0) {
+        moved = __builtin_amdgcn_mov_dpp(bits, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+    } else if constexpr (STAGE == 1) {
+        moved = __builtin_amdgcn_mov_dpp(bits, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+    } else if constexpr (STAGE == 2) {
+        // lanes 0-3 and 8-11 of a row read four lanes up, lanes 4-7 and 12-15 four lanes down
+        moved = __builtin_amdgcn_update_dpp(bits, bits, 0x104, 0xf, 0x5, false);   // row_shl:4
+        moved = __builtin_amdgcn_update_dpp(moved, bits, 0x114, 0xf, 0xa, false);  // row_shr:4
+    } else if constexpr (STAGE == 3) {
+        moved = __builtin_amdgcn_mov_dpp(bits, 0x128, 0xf, 0xf, true);  // row_ror:8
+    } else if constexpr (STAGE == 4) {
+        const auto swapped = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+        moved = (lane & 16) ? swapped[0] : swapped[1];
+    } else {
+        const auto swapped = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+        moved = (lane & 32) ? swapped[0] : swapped[1];
+    }
+    return __builtin_bit_cast(float, moved);
+}
+
+// Sums each of V per-lane values over the 64 lanes of a wavefront.  While more than one
+// value is left, every stage halves them: the lane whose bit STAGE is clear keeps the
+// lower half and receives its partner's lower half, the other lane the upper half.  On
+// return v[0] of lane L is the total of value number
+//     sum over s < log2(V) of bit_s(L) * (V >> (s + 1)).
+template <int V, int STAGE = 0>
+__device__ __forceinline__ void transposed_wave_sum(float (&v)[V], int lane) {
+    if constexpr (STAGE < 6) {
+        if constexpr (V > 1) {
+            constexpr int H = V / 2;
+            const bool upper = (lane >> STAGE) & 1;
+            float next[H];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int row = row_base + (pass + u) * a.rows_parallel + row_phase;
-            row = row < a.rows ? row : a.rows - 1;
-            const uint8_t *row_ptr = a.packed + static_cast<size_t>(row) * row_bytes;
-#pragma unroll
-            for (int c = 0; c < C; ++c) {
-                if (chunk_active[c]) {
-                    const int chunk = lane_in_row + c * a.seg_lanes;
-                    load_codes<BITS>(codes[u][c], row_ptr + static_cast<size_t>(chunk) * (4 * BITS));
-                } else {
-#pragma unroll
-                    for (int i = 0; i < BITS; ++i) codes[u][c].w[i] = 0u;
-                }
+            for (int j = 0; j < H; ++j) {
+                const float keep = upper ? v[j + H] : v[j];
+                const float send = upper ? v[j] : v[j + H];
+                next[j] = keep + lane_exchange<STAGE>(send, lane);
             }
+            transposed_wave_sum<H, STAGE + 1>(next, lane);
+            v[0] = next[0];
+        } else {
+            v[0] += lane_exchange<STAGE>(v[0], lane);
+            transposed_wave_sum<1, STAGE + 1>(v, lane);
         }
     }
-};
+}
 
+template <int V>
+__device__ __forceinline__ int transposed_value_of_lane(int lane) {
+    int value = 0;
+#pragma unroll
+    for (int s = 0; (V >> (s + 1)) > 0; ++s) value += ((lane >> s) & 1) * (V >> (s + 1));
+    return value;
+}
+
+// Sum over aligned groups of 32 lanes by DPP adds; valid in the LAST lane of each group
+// (for `lanes` < 32, a power of two: in the last lane of each group of `lanes`).
+__device__ __forceinline__ float dpp_group_sum(float v, int lanes) {
+#define MK_DPP_ADD(ctrl, row_mask)                                                               \
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, \
+                                                               row_mask, 0xf, true))
+    if (lanes >= 2) MK_DPP_ADD(0xB1, 0xf);    // quad_perm [1,0,3,2]
+    if (lanes >= 4) MK_DPP_ADD(0x4E, 0xf);    // quad_perm [2,3,0,1]
+    if (lanes >= 8) MK_DPP_ADD(0x141, 0xf);   // row_half_mirror
+    if (lanes >= 16) MK_DPP_ADD(0x140, 0xf);  // row_mirror
+    if (lanes >= 32) MK_DPP_ADD(0x142, 0xa);  // row_bcast:15 into rows 1 and 3
+#undef MK_DPP_ADD
+    return v;
+}
+
+// One workgroup multiplies a tile of rows_parallel * kThreadRows adjacent rows.  The grid
+// covers whole tiles only (rows left over go to the word kernel), so a row's address is a
+// uniform base plus a per-lane constant and the streaming part has no branches at all.
+//
+// Timeline of a wavefront: align with the workgroup; request activations, scales and the
+// first rows_ahead() rows of codes; then, for each group of rows: wait for a row,
+// accumulate its unscaled dot products, request the row rows_ahead() further on; apply
+// the scales and put the per-lane sums in LDS.  After a barrier a few threads add up the
+// lanes of each row and store the outputs while the other wavefronts are already summing
+// the next rows.  Only the last group's sums are not hidden behind the stream.
 template <int BITS, int XT, int MT, int C, bool UNIFORM>
-__global__ void packed_matvec_kernel(const MatvecArgs a) {
+__global__ void __launch_bounds__(512) packed_matvec_kernel(const MatvecArgs a) {
     extern __shared__ float lds[];
-    using Batch = RowBatch<BITS, XT, MT, C, UNIFORM>;
-    constexpr int U = Batch::U;
+    constexpr int kRows = kThreadRows;
+    constexpr int kGroupRows = group_rows<MT>();
+    constexpr int kGroups = kRows / kGroupRows;
+    constexpr int kSums = kGroupRows * MT;  // row sums per thread and group
+    constexpr int kAhead = rows_ahead<BITS, C>();
     constexpr bool kNibblePairs = (BITS == 4 && XT == MK_F16 && UNIFORM);
 
     const int tid = threadIdx.x;
     const int threads = blockDim.x;
-    const int lane_in_row = tid % a.seg_lanes;
-    const int row_phase = tid / a.seg_lanes;
-    const int tile_rows = a.rows_parallel * a.rows_per_thread;
+    const int seg = a.seg_lanes;
+    const int row_phase = a.rows_parallel == 1 ? 0 : tid / seg;
+    const int lane_in_row = a.rows_parallel == 1 ? tid : tid - row_phase * seg;
+    const int tile_rows = a.rows_parallel * kRows;
     const int row_base = blockIdx.x * tile_rows;
     const int sample_base = blockIdx.y * MT;
     const bool has_zero = a.zeros != nullptr;
-    const int waves_per_row = a.seg_lanes > 64 ? a.seg_lanes / 64 : 1;
+    const uint32_t row_bytes = static_cast<uint32_t>(a.chunks_per_row) * (4 * BITS);
+    const uint8_t *tile_codes = a.packed + static_cast<size_t>(row_base) * row_bytes;
+    const uint32_t pass_stride = static_cast<uint32_t>(a.rows_parallel) * row_bytes;
 
+    // Lanes past the end of a row read chunk 0 and multiply it by zero activations.
     bool chunk_active[C];
-    int group_of[C];
+    uint32_t lane_offset[C];
+    int slot_of[C];
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-        const int chunk = lane_in_row + c * a.seg_lanes;
+        const int chunk = lane_in_row + c * seg;
         chunk_active[c] = chunk < a.chunks_per_row;
-        group_of[c] = chunk_active[c] ? (chunk * kChunkCodes) / a.group : 0;
+        const int safe_chunk = chunk_active[c] ? chunk : 0;
+        lane_offset[c] = static_cast<uint32_t>(row_phase) * row_bytes + static_cast<uint32_t>(safe_chunk) * (4 * BITS);
+        slot_of[c] = row_phase * a.groups + (safe_chunk * kChunkCodes) / a.group;
     }
 
-    // The code stream depends on nothing: its first loads go out before anything else.
-    Batch even, odd;
-    even.load(a, 0, row_base, row_phase, lane_in_row, chunk_active);
-
-    // LDS: [value table][scale tile][zero tile][cross-wave partial sums]
+    // LDS: [value table][scale tile][zero tile][bias tile][two buffers of per-lane row
+    // sums, sums[value][thread]]; the tiles are padded so staging needs no bounds checks.
+    constexpr int kStaged = 4;
+    const int slot_count = tile_rows * a.groups;
+    const int tile_slots = slot_count > kStaged * threads ? slot_count : kStaged * threads;
     float *table = lds;
     float *scale_tile = table + (UNIFORM ? 0 : kMaxTableEntries);
-    float *zero_tile = scale_tile + tile_rows * a.groups;
-    float *partials = zero_tile + (has_zero ? tile_rows * a.groups : 0);
+    float *zero_tile = scale_tile + tile_slots;
+    float *bias_tile = zero_tile + tile_slots;  // [max(tile_rows, threads)]
+    float *lane_sums = bias_tile + (tile_rows > threads ? tile_rows : threads);
 
-    if constexpr (!UNIFORM) {
-        for (int i = tid; i < kMaxTableEntries; i += threads)
-            table[i] = i < a.n_values ? a.values[i] : 0.0f;
-    }
-    {
-        const size_t first = static_cast<size_t>(row_base) * a.groups;
-        const size_t last = static_cast<size_t>(a.rows) * a.groups - 1;
-        const int count = tile_rows * a.groups;
-        for (int i = tid; i < count; i += threads) {
-            size_t index = first + i;
-            index = index > last ? last : index;
-            scale_tile[i] = mk_load_as_float(a.scales, index, a.scale_dtype);
-            if (has_zero) zero_tile[i] = mk_load_as_float(a.zeros, index, a.scale_dtype);
-        }
-    }
+    // A compute unit serves its wavefronts' loads first come, first served, and a
+    // wavefront receives its loads in issue order.  So the workgroup is aligned first,
+    // then every wavefront issues its few small loads and only then the code stream.
+    // Everything up to the stream is unconditional straight-line code: a load whose only
+    // use sits in a branch would be moved into that branch, behind the stream.
+    __syncthreads();
 
-    // Activations of this lane's chunks, resident for the whole workgroup.
+    // Activations of this lane's chunks, resident for the whole workgroup (L2 hits).
     XChunk<XT> x[C][MT];
-    float x_sum[C][MT];
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-        const int chunk = lane_in_row + c * a.seg_lanes;
+        const int chunk = lane_in_row + c * seg;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             const int sample = sample_base + m;
-            const bool active = chunk_active[c] && sample < a.samples;
+            const int safe_sample = sample < a.samples ? sample : a.samples - 1;
             load_x_chunk<XT>(x[c][m], a.x,
-                             static_cast<size_t>(sample) * a.width + static_cast<size_t>(chunk) * kChunkCodes,
-                             active, x_sum[c][m]);
-            if constexpr (kNibblePairs) pair_for_nibbles(x[c][m]);
+                             static_cast<size_t>(safe_sample) * a.width +
+                                 static_cast<size_t>(chunk_active[c] ? chunk : 0) * kChunkCodes);
         }
     }
-    __syncthreads();
-
-    auto consume = [&](const Batch &batch, int pass) {
+    // Scales, offsets, bias and table entries (first touch, from HBM): only needed once
+    // the first group of rows is summed, so they queue behind the activations.
+    const int scale_bytes = a.scale_dtype == MK_F32 ? 4 : 2;
+    const size_t first_slot_byte = static_cast<size_t>(a.scale_row_offset + row_base) * a.groups * scale_bytes;
+    const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + first_slot_byte;
+    const uint8_t *zero_base = has_zero ? static_cast<const uint8_t *>(a.zeros) + first_slot_byte : scale_base;
+    MkRaw staged_scale[kStaged], staged_zero[kStaged];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int local_row = (pass + u) * a.rows_parallel + row_phase;
+    for (int j = 0; j < kStaged; ++j) {
+        const int i = tid + j * threads;
+        const uint32_t slot = i < slot_count ? i : 0;
+        staged_scale[j] = load_raw_near(scale_base, slot, a.scale_dtype);
+        staged_zero[j] = load_raw_near(zero_base, slot, a.scale_dtype);
+    }
+    const int bias_dtype = a.bias ? a.bias_dtype : a.scale_dtype;
+    const uint8_t *bias_base =
+        a.bias ? static_cast<const uint8_t *>(a.bias) +
+                     static_cast<size_t>(a.scale_row_offset + row_base) * (bias_dtype == MK_F32 ? 4 : 2)
+               : scale_base;
+    const MkRaw staged_bias = load_raw_near(bias_base, a.bias && tid < tile_rows ? tid : 0, bias_dtype);
+    float staged_table[UNIFORM ? 1 : kStaged];
+    if constexpr (!UNIFORM) {
+#pragma unroll
+        for (int j = 0; j < kStaged; ++j) {
+            const int i = tid + j * threads;
+            staged_table[j] = a.values[i < a.n_values ? i : a.n_values - 1];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // The code stream starts kAhead rows deep; each row summed below requests the next.
+    CodeChunk<BITS> codes[kRows][C];
+    auto issue_row = [&](int r) __attribute__((always_inline)) {
+        const uint8_t *pass_codes = tile_codes + static_cast<size_t>(r) * pass_stride;
+#pragma unroll
+        for (int c = 0; c < C; ++c) load_codes<BITS>(codes[r][c], pass_codes + lane_offset[c]);
+    };
+#pragma unroll
+    for (int r = 0; r < kAhead; ++r) {
+        issue_row(r);
+        __builtin_amdgcn_sched_barrier(0);  // in row order
+    }
+
+    // Per-chunk constants of the affine grid map: sum_k (min + step c_k) x_k
+    //   = step * dot + min * sum(x)   (minus step * the code-free part of dot on the nibble path).
+    float x_sum[C][MT];
+    float grid_term[C][MT];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const uint32_t keep = (chunk_active[c] && sample_base + m < a.samples) ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int i = 0; i < (XT == MK_F32 ? 32 : 16); ++i) x[c][m].r[i] &= keep;
+            x_sum[c][m] = chunk_sum<XT>(x[c][m]);
+            if constexpr (kNibblePairs) {
+                const float code_free = pair_for_nibbles(x[c][m]);
+                grid_term[c][m] = a.grid_min * x_sum[c][m] - a.grid_step * code_free;
+            } else {
+                grid_term[c][m] = a.grid_min * x_sum[c][m];
+            }
+        }
+    }
+    if constexpr (!UNIFORM) {
+        // The table is needed by the stream itself (a short wait: requested before the codes).
+#pragma unroll
+        for (int j = 0; j < kStaged; ++j) {
+            const int i = tid + j * threads;
+            table[i < kMaxTableEntries ? i : kMaxTableEntries - 1] = staged_table[j];
+        }
+        for (int i = tid + kStaged * threads; i < kMaxTableEntries; i += threads)
+            table[i] = a.values[i < a.n_values ? i : a.n_values - 1];
+        __syncthreads();
+    }
+
+    // Who adds up the lanes of a row: `team` consecutive threads per output, each summing
+    // every team-th lane of the row, then a DPP sum inside the team.
+    const int team = seg < 32 ? seg : 32;                    // a power of two
+    const int team_shift = 31 - __builtin_clz(team);
+    const int phase_shift = 31 - __builtin_clz(a.rows_parallel);  // rows_parallel is a power of two
+    const int group_outputs = a.rows_parallel * kSums;  // (row in group, phase, sample)
+    const int pass_slots = a.rows_parallel * a.groups;
+#pragma unroll
+    for (int g = 0; g < kGroups; ++g) {
+        // The stream: unscaled dot products, row by row as the codes arrive.
+        float dots[kGroupRows][C][MT];
+#pragma unroll
+        for (int j = 0; j < kGroupRows; ++j) {
+            const int r = g * kGroupRows + j;
+#pragma unroll
+            for (int c = 0; c < C; ++c) chunk_dot<BITS, XT, MT, UNIFORM>(codes[r][c], x[c], table, dots[j][c]);
+            if (r + kAhead < kRows) issue_row(r + kAhead);
+            // Keeps the rows in arrival order and their temporaries short-lived.
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        if (g == 0) {
+            // Scales, offsets and bias go through LDS as fp32 (they arrived long ago).  The
+            // empty asm pins their first use here, so no wait for them moves above the stream.
+#pragma unroll
+            for (int j = 0; j < kStaged; ++j) {
+                asm volatile("" : "+v"(staged_scale[j].word), "+v"(staged_zero[j].word));
+                const int i = tid + j * threads;
+                scale_tile[i] = mk_raw_to_float(staged_scale[j], a.scale_dtype);
+                zero_tile[i] = has_zero ? mk_raw_to_float(staged_zero[j], a.scale_dtype) : 0.0f;
+            }
+            for (int i = tid + kStaged * threads; i < slot_count; i += threads) {
+                scale_tile[i] = mk_load_as_float(scale_base, i, a.scale_dtype);
+                zero_tile[i] = has_zero ? mk_load_as_float(zero_base, i, a.scale_dtype) : 0.0f;
+            }
+            bias_tile[tid] = a.bias ? mk_raw_to_float(staged_bias, bias_dtype) : 0.0f;
+            for (int i = tid + threads; i < tile_rows; i += threads)
+                bias_tile[i] = a.bias ? mk_load_as_float(bias_base, i, bias_dtype) : 0.0f;
+            __syncthreads();
+        }
+
+        // Scaled per-lane sums into LDS: buffer[(j * MT + m) * threads + tid].
+        float *buffer = lane_sums + (g & 1) * (kSums * threads);
+#pragma unroll
+        for (int j = 0; j < kGroupRows; ++j) {
+            const int r = g * kGroupRows + j;
             float acc[MT];
 #pragma unroll
             for (int m = 0; m < MT; ++m) acc[m] = 0.0f;
 #pragma unroll
             for (int c = 0; c < C; ++c) {
-                if (chunk_active[c]) {
-                    float dot[MT];
-                    chunk_dot<BITS, XT, MT, UNIFORM>(batch.codes[u][c], x[c], table, dot);
-                    const int slot = local_row * a.groups + group_of[c];
-                    const float scale = scale_tile[slot];
-                    const float zero = has_zero ? zero_tile[slot] : 0.0f;
+                const float scale = scale_tile[r * pass_slots + slot_of[c]];
+                const float zero = zero_tile[r * pass_slots + slot_of[c]];
 #pragma unroll
-                    for (int m = 0; m < MT; ++m) {
-                        float value = dot[m];
-                        if constexpr (UNIFORM)
-                            value = __builtin_fmaf(a.grid_step, value, a.grid_min * x_sum[c][m]);
-                        acc[m] = __builtin_fmaf(scale, value, acc[m]);
-                        acc[m] = __builtin_fmaf(zero, x_sum[c][m], acc[m]);
-                    }
+                for (int m = 0; m < MT; ++m) {
+                    float value = dots[j][c][m];
+                    if constexpr (UNIFORM) value = __builtin_fmaf(a.grid_step, value, grid_term[c][m]);
+                    acc[m] = __builtin_fmaf(scale, value, acc[m]);
+                    acc[m] = __builtin_fmaf(zero, x_sum[c][m], acc[m]);
                 }
             }
-            // Meet the lanes of this row inside the wavefront.
 #pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                float total = acc[m];
-                if (a.seg_lanes >= 64) total = mk_segment_sum<64>(total);
-                else if (a.seg_lanes == 32) total = mk_segment_sum<32>(total);
-                else if (a.seg_lanes == 16) total = mk_segment_sum<16>(total);
-                else if (a.seg_lanes == 8) total = mk_segment_sum<8>(total);
-                else if (a.seg_lanes == 4) total = mk_segment_sum<4>(total);
-                else if (a.seg_lanes == 2) total = mk_segment_sum<2>(total);
-                acc[m] = total;
-            }
-            const int row = row_base + local_row;
-            if (waves_per_row == 1) {
-                if (lane_in_row == 0 && row < a.rows) {
-#pragma unroll
-                    for (int m = 0; m < MT; ++m) {
-                        const int sample = sample_base + m;
-                        if (sample < a.samples) {
-                            float result = acc[m];
-                            if (a.bias) result += mk_load_as_float(a.bias, row, a.bias_dtype);
-                            mk_store_from_float(a.y, static_cast<size_t>(sample) * a.rows + row, XT, result);
-                        }
-                    }
-                }
-            } else if ((lane_in_row & 63) == 0) {
-                const int wave_in_row = lane_in_row >> 6;
-#pragma unroll
-                for (int m = 0; m < MT; ++m)
-                    partials[(local_row * MT + m) * waves_per_row + wave_in_row] = acc[m];
-            }
+            for (int m = 0; m < MT; ++m) buffer[(j * MT + m) * threads + tid] = acc[m];
         }
-    };
-
-    // Two register batches alternate: the next rows are in flight while these are summed.
-    for (int pass = 0; pass < a.rows_per_thread; pass += 2 * U) {
-        const bool more = pass + U < a.rows_per_thread;
-        if (more) odd.load(a, pass + U, row_base, row_phase, lane_in_row, chunk_active);
-        consume(even, pass);
-        if (more) {
-            if (pass + 2 * U < a.rows_per_thread)
-                even.load(a, pass + 2 * U, row_base, row_phase, lane_in_row, chunk_active);
-            consume(odd, pass + U);
-        }
-    }
-
-    if (waves_per_row > 1) {
+        // After this barrier the group's sums are complete; the buffer is written again
+        // two groups later, behind the next barrier, so its readers below are done by then.
         __syncthreads();
-        for (int i = tid; i < tile_rows * MT; i += threads) {
-            const int local = i / MT, m = i % MT;
-            const int row = row_base + local, sample = sample_base + m;
-            if (row < a.rows && sample < a.samples) {
-                float result = 0.0f;
-                for (int w = 0; w < waves_per_row; ++w) result += partials[i * waves_per_row + w];
-                if (a.bias) result += mk_load_as_float(a.bias, row, a.bias_dtype);
-                mk_store_from_float(a.y, static_cast<size_t>(sample) * a.rows + row, XT, result);
+
+        // Output o = (j * MT + m) * rows_parallel + phase: its lanes are threads
+        // phase * seg .. phase * seg + seg - 1 of value (j * MT + m).
+        for (int t = tid; t < group_outputs * team; t += threads) {
+            const int output = t >> team_shift, part = t & (team - 1);
+            const int value = output >> phase_shift, phase = output & (a.rows_parallel - 1);
+            const float *in = buffer + value * threads + phase * seg;
+            float total = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {  // seg <= 512 = 16 * 32
+                const int lane_k = part + k * team;
+                const float term = in[lane_k < seg ? lane_k : seg - 1];
+                total += lane_k < seg ? term : 0.0f;
+            }
+            total = dpp_group_sum(total, team);
+            if (part == team - 1) {
+                const int j = value / MT, m = value - j * MT;
+                const int local = (g * kGroupRows + j) * a.rows_parallel + phase;
+                const int sample = sample_base + m;
+                if (sample < a.samples)
+                    mk_store_from_float(a.y, static_cast<size_t>(sample) * a.rows + row_base + local, XT,
+                                        total + bias_tile[local]);
             }
         }
     }
@@ -433,10 +629,9 @@ bool dispatch_tile(const MatvecArgs &a, const Plan &p, hipStream_t stream) {
         launch_chunked<BITS, XT, MT_, C_, UNIFORM>(a, p, stream);     \
         return true;                                                  \
     }
-    MK_CASE(1, 1) MK_CASE(1, 2) MK_CASE(1, 4) MK_CASE(1, 8)
-    MK_CASE(2, 1) MK_CASE(2, 2) MK_CASE(2, 4)
-    MK_CASE(4, 1) MK_CASE(4, 2)
-    if constexpr (XT != MK_F32) { MK_CASE(8, 1) }
+    MK_CASE(1, 1) MK_CASE(2, 1) MK_CASE(4, 1)
+    MK_CASE(1, 2) MK_CASE(2, 2)
+    if constexpr (XT != MK_F32) { MK_CASE(8, 1) MK_CASE(4, 2) }
 #undef MK_CASE
     return false;
 }

@@ -6,13 +6,17 @@ or raises.  Build it with ``python -m mlkit_amd.build`` (hipcc, gfx950).
 """
 
 import ctypes
+import os
 import pathlib
 from typing import Any
 
 import torch
 from torch import Tensor
 
-LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "libmlkit_amd.so"
+# MLKIT_AMD_LIBRARY selects another build of the same library (e.g. a profiling build).
+LIBRARY_PATH = pathlib.Path(
+    os.environ.get("MLKIT_AMD_LIBRARY") or pathlib.Path(__file__).resolve().parent / "libmlkit_amd.so"
+)
 
 MK_F32, MK_F16, MK_BF16 = 0, 1, 2
 DTYPE_CODES = {torch.float32: MK_F32, torch.float16: MK_F16, torch.bfloat16: MK_BF16}
