@@ -24,8 +24,8 @@ SCALE_BYTES = ROWS * (WIDTH // GROUP) * 2
 WEIGHT_BYTES = CODE_BYTES + SCALE_BYTES
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
-# profiles/); None until such a run has been recorded for the current kernel.
-MEASURED_TRAFFIC_BYTES = None
+# profiles/packed_matvec_stream4_int4_g128_4096x14336_m1.md), M=1.
+MEASURED_TRAFFIC_BYTES = 30_635_000
 
 
 def algorithmic_bytes(samples: int) -> int:
@@ -148,6 +148,9 @@ def main() -> None:
     parser.add_argument("--copies", type=int, default=18)
     parser.add_argument("--no-graph", action="store_true")
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--profile-launches", type=int, default=0,
+                        help="for rocprofv3: only launch the M=1 matvec this many times, plus three "
+                             "256 MiB device copies whose counters calibrate FETCH_SIZE / WRITE_SIZE")
     options = parser.parse_args()
     if options.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -158,6 +161,20 @@ def main() -> None:
     values = torch.arange(-8, 8, dtype=torch.float32, device=device)
     copies = make_copies(options.copies, device)
     generator = torch.Generator(device=device).manual_seed(5)
+
+    if options.profile_launches:
+        x = torch.randn((1, WIDTH), device=device, generator=generator).half()
+        y = torch.empty((1, ROWS), device=device, dtype=torch.float16)
+        launchers = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
+        raw = torch.cuda.current_stream().cuda_stream
+        for step in range(options.profile_launches):
+            launchers[step % len(launchers)](raw)
+        source = torch.empty(256 * 2**20, dtype=torch.uint8, device=device)
+        target = torch.empty_like(source)
+        for _ in range(3):
+            target.copy_(source)
+        torch.cuda.synchronize()
+        return
 
     results = {}
     for samples in (1, 2, 4, 8):
