@@ -68,6 +68,109 @@ int mk_packed_decode(const uint8_t *packed, const void *scales, int scale_dtype,
                      int out_dtype, int output_width, int input_width, int group, int bits,
                      int uniform, float grid_min, float grid_step, void *stream);
 
+/* Scale storage formats of the scalar codec (formats/scale_storage.py:11-26). */
+#define MK_SCALE_FP32 0
+#define MK_SCALE_FP16 1
+#define MK_SCALE_BF16 2
+#define MK_SCALE_FP8 3  /* e4m3 */
+#define MK_SCALE_E8M0 4 /* power of two */
+
+/* codes[r, c] = code of the grid value nearest to (value[r, c] - zeros[r, c/group]) / scales[r, c/group]
+ * (IEEE division).  integer != 0: round half to even, clamp to [minimum, maximum], subtract
+ * minimum; otherwise the nearest entry of the ascending table `values`, ties to the lower
+ * index.  value [rows, width] fp32; scales, zeros (NULL or) [rows, groups_per_row] fp32;
+ * codes [rows, width] uint8.
+ * Replaces: kernels/scalar_encode.py:110-146 (encode). */
+int mk_scalar_encode(const float *value, const float *scales, const float *zeros, const float *values,
+                     int n_values, uint8_t *codes, int rows, int width, int group, int groups_per_row,
+                     int integer, float minimum, float maximum, void *stream);
+
+/* out[r, c] = values[codes[r, c]] * scales[r, s(c)] (+ zeros[r, s(c)]), multiply and add
+ * separately rounded.  refit == 0: s(c) = c / group; refit > 0 (error-feedback codec):
+ * s(c) = (c / refit) * ceil(refit / group) + (c % refit) / group.
+ * Replaces: kernels/scalar_decode.py:70-97 (decode) and the scale indexing of
+ * quantization/codecs/scaled.py:67-101 (decode_feedback). */
+int mk_scalar_decode(const uint8_t *codes, const float *scales, const float *values, int n_values,
+                     const float *zeros, float *out, int rows, int width, int group, int groups_per_row,
+                     int refit, void *stream);
+
+/* selected[r, g] = the candidate among scales[r, g] and store(scales[r, g] * fractions[i]),
+ * i ascending, with the least squared rounding error over the group; a later candidate
+ * wins only if strictly better.  `scale_format` is one of MK_SCALE_*.  Per-group errors
+ * are summed by P = min(64, largest power of two dividing group) strided partial sums
+ * folded by halving.
+ * Replaces: kernels/scalar_encode.py:261-304 (search_scales). */
+int mk_search_scales(const float *value, const float *scales, const float *zeros, const float *values,
+                     int n_values, const float *fractions, int n_fractions, float *selected, int rows,
+                     int width, int group, int groups_per_row, int scale_format, int integer,
+                     float minimum, float maximum, void *stream);
+
+/* out[i] = nearest entry of the ascending table `values` to value[i] (ties to the lower entry).
+ * Replaces: kernels/scalar_encode.py:327-345 (snap). */
+int mk_snap(const float *value, const float *values, int n_values, float *out, long long count,
+            void *stream);
+
+/* Per-group scales (and offsets) from each group's range, over columns [0, span) of rows
+ * that lie row_stride elements apart:
+ *   symmetric:  scale = max(max, -min, 1e-12) * reciprocal
+ *   asymmetric: scale = max(max - min, 1e-12) * reciprocal, zero = min - value_minimum * scale
+ * scales are rounded to `scale_format`; zeros are stored raw, or with store_zero != 0 as the
+ * rounded magnitude carrying the sign.  A group holding a non-finite value yields NaN.
+ * scales, zeros: [rows, ceil(span / group)] fp32.
+ * Replaces: the tensor reductions of formats/grouped_scaling.py:30-43,274-289
+ * (group_extrema, Scaled._initial_scales) and the storage rounding of :160-175. */
+int mk_fit_scales(const float *value, long long row_stride, float *scales, float *zeros, int rows,
+                  int span, int group, int asym, float reciprocal, float value_minimum,
+                  int scale_format, int store_zero, void *stream);
+
+/* Walsh-Hadamard transform of `rows` rows of `width` = 2^S values: radix-2 butterflies in
+ * ascending stride in fp32, then one multiplication by `scale`.  Input and output may be
+ * fp32, fp16 or bf16 and may alias.  signs_before / signs_after (NULL or fp32 vectors of
+ * +-1 with `sign_period` entries, a multiple of width) multiply the input / the output;
+ * element (r, i) uses sign (r * width + i) mod sign_period, which lets a tensor of wider
+ * rows be transformed block by block.
+ * Replaces: kernels/hadamard.py:108-136 (transform). */
+int mk_fwht(const void *source, int source_dtype, void *target, int target_dtype, long long rows,
+            int width, const float *signs_before, const float *signs_after, int sign_period,
+            float scale, void *stream);
+
+/* target[r, f', p] = sum_f mix[f', f] * source[r, f, p] for fp32 tensors [rows, order, power];
+ * mix = basis (transpose == 0) or its transpose; signs_after (NULL or [order * power])
+ * multiplies the result.  order <= 256.  source and target must not alias.
+ * Replaces: the basis product of quantization/operations/orthogonal_transforms.py:101-109
+ * (structured_transform). */
+int mk_basis_mix(const float *source, float *target, const float *basis, long long rows, int order,
+                 int power, int transpose, const float *signs_after, void *stream);
+
+/* Error-feedback sweep over columns [tile_start, tile_start + tile_width) of every row:
+ * target = original + correction; the nearest grid value (as in mk_scalar_encode, with the
+ * table's nearest entry taken as the lowest index of the least distance) times scale plus
+ * zero is written to output, its code to encoded, and (original - reconstruction) times
+ * coeff[column, later columns of the tile] is added to the later corrections, which start
+ * from feedback[:, tile].  scales / zeros: [rows, groups_per_row] of the region starting at
+ * column region_start.  tile_width <= 1024.
+ * Replaces: kernels/error_feedback.py:99-143 (round_tile). */
+int mk_feedback_round_tile(const float *original, const float *feedback, const float *coeff,
+                           const float *scales, const float *zeros, const float *values, int n_values,
+                           float *output, uint8_t *encoded, int rows, int width, int region_start,
+                           int tile_start, int tile_width, int group, int groups_per_row,
+                           int integer_grid, float code_min, float code_max, void *stream);
+
+/* out[rows, stop - start] = feedback[:, start:stop] * U^-1 (+ original[:, start:stop] when
+ * original is not NULL), U = coeff[start:stop, start:stop] unit upper triangular, by
+ * right-looking substitution (x[c] -= x[j] * U[j, c], j ascending).  stop - start <= 1024.
+ * Replaces: quantization/algorithms/error_feedback.py:373-393 (_pending_continuation). */
+int mk_feedback_pending(const float *feedback, const float *coeff, const float *original, float *out,
+                        int rows, int width, int region_start, int region_stop, void *stream);
+
+/* feedback[:, tile_stop:] += (original - output)[:, tile_start:tile_stop] @ coeff[tile_start:tile_stop, tile_stop:]
+ * on the fp32 matrix cores; each product sum starts at zero, accumulates over ascending k
+ * and is added to feedback once.
+ * Replaces: the addmm_ of quantization/algorithms/error_feedback.py:366-370. */
+int mk_feedback_block_update(float *feedback, const float *original, const float *output,
+                             const float *coeff, int rows, int width, int tile_start, int tile_stop,
+                             void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,359 @@
+// LDL-form error feedback (GPTQ / LDLQ) on gfx950: the sequential column sweep of a tile,
+// the triangular solve that predicts a region's targets, and the trailing block update.
+//
+// Sweep and solve.  One wavefront owns one weight row; lane l keeps columns l, l + 64, ...
+// of the tile in registers.  Step j takes one value from the lane that owns column j
+// (v_readlane) and every lane adds its multiple of coefficient row j to its columns.
+// Each column therefore receives exactly the sequence of separately rounded multiplies
+// and adds that a scalar loop over j gives it.  Coefficient rows reach the wavefronts of
+// a workgroup through LDS, a chunk of rows at a time, with the next chunk's global loads
+// in flight while the current one is used; entries at or left of the diagonal are stored
+// as zero, which makes the update of finished columns a no-op.
+//
+// Trailing update.  feedback[:, stop:] += (original - output)[:, tile] @ coeff[tile, stop:]
+// runs on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).  Each product sum starts from
+// zero and accumulates over ascending k, which on this hardware equals a chain of fused
+// multiply-adds in the same order; the sum is then added to feedback once.
+//
+// Replaces, in /root/reference/src/mlkit:
+//   kernels/error_feedback.py:22-143                    round_feedback_tile / round_tile
+//   quantization/algorithms/error_feedback.py:373-393   _pending_continuation (solve_triangular)
+//   quantization/algorithms/error_feedback.py:366-370   trailing addmm_
+
+#include "mk_common.h"
+
+namespace {
+
+constexpr int kSweepThreads = 256;  // four wavefronts = four rows
+constexpr int kModeInteger = 0, kModeCodebook = 1, kModeSolve = 2;
+
+struct SweepArgs {
+    const float *original;
+    const float *feedback;
+    const float *coeff;
+    const float *scales;
+    const float *zeros;
+    const float *values;
+    float *output;     // reconstruction [rows, width]; solve: [rows, span]
+    uint8_t *encoded;  // [rows, width]
+    int rows, width;
+    int region_start, tile_start, tile_width;
+    int group, groups_per_row, n_values;
+    float code_min, code_max;
+};
+
+template <int S>
+struct SweepShape {
+    static constexpr int kWidth = 64 * S;                      // padded tile width
+    static constexpr int kChunk = S <= 4 ? 16 : 4;             // coefficient rows per LDS chunk
+    static constexpr int kPerThread = kChunk * kWidth / kSweepThreads;
+};
+
+template <int S>
+__device__ __forceinline__ void fetch_chunk(const SweepArgs &a, int first, float (&held)[SweepShape<S>::kPerThread]) {
+    using Shape = SweepShape<S>;
+#pragma unroll
+    for (int p = 0; p < Shape::kPerThread; ++p) {
+        const int flat = p * kSweepThreads + threadIdx.x;
+        const int j = first + flat / Shape::kWidth;
+        const int c = flat % Shape::kWidth;
+        const bool wanted = j < a.tile_width && c > j && c < a.tile_width;
+        const size_t index = static_cast<size_t>(a.tile_start + (wanted ? j : 0)) * a.width + a.tile_start + (wanted ? c : 0);
+        const float loaded = a.coeff[index];
+        held[p] = wanted ? loaded : 0.0f;
+    }
+}
+
+template <int S>
+__device__ __forceinline__ void keep_chunk(float *buffer, const float (&held)[SweepShape<S>::kPerThread]) {
+#pragma unroll
+    for (int p = 0; p < SweepShape<S>::kPerThread; ++p) buffer[p * kSweepThreads + threadIdx.x] = held[p];
+}
+
+__device__ __forceinline__ float lane_value(float value, int lane) {
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(value), lane));
+}
+
+// Smallest (distance, index) over the table for one wavefront-uniform x: lane e scans
+// entries e, e + 64, ...; keys order by distance first, then by index.
+__device__ __forceinline__ int nearest_by_scan(float x, const float *table, int count, int lane) {
+    unsigned long long best = ~0ull;
+    for (int e = lane; e < count; e += 64) {
+        const float distance = fabsf(__fsub_rn(x, table[e]));
+        const unsigned long long key = (static_cast<unsigned long long>(__float_as_uint(distance)) << 32) | static_cast<unsigned>(e);
+        best = key < best ? key : best;
+    }
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+        const unsigned long long other = __shfl_xor(best, offset, 64);
+        best = other < best ? other : best;
+    }
+    const int index = static_cast<int>(best & 0xffffffffu);
+    return index < count ? index : count - 1;
+}
+
+template <int S, int MODE>
+__global__ void __launch_bounds__(kSweepThreads) sweep_kernel(const SweepArgs a) {
+    using Shape = SweepShape<S>;
+    __shared__ float chunks[2][Shape::kChunk * Shape::kWidth];
+    __shared__ float table[MODE == kModeCodebook ? 256 : 1];
+    const int lane = threadIdx.x & 63;
+    const int wanted_row = blockIdx.x * (kSweepThreads / 64) + (threadIdx.x >> 6);
+    const bool active = wanted_row < a.rows;
+    const int row = active ? wanted_row : a.rows - 1;
+    const size_t row_base = static_cast<size_t>(row) * a.width;
+
+    if constexpr (MODE == kModeCodebook)
+        for (int i = threadIdx.x; i < a.n_values; i += kSweepThreads) table[i] = a.values[i];
+
+    float held[Shape::kPerThread];
+    fetch_chunk<S>(a, 0, held);
+
+    // This lane's columns: weight, running correction, and the scale and offset of each.
+    float weight[S], running[S], scale[S], zero[S], finished[S];
+    uint32_t code[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const int c = 64 * s + lane;
+        const bool inside = c < a.tile_width;
+        const int position = a.tile_start + (inside ? c : 0);
+        running[s] = inside ? a.feedback[row_base + position] : 0.0f;
+        weight[s] = 0.0f; scale[s] = 1.0f; zero[s] = 0.0f; finished[s] = 0.0f; code[s] = 0;
+        if constexpr (MODE != kModeSolve) {
+            weight[s] = inside ? a.original[row_base + position] : 0.0f;
+            const int slot = row * a.groups_per_row + (position - a.region_start) / a.group;
+            scale[s] = inside ? a.scales[slot] : 1.0f;
+            if (a.zeros) zero[s] = inside ? a.zeros[slot] : 0.0f;
+        }
+    }
+    keep_chunk<S>(chunks[0], held);
+    __syncthreads();
+
+    int chunk_index = 0;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        for (int first = 64 * s; first < 64 * (s + 1) && first < a.tile_width; first += Shape::kChunk) {
+            const bool more = first + Shape::kChunk < a.tile_width;
+            if (more) fetch_chunk<S>(a, first + Shape::kChunk, held);
+            const float *rows_of_chunk = chunks[chunk_index & 1];
+            for (int i = 0; i < Shape::kChunk; ++i) {
+                const int j = first + i;
+                if (j >= a.tile_width) break;
+                const int owner = j & 63;
+                float pushed;
+                if constexpr (MODE == kModeSolve) {
+                    pushed = -lane_value(running[s], owner);
+                } else {
+                    const float target = __fadd_rn(weight[s], running[s]);
+                    const float normalized = __fdiv_rn(__fsub_rn(target, zero[s]), scale[s]);
+                    float chosen;
+                    uint32_t index;
+                    if constexpr (MODE == kModeInteger) {
+                        chosen = fminf(fmaxf(rintf(normalized), a.code_min), a.code_max);
+                        index = static_cast<uint32_t>(static_cast<int>(__fsub_rn(chosen, a.code_min)));
+                    } else {
+                        index = nearest_by_scan(lane_value(normalized, owner), table, a.n_values, lane);
+                        chosen = table[index];
+                    }
+                    const float reconstruction = __fadd_rn(__fmul_rn(chosen, scale[s]), zero[s]);
+                    const bool mine = lane == owner;
+                    finished[s] = mine ? reconstruction : finished[s];
+                    code[s] = mine ? index : code[s];
+                    pushed = lane_value(__fsub_rn(weight[s], reconstruction), owner);
+                }
+                const float *coefficient_row = rows_of_chunk + i * Shape::kWidth + lane;
+#pragma unroll
+                for (int later = s; later < S; ++later)
+                    running[later] = __fadd_rn(running[later], __fmul_rn(pushed, coefficient_row[64 * later]));
+            }
+            if (more) keep_chunk<S>(chunks[(chunk_index + 1) & 1], held);
+            __syncthreads();
+            ++chunk_index;
+        }
+    }
+
+    if (!active) return;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const int c = 64 * s + lane;
+        if (c >= a.tile_width) continue;
+        if constexpr (MODE == kModeSolve) {
+            // a.output is [rows, tile_width]; with `original` given the solved adjustment is
+            // added to the region's weights (the targets a region's scales are fitted to).
+            float value = running[s];
+            if (a.original) value = __fadd_rn(a.original[row_base + a.tile_start + c], value);
+            a.output[static_cast<size_t>(row) * a.tile_width + c] = value;
+        } else {
+            a.output[row_base + a.tile_start + c] = finished[s];
+            a.encoded[row_base + a.tile_start + c] = static_cast<uint8_t>(code[s]);
+        }
+    }
+}
+
+template <int MODE>
+int launch_sweep(const SweepArgs &a, hipStream_t stream) {
+    const dim3 grid(mk_cdiv(a.rows, kSweepThreads / 64)), block(kSweepThreads);
+    if (a.tile_width <= 128)
+        hipLaunchKernelGGL((sweep_kernel<2, MODE>), grid, block, 0, stream, a);
+    else if (a.tile_width <= 256)
+        hipLaunchKernelGGL((sweep_kernel<4, MODE>), grid, block, 0, stream, a);
+    else
+        hipLaunchKernelGGL((sweep_kernel<16, MODE>), grid, block, 0, stream, a);
+    return MK_OK;
+}
+
+// ---- trailing block update on the fp32 matrix cores ------------------------------------
+
+typedef float mk_f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kTileRows = 128, kTileColumns = 128, kDepthChunk = 32, kUpdateThreads = 256;
+
+struct UpdateArgs {
+    float *feedback;
+    const float *original;
+    const float *output;
+    const float *coeff;
+    int rows, width, tile_start, tile_stop;
+};
+
+__global__ void __launch_bounds__(kUpdateThreads) block_update_kernel(const UpdateArgs a) {
+    __shared__ float deviation_t[kDepthChunk][kTileRows + 1];  // [k][row]
+    __shared__ float coefficient[kDepthChunk][kTileColumns];   // [k][column]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int row0 = blockIdx.y * kTileRows;
+    const int column0 = a.tile_stop + blockIdx.x * kTileColumns;
+    const int wave_row = (wave >> 1) * 64, wave_column = (wave & 1) * 64;
+    const int depth = a.tile_stop - a.tile_start;
+
+    mk_f32x16 sums[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sums[mi][ni][r] = 0.0f;
+
+    for (int k0 = 0; k0 < depth; k0 += kDepthChunk) {
+#pragma unroll
+        for (int p = 0; p < kTileRows * kDepthChunk / kUpdateThreads; ++p) {
+            const int flat = p * kUpdateThreads + threadIdx.x;
+            const int r = flat / kDepthChunk, k = flat % kDepthChunk;
+            const bool wanted = row0 + r < a.rows && k0 + k < depth;
+            const size_t index = static_cast<size_t>(wanted ? row0 + r : 0) * a.width + a.tile_start + (wanted ? k0 + k : 0);
+            const float difference = __fsub_rn(a.original[index], a.output[index]);
+            deviation_t[k][r] = wanted ? difference : 0.0f;
+        }
+#pragma unroll
+        for (int p = 0; p < kDepthChunk * kTileColumns / kUpdateThreads; ++p) {
+            const int flat = p * kUpdateThreads + threadIdx.x;
+            const int k = flat / kTileColumns, c = flat % kTileColumns;
+            const bool wanted = column0 + c < a.width && k0 + k < depth;
+            const size_t index = static_cast<size_t>(a.tile_start + (wanted ? k0 + k : 0)) * a.width + (wanted ? column0 + c : 0);
+            const float loaded = a.coeff[index];
+            coefficient[k][c] = wanted ? loaded : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < kDepthChunk; kk += 2) {
+            const int k = kk + (lane >> 5);
+            float left[2], right[2];
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi) left[mi] = deviation_t[k][wave_row + mi * 32 + (lane & 31)];
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) right[ni] = coefficient[k][wave_column + ni * 32 + (lane & 31)];
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    sums[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(left[mi], right[ni], sums[mi][ni], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = row0 + wave_row + mi * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                const int column = column0 + wave_column + ni * 32 + (lane & 31);
+                if (row < a.rows && column < a.width) {
+                    const size_t index = static_cast<size_t>(row) * a.width + column;
+                    a.feedback[index] = __fadd_rn(a.feedback[index], sums[mi][ni][r]);
+                }
+            }
+}
+
+int check_tile(const char *name, int rows, int width, int tile_start, int tile_width) {
+    MK_REQUIRE(rows >= 1 && width >= 1, MK_ERR_INVALID, "%s: sizes must be positive", name);
+    MK_REQUIRE(tile_start >= 0 && tile_width >= 1 && tile_start + tile_width <= width, MK_ERR_INVALID,
+               "%s: columns [%d, %d) lie outside a row of %d", name, tile_start, tile_start + tile_width, width);
+    MK_REQUIRE(tile_width <= 1024, MK_ERR_UNSUPPORTED, "%s: at most 1024 columns per call (got %d)", name, tile_width);
+    return MK_OK;
+}
+
+}  // namespace
+
+extern "C" int mk_feedback_round_tile(const float *original, const float *feedback, const float *coeff,
+                                      const float *scales, const float *zeros, const float *values, int n_values,
+                                      float *output, uint8_t *encoded, int rows, int width, int region_start,
+                                      int tile_start, int tile_width, int group, int groups_per_row,
+                                      int integer_grid, float code_min, float code_max, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(original && feedback && coeff && scales && output && encoded, MK_ERR_INVALID,
+               "mk_feedback_round_tile: null tensor pointer");
+    if (int status = check_tile("mk_feedback_round_tile", rows, width, tile_start, tile_width)) return status;
+    MK_REQUIRE(group >= 1 && region_start >= 0 && region_start <= tile_start, MK_ERR_INVALID,
+               "mk_feedback_round_tile: the tile must start inside its region");
+    MK_REQUIRE((tile_start + tile_width - 1 - region_start) / group < groups_per_row, MK_ERR_INVALID,
+               "mk_feedback_round_tile: %d scale groups per row do not reach column %d of the region", groups_per_row,
+               tile_start + tile_width - 1 - region_start);
+    SweepArgs a{};
+    a.original = original; a.feedback = feedback; a.coeff = coeff; a.scales = scales; a.zeros = zeros;
+    a.values = values; a.output = output; a.encoded = encoded; a.rows = rows; a.width = width;
+    a.region_start = region_start; a.tile_start = tile_start; a.tile_width = tile_width; a.group = group;
+    a.groups_per_row = groups_per_row; a.n_values = n_values; a.code_min = code_min; a.code_max = code_max;
+    if (integer_grid) {
+        MK_REQUIRE(code_max >= code_min && code_max - code_min <= 255.0f, MK_ERR_INVALID,
+                   "mk_feedback_round_tile: integer grid must span at most 256 codes");
+        launch_sweep<kModeInteger>(a, stream);
+    } else {
+        MK_REQUIRE(values && n_values >= 1 && n_values <= 256, MK_ERR_INVALID,
+                   "mk_feedback_round_tile: a value table of 1..256 entries is required");
+        launch_sweep<kModeCodebook>(a, stream);
+    }
+    MK_LAUNCH_CHECK("mk_feedback_round_tile");
+    return MK_OK;
+}
+
+extern "C" int mk_feedback_pending(const float *feedback, const float *coeff, const float *original, float *out,
+                                   int rows, int width, int region_start, int region_stop, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(feedback && coeff && out, MK_ERR_INVALID, "mk_feedback_pending: null tensor pointer");
+    if (int status = check_tile("mk_feedback_pending", rows, width, region_start, region_stop - region_start)) return status;
+    SweepArgs a{};
+    a.original = original; a.feedback = feedback; a.coeff = coeff; a.output = out; a.rows = rows; a.width = width;
+    a.region_start = region_start; a.tile_start = region_start; a.tile_width = region_stop - region_start;
+    a.group = 1; a.groups_per_row = 0;
+    launch_sweep<kModeSolve>(a, stream);
+    MK_LAUNCH_CHECK("mk_feedback_pending");
+    return MK_OK;
+}
+
+extern "C" int mk_feedback_block_update(float *feedback, const float *original, const float *output,
+                                        const float *coeff, int rows, int width, int tile_start, int tile_stop,
+                                        void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(feedback && original && output && coeff, MK_ERR_INVALID, "mk_feedback_block_update: null tensor pointer");
+    MK_REQUIRE(rows >= 1 && width >= 1 && tile_start >= 0 && tile_start < tile_stop && tile_stop <= width,
+               MK_ERR_INVALID, "mk_feedback_block_update: columns [%d, %d) lie outside a row of %d", tile_start, tile_stop, width);
+    if (tile_stop == width) return MK_OK;
+    MK_REQUIRE(mk_cdiv(rows, kTileRows) <= 65535, MK_ERR_UNSUPPORTED, "mk_feedback_block_update: too many rows");
+    UpdateArgs a{feedback, original, output, coeff, rows, width, tile_start, tile_stop};
+    const dim3 grid(mk_cdiv(width - tile_stop, kTileColumns), mk_cdiv(rows, kTileRows));
+    hipLaunchKernelGGL(block_update_kernel, grid, dim3(kUpdateThreads), 0, stream, a);
+    MK_LAUNCH_CHECK("mk_feedback_block_update");
+    return MK_OK;
+}

@@ -1,0 +1,224 @@
+// Fast Walsh-Hadamard transform along rows on gfx950, one launch per tensor.
+//
+// A row of n = 2^S values goes through S radix-2 butterfly stages in ascending stride
+// (1, 2, 4, ...): out[i] = a + b, out[i + stride] = a - b.  Every output of a stage depends
+// on exactly two outputs of the stage before it, so grouping stages (several in registers,
+// exchanges through LDS between groups) changes no bit of the result as long as the stage
+// order is kept.  The last step multiplies by `scale` (fp32(1)/fp32(sqrt n) to normalise).
+//
+// One workgroup owns whole rows: a row is read from HBM once (coalesced, cast to fp32,
+// optionally multiplied by a +-1 sign vector), lives in LDS between stage groups, and is
+// written once (optionally multiplied by the sign vector, cast to the output type).
+// Rows shorter than a workgroup's worth of elements share a workgroup.
+//
+// The blocked transform of a width that is not a power of two (order x power, e.g.
+// 14336 = 28 x 512) runs this kernel on rows * order rows of `power` values and then
+// `mk_basis_mix`, which multiplies the `order` blocks of every row by a dense orthonormal
+// basis.
+//
+// Replaces, in /root/reference/src/mlkit:
+//   kernels/hadamard.py:21-136                            hadamard_pass / transform -> mk_fwht
+//   quantization/operations/orthogonal_transforms.py:101-109  basis product of
+//                                                         structured_transform      -> mk_basis_mix
+
+#include "mk_common.h"
+
+namespace {
+
+constexpr int kMaxThreads = 1024;
+
+struct FwhtArgs {
+    const void *source;
+    void *target;
+    const float *signs_before;  // multiplied into the input, or null
+    const float *signs_after;   // multiplied into the output, or null
+    long long rows;
+    int width, log_width;
+    int source_dtype, target_dtype;
+    int sign_period;  // signs repeat every sign_period elements of the flattened tensor
+    int rows_per_block, threads_per_row;
+    float scale;
+};
+
+__host__ __device__ __forceinline__ int padded(int index) { return index + (index >> 4); }
+
+// E values per thread; stage group `g` covers index bits [base, base + log2 E).
+template <int E>
+__global__ void __launch_bounds__(kMaxThreads) fwht_kernel(const FwhtArgs a) {
+    extern __shared__ float tile[];
+    constexpr int kLogE = E == 1 ? 0 : E == 2 ? 1 : E == 4 ? 2 : E == 8 ? 3 : E == 16 ? 4 : 5;
+    const int threads_per_row = a.threads_per_row;
+    const int local_row = threadIdx.x / threads_per_row;
+    const int t = threadIdx.x - local_row * threads_per_row;
+    const long long row = static_cast<long long>(blockIdx.x) * a.rows_per_block + local_row;
+    const bool active = row < a.rows;
+    float *mine = tile + local_row * padded(a.width);
+    const size_t row_base = static_cast<size_t>(active ? row : 0) * a.width;
+    const int sign_base = a.sign_period ? static_cast<int>(row_base % static_cast<size_t>(a.sign_period)) : 0;
+
+    // HBM -> LDS, consecutive lanes read consecutive elements.
+    if (active) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            const int index = j * threads_per_row + t;
+            float value = mk_load_as_float(a.source, row_base + index, a.source_dtype);
+            if (a.signs_before) value *= a.signs_before[sign_base + index];
+            mine[padded(index)] = value;
+        }
+    }
+    __syncthreads();
+
+    float v[E];
+    int done = 0;
+    while (true) {
+        // This group holds index bits [base, base + kLogE) in registers; the last group is
+        // shifted down to stay inside the row and skips the stages already done.
+        int base = done;
+        if (base + kLogE > a.log_width) base = a.log_width - kLogE;
+        const int low = t & ((1 << base) - 1);
+        const int high = t >> base;
+        const int origin = (high << (base + kLogE)) | low;
+#pragma unroll
+        for (int j = 0; j < E; ++j) v[j] = mine[padded(origin | (j << base))];
+#pragma unroll
+        for (int bit = 0; bit < kLogE; ++bit) {
+            if (base + bit >= done) {
+#pragma unroll
+                for (int j = 0; j < E; ++j) {
+                    if ((j >> bit) & 1) continue;
+                    const float first = v[j], second = v[j | (1 << bit)];
+                    v[j] = first + second;
+                    v[j | (1 << bit)] = first - second;
+                }
+            }
+        }
+        done = base + kLogE;
+        if (done >= a.log_width) {
+            if (active) {
+#pragma unroll
+                for (int j = 0; j < E; ++j) {
+                    const int index = origin | (j << base);
+                    float value = v[j] * a.scale;
+                    if (a.signs_after) value *= a.signs_after[sign_base + index];
+                    mk_store_from_float(a.target, row_base + index, a.target_dtype, value);
+                }
+            }
+            break;
+        }
+#pragma unroll
+        for (int j = 0; j < E; ++j) mine[padded(origin | (j << base))] = v[j];
+        __syncthreads();
+    }
+}
+
+template <int E>
+int launch_fwht(FwhtArgs a, hipStream_t stream) {
+    a.threads_per_row = a.width / E;
+    a.rows_per_block = a.threads_per_row >= 256 ? 1 : 256 / a.threads_per_row;
+    if (a.rows_per_block > a.rows) a.rows_per_block = static_cast<int>(a.rows);
+    const int threads = a.rows_per_block * a.threads_per_row;
+    const size_t lds = static_cast<size_t>(a.rows_per_block) * padded(a.width) * sizeof(float);
+    static size_t allowed = 48 * 1024;  // raised once per instantiation when a row needs more
+    if (lds > allowed) {
+        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwht_kernel<E>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (status != hipSuccess)
+            return mk_fail(MK_ERR_HIP, "mk_fwht: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(status));
+        allowed = 160 * 1024;
+    }
+    const long long blocks = (a.rows + a.rows_per_block - 1) / a.rows_per_block;
+    hipLaunchKernelGGL((fwht_kernel<E>), dim3(static_cast<unsigned>(blocks)), dim3(threads), lds, stream, a);
+    return MK_OK;
+}
+
+struct MixArgs {
+    const float *source;
+    float *target;
+    const float *basis;  // [order, order] row-major
+    const float *signs_after;
+    long long rows;
+    int order, power, transpose;
+};
+
+// target[r, f', p] = sum_f mix[f', f] * source[r, f, p], mix = basis or its transpose;
+// the sum runs over ascending f with fused multiply-adds starting from zero.
+// One thread owns one (r, p) column of `order` values, kept in a private column of LDS
+// (dynamically indexed registers would live in scratch memory); consecutive lanes take
+// consecutive p, and the basis entries are wavefront-uniform scalar loads.
+constexpr int kMaxOrder = 256;
+
+__global__ void __launch_bounds__(256) basis_mix_kernel(const MixArgs a) {
+    extern __shared__ float columns_tile[];  // [order][blockDim.x]
+    float *mine = columns_tile + threadIdx.x;
+    const long long columns = a.rows * a.power;
+    const int row_stride = a.transpose ? 1 : a.order;
+    const int column_stride = a.transpose ? a.order : 1;
+    for (long long column = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; column < columns;
+         column += static_cast<long long>(gridDim.x) * blockDim.x) {
+        const long long row = column / a.power;
+        const int p = static_cast<int>(column - row * a.power);
+        const size_t base = static_cast<size_t>(row) * a.order * a.power + p;
+        for (int f = 0; f < a.order; ++f) mine[f * blockDim.x] = a.source[base + static_cast<size_t>(f) * a.power];
+        for (int out = 0; out < a.order; ++out) {
+            const float *mix_row = a.basis + out * row_stride;
+            float sum = 0.0f;
+            for (int f = 0; f < a.order; ++f) sum = __builtin_fmaf(mix_row[f * column_stride], mine[f * blockDim.x], sum);
+            if (a.signs_after) sum *= a.signs_after[out * a.power + p];
+            a.target[base + static_cast<size_t>(out) * a.power] = sum;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int mk_fwht(const void *source, int source_dtype, void *target, int target_dtype, long long rows,
+                       int width, const float *signs_before, const float *signs_after, int sign_period,
+                       float scale, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(rows >= 0, MK_ERR_INVALID, "mk_fwht: negative row count");
+    MK_REQUIRE(width >= 1 && (width & (width - 1)) == 0, MK_ERR_INVALID,
+               "mk_fwht: hadamard currently requires a power-of-two final dimension (got %d)", width);
+    MK_REQUIRE(width <= 32768, MK_ERR_UNSUPPORTED, "mk_fwht: rows longer than 32768 values are not supported");
+    if (rows == 0) return MK_OK;
+    MK_REQUIRE(source && target, MK_ERR_INVALID, "mk_fwht: null tensor pointer");
+    MK_REQUIRE(mk_dtype_valid(source_dtype) && mk_dtype_valid(target_dtype), MK_ERR_INVALID,
+               "mk_fwht: unknown dtype code");
+    MK_REQUIRE(!(signs_before || signs_after) || (sign_period >= width && sign_period % width == 0), MK_ERR_INVALID,
+               "mk_fwht: the sign period must be a multiple of the row width");
+    MK_REQUIRE((rows + 255) / 256 < (1ll << 31), MK_ERR_INVALID, "mk_fwht: too many rows");
+    FwhtArgs a{};
+    a.source = source; a.target = target; a.signs_before = signs_before; a.signs_after = signs_after;
+    a.rows = rows; a.width = width; a.source_dtype = source_dtype; a.target_dtype = target_dtype;
+    a.sign_period = (signs_before || signs_after) ? sign_period : 0; a.scale = scale;
+    a.log_width = 0;
+    while ((1 << a.log_width) < width) ++a.log_width;
+    int status;
+    if (width >= 32768) status = launch_fwht<32>(a, stream);
+    else if (width >= 16) status = launch_fwht<16>(a, stream);
+    else if (width == 8) status = launch_fwht<8>(a, stream);
+    else if (width == 4) status = launch_fwht<4>(a, stream);
+    else if (width == 2) status = launch_fwht<2>(a, stream);
+    else status = launch_fwht<1>(a, stream);
+    if (status) return status;
+    MK_LAUNCH_CHECK("mk_fwht");
+    return MK_OK;
+}
+
+extern "C" int mk_basis_mix(const float *source, float *target, const float *basis, long long rows, int order,
+                            int power, int transpose, const float *signs_after, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(rows >= 0 && order >= 1 && power >= 1, MK_ERR_INVALID, "mk_basis_mix: sizes must be positive");
+    MK_REQUIRE(order <= kMaxOrder, MK_ERR_UNSUPPORTED, "mk_basis_mix: basis order %d exceeds %d", order, kMaxOrder);
+    if (rows == 0) return MK_OK;
+    MK_REQUIRE(source && target && basis, MK_ERR_INVALID, "mk_basis_mix: null tensor pointer");
+    MK_REQUIRE(source != target, MK_ERR_INVALID, "mk_basis_mix: source and target must not alias");
+    MixArgs a{source, target, basis, signs_after, rows, order, power, transpose};
+    // One LDS column of `order` floats per thread: fewer threads for larger bases (64 KB).
+    const int threads = order <= 64 ? 256 : order <= 128 ? 128 : 64;
+    long long blocks = (rows * power + threads - 1) / threads;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    hipLaunchKernelGGL(basis_mix_kernel, dim3(static_cast<unsigned>(blocks)), dim3(threads),
+                       static_cast<size_t>(order) * threads * sizeof(float), stream, a);
+    MK_LAUNCH_CHECK("mk_basis_mix");
+    return MK_OK;
+}

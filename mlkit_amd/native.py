@@ -23,7 +23,9 @@ DTYPE_CODES = {torch.float32: MK_F32, torch.float16: MK_F16, torch.bfloat16: MK_
 
 MK_ERR_INVALID, MK_ERR_UNSUPPORTED, MK_ERR_HIP = 1, 2, 3
 
-_c_int, _c_float, _c_void_p = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+_c_int, _c_float, _c_void_p, _c_longlong = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
+
+SCALE_FORMAT_CODES = {"fp32": 0, "fp16": 1, "bf16": 2, "fp8": 3, "e8m0": 4}
 
 # name -> (restype, argtypes); mirrors include/mlkit_amd.h declaration by declaration.
 SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
@@ -38,6 +40,41 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "mk_packed_decode": (_c_int, [
         _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
+    ]),
+    "mk_scalar_encode": (_c_int, [
+        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int,
+        _c_int, _c_int, _c_float, _c_float, _c_void_p,
+    ]),
+    "mk_scalar_decode": (_c_int, [
+        _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+        _c_int, _c_int, _c_void_p,
+    ]),
+    "mk_search_scales": (_c_int, [
+        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
+    ]),
+    "mk_snap": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_longlong, _c_void_p]),
+    "mk_fit_scales": (_c_int, [
+        _c_void_p, _c_longlong, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_float,
+        _c_float, _c_int, _c_int, _c_void_p,
+    ]),
+    "mk_fwht": (_c_int, [
+        _c_void_p, _c_int, _c_void_p, _c_int, _c_longlong, _c_int, _c_void_p, _c_void_p, _c_int,
+        _c_float, _c_void_p,
+    ]),
+    "mk_basis_mix": (_c_int, [
+        _c_void_p, _c_void_p, _c_void_p, _c_longlong, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
+    ]),
+    "mk_feedback_round_tile": (_c_int, [
+        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
+        _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+        _c_float, _c_void_p,
+    ]),
+    "mk_feedback_pending": (_c_int, [
+        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+    ]),
+    "mk_feedback_block_update": (_c_int, [
+        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p,
     ]),
 }
 

@@ -59,8 +59,11 @@ def store_scale(value: np.ndarray, fmt: str) -> tuple[np.ndarray, int]:
     if fmt == "fp8":
         return round_e4m3(value), 8
     if fmt == "e8m0":
-        exponent = np.clip(np.rint(np.log2(np.maximum(value, F32(2.0**-127)))), -127, 127)
-        return np.exp2(exponent.astype(F32)).astype(F32), 8
+        # log2 in float64: the rounding thresholds 2^(k+1/2) are irrational, so no fp32
+        # value sits close enough to one for the float64 error to matter.
+        clamped = np.maximum(value, F32(2.0**-127)).astype(np.float64)
+        exponent = np.clip(np.rint(np.log2(clamped)), -127, 127)
+        return np.ldexp(np.float64(1.0), exponent.astype(np.int32)).astype(F32), 8
     raise ValueError(f"unsupported scale storage format {fmt!r}")
 
 

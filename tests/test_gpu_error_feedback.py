@@ -1,0 +1,108 @@
+"""GPU parity (through the C ABI) of the error-feedback kernels against the C oracle:
+reconstructions, codes, solved continuations and the trailing update bit for bit."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import feedback as oracle_feedback, scaling
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+F32 = np.float32
+INT4 = scaling.int_values(4)
+SEVEN = np.array([-1, -0.5, -0.25, 0, 0.25, 0.5, 1], dtype=F32)
+
+
+def dev(array):
+    return None if array is None else torch.from_numpy(np.ascontiguousarray(array)).cuda()
+
+
+def host(tensor):
+    torch.cuda.synchronize()
+    return tensor.cpu().numpy()
+
+
+def problem(rows, width, seed, samples=None):
+    """Weights and the unit upper coefficient matrix of a correlated synthetic Hessian."""
+    rng = np.random.default_rng(seed)
+    weight = helpers.normal_weight(rows, width, seed=seed)
+    samples = samples or 2 * width
+    inputs = rng.standard_normal((samples, width)).astype(F32)
+    inputs[:, ::7] *= 4
+    inputs += 0.5 * np.roll(inputs, 1, axis=1)
+    hessian = (inputs.T @ inputs / samples).astype(F32)
+    coeff, status = oracle_feedback.coefficients(hessian, 0.01)
+    assert status == 0
+    return weight, coeff, hessian
+
+
+@pytest.mark.parametrize("rows,width,tile_start,tile_width,group,values,integer,asym", [
+    (71, 96, 0, 96, 32, INT4, True, False),          # the reference's own tile test shape
+    (64, 256, 128, 128, 128, INT4, True, False),
+    (64, 256, 0, 128, 64, INT4, True, True),
+    (35, 512, 128, 200, 128, INT4, True, False),     # four-slot kernel
+    (19, 640, 64, 300, 50, INT4, True, True),        # sixteen-slot kernel, ragged groups
+    (64, 256, 128, 128, 64, scaling.NF4_VALUES, False, False),
+    (33, 128, 0, 100, 128, SEVEN, False, True),
+])
+def test_round_tile_matches_oracle(rows, width, tile_start, tile_width, group, values, integer, asym):
+    from mlkit_amd.kernels import error_feedback
+
+    weight, coeff, _ = problem(rows, width, seed=rows + tile_width)
+    rng = np.random.default_rng(1)
+    feedback = (rng.standard_normal((rows, width)) * 0.004).astype(F32)
+    region_start = tile_start - (group if tile_start >= group and tile_start % group == 0 else 0)
+    region = weight[:, region_start:tile_start + tile_width]
+    scales, zeros = oracle_feedback.fit_scales(region, values, group, asym)
+    expected_out = np.zeros_like(weight)
+    expected_codes = np.zeros(weight.shape, dtype=np.uint8)
+    oracle_feedback.round_tile(weight, feedback, coeff, scales, zeros, values, expected_out, expected_codes,
+                               region_start=region_start, tile_start=tile_start, tile_width=tile_width,
+                               group=group, integer=integer)
+    output = torch.zeros((rows, width), device="cuda")
+    encoded = torch.zeros((rows, width), device="cuda", dtype=torch.uint8)
+    bits = 4 if integer else int(np.ceil(np.log2(len(values))))
+    error_feedback.round_tile(dev(weight), dev(feedback), dev(coeff), dev(scales), dev(zeros), output, encoded,
+                              region_start=region_start, tile_start=tile_start, tile_width=tile_width,
+                              group=group, bits=bits, values=dev(values), integer_grid=integer)
+    np.testing.assert_array_equal(host(encoded), expected_codes)
+    np.testing.assert_array_equal(host(output), expected_out)
+
+
+@pytest.mark.parametrize("rows,width,start,stop", [(64, 384, 128, 256), (37, 512, 192, 492), (16, 1024, 0, 1024)])
+def test_pending_continuation_matches_oracle(rows, width, start, stop):
+    from mlkit_amd.kernels import error_feedback
+
+    weight, coeff, _ = problem(rows, width, seed=width + start)
+    rng = np.random.default_rng(2)
+    feedback = (rng.standard_normal((rows, width)) * 0.01).astype(F32)
+    expected = oracle_feedback.pending(feedback, coeff, start, stop)
+    solved = error_feedback.pending_continuation(dev(feedback), dev(coeff), start, stop)
+    np.testing.assert_array_equal(host(solved), expected)
+    targets = error_feedback.pending_continuation(dev(feedback), dev(coeff), start, stop, original=dev(weight))
+    np.testing.assert_array_equal(host(targets), (weight[:, start:stop] + expected).astype(F32))
+    # the textbook definition: x U = feedback[:, region]
+    block = coeff[start:stop, start:stop].astype(np.float64)
+    np.testing.assert_allclose(expected @ block, feedback[:, start:stop], rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("rows,width,start,stop", [(128, 512, 0, 128), (200, 700, 128, 256), (71, 333, 64, 101),
+                                                   (64, 256, 0, 255)])
+def test_block_update_matches_fma_chain(rows, width, start, stop):
+    from mlkit_amd.kernels import error_feedback
+
+    weight, coeff, _ = problem(rows, width, seed=width + stop)
+    rng = np.random.default_rng(3)
+    output = (weight + rng.standard_normal(weight.shape).astype(F32) * 0.003).astype(F32)
+    feedback = (rng.standard_normal(weight.shape) * 0.01).astype(F32)
+    expected = feedback.copy()
+    oracle_feedback.block_update(expected, weight, output, coeff, start, stop, mode=0)
+    updated = dev(feedback)
+    error_feedback.block_update(updated, dev(weight), dev(output), dev(coeff), start, stop)
+    np.testing.assert_array_equal(host(updated), expected)
+    exact = feedback[:, stop:].astype(np.float64) + (weight - output)[:, start:stop].astype(np.float64) @ coeff[start:stop, stop:].astype(np.float64)
+    np.testing.assert_allclose(host(updated)[:, stop:], exact, rtol=1e-4, atol=1e-6)
+    np.testing.assert_array_equal(host(updated)[:, :stop], feedback[:, :stop])

@@ -1,0 +1,118 @@
+"""GPU parity (through the C ABI) of the Walsh-Hadamard kernels against the oracle:
+bit for bit against the stage-by-stage fp32 restatement, to 1e-4 against the Sylvester
+matrix product in float64 (the reference's own bound, tests/quantization/test_operations.py:99-100)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import transforms
+
+pytestmark = pytest.mark.gpu
+
+F32 = np.float32
+
+
+def dev(array):
+    return torch.from_numpy(np.ascontiguousarray(array)).cuda()
+
+
+def host(tensor):
+    torch.cuda.synchronize()
+    return tensor.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("width", [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 16384, 32768])
+@pytest.mark.parametrize("normalize", [True, False])
+def test_transform_is_bit_exact(width, normalize):
+    from mlkit_amd.kernels import hadamard
+
+    rng = np.random.default_rng(width)
+    rows = 5 if width >= 4096 else 37
+    value = rng.standard_normal((rows, width)).astype(F32)
+    out = host(hadamard.transform(dev(value), normalize=normalize))
+    np.testing.assert_array_equal(out, transforms.fwht(value, normalize))
+    if width <= 2048:
+        exact = value.astype(np.float64) @ transforms.sylvester(width)
+        if normalize:
+            exact = exact / np.sqrt(width)
+        np.testing.assert_allclose(out, exact, rtol=1e-4, atol=1e-4)
+
+
+def test_leading_dimensions_and_involution():
+    from mlkit_amd.kernels import hadamard
+
+    rng = np.random.default_rng(1)
+    value = rng.standard_normal((3, 7, 256)).astype(F32)
+    once = hadamard.transform(dev(value))
+    np.testing.assert_array_equal(host(once), transforms.fwht(value))
+    np.testing.assert_allclose(host(hadamard.transform(once)), value, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(np.linalg.norm(host(once)), np.linalg.norm(value), rtol=1e-5)
+
+
+def test_rejects_other_widths():
+    from mlkit_amd.kernels import hadamard
+
+    with pytest.raises(ValueError, match="power-of-two"):
+        hadamard.transform(torch.zeros((4, 12), device="cuda"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_half_precision_rows_compute_in_fp32(dtype):
+    from mlkit_amd.kernels import hadamard
+
+    generator = torch.Generator().manual_seed(2)
+    value = torch.randn((8, 4096), generator=generator).to(dtype)
+    out = hadamard.transform(value.cuda())
+    assert out.dtype == dtype
+    expected = torch.from_numpy(transforms.fwht(value.float().numpy())).to(dtype)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), expected)
+
+
+def test_fused_signs_match_separate_multiplication():
+    from mlkit_amd.kernels import hadamard
+
+    rng = np.random.default_rng(3)
+    value = rng.standard_normal((9, 1024)).astype(F32)
+    signs = transforms.deterministic_signs(1024, seed=77)
+    forward = hadamard.transform(dev(value), signs_before=dev(signs))
+    np.testing.assert_array_equal(host(forward), transforms.fwht((value * signs).astype(F32)))
+    inverse = hadamard.transform(forward, signs_after=dev(signs))
+    np.testing.assert_allclose(host(inverse), value, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("width", [12, 20, 28, 96, 896, 4864, 7, 14336])
+def test_blocked_transform_matches_oracle(width):
+    from mlkit_amd.kernels import hadamard
+
+    order, power, basis = transforms.transform_factor(width)
+    rng = np.random.default_rng(width)
+    rows = 6
+    value = rng.standard_normal((rows, width)).astype(F32)
+    signs = transforms.deterministic_signs(width, seed=5)
+    blocks = hadamard.transform(dev(value).view(rows, order, power), signs_before=dev(signs))
+    np.testing.assert_array_equal(host(blocks).reshape(rows, width),
+                                  transforms.fwht((value * signs).astype(F32).reshape(rows, order, power)).reshape(rows, width))
+    mixed = hadamard.mix_blocks(blocks, dev(basis), transpose=False).view(rows, width)
+    expected = transforms.randomized(value, signs)
+    np.testing.assert_allclose(host(mixed), expected, rtol=1e-5, atol=1e-5)
+    # inverse: H blocks, transposed basis, signs afterwards
+    back = hadamard.transform(mixed.view(rows, order, power))
+    back = hadamard.mix_blocks(back, dev(basis), transpose=True, signs_after=dev(signs)).view(rows, width)
+    np.testing.assert_allclose(host(back), value, rtol=1e-5, atol=2e-5)
+    np.testing.assert_allclose(host(back), transforms.randomized(expected, signs, inverse=True), rtol=1e-5, atol=2e-5)
+
+
+def test_weight_sized_rotation_keeps_norms():
+    """4096 x 14336 fp32 along K as 7 x 2048 blocks (the literal blocked FWHT) and along
+    4096: row norms are preserved and the transform is its own inverse."""
+    from mlkit_amd.kernels import hadamard
+
+    generator = torch.Generator(device="cuda").manual_seed(4)
+    weight = torch.randn((4096, 14336), device="cuda", generator=generator) * 0.02
+    blocks = hadamard.transform(weight.view(4096, 7, 2048))
+    torch.testing.assert_close(blocks.view(4096, -1).norm(dim=1), weight.norm(dim=1), rtol=1e-5, atol=0)
+    torch.testing.assert_close(hadamard.transform(blocks).view_as(weight), weight, rtol=1e-5, atol=1e-6)
+    sample = weight[:3].cpu().numpy().reshape(3, 7, 2048)
+    np.testing.assert_array_equal(host(blocks[:3]), transforms.fwht(sample))
