@@ -1,0 +1,103 @@
+"""Minimal model wrappers: what ``optimize`` and the checkpoint functions need.
+
+``Model`` / ``QModel`` keep the attribute names of the reference's wrappers
+(/root/reference/src/mlkit/models/model.py:18-166: ``module``, ``quantized``,
+``tied_weights``, ``execution_backend``, ``bpw``) without its architecture adapters,
+calibration engine or reports, which are outside this package's path.  ``quantize`` rounds
+every ``nn.Linear`` of a module with one quantizer, collecting layer inputs for calibrated
+quantizers from the batches it is given.
+"""
+
+from collections.abc import Callable, Iterable
+from typing import Any
+
+import torch
+from torch import Tensor, nn
+
+from mlkit_amd.quantization.core import Ctx, Q, as_q
+
+
+class Model(nn.Module):
+    def __init__(self, module: nn.Module, tokenizer: Any = None, *, name: str | None = None) -> None:
+        super().__init__()
+        self.module = module.cuda()
+        self.tokenizer = tokenizer
+        self.name = name or type(module).__name__
+        self.execution_backend = "dense"
+
+    def forward(self, *args: Any, **kwargs: Any) -> Any:
+        device = self.device
+        move = lambda value: value.to(device) if isinstance(value, Tensor) else value  # noqa: E731
+        return self.module(*[move(a) for a in args], **{k: move(v) for k, v in kwargs.items()})
+
+    @property
+    def device(self) -> torch.device:
+        tensor = next(self.module.parameters(), None)
+        if tensor is None:
+            tensor = next(self.module.buffers(), None)
+        return torch.device("cuda") if tensor is None else tensor.device
+
+
+class QModel(Model):
+    """A converted model with the representation of every rounded layer.
+
+    ``tied_weights`` maps the name of a parameter that shares a rounded weight (a tied input
+    embedding) to the name of the layer that owns its codes.
+    """
+
+    def __init__(self, *args: Any, **kwargs: Any) -> None:
+        super().__init__(*args, **kwargs)
+        self.quantized: dict[str, Q] = {}
+        self.tied_weights: dict[str, str] = {}
+        self.transforms: list[dict[str, Any]] = []
+
+    @property
+    def bpw(self) -> float | None:
+        if not self.quantized or any(q.bits is None for q in self.quantized.values()):
+            return None
+        bits = sum(float(q.bits) for q in self.quantized.values())
+        return bits / sum(self.module.get_submodule(name).weight.numel() for name in self.quantized)
+
+    model_bpw = bpw
+
+
+def quantize(model: "Model | nn.Module", quantization: Callable[..., "Q | Tensor"],
+             calib: Iterable[Any] | None = None, *, skip: Iterable[str] = (), seed: int = 0,
+             cache_dir: Any = None) -> QModel:
+    """Round every ``nn.Linear`` (except ``skip``) in place and record its ``Q``.
+
+    ``calib`` is an iterable of positional-argument tuples (or single tensors) the module is
+    called with once; each layer's flattened inputs become ``Ctx.X``.  ``cache_dir`` is
+    accepted for call compatibility and unused (statistics are not cached on disk).
+    """
+    calibration = calib
+    module = model.module if isinstance(model, Model) else model
+    converted = QModel(module, getattr(model, "tokenizer", None), name=getattr(model, "name", None))
+    skipped = set(skip)
+    layers = {name: layer for name, layer in converted.module.named_modules()
+              if isinstance(layer, nn.Linear) and name not in skipped}
+    seen: dict[str, list[Tensor]] = {name: [] for name in layers}
+    if calibration is not None:
+        hooks = [layer.register_forward_pre_hook(
+            lambda _, inputs, key=name: seen[key].append(inputs[0].detach().reshape(-1, inputs[0].shape[-1])))
+            for name, layer in layers.items()]
+        with torch.no_grad():
+            for batch in calibration:
+                converted(*batch) if isinstance(batch, (tuple, list)) else converted(batch)
+        for hook in hooks:
+            hook.remove()
+    owners = {id(layer.weight): name for name, layer in layers.items()}
+    for name, parameter in converted.module.named_parameters(remove_duplicate=False):
+        owner = owners.get(id(parameter))
+        if owner is not None and name != (f"{owner}.weight" if owner else "weight"):
+            converted.tied_weights[name] = owner
+    for name, layer in layers.items():
+        inputs = torch.cat(seen[name]) if seen[name] else None
+        context = Ctx(name, module=layer, X=inputs, seed=seed, device=layer.weight.device)
+        with torch.no_grad():
+            result = as_q(quantization(layer.weight.detach(), context))
+            layer.weight.copy_(result.w.to(layer.weight.dtype))
+        if result.bits is not None:
+            result.bits = result.bits + context.additional_bits
+        converted.quantized[name] = result
+    return converted

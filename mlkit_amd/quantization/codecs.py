@@ -1,0 +1,135 @@
+"""Named decoders: checkpoints and ``Q`` objects refer to a decoder by name.
+
+Mirrors, in /root/reference/src/mlkit/quantization/codecs:
+  registry.py:1-46        codec, decoder, registered, row_parameters
+  scaled.py:19-101        decode_grouped, decode_scaled ("scaled"), decode_feedback ("feedback")
+  composition.py:14-20    deterministic_signs
+  composition.py:87-116   concatenate_rows
+Decoding uint8 codes with FP32 parameters on a HIP device runs ``mk_scalar_decode``; tensors
+that track gradients, or live on the host, use the same expression in tensor operations.
+"""
+
+from collections.abc import Callable, Sequence
+
+import torch
+from torch import Tensor
+
+from mlkit_amd.quantization.core import Q
+
+_DECODERS: dict[str, Callable[..., Tensor]] = {}
+_ROW_PARAMETERS: dict[str, tuple[str, ...]] = {}
+
+
+def codec(name: str, *, row_parameters: tuple[str, ...] | None = None) -> Callable[[Callable], Callable]:
+    """Register ``function(codes, **params) -> Tensor`` under ``name``.
+
+    ``row_parameters`` names the parameters holding one entry per weight row; declaring
+    them lets row chunks of one matrix be joined (``concatenate_rows``).
+    """
+    def register(function: Callable[..., Tensor]) -> Callable[..., Tensor]:
+        if not name or name in _DECODERS:
+            raise ValueError(f"codec name {name!r} is empty or already registered")
+        _DECODERS[name] = function
+        if row_parameters is not None:
+            _ROW_PARAMETERS[name] = tuple(row_parameters)
+        return function
+
+    return register
+
+
+def decoder(name: str) -> Callable[..., Tensor]:
+    try:
+        return _DECODERS[name]
+    except KeyError:
+        raise ValueError(f"checkpoint requires registered codec {name!r}") from None
+
+
+def registered(name: str | None) -> bool:
+    return name in _DECODERS
+
+
+def row_parameters(name: str | None) -> tuple[str, ...] | None:
+    return None if name is None else _ROW_PARAMETERS.get(name)
+
+
+def _tracked(*tensors: Tensor | None) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def _kernel_ready(codes: Tensor, scales: Tensor, values: Tensor, zero: Tensor | None) -> bool:
+    return (codes.is_cuda and codes.dtype == torch.uint8 and codes.dim() == 2 and codes.is_contiguous()
+            and scales.dtype == torch.float32 and values.dtype == torch.float32 and values.numel() <= 256
+            and (zero is None or zero.dtype == torch.float32) and not _tracked(scales, values, zero))
+
+
+def _expand(codes: Tensor, values: Tensor, scales: Tensor, zero: Tensor | None, index: Tensor) -> Tensor:
+    out = values[codes.int()] * scales[:, index]
+    return out if zero is None else out + zero[:, index]
+
+
+def decode_grouped(codes: Tensor, scales: Tensor, values: Tensor, group: int, zero: Tensor | None) -> Tensor:
+    """``values[codes] * scales[:, c // group] (+ zero[:, c // group])`` as FP32."""
+    if _kernel_ready(codes, scales, values, zero):
+        from mlkit_amd.kernels import scalar_decode
+
+        return scalar_decode.decode(codes, scales.contiguous(), values.contiguous(),
+                                    None if zero is None else zero.contiguous(), group)
+    index = torch.arange(codes.shape[1], device=codes.device) // group
+    return _expand(codes, values, scales, zero, index)
+
+
+@codec("scaled", row_parameters=("scales", "zero"))
+def decode_scaled(codes: Tensor, *, scales: Tensor, values: Tensor, group: int, offset: int = 0,
+                  zero: Tensor | None = None) -> Tensor:
+    if offset == 0:
+        return decode_grouped(codes, scales, values, group, zero)
+    index = torch.arange(offset, offset + codes.shape[1], device=codes.device) // group
+    return _expand(codes, values, scales, zero, index)
+
+
+@codec("feedback", row_parameters=("scales", "zero"))
+def decode_feedback(codes: Tensor, *, scales: Tensor, values: Tensor, group: int, refit: int,
+                    zero: Tensor | None = None, permutation: Tensor | None = None) -> Tensor:
+    """Codes of an error-feedback sweep: scales are laid out region by region of ``refit``
+    columns, ``ceil(refit / group)`` per region."""
+    if refit % group == 0:
+        out = decode_grouped(codes, scales, values, group, zero)
+    elif _kernel_ready(codes, scales, values, zero):
+        from mlkit_amd.kernels import scalar_decode
+
+        out = scalar_decode.decode(codes, scales.contiguous(), values.contiguous(),
+                                   None if zero is None else zero.contiguous(), group, refit=refit)
+    else:
+        columns = torch.arange(codes.shape[1], device=codes.device)
+        index = (columns // refit) * (-(-refit // group)) + (columns % refit) // group
+        out = _expand(codes, values, scales, zero, index)
+    return out if permutation is None else out[:, permutation.argsort()]
+
+
+def deterministic_signs(width: int, seed: int, device: torch.device | str) -> Tensor:
+    """Rademacher signs from an integer hash of ``index + seed``: identical on every device."""
+    v = (torch.arange(width, device=device, dtype=torch.int64) + seed) & 0xFFFFFFFF
+    for _ in range(2):
+        v = ((v ^ (v >> 16)) * 0x45D9F3B) & 0xFFFFFFFF
+    v = v ^ (v >> 16)
+    return (v & 1).float() * 2 - 1
+
+
+def concatenate_rows(parts: Sequence[Q]) -> Q:
+    """Join the representations of consecutive row chunks of one matrix."""
+    head = parts[0]
+    known = [part.bits for part in parts if part.bits is not None]
+    bits = sum(known) if len(known) == len(parts) else None
+    if any(part.codes is None for part in parts):
+        return Q(torch.cat([part.w for part in parts]), bits=bits)
+    per_row = row_parameters(head.codec)
+    if per_row is None:
+        raise ValueError(
+            f"codec {head.codec!r} does not declare row parameters, so a row-separable "
+            "quantizer cannot use it; register it with mk.codec(name, row_parameters=...)")
+    params = dict(head.params)
+    for key in per_row:
+        if isinstance(head.params.get(key), Tensor):
+            params[key] = torch.cat([part.params[key] for part in parts])
+    return Q(codes=torch.cat([part.codes for part in parts]), params=params, decode=head.decode,
+             codec=head.codec, bits=bits, metadata=head.metadata)

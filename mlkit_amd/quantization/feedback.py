@@ -1,0 +1,295 @@
+"""Hessian error feedback in LDL form: GPTQ (one column at a time) and LDLQ (blocks).
+
+With the damped Hessian factored as ``H = R R^T`` (``R`` upper triangular), column block
+``k`` is rounded after adding ``sum_{j<k} d_j R_jk R_kk^-1`` to its weights, ``d = w - q``.
+``feedback_coefficients`` returns ``A = R blockdiag(R)^-1`` once; the sweep then needs no
+inverse.  Mirrors /root/reference/src/mlkit/quantization/algorithms/error_feedback.py
+(:37-83 feedback_coefficients, :107-233 CodecAccumulator, :236-467 ErrorFeedback,
+:473-489 ldlq / gptq) and operations/losses.py:9-15 (proxy_loss).
+
+On a HIP device, scalar grids with ``step == 1`` run entirely in kernels: per region one
+triangular solve (``mk_feedback_pending``), one scale fit, then per tile the column sweep
+(``mk_feedback_round_tile``) and the trailing update on the matrix cores
+(``mk_feedback_block_update``).  Other rounders take the block-by-block tensor path.
+"""
+
+import math
+from collections.abc import Callable
+from typing import Any
+
+import torch
+from torch import Tensor
+
+from mlkit_amd.quantization.codecs import decode_feedback
+from mlkit_amd.quantization.core import Ctx, FittedRounder, Q, Quantizer, ScalarRounding, as_q, fit_quantizer
+
+FUSED_CODEBOOK_LIMIT = 256
+FUSED_VECTOR_DIMENSIONS = {2, 4, 8, 16}
+FUSED_VECTOR_CODEBOOK_LIMIT = 65536
+UPPER_FACTORIZATION_WIDTH = 4096
+MAXIMUM_FUSED_TILE = 1024
+
+
+def feedback_coefficients(hessian: Tensor, step: int, *, damp: float = 0.01,
+                          permutation: Tensor | None = None) -> tuple[Tensor, int]:
+    """``(A, status)``: ``A = R blockdiag(R)^-1`` for the damped ``H = R R^T``, row-major;
+    only entries above the block diagonal are meaningful.  ``status != 0``: H is indefinite.
+
+    Zero diagonal entries (channels never activated) become one before damping by
+    ``damp * mean(diag)``.  The lower Cholesky factor of the index-reversed matrix,
+    reversed back, is the upper factor ``R``.
+    """
+    width = hessian.shape[0]
+    if permutation is None:
+        flipped = hessian.flip(0, 1)
+    else:
+        order = permutation.flip(0)
+        flipped = hessian[order][:, order]
+    diagonal = flipped.diagonal()
+    diagonal.masked_fill_(diagonal == 0, 1)
+    diagonal.add_(damp * diagonal.mean().clamp_min(1e-12))
+    if width >= UPPER_FACTORIZATION_WIDTH:
+        # column-major solvers factor the upper triangle faster; its transpose is the lower factor
+        factor, status = torch.linalg.cholesky_ex(flipped, upper=True)
+        lower = factor.T
+    else:
+        lower, status = torch.linalg.cholesky_ex(flipped)
+    if int(status.item()) != 0:
+        return lower, int(status.item())
+    if step == 1:
+        lower = lower / lower.diagonal().clone()
+        return lower.flip(0, 1).contiguous(), 0
+    upper = lower.flip(0, 1).contiguous()
+    blocks = width // step
+    pick = torch.arange(blocks, device=upper.device)
+    diagonal_blocks = upper.reshape(blocks, step, blocks, step)[pick, :, pick, :]
+    block_columns = upper.reshape(width, blocks, step).transpose(0, 1)
+    solved = torch.linalg.solve_triangular(diagonal_blocks, block_columns, upper=True, left=False)
+    return solved.transpose(0, 1).reshape(width, width).contiguous(), 0
+
+
+def proxy_loss(weight: Tensor, reconstruction: Tensor, hessian: Tensor) -> Tensor:
+    """``tr(E H E^T) / rows`` with ``E = W - W_hat``: the layer-output error the sweep minimises."""
+    error = (weight - reconstruction).float()
+    return ((error @ hessian.float()) * error).sum() / weight.shape[0]
+
+
+class _PermutedStatistics:
+    """Calibration statistics in the column order of permuted weights."""
+
+    def __init__(self, ctx: Ctx, permutation: Tensor) -> None:
+        self.ctx, self.permutation, self.seen = ctx, permutation, {}
+
+    def __call__(self, name: str, function: Callable | None, reduction: str) -> Tensor:
+        if name not in self.seen:
+            value = self.ctx.stat(name, function, reduction)
+            if name == "H":
+                value = value[self.permutation][:, self.permutation]
+            elif name == "X":
+                value = value[:, self.permutation]
+            elif name in {"act_absmean", "act_absmax"}:
+                value = value[self.permutation]
+            self.seen[name] = value
+        return self.seen[name]
+
+
+class _Collected:
+    """Codes and fitted parameters of all regions, so the result stays a portable codec."""
+
+    def __init__(self, rows: int, width: int, device: torch.device) -> None:
+        self.rows, self.width, self.device = rows, width, device
+        self.codes: Tensor | None = None
+        self.shared: dict[str, Any] = {}
+        self.metadata: dict[str, Any] = {}
+        self.scales: list[Tensor] = []
+        self.zeros: list[Tensor] = []
+        self.portable = True
+        self.bits: float | None = 0.0
+
+    def count(self, bits: float | None) -> None:
+        self.bits = None if self.bits is None or bits is None else self.bits + bits
+
+    def open_scalar_region(self, scalar: ScalarRounding) -> Tensor:
+        if self.codes is None:
+            self.codes = torch.empty((self.rows, self.width), dtype=torch.uint8, device=self.device)
+            self.shared = {"values": scalar.values, "group": scalar.group}
+            self.metadata = scalar.metadata
+        self.scales.append(scalar.scales)
+        if scalar.zero is not None:
+            self.zeros.append(scalar.zero)
+        self.count(scalar.bits)
+        return self.codes
+
+    def add_block(self, quantized: Q, column: int, stop: int, region_start: int) -> None:
+        self.count(quantized.bits)
+        if not self.portable:
+            return
+        if quantized.codec != "scaled" or quantized.codes is None:
+            self.portable = False
+            return
+        if self.codes is None:
+            self.codes = torch.empty((self.rows, self.width), dtype=quantized.codes.dtype, device=self.device)
+            self.shared = quantized.params
+            self.metadata = quantized.metadata
+        self.codes[:, column:stop] = quantized.codes
+        if column == region_start:
+            self.scales.append(quantized.params["scales"])
+            if quantized.params["zero"] is not None:
+                self.zeros.append(quantized.params["zero"])
+
+    def result(self, output: Tensor, permutation: Tensor | None, refit_width: int, ctx: Ctx) -> Q:
+        if self.portable and self.codes is not None:
+            if permutation is not None:
+                ctx.add_bits(self.width * math.ceil(math.log2(self.width)))
+            params = {"scales": torch.cat(self.scales, dim=1), "values": self.shared["values"],
+                      "group": self.shared["group"], "refit": refit_width,
+                      "zero": torch.cat(self.zeros, dim=1) if self.zeros else None, "permutation": permutation}
+            return Q(codes=self.codes, bits=self.bits, codec="feedback", decode=decode_feedback, params=params,
+                     metadata=self.metadata)
+        if permutation is not None:
+            output = output[:, permutation.argsort()]
+        return Q(output, bits=self.bits)
+
+
+class ErrorFeedback(Quantizer):
+    """LDL error feedback around an inner quantizer, with per-region refits of its format."""
+
+    def __init__(self, inner: Callable[..., "Q | Tensor"], *, step: int = 8, refit: int | None = None,
+                 damp: float = 0.01, order: str = "natural", block_size: int = 128, backend: str = "auto") -> None:
+        if step < 1 or block_size < step or block_size % step:
+            raise ValueError("block_size must be a positive multiple of step")
+        if refit is not None and (refit < step or refit % step):
+            raise ValueError("refit must be a positive multiple of step or None")
+        if damp < 0 or order not in {"natural", "activation"}:
+            raise ValueError("damp must be nonnegative and order must be natural or activation")
+        if backend not in {"auto", "torch", "hip", "triton"}:
+            raise ValueError("error-feedback backend must be auto, torch, or hip")
+        self.inner, self.step, self.refit, self.damp = inner, step, refit, damp
+        self.order, self.block_size = order, block_size
+        self.backend = "hip" if backend == "triton" else backend
+
+    @property
+    def row_separable(self) -> bool:  # type: ignore[override]
+        return bool(getattr(self.inner, "row_separable", False))
+
+    def __repr__(self) -> str:
+        return f"ldlq({self.inner!r}, step={self.step}, refit={self.refit})"
+
+    # -- pieces --------------------------------------------------------------------------
+
+    def _kernel_state(self, rounder: Callable[[Tensor, slice], Q], device: torch.device) -> ScalarRounding | None:
+        """The fitted scalar state when the HIP kernels can round this region."""
+        scalar = rounder.scalar if isinstance(rounder, FittedRounder) else None
+        usable = (scalar is not None and device.type == "cuda" and self.backend != "torch" and self.step == 1
+                  and scalar.grid.bits <= 8 and 1 <= scalar.values.numel() <= FUSED_CODEBOOK_LIMIT
+                  and self.block_size <= MAXIMUM_FUSED_TILE)
+        if usable:
+            return scalar
+        if self.backend == "hip":
+            raise ValueError("fused error feedback requires a HIP device and a native scalar rounder with step=1")
+        return None
+
+    @staticmethod
+    def _pending_continuation(feedback: Tensor, coefficients: Tensor, start: int, stop: int) -> Tensor:
+        """The adjustment the region's columns would take if nothing more were rounded:
+        accumulated feedback is that adjustment times the region's unit-triangular block."""
+        if feedback.is_cuda and stop - start <= MAXIMUM_FUSED_TILE:
+            from mlkit_amd.kernels import error_feedback as kernel
+
+            return kernel.pending_continuation(feedback, coefficients, start, stop)
+        return torch.linalg.solve_triangular(coefficients[start:stop, start:stop], feedback[:, start:stop],
+                                             upper=True, left=False, unitriangular=True)
+
+    def _round_tile_by_blocks(self, rounder, original, feedback, coefficients, output, collected,
+                              region_start: int, tile_start: int, tile_stop: int) -> None:
+        corrections = feedback[:, tile_start:tile_stop].clone()
+        for column in range(tile_start, tile_stop, self.step):
+            stop = column + self.step
+            local = slice(column - tile_start, stop - tile_start)
+            weights = original[:, column:stop]
+            quantized = as_q(rounder(weights + corrections[:, local], slice(column - region_start, stop - region_start)))
+            restored = quantized.w
+            if restored.shape != weights.shape:
+                raise ValueError("inner quantizer changed the shape of a column slice")
+            output[:, column:stop] = restored
+            collected.add_block(quantized, column, stop, region_start)
+            if stop < tile_stop:
+                deviation = weights - restored
+                later = coefficients[column:stop, stop:tile_stop]
+                if self.step == 1:
+                    corrections[:, local.stop:] += deviation * later
+                else:
+                    corrections[:, local.stop:] += deviation @ later
+
+    # -- the sweep -----------------------------------------------------------------------
+
+    def __call__(self, w: Tensor, ctx: Ctx | None = None) -> Q:
+        ctx = ctx or Ctx(device=w.device)
+        rows, width = w.shape
+        hessian = ctx.H.to(device=w.device, dtype=torch.float32).detach()
+        if hessian.shape != (width, width):
+            raise ValueError("Hessian dimensions must match the weight input width")
+        if width % self.step:
+            raise ValueError("weight input width must be divisible by the error-feedback step")
+        dead = hessian.diagonal() == 0
+        original = w.detach().to(torch.float32, copy=True)
+        original[:, dead] = 0
+        permutation = None
+        if self.order == "activation":
+            permutation = hessian.diagonal().masked_fill(dead, 1).argsort(descending=True)
+            original = original[:, permutation].contiguous()
+        coefficients, status = feedback_coefficients(hessian.clone(), self.step, damp=self.damp, permutation=permutation)
+        if status != 0:
+            raise ValueError(f"calibration Hessian for {ctx.name!r} is not positive definite; increase damp")
+        del hessian
+        statistics = None if permutation is None else _PermutedStatistics(ctx, permutation)
+        feedback = torch.zeros_like(original)
+        output = torch.empty_like(original)
+        collected = _Collected(rows, width, w.device)
+        refit_width = width if self.refit is None else self.refit
+        on_device = w.is_cuda
+        if on_device:
+            from mlkit_amd.kernels import error_feedback as kernel
+        for region_start in range(0, width, refit_width):
+            region_stop = min(width, region_start + refit_width)
+            targets = original[:, region_start:region_stop]
+            if region_start:
+                if on_device and region_stop - region_start <= MAXIMUM_FUSED_TILE:
+                    targets = kernel.pending_continuation(feedback, coefficients, region_start, region_stop,
+                                                          original=original)
+                else:
+                    targets = targets + self._pending_continuation(feedback, coefficients, region_start, region_stop)
+            fitted_ctx = ctx if statistics is None else ctx.derive(statistics)
+            rounder = fit_quantizer(self.inner, targets, fitted_ctx)
+            del targets
+            if fitted_ctx is not ctx:
+                ctx.add_bits(fitted_ctx.additional_bits)
+            scalar = self._kernel_state(rounder, w.device)
+            encoded = None if scalar is None else collected.open_scalar_region(scalar)
+            for tile_start in range(region_start, region_stop, self.block_size):
+                tile_stop = min(region_stop, tile_start + self.block_size)
+                if scalar is not None:
+                    kernel.round_tile(original, feedback, coefficients, scalar.scales.contiguous(),
+                                      None if scalar.zero is None else scalar.zero.contiguous(), output, encoded,
+                                      region_start=region_start, tile_start=tile_start,
+                                      tile_width=tile_stop - tile_start, group=scalar.group, bits=scalar.grid.bits,
+                                      values=scalar.values, integer_grid=scalar.grid.integer)
+                else:
+                    self._round_tile_by_blocks(rounder, original, feedback, coefficients, output, collected,
+                                               region_start, tile_start, tile_stop)
+                if tile_stop < width:
+                    if on_device:
+                        kernel.block_update(feedback, original, output, coefficients, tile_start, tile_stop)
+                    else:
+                        deviations = original[:, tile_start:tile_stop] - output[:, tile_start:tile_stop]
+                        feedback[:, tile_stop:].addmm_(deviations, coefficients[tile_start:tile_stop, tile_stop:])
+        return collected.result(output, permutation, refit_width, ctx)
+
+
+def ldlq(inner: Callable[..., "Q | Tensor"], **options: Any) -> ErrorFeedback:
+    return ErrorFeedback(inner, **options)
+
+
+def gptq(inner: Callable[..., "Q | Tensor"], refit: int | None = 128, act_order: bool = False,
+         **options: Any) -> ErrorFeedback:
+    return ldlq(inner, step=1, refit=refit, order="activation" if act_order else "natural", **options)

@@ -1,0 +1,165 @@
+"""Orthogonal structured transforms of ordinary transformer widths.
+
+Mirrors /root/reference/src/mlkit/quantization/operations/orthogonal_transforms.py:
+  :12-31     hadamard                 :34-67    prime, paley_matrix
+  :70-98     transform_factor         :101-109  structured_transform
+  :112-122   randomized_transform, rht
+FP32 / FP16 / BF16 tensors on a HIP device run ``mk_fwht`` (one launch per tensor) and
+``mk_basis_mix``; ``rotate`` additionally fuses the sign flips into those launches.
+Host tensors and tensors that track gradients use the stage-by-stage tensor operations.
+"""
+
+import functools
+import math
+
+import torch
+from torch import Tensor
+
+_KERNEL_DTYPES = {torch.float32, torch.float16, torch.bfloat16}
+MAXIMUM_KERNEL_WIDTH = 32768
+MAXIMUM_KERNEL_ORDER = 256
+
+
+def _on_kernel(value: Tensor) -> bool:
+    tracked = torch.is_grad_enabled() and value.requires_grad
+    return value.is_cuda and value.dtype in _KERNEL_DTYPES and not tracked and value.shape[-1] <= MAXIMUM_KERNEL_WIDTH
+
+
+def hadamard(value: Tensor, *, normalize: bool = True) -> Tensor:
+    """Fast Walsh-Hadamard transform along the final dimension (natural order)."""
+    width = value.shape[-1]
+    if width <= 0 or width & (width - 1):
+        raise ValueError("hadamard currently requires a power-of-two final dimension")
+    if _on_kernel(value):
+        from mlkit_amd.kernels import hadamard as kernel
+
+        return kernel.transform(value.contiguous(), normalize=normalize)
+    out = value.clone()
+    stride = 1
+    while stride < width:
+        pairs = out.reshape(*value.shape[:-1], -1, 2, stride)
+        low, high = pairs[..., 0, :], pairs[..., 1, :]
+        out = torch.stack((low + high, low - high), dim=-2).reshape_as(value)
+        stride *= 2
+    return out / math.sqrt(width) if normalize else out
+
+
+def prime(value: int) -> bool:
+    return value >= 2 and all(value % divisor for divisor in range(2, math.isqrt(value) + 1))
+
+
+def _quadratic_characters(field: int) -> Tensor:
+    """chi(i - j) over the prime field: +1 for nonzero squares, -1 for non-squares, 0 on the diagonal."""
+    index = torch.arange(field)
+    is_square = torch.zeros(field)
+    is_square[(index[1:] ** 2) % field] = 1
+    difference = (index[:, None] - index[None, :]) % field
+    return torch.where(difference == 0, 0.0, 2 * is_square[difference] - 1)
+
+
+@functools.lru_cache(maxsize=32)
+def paley_matrix(order: int) -> Tensor:
+    """An orthonormal Hadamard matrix of a Paley order: q + 1 (q = 3 mod 4) or 2(q + 1) (q = 1 mod 4)."""
+    if prime(order - 1) and (order - 1) % 4 == 3:
+        field = order - 1
+        matrix = torch.ones(order, order)
+        matrix[1:, 0] = -1
+        matrix[1:, 1:] = _quadratic_characters(field) + torch.eye(field)
+        return matrix / math.sqrt(order)
+    field = order // 2 - 1
+    if order % 2 == 0 and prime(field) and field % 4 == 1:
+        conference = torch.ones(field + 1, field + 1)
+        conference[0, 0] = 0
+        conference[1:, 1:] = _quadratic_characters(field)
+        eye = torch.eye(field + 1)
+        top = torch.cat((conference + eye, conference - eye), dim=1)
+        bottom = torch.cat((conference - eye, -conference - eye), dim=1)
+        return torch.cat((top, bottom), dim=0) / math.sqrt(order)
+    raise ValueError(f"no prime-field Paley construction for order {order}")
+
+
+@functools.lru_cache(maxsize=128)
+def transform_factor(width: int) -> tuple[int, int, Tensor | None]:
+    """``(order, power, basis)`` with ``width = order * power``: a dense orthonormal basis of
+    ``order`` and a Hadamard power of two.  Widths without a Paley construction keep their
+    odd factor as an orthonormal DCT-II basis."""
+    if width < 1:
+        raise ValueError("transform width must be positive")
+    if width & (width - 1) == 0:
+        return 1, width, None
+    odd = width
+    while odd % 2 == 0:
+        odd //= 2
+    power = width // odd
+    for multiplier in (1, 2, 4, 8, 16):
+        if power % multiplier:
+            continue
+        try:
+            return odd * multiplier, power // multiplier, paley_matrix(odd * multiplier)
+        except ValueError:
+            continue
+    index = torch.arange(odd, dtype=torch.float64)
+    matrix = torch.cos(math.pi / odd * (index[None, :] + 0.5) * index[:, None])
+    matrix[0] *= 1 / math.sqrt(odd)
+    matrix[1:] *= math.sqrt(2 / odd)
+    return odd, power, matrix.float()
+
+
+@functools.lru_cache(maxsize=64)
+def _basis_on(width: int, device: torch.device) -> Tensor:
+    basis = transform_factor(width)[2]
+    assert basis is not None
+    return basis.to(device).contiguous()
+
+
+def rotate(value: Tensor, *, inverse: bool = False, signs: Tensor | None = None) -> Tensor:
+    """``structured_transform`` with optional fused sign flips: forward ``T(value * signs)``,
+    inverse ``T^-1(value) * signs``.  Two launches at most on a HIP device."""
+    order, power, basis = transform_factor(value.shape[-1])
+    if not (_on_kernel(value) and power <= MAXIMUM_KERNEL_WIDTH and order <= MAXIMUM_KERNEL_ORDER):
+        if signs is not None and not inverse:
+            value = value * signs
+        out = _structured_on_host(value, order, power, basis, inverse)
+        return out * signs if signs is not None and inverse else out
+    from mlkit_amd.kernels import hadamard as kernel
+
+    if signs is not None:
+        signs = signs.to(device=value.device, dtype=torch.float32).contiguous()
+    before, after = (None, signs) if inverse else (signs, None)
+    value = value.contiguous()
+    if basis is None:
+        return kernel.transform(value, signs_before=before, signs_after=after)
+    blocks = value.reshape(*value.shape[:-1], order, power)
+    staged = torch.empty(blocks.shape, device=value.device, dtype=torch.float32)
+    kernel.transform(blocks, signs_before=before, out=staged)
+    mixed = kernel.mix_blocks(staged, _basis_on(value.shape[-1], value.device), transpose=inverse, signs_after=after)
+    return mixed.reshape(value.shape).to(value.dtype)
+
+
+def _structured_on_host(value: Tensor, order: int, power: int, basis: Tensor | None, inverse: bool) -> Tensor:
+    if basis is None:
+        return hadamard(value)
+    blocks = hadamard(value.reshape(*value.shape[:-1], order, power)).transpose(-1, -2)
+    basis = basis.to(device=value.device, dtype=value.dtype)
+    mixed = blocks @ (basis if inverse else basis.T)
+    return mixed.transpose(-1, -2).reshape_as(value)
+
+
+def structured_transform(value: Tensor, *, inverse: bool = False) -> Tensor:
+    """``(basis (x) H_power)`` along the final dimension; ``inverse`` applies its transpose."""
+    return rotate(value, inverse=inverse)
+
+
+def random_signs(width: int, seed: int, device: torch.device | str, dtype: torch.dtype = torch.float32) -> Tensor:
+    """The +-1 vector ``randomized_transform`` draws for ``seed`` on ``device``."""
+    generator = torch.Generator(device=device).manual_seed(seed)
+    return torch.randint(2, (width,), generator=generator, device=device).to(dtype) * 2 - 1
+
+
+def randomized_transform(value: Tensor, *, seed: int = 0, inverse: bool = False) -> Tensor:
+    signs = random_signs(value.shape[-1], seed, value.device, value.dtype)
+    return rotate(value, inverse=inverse, signs=signs)
+
+
+def rht(value: Tensor, *, seed: int = 0, inverse: bool = False) -> Tensor:
+    return randomized_transform(value, seed=seed, inverse=inverse)
