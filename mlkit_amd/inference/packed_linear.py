@@ -128,19 +128,20 @@ class PackedLinear(nn.Module):
         """One call into the C ABI with the layer's constant arguments bound once
         (rebuilt after the buffers move or change dtype)."""
         launch = self._launch
-        if launch is None:
+        if launch is None or launch[0] != self.packed.data_ptr():  # a copy owns other buffers
             scales, zeros, bias = self.scales, self.zeros, self.bias
             launch = self._launch = (
-                native.library().mk_packed_matvec,
+                self.packed.data_ptr(),
                 (self.packed.data_ptr(), scales.data_ptr(), native.dtype_code(scales), self.values.data_ptr(),
                  self.values.numel(), native.pointer(zeros), native.pointer(bias),
                  0 if bias is None else native.dtype_code(bias)),
                 (self.out_features, self.in_features, self.group, self.code_bits, int(self.uniform_grid),
                  self.grid_minimum, self.grid_step),
             )
-        function, tensors, constants = launch
-        status = function(inputs.data_ptr(), native.DTYPE_CODES[inputs.dtype], *tensors, output.data_ptr(), rows,
-                          *constants, torch.cuda.current_stream(inputs.device).cuda_stream)
+        _, tensors, constants = launch
+        status = native.library().mk_packed_matvec(
+            inputs.data_ptr(), native.DTYPE_CODES[inputs.dtype], *tensors, output.data_ptr(), rows, *constants,
+            torch.cuda.current_stream(inputs.device).cuda_stream)
         if status:
             native.check(status)
 

@@ -1,0 +1,344 @@
+"""GPU tests of the public API on HIP tensors: the kernels behind ``mk.scaled``, ``mk.gptq``,
+``mk.rht``, ``PackedLinear`` and ``mk.optimize`` against the oracle (bit for bit where the
+arithmetic is fixed) and with the reference's own module-level assertions
+(tests/inference/test_packed_linear.py, tests/evaluation/test_capability_report.py,
+tests/conversion/test_head_quantization.py:76-81, tests/checkpoints/test_checkpoints.py in
+/root/reference)."""
+
+import copy
+
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+import mlkit_amd as mk
+from mlkit_amd.quantization.core import Ctx
+from oracle import feedback as oracle_feedback, scaling, transforms as oracle_transforms
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+F32 = np.float32
+SEVEN = np.array([-1, -0.5, -0.25, 0, 0.25, 0.5, 1], dtype=F32)
+
+
+def dev(array):
+    return torch.from_numpy(np.ascontiguousarray(array)).cuda()
+
+
+def host(tensor):
+    torch.cuda.synchronize()
+    return tensor.detach().cpu().numpy()
+
+
+@pytest.mark.parametrize("name,make,values,integer,kwargs", [
+    ("int4-asym-g128", lambda: mk.int(4, group=128, asym=True), scaling.int_values(4), True, dict(group=128, asym=True)),
+    ("int2-g64", lambda: mk.int(2, group=64), scaling.int_values(2), True, dict(group=64)),
+    ("int3-g64", lambda: mk.int(3, group=64), scaling.int_values(3), True, dict(group=64)),
+    ("nf4-g64", lambda: mk.nf4(group=64), scaling.NF4_VALUES, False, dict(group=64)),
+    ("cb3-g64-mse", lambda: mk.scaled(mk.grid.values(SEVEN, bits=3), group=64, scale="mse"), SEVEN, False,
+     dict(group=64, scale="mse")),
+    ("int4-g128-mse", lambda: mk.int(4, group=128, scale="mse"), scaling.int_values(4), True, dict(group=128, scale="mse")),
+    ("int4-rowwise-bf16", lambda: mk.int(4, group=None, scale_fmt="bf16"), scaling.int_values(4), True,
+     dict(group=None, fmt="bf16")),
+])
+def test_scaled_formats_match_oracle_bit_for_bit(name, make, values, integer, kwargs):
+    weight = helpers.normal_weight(96, 1024, seed=31, student_t=True)
+    result = make()(dev(weight))
+    expected = scaling.quantize(weight, values, integer=integer, **kwargs)
+    np.testing.assert_array_equal(host(result.params["scales"]), expected["scales"])
+    np.testing.assert_array_equal(host(result.codes), expected["codes"])
+    if expected["zero"] is not None:
+        np.testing.assert_array_equal(host(result.params["zero"]), expected["zero"])
+    dense = scaling.decode_grouped(expected["codes"], expected["scales"], values, expected["group"], expected["zero"])
+    np.testing.assert_array_equal(host(result.w), dense)
+    assert result.bits == make().logical_bits(weight.shape)
+
+
+def test_scaled_rejects_non_finite_weights_on_device():
+    weight = torch.randn(8, 256, device="cuda")
+    weight[3, 17] = float("nan")
+    with pytest.raises(ValueError, match="finite"):
+        mk.int(4)(weight)
+
+
+def test_online_activation_reconstruction_equals_quantize_dequantize():
+    x = torch.randn(5, 512, device="cuda").half()
+    fmt = mk.int(8, group=128)
+    torch.testing.assert_close(fmt.reconstruct_activations(x), fmt(x.float()).w.half(), rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("values,integer,asym,group,refit,block", [
+    (scaling.int_values(4), True, False, 128, 128, 128),
+    (scaling.int_values(4), True, True, 64, 128, 64),      # two tiles per region
+    (scaling.NF4_VALUES, False, False, 64, 64, 128),
+    (scaling.int_values(3), True, False, 32, None, 128),   # one region: no refits
+])
+def test_gptq_on_device_matches_oracle_sweep(values, integer, asym, group, refit, block, rng):
+    rows, width = 80, 512
+    weight = helpers.normal_weight(rows, width, seed=32)
+    inputs = rng.standard_normal((1536, width)).astype(F32)
+    inputs[:, ::9] *= 5
+    inputs[:, 100] = 0
+    hessian = (inputs.T @ inputs / 1536).astype(F32)
+    grid = mk.grid.int(int(np.log2(len(values)))) if integer else mk.grid.values(values, bits=4)
+    inner = mk.scaled(grid, group=group, asym=asym)
+    quantizer = mk.gptq(inner, refit=refit, block_size=block)
+    context = Ctx("layer", H=dev(hessian))
+    result = quantizer(dev(weight), context)
+    # the coefficient matrix is an input of the sweep: hand the oracle the very same one
+    coeff = host(mk.feedback_coefficients(dev(hessian).clone(), 1)[0])
+    expected = oracle_feedback.sweep(weight, coeff, values, group=group, integer=integer, refit=refit, block=block,
+                                     asym=asym, dead=np.diag(hessian) == 0, update_mode=0)
+    np.testing.assert_array_equal(host(result.params["scales"]), expected["scales"])
+    np.testing.assert_array_equal(host(result.codes), expected["codes"])
+    np.testing.assert_array_equal(host(result.w), expected["w"])
+    assert result.codec == "feedback"
+    loss = float(mk.proxy_loss(dev(weight), result.w, dev(hessian)))
+    assert loss < float(mk.proxy_loss(dev(weight), inner(dev(weight)).w, dev(hessian)))
+    assert loss == pytest.approx(oracle_feedback.proxy_loss(weight, expected["w"], hessian), rel=1e-3)
+
+
+def test_gptq_full_width_layer_rows_match_oracle():
+    """N = 512 rows of the K = 11008 layer of the benchmark configuration (rows are
+    independent): the oracle sweeps the first 16 rows with the same coefficient matrix."""
+    rows, width, checked = 512, 11008, 16
+    generator = torch.Generator(device="cuda").manual_seed(33)
+    weight = (torch.randn((rows, width), device="cuda", generator=generator) * 0.02).half().float()
+    inputs = torch.randn((16384, width), device="cuda", generator=generator).half()
+    hot = torch.randperm(width, device="cuda", generator=generator)[: width // 100]
+    inputs[:, hot] *= 30
+    hessian = (inputs.float().T @ inputs.float()) / inputs.shape[0]
+    del inputs
+    result = mk.gptq(mk.int(4, group=128))(weight, Ctx("down_proj", H=hessian))
+    coeff = host(mk.feedback_coefficients(hessian.clone(), 1)[0])
+    expected = oracle_feedback.sweep(host(weight[:checked]), coeff, scaling.int_values(4), group=128, integer=True,
+                                     refit=128, block=128)
+    np.testing.assert_array_equal(host(result.codes[:checked]), expected["codes"])
+    np.testing.assert_array_equal(host(result.params["scales"][:checked]), expected["scales"])
+    rtn = mk.int(4, group=128)(weight).w
+    assert float(mk.proxy_loss(weight, result.w, hessian)) < 0.9 * float(mk.proxy_loss(weight, rtn, hessian))
+
+
+@pytest.mark.parametrize("width", [28, 96, 896, 4864, 4096, 14336])
+def test_rht_round_trip_and_oracle(width):
+    value = torch.randn((6, width), device="cuda")
+    rotated = mk.rht(value, seed=5)
+    torch.testing.assert_close(mk.rht(rotated, seed=5, inverse=True), value, rtol=1e-5, atol=2e-5)
+    torch.testing.assert_close(rotated.norm(dim=1), value.norm(dim=1), rtol=1e-5, atol=0)
+    from mlkit_amd.quantization.transforms import random_signs
+
+    signs = host(random_signs(width, 5, "cuda"))
+    np.testing.assert_allclose(host(rotated), oracle_transforms.randomized(host(value), signs), rtol=1e-5, atol=2e-5)
+
+
+def test_rotated_layer_keeps_its_outputs():
+    """Offline rotation of the weight columns plus online rotation of the inputs leaves the
+    product unchanged (14336-wide down projection, 28 x 512 Paley factorisation)."""
+    weight = torch.randn((256, 14336), device="cuda") * 0.02
+    x = torch.randn((2, 14336), device="cuda")
+    torch.testing.assert_close(mk.rht(x, seed=9) @ mk.rht(weight, seed=9).T, x @ weight.T, rtol=1e-3, atol=2e-3)
+    half = mk.rht(x.half(), seed=9)
+    assert half.dtype == torch.float16
+    torch.testing.assert_close(half.float(), mk.rht(x.half().float(), seed=9), rtol=2e-3, atol=2e-3)
+
+
+# ---- module level: mirrors of the reference's PackedLinear tests ---------------------------
+
+def packed_and_reference(fmt, *, input_width=256, output_width=37, dtype=torch.float32, calibration=None):
+    torch.manual_seed(40)
+    module = nn.Sequential(nn.Linear(input_width, output_width, dtype=dtype))
+    converted = mk.quantize(module, fmt, calib=None if calibration is None else [calibration], cache_dir=None)
+    packed = mk.optimize(converted, backend="packed")
+    assert isinstance(packed.module[0], mk.PackedLinear)
+    return packed, converted
+
+
+@pytest.mark.parametrize("name", ["int4", "nf4"])
+@pytest.mark.parametrize("batch", [1, 3, 7])
+def test_packed_linear_matches_dense(name, batch):
+    fmt = {"int4": mk.int(4, group=32), "nf4": mk.nf4(group=32)}[name]
+    torch.manual_seed(41)
+    module = nn.Sequential(nn.Linear(130, 71, dtype=torch.float16))
+    converted = mk.quantize(module, fmt, calib=None)
+    packed = mk.optimize(converted, backend="packed")
+    inputs = torch.randn(batch, 130, dtype=torch.float16)
+    with torch.inference_mode():
+        torch.testing.assert_close(packed(inputs), converted(inputs), rtol=0.002, atol=0.002)
+    assert isinstance(packed.module[0], mk.PackedLinear)
+    assert packed.module[0].packed.numel() == (130 * 71 + 1) // 2
+    assert packed.execution_backend == "packed:1"
+
+
+@pytest.mark.parametrize("rows", [1, 2, 5, 8, 9, 33])
+def test_packed_linear_handles_every_row_count(rows):
+    packed, converted = packed_and_reference(mk.int(4, group=64))
+    inputs = torch.randn(rows, 256)
+    with torch.inference_mode():
+        torch.testing.assert_close(packed(inputs), converted(inputs), rtol=1e-4, atol=1e-5)
+        nested = inputs.reshape(1, rows, 256)
+        torch.testing.assert_close(packed(nested), converted(nested), rtol=1e-4, atol=1e-5)
+
+
+def test_packed_linear_applies_asymmetric_offsets():
+    packed, converted = packed_and_reference(mk.int(4, group=64, asym=True))
+    assert packed.module[0].zeros is not None
+    for rows in (1, 3, 20):
+        inputs = torch.randn(rows, 256)
+        with torch.inference_mode():
+            torch.testing.assert_close(packed(inputs), converted(inputs), rtol=1e-4, atol=1e-5)
+
+
+def test_packed_linear_executes_error_feedback_codecs():
+    calibration = torch.randn(512, 256)
+    packed, converted = packed_and_reference(mk.gptq(mk.int(4, group=64), refit=64), calibration=calibration)
+    assert converted.quantized["0"].codec == "feedback"
+    inputs = torch.randn(3, 256)
+    with torch.inference_mode():
+        torch.testing.assert_close(packed(inputs), converted(inputs), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("input_width,group", [(255, 64), (256, 5), (250, 20)])
+def test_layouts_that_split_a_packing_word_use_dense_reconstruction(input_width, group):
+    packed, converted = packed_and_reference(mk.int(4, group=group), input_width=input_width)
+    layer = packed.module[0]
+    assert layer.layout is None and layer.maximum_fused_rows == 0
+    inputs = torch.randn(2, input_width)
+    with torch.inference_mode():
+        torch.testing.assert_close(packed(inputs), converted(inputs), rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(layer.weight, converted.module[0].weight, rtol=1e-6, atol=1e-7)
+
+
+def test_packed_weight_reconstruction_matches_the_converted_layer():
+    for fmt in (mk.int(4, group=64), mk.nf4(group=32), mk.int(4, group=64, asym=True)):
+        packed, converted = packed_and_reference(fmt)
+        torch.testing.assert_close(packed.module[0].weight, converted.module[0].weight, rtol=1e-6, atol=1e-7)
+
+
+def test_packed_linear_can_be_copied_and_cast_after_launching():
+    packed, converted = packed_and_reference(mk.int(4, group=64), dtype=torch.float16)
+    inputs = torch.randn(1, 256, dtype=torch.float16)
+    with torch.inference_mode():
+        expected = packed(inputs)
+        duplicate = copy.deepcopy(packed)
+        torch.testing.assert_close(duplicate(inputs), expected, rtol=0, atol=0)
+        single = duplicate.module[0].float()
+        result = single(inputs.float().cuda())
+        torch.testing.assert_close(result, expected.float(), rtol=2e-3, atol=2e-3)
+        assert result.dtype == torch.float32
+
+
+WIDTH_FORMATS = {
+    "int2": lambda: mk.int(2, group=64),
+    "int3": lambda: mk.int(3, group=64),
+    "int5": lambda: mk.int(5, group=64),
+    "int6": lambda: mk.int(6, group=32),
+    "int7": lambda: mk.int(7, group=64),
+    "int8": lambda: mk.int(8, group=128),
+    "int3-asymmetric": lambda: mk.int(3, group=64, asym=True),
+    "e4m3": lambda: mk.scaled(mk.grid.fp("e4m3"), group=64),
+    "codebook3": lambda: mk.scaled(mk.grid.values(torch.linspace(-1, 1, 7).pow(3), bits=3), group=32),
+}
+
+
+@pytest.mark.parametrize("name", WIDTH_FORMATS)
+@pytest.mark.parametrize("rows", [1, 3, 20])
+def test_packed_linear_executes_every_code_width(name, rows):
+    packed, converted = packed_and_reference(WIDTH_FORMATS[name]())
+    layer = packed.module[0]
+    bits = converted.quantized["0"].metadata["code_bits"]
+    assert layer.layout is not None
+    assert layer.packed.numel() == 37 * 256 * bits // 8
+    inputs = torch.randn(rows, 256)
+    with torch.inference_mode():
+        torch.testing.assert_close(packed(inputs), converted(inputs), rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(layer.weight, converted.module[0].weight, rtol=1e-6, atol=1e-7)
+
+
+def test_three_bit_rows_that_split_a_word_use_dense_reconstruction():
+    packed, converted = packed_and_reference(mk.int(3, group=50), input_width=250)
+    assert packed.module[0].layout is None
+    inputs = torch.randn(2, 250)
+    with torch.inference_mode():
+        torch.testing.assert_close(packed(inputs), converted(inputs), rtol=1e-4, atol=1e-5)
+
+
+def test_wide_codes_remain_dense():
+    converted = mk.quantize(nn.Sequential(nn.Linear(64, 16)), mk.int(12, group=32), calib=None)
+    packed = mk.optimize(converted, backend="packed")
+    assert isinstance(packed.module[0], nn.Linear)
+    assert packed.execution_backend == "packed:0"
+    assert mk.optimize(converted, backend="dense").execution_backend == "dense"
+    with pytest.raises(ValueError, match="backend must be"):
+        mk.optimize(converted, backend="other")
+    with pytest.raises(ValueError, match="QModel"):
+        mk.optimize(nn.Linear(4, 4), backend="packed")
+
+
+def test_packed_linear_input_validation():
+    packed, _ = packed_and_reference(mk.int(4, group=64))
+    layer = packed.module[0]
+    with pytest.raises(ValueError, match="input width"):
+        layer(torch.randn(1, 128, device="cuda"))
+    with pytest.raises(ValueError, match="CUDA inputs"):
+        layer(torch.randn(1, 256))
+    with pytest.raises(RuntimeError, match="autograd"):
+        layer(torch.randn(1, 256, device="cuda", requires_grad=True))
+    with pytest.raises(ValueError, match="PackedLinear requires"):
+        mk.PackedLinear(nn.Linear(8, 8).cuda(), mk.Q(torch.zeros(8, 8)))
+
+
+class TiedHead(nn.Module):
+    def __init__(self, vocabulary=300, width=128):
+        super().__init__()
+        self.embed = nn.Embedding(vocabulary, width)
+        self.head = nn.Linear(width, vocabulary, bias=False)
+        self.head.weight = self.embed.weight
+
+    def forward(self, tokens):
+        return self.head(self.embed(tokens))
+
+
+def test_embedding_tied_to_a_packed_head_reads_the_packed_rows():
+    torch.manual_seed(42)
+    converted = mk.quantize(TiedHead(), mk.int(4, group=64), calib=None)
+    assert converted.tied_weights == {"embed.weight": "head"}
+    packed = mk.optimize(converted, backend="packed")
+    assert isinstance(packed.module.embed, mk.PackedEmbedding) and isinstance(packed.module.head, mk.PackedLinear)
+    tokens = torch.tensor([[0, 5, 299], [17, 17, 1]], device="cuda")
+    dense = converted.quantized["head"].w.cuda()
+    torch.testing.assert_close(packed.module.embed(tokens), dense[tokens], rtol=0, atol=0)
+    with torch.inference_mode():
+        torch.testing.assert_close(packed(tokens), converted(tokens), rtol=1e-4, atol=1e-4)
+
+
+def test_checkpoint_round_trip(tmp_path):
+    torch.manual_seed(43)
+    module = nn.Sequential(nn.Linear(64, 48), nn.ReLU(), nn.Linear(48, 16, bias=False))
+    converted = mk.quantize(module, mk.int(4, group=16, asym=True), calib=None)
+    inputs = torch.randn(4, 64)
+    expected = converted(inputs)
+    mk.save(converted, tmp_path / "checkpoint")
+    with pytest.raises(FileExistsError):
+        mk.save(converted, tmp_path / "checkpoint")
+    restored = mk.load_checkpoint(tmp_path / "checkpoint",
+                                  model=lambda: nn.Sequential(nn.Linear(64, 48), nn.ReLU(), nn.Linear(48, 16, bias=False)))
+    torch.testing.assert_close(restored(inputs), expected, rtol=0, atol=0)
+    assert restored.quantized["0"].codec == "scaled" and restored.quantized["0"].bits == converted.quantized["0"].bits
+    packed = mk.optimize(restored)
+    assert packed.execution_backend == "packed:2"
+    with torch.inference_mode():
+        torch.testing.assert_close(packed(inputs), expected, rtol=1e-4, atol=1e-5)
+    mk.save(converted, tmp_path / "checkpoint", overwrite=True)
+    assert (tmp_path / "checkpoint" / "mlkit.json").exists() and (tmp_path / "checkpoint" / "weights.safetensors").exists()
+
+
+def test_capabilities_on_device():
+    report = mk.capabilities(mk.int(4, group=128))
+    assert report.bits_per_weight == 4.125 and report.codec == "scaled"
+    assert report.error_feedback == "fused scalar kernel at step=1"
+    assert report.packed_inference == "fused kernel" and report.online_activations == "fused kernel"
+    assert mk.capabilities(mk.gptq(mk.int(4))).packed_inference == "fused kernel"
+    assert mk.capabilities(mk.int(3, group=50), shape=(16, 250)).packed_inference.startswith("packed storage with dense")
