@@ -140,6 +140,136 @@ def cpu_baseline():
     }
 
 
+def _time(function, repeats=20, warmup=3):
+    """Milliseconds per call by HIP events on the current stream (where the kernels launch)."""
+    for _ in range(warmup):
+        function()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    begin.record()
+    for _ in range(repeats):
+        function()
+    end.record()
+    torch.cuda.synchronize()
+    return begin.elapsed_time(end) / repeats
+
+
+def other_kernels(device: torch.device) -> dict:
+    """Timings of the other kernels of the path at the shapes of the benchmark configurations
+    (`--kernels`); each entry carries its algorithmic bytes or flops and the rate they give."""
+    import mlkit_amd as mk
+    from mlkit_amd.kernels import hadamard, packed_linear, scalar_decode, scalar_encode
+    from mlkit_amd.quantization.core import Ctx
+
+    out = {}
+    generator = torch.Generator(device=device).manual_seed(1)
+    weight = (torch.randn((ROWS, WIDTH), device=device, generator=generator) * 0.02).half().float()
+    elements = ROWS * WIDTH
+    values = torch.arange(-8, 8, dtype=torch.float32, device=device)
+
+    def entry(ms, nbytes=None, flops=None, **extra):
+        record = {"ms": ms, **extra}
+        if nbytes is not None:
+            record.update(bytes=nbytes, GBps=nbytes / ms / 1e6, hbm_frac=nbytes / ms / 1e6 / HBM_PEAK_GBPS)
+        if flops is not None:
+            record.update(flops=flops, TFLOPs=flops / ms / 1e9)
+        return record
+
+    fit = lambda: scalar_encode.fit_scales(weight, GROUP, asym=False, reciprocal=0.125, value_minimum=-8.0,  # noqa: E731
+                                           scale_format="fp16", store_zero=False)
+    scales, _ = fit()
+    out["fit_scales 4096x14336 g128"] = entry(_time(fit), elements * 4 + scales.numel() * 4)
+    encode = lambda: scalar_encode.encode(weight, scales, None, values, GROUP, None, integer=True,  # noqa: E731
+                                          minimum=-8.0, maximum=7.0)
+    codes = encode()
+    out["encode int4 4096x14336 g128"] = entry(_time(encode), elements * 5 + scales.numel() * 4)
+    out["decode codes 4096x14336 g128"] = entry(
+        _time(lambda: scalar_decode.decode(codes, scales, values, None, GROUP)), elements * 5 + scales.numel() * 4)
+    seven = torch.tensor([-1, -0.5, -0.25, 0, 0.25, 0.5, 1], device=device)
+    fractions = torch.linspace(0.5, 1.0, 20, device=device)
+    square = weight[:, :4096].contiguous()
+    base, _ = scalar_encode.fit_scales(square, 64, asym=False, reciprocal=1.0, value_minimum=-1.0,
+                                       scale_format="fp16", store_zero=False)
+    out["search_scales codebook7 4096x4096 g64, 21 candidates"] = entry(
+        _time(lambda: scalar_encode.search_scales(square, base, None, seven, fractions, 64, None, "fp16",
+                                                  integer=False, minimum=-1.0, maximum=1.0), repeats=5),
+        4096 * 4096 * 4 + 2 * base.numel() * 4)
+    packed = mk.pack(codes[:8], 4)  # layout only; the timed stream is synthetic
+    packed = torch.randint(0, 256, (CODE_BYTES,), dtype=torch.uint8, device=device, generator=generator)
+    dense = torch.empty((ROWS, WIDTH), device=device, dtype=torch.float16)
+    layout = packed_linear.layout_for(BITS, WIDTH, GROUP)
+    half_scales = scales.half()
+    out["packed decode int4 4096x14336 -> fp16"] = entry(
+        _time(lambda: packed_linear.decode(packed, half_scales, values, None, dense, GROUP, layout, True, -8.0, 1.0)),
+        CODE_BYTES + SCALE_BYTES + elements * 2)
+
+    rotated = torch.empty_like(weight)
+    out["fwht 4096x14336 fp32 as 7x2048 blocks"] = entry(
+        _time(lambda: hadamard.transform(weight.view(ROWS, 7, 2048), out=rotated.view(ROWS, 7, 2048))), elements * 8)
+    tall = weight.view(WIDTH, ROWS)
+    out["fwht 14336x4096 fp32"] = entry(_time(lambda: hadamard.transform(tall, out=rotated.view(WIDTH, ROWS))), elements * 8)
+    out["rht 4096x14336 fp32 (28x512 Paley: fwht + basis mix)"] = entry(
+        _time(lambda: mk.rht(weight, seed=3), repeats=5), elements * 8, launches=2)
+    for samples in (1, 8):
+        for width in (4096, 14336):
+            x = torch.randn((samples, width), device=device, generator=generator).half()
+            out[f"rht activations M={samples} K={width} fp16"] = {"us": _time(lambda: mk.rht(x, seed=3), 50) * 1e3}
+
+    # other matvec shapes and codecs, M = 1 and 8 (eager launches, one weight copy each)
+    def matvec(rows, width, group, bits, table, uniform, asym, label):
+        layout = packed_linear.layout_for(bits, width, group)
+        stream = torch.randint(0, 256, (rows * width * bits // 8,), dtype=torch.uint8, device=device, generator=generator)
+        side = (torch.rand((rows, width // group), device=device, generator=generator) * 0.004 + 0.005).half()
+        zeros = side.clone() if asym else None
+        for samples in (1, 8):
+            x = torch.randn((samples, width), device=device, generator=generator).half()
+            y = torch.empty((samples, rows), device=device, dtype=torch.float16)
+            ms = _time(lambda: packed_linear.matrix_vector(x, stream, side, table, zeros, None, y, group, layout,
+                                                           uniform_grid=uniform, grid_minimum=float(table[0]),
+                                                           grid_step=float(table[1] - table[0])), 200, 20)
+            nbytes = stream.numel() + side.numel() * 2 * (2 if asym else 1) + samples * (width + rows) * 2
+            out[f"matvec {label} {rows}x{width} M={samples}"] = entry(ms, nbytes)
+
+    nf4 = mk.NF4_VALUES.to(device)
+    matvec(4096, 4096, 128, 4, values, True, True, "int4 asym g128")
+    matvec(ROWS, WIDTH, 64, 2, torch.arange(-2, 2, dtype=torch.float32, device=device), True, False, "int2 g64")
+    matvec(ROWS, WIDTH, 64, 3, torch.arange(-4, 4, dtype=torch.float32, device=device), True, False, "int3 g64")
+    matvec(ROWS, WIDTH, 64, 4, nf4, False, False, "nf4 g64")
+    matvec(ROWS, WIDTH, 64, 3, seven, False, False, "codebook7 g64")
+    matvec(151936, 896, 128, 4, values, True, False, "int4 g128 (tied head)")
+    del weight, rotated, dense, codes
+
+    # GPTQ, INT4 g128, 4096 x 11008, refit = block = 128 (Hessian and Cholesky timed apart)
+    rows, width = 4096, 11008
+    target = (torch.randn((rows, width), device=device, generator=generator) * 0.02).half().float()
+    inputs = torch.randn((16384, width), device=device, generator=generator).half()
+    hot = torch.randperm(width, device=device, generator=generator)[: width // 100]
+    inputs[:, hot] *= 30
+    hessian = (inputs.float().T @ inputs.float()) / inputs.shape[0]
+    del inputs
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    mk.feedback_coefficients(hessian.clone(), 1)
+    torch.cuda.synchronize()
+    factor_ms = (time.perf_counter() - started) * 1e3
+    quantizer = mk.gptq(mk.int(4, group=128))
+    quantizer(target, Ctx("warmup", H=hessian))
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    result = quantizer(target, Ctx("down_proj", H=hessian))
+    torch.cuda.synchronize()
+    total_ms = (time.perf_counter() - started) * 1e3
+    update_flops = sum(2 * rows * 128 * (width - stop) for stop in range(128, width, 128))
+    rtn = mk.int(4, group=128)(target)
+    out["gptq int4 g128 4096x11008"] = {
+        "total_ms": total_ms, "coefficients_ms": factor_ms, "sweep_and_update_ms": total_ms - factor_ms,
+        "columns_per_s": width / ((total_ms - factor_ms) / 1e3), "trailing_update_flops": update_flops,
+        "proxy_loss": float(mk.proxy_loss(target, result.w, hessian)),
+        "rtn_proxy_loss": float(mk.proxy_loss(target, rtn.w, hessian)),
+    }
+    return out
+
+
 def main() -> None:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -148,6 +278,8 @@ def main() -> None:
     parser.add_argument("--copies", type=int, default=18)
     parser.add_argument("--no-graph", action="store_true")
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--kernels", action="store_true",
+                        help="also time the other kernels of the path (adds a `kernels` object to the line)")
     parser.add_argument("--profile-launches", type=int, default=0,
                         help="for rocprofv3: only launch the M=1 matvec this many times, plus three "
                              "256 MiB device copies whose counters calibrate FETCH_SIZE / WRITE_SIZE")
@@ -227,6 +359,10 @@ def main() -> None:
         },
         "cpu_baseline": None if options.no_cpu_baseline else cpu_baseline(),
     }
+    if options.kernels:
+        del copies, launchers
+        torch.cuda.empty_cache()
+        line["kernels"] = other_kernels(device)
     print(json.dumps(line))
 
 
