@@ -47,15 +47,16 @@ def make_copies(count: int, device: torch.device):
 class Launcher:
     """Pre-bound arguments of mk_packed_matvec for one (weight copy, M)."""
 
-    def __init__(self, x, packed, scales, values, y):
+    def __init__(self, x, packed, scales, values, y, *, zeros=None, rows=ROWS, width=WIDTH, group=GROUP,
+                 bits=BITS, uniform=True, grid_min=-8.0, grid_step=1.0):
         from mlkit_amd import native
 
         self.function = native.library().mk_packed_matvec
-        self.keep = (x, packed, scales, values, y)
+        self.keep = (x, packed, scales, values, y, zeros)
         self.arguments = (
             x.data_ptr(), native.MK_F16, packed.data_ptr(), scales.data_ptr(), native.MK_F16,
-            values.data_ptr(), 16, None, None, 0, y.data_ptr(), x.shape[0], ROWS, WIDTH, GROUP,
-            BITS, 1, -8.0, 1.0,
+            values.data_ptr(), values.numel(), None if zeros is None else zeros.data_ptr(), None, 0,
+            y.data_ptr(), x.shape[0], rows, width, group, bits, int(uniform), grid_min, grid_step,
         )
 
     def __call__(self, stream: int) -> None:
@@ -215,20 +216,24 @@ def other_kernels(device: torch.device) -> dict:
             x = torch.randn((samples, width), device=device, generator=generator).half()
             out[f"rht activations M={samples} K={width} fp16"] = {"us": _time(lambda: mk.rht(x, seed=3), 50) * 1e3}
 
-    # other matvec shapes and codecs, M = 1 and 8 (eager launches, one weight copy each)
+    # other matvec shapes and codecs, M = 1 and 8: HIP-graph launches through the C ABI over
+    # enough distinct weight copies (> 512 MB) that the Infinity Cache cannot serve them
     def matvec(rows, width, group, bits, table, uniform, asym, label):
-        layout = packed_linear.layout_for(bits, width, group)
-        stream = torch.randint(0, 256, (rows * width * bits // 8,), dtype=torch.uint8, device=device, generator=generator)
+        code_bytes = rows * width * bits // 8
+        count = max(2, min(40, -(-(512 * 2**20) // code_bytes)))
+        streams = [torch.randint(0, 256, (code_bytes,), dtype=torch.uint8, device=device, generator=generator)
+                   for _ in range(count)]
         side = (torch.rand((rows, width // group), device=device, generator=generator) * 0.004 + 0.005).half()
         zeros = side.clone() if asym else None
         for samples in (1, 8):
             x = torch.randn((samples, width), device=device, generator=generator).half()
             y = torch.empty((samples, rows), device=device, dtype=torch.float16)
-            ms = _time(lambda: packed_linear.matrix_vector(x, stream, side, table, zeros, None, y, group, layout,
-                                                           uniform_grid=uniform, grid_minimum=float(table[0]),
-                                                           grid_step=float(table[1] - table[0])), 200, 20)
-            nbytes = stream.numel() + side.numel() * 2 * (2 if asym else 1) + samples * (width + rows) * 2
-            out[f"matvec {label} {rows}x{width} M={samples}"] = entry(ms, nbytes)
+            launchers = [Launcher(x, stream, side, table, y, zeros=zeros, rows=rows, width=width, group=group,
+                                  bits=bits, uniform=uniform, grid_min=float(table[0]),
+                                  grid_step=float(table[1] - table[0])) for stream in streams]
+            _, seconds, _ = timed_region(launchers, 400, 40)
+            nbytes = code_bytes + side.numel() * 2 * (2 if asym else 1) + samples * (width + rows) * 2
+            out[f"matvec {label} {rows}x{width} M={samples}"] = entry(seconds / 400 * 1e3, nbytes, copies=count)
 
     nf4 = mk.NF4_VALUES.to(device)
     matvec(4096, 4096, 128, 4, values, True, True, "int4 asym g128")

@@ -203,6 +203,16 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
         s4.groups = groups; s4.bias_dtype = bias_dtype; s4.grid_min = grid_min; s4.grid_step = grid_step;
         done_rows = mk_matvec::stream4_launch(s4, stream);
         if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
+    } else if (aligned && !tuning("MK_MATVEC_NO_PAIRS", 0) &&
+               mk_matvec::pairs_accepts(input_width, group, bits, x_dtype, scale_dtype) &&
+               (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
+        mk_matvec::Stream4Args s4;
+        s4.x = x; s4.packed = packed; s4.scales = scales; s4.zeros = zeros; s4.bias = bias; s4.y = y;
+        s4.samples = samples; s4.rows = output_width; s4.width = input_width; s4.group = group;
+        s4.groups = groups; s4.bias_dtype = bias_dtype; s4.grid_min = grid_min; s4.grid_step = grid_step;
+        s4.values = values; s4.n_values = n_values; s4.uniform = uniform; s4.bits = bits;
+        done_rows = mk_matvec::pairs_launch(s4, stream);
+        if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
     } else if (aligned && plan_chunked(samples, output_width, input_width, group, groups, bits, x_dtype,
                                 uniform != 0, zeros != nullptr, plan)) {
         const int tile_rows = plan.rows_parallel * plan.rows_per_thread;

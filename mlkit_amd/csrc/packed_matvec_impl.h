@@ -63,7 +63,12 @@ struct Stream4Args {
     void *y;              // fp16 [samples, rows]
     int samples, rows, width, group, groups, bias_dtype;
     float grid_min, grid_step;
+    const float *values;  // fp32 table (pair-table kernel, when uniform == 0)
+    int n_values, uniform, bits;
 };
+// Pair-table kernel (packed_matvec_pairs.hip): 2-, 3- and 4-bit codes of any scalar grid.
+bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype);
+int pairs_launch(const Stream4Args &a, hipStream_t stream);
 bool stream4_accepts(int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
 

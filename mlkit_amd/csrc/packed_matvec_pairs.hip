@@ -1,0 +1,213 @@
+// Packed matvec for 2-, 3- and 4-bit codes of any scalar grid (integer grids, NF4, small
+// codebooks) with fp16 activations and fp16 scales, rows of K = 32 ... 16384 codes (K % 32 == 0).
+//
+// Two adjacent codes index a table of fp16 pairs (value[low], value[high]) held in LDS, so
+// one LDS read decodes two weights and one v_dot2_f32_f16 multiplies them with the
+// matching pair of activations, accumulating in fp32.  Table entries are the grid values
+// rounded to fp16 (exact for integer grids and minifloats; NF4-like tables lose at most
+// 2^-11 relative per weight, inside the fp16 output's own rounding).  Entries of different
+// pairs fall in different LDS banks except by coincidence, so the lookups mostly proceed
+// at full rate.  Work split, load order and the reduction are those of the 4-bit streaming
+// kernel: a workgroup of ceil(K/2048) wavefronts owns 16 rows; lane t owns codes [32t, 32t + 32)
+// of every row; codes are requested eight rows ahead; per-wavefront row sums meet in LDS in
+// a fixed order.
+//
+// Replaces the reference's Triton kernel `packed_matrix_vector`
+// (kernels/packed_linear.py:107-173 in /root/reference/src/mlkit) for these layouts.
+
+#include "packed_matvec_impl.h"
+
+namespace mk_matvec {
+
+namespace {
+
+constexpr int kPairRows = 16;
+constexpr int kPairAhead = 8;
+
+template <int MT>
+constexpr int pair_reduce_rows() {
+    return kPairRows * MT <= 64 ? kPairRows : 64 / MT;
+}
+
+// Field i (0..15) of 2*BITS bits out of a chunk of BITS dwords, times four (a byte offset
+// into the table).  i is a compile-time constant after unrolling.
+template <int BITS>
+__device__ __forceinline__ uint32_t pair_offset(const CodeChunk<BITS> &c, int i) {
+    constexpr int kField = 2 * BITS;
+    constexpr uint32_t mask = ((1u << kField) - 1u) << 2;
+    const int bit = i * kField;
+    const int word = bit >> 5, shift = bit & 31;
+    if (shift + kField <= 32) {
+        if (shift >= 2) return (c.w[word] >> (shift - 2)) & mask;
+        return (c.w[word] << (2 - shift)) & mask;
+    }
+    return (__builtin_amdgcn_alignbit(c.w[(word + 1) % BITS], c.w[word], shift) << 2) & mask;
+}
+
+template <int BITS, int MT, bool HAS_ZERO>
+__global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
+    constexpr int kEntries = 1 << (2 * BITS);
+    __shared__ uint32_t table[kEntries];  // fp16 pairs
+    __shared__ float partials[64 * 8];    // [row sum][wavefront]
+    constexpr int kReduceRows = pair_reduce_rows<MT>();
+    constexpr int kSums = kReduceRows * MT;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int waves = blockDim.x >> 6;
+    const int row_base = blockIdx.x * kPairRows;
+    const int sample_base = blockIdx.y * MT;
+    const uint32_t row_bytes = (static_cast<uint32_t>(a.width) * BITS) >> 3;
+    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
+    // Lanes past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
+    // activations: they add nothing.
+    const bool in_row = tid * kChunkCodes < a.width;
+    const int chunk = in_row ? tid : 0;
+    const uint32_t code_offset = static_cast<uint32_t>(chunk) * (4u * BITS);
+
+    for (int entry = tid; entry < kEntries; entry += blockDim.x) {
+        const int low = entry & ((1 << BITS) - 1), high = entry >> BITS;
+        float first, second;
+        if (a.uniform) {
+            first = __builtin_fmaf(static_cast<float>(low), a.grid_step, a.grid_min);
+            second = __builtin_fmaf(static_cast<float>(high), a.grid_step, a.grid_min);
+        } else {
+            first = low < a.n_values ? a.values[low] : 0.0f;
+            second = high < a.n_values ? a.values[high] : 0.0f;
+        }
+        const mk_h2 pair = {static_cast<_Float16>(first), static_cast<_Float16>(second)};
+        table[entry] = __builtin_bit_cast(uint32_t, pair);
+    }
+    // Also aligns the wavefronts, so that nobody's small loads queue behind another's codes.
+    __syncthreads();
+
+    XChunk<MK_F16> x[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int sample = sample_base + m < a.samples ? sample_base + m : a.samples - 1;
+        load_x_chunk<MK_F16>(x[m], a.x, static_cast<size_t>(sample) * a.width + static_cast<size_t>(chunk) * kChunkCodes);
+    }
+    const uint32_t group_offset = ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
+    const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
+    const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
+    const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
+                                        : nullptr;
+    uint16_t scale_raw[kPairRows], zero_raw[HAS_ZERO ? kPairRows : 1];
+#pragma unroll
+    for (int r = 0; r < kPairRows; ++r) {
+        scale_raw[r] = *reinterpret_cast<const uint16_t *>(scale_base + static_cast<size_t>(r) * scale_row_bytes + group_offset);
+        if constexpr (HAS_ZERO)
+            zero_raw[r] = *reinterpret_cast<const uint16_t *>(zero_base + static_cast<size_t>(r) * scale_row_bytes + group_offset);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    CodeChunk<BITS> codes[kPairRows];
+#pragma unroll
+    for (int r = 0; r < kPairAhead; ++r) {
+        load_codes<BITS>(codes[r], codes_base + static_cast<size_t>(r) * row_bytes + code_offset);
+        __builtin_amdgcn_sched_barrier(0);  // in row order
+    }
+
+    float x_sum[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const uint32_t keep = in_row && sample_base + m < a.samples ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) x[m].r[i] &= keep;
+        x_sum[m] = HAS_ZERO ? chunk_sum<MK_F16>(x[m]) : 0.0f;
+    }
+
+    const uint8_t *table_bytes = reinterpret_cast<const uint8_t *>(table);
+#pragma unroll
+    for (int pass = 0; pass < kPairRows / kReduceRows; ++pass) {
+        float sums[kSums];
+#pragma unroll
+        for (int j = 0; j < kReduceRows; ++j) {
+            const int r = pass * kReduceRows + j;
+            float dot[MT];
+#pragma unroll
+            for (int m = 0; m < MT; ++m) dot[m] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t entry = *reinterpret_cast<const uint32_t *>(table_bytes + pair_offset<BITS>(codes[r], i));
+                const mk_h2 weights = __builtin_bit_cast(mk_h2, entry);
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    dot[m] = __builtin_amdgcn_fdot2(weights, __builtin_bit_cast(mk_h2, x[m].r[i]), dot[m], false);
+            }
+            if (r + kPairAhead < kPairRows)
+                load_codes<BITS>(codes[r + kPairAhead],
+                                 codes_base + static_cast<size_t>(r + kPairAhead) * row_bytes + code_offset);
+            const float scale = static_cast<float>(__builtin_bit_cast(_Float16, scale_raw[r]));
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                float value = scale * dot[m];
+                if constexpr (HAS_ZERO)
+                    value = __builtin_fmaf(static_cast<float>(__builtin_bit_cast(_Float16, zero_raw[r])), x_sum[m], value);
+                sums[j * MT + m] = value;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        transposed_wave_sum<kSums>(sums, lane);
+        if (pass > 0) __syncthreads();
+        if (lane < kSums) partials[transposed_value_of_lane<kSums>(lane) * 8 + wave] = sums[0];
+        __syncthreads();
+        if (tid < kSums) {
+            float total = partials[tid * 8];
+#pragma unroll
+            for (int w = 1; w < 8; ++w) total += w < waves ? partials[tid * 8 + w] : 0.0f;
+            const int j = tid / MT, m = tid - j * MT;
+            const int row = row_base + pass * kReduceRows + j;
+            const int sample = sample_base + m;
+            if (sample < a.samples) {
+                if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
+                static_cast<_Float16 *>(a.y)[static_cast<size_t>(sample) * a.rows + row] = static_cast<_Float16>(total);
+            }
+        }
+    }
+}
+
+template <int BITS, int MT>
+void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
+    const dim3 grid(tiles, mk_cdiv(a.samples, MT));
+    const dim3 block(mk_cdiv(a.width, 2048) * 64);
+    if (a.zeros)
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true>), grid, block, 0, stream, a);
+    else
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false>), grid, block, 0, stream, a);
+}
+
+template <int BITS>
+void launch_bits(const Stream4Args &a, int tiles, hipStream_t stream) {
+    int tile = 1;
+    while (tile < a.samples && tile < 8) tile <<= 1;
+    switch (tile) {
+        case 1: launch_tile<BITS, 1>(a, tiles, stream); break;
+        case 2: launch_tile<BITS, 2>(a, tiles, stream); break;
+        case 4: launch_tile<BITS, 4>(a, tiles, stream); break;
+        default: launch_tile<BITS, 8>(a, tiles, stream); break;
+    }
+}
+
+}  // namespace
+
+bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype) {
+    return bits >= 2 && bits <= 4 && x_dtype == MK_F16 && scale_dtype == MK_F16 && width % kChunkCodes == 0 &&
+           width <= 16384 && (group % kChunkCodes == 0 || group >= width);
+}
+
+// Multiplies rows [0, 16 * tiles); returns the number of rows covered.
+int pairs_launch(const Stream4Args &a, hipStream_t stream) {
+    const int tiles = a.rows / kPairRows;
+    if (tiles == 0) return 0;
+    switch (a.bits) {
+        case 2: launch_bits<2>(a, tiles, stream); break;
+        case 3: launch_bits<3>(a, tiles, stream); break;
+        default: launch_bits<4>(a, tiles, stream); break;
+    }
+    return tiles * kPairRows;
+}
+
+}  // namespace mk_matvec

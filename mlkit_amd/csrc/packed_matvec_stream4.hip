@@ -1,5 +1,5 @@
 // 4-bit uniform-grid packed matvec with fp16 activations and fp16 scales: the decode-time
-// kernel for INT4 layers whose rows are whole multiples of 2048 codes (K = 2048 ... 16384).
+// kernel for INT4 layers whose rows are whole multiples of 32 codes (K = 32 ... 16384).
 //
 // The kernel is bound by whichever is larger: the HBM stream of the codes, or the vector
 // ALU time of the busiest SIMD (a wavefront issues one vector instruction per four
@@ -9,7 +9,7 @@
 // loaded by the lane that uses them, nine vector instructions per eight codes, and one
 // transposed reduction for all rows of a wavefront instead of one reduction per row.
 //
-// Work split: a workgroup of K/2048 wavefronts multiplies 16 adjacent rows; lane `tid`
+// Work split: a workgroup of ceil(K/2048) wavefronts multiplies 16 adjacent rows; lane `tid`
 // owns codes [32 tid, 32 tid + 32) of every row and keeps the matching activations of
 // all samples in registers.  Codes are requested eight rows ahead of the row being
 // summed.  Per-wavefront row sums meet in LDS in a fixed order, so results do not depend
@@ -48,7 +48,11 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     const int sample_base = blockIdx.y * MT;
     const uint32_t row_bytes = static_cast<uint32_t>(a.width) >> 1;
     const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
-    const uint32_t code_offset = static_cast<uint32_t>(tid) * 16u;
+    // Lanes past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
+    // activations: they add nothing.
+    const bool in_row = tid * kChunkCodes < a.width;
+    const int chunk = in_row ? tid : 0;
+    const uint32_t code_offset = static_cast<uint32_t>(chunk) * 16u;
 
     // The workgroup is aligned first: a compute unit serves loads first come, first served,
     // and a wavefront that starts late would queue its small loads behind the others' codes.
@@ -59,10 +63,10 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int sample = sample_base + m < a.samples ? sample_base + m : a.samples - 1;
-        load_x_chunk<MK_F16>(x[m], a.x, static_cast<size_t>(sample) * a.width + static_cast<size_t>(tid) * kChunkCodes);
+        load_x_chunk<MK_F16>(x[m], a.x, static_cast<size_t>(sample) * a.width + static_cast<size_t>(chunk) * kChunkCodes);
     }
     // The scale (and offset) of this lane's chunk in every row, 2 bytes each.
-    const uint32_t group_offset = ((static_cast<uint32_t>(tid) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
+    const uint32_t group_offset = ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
     const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
     const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
@@ -87,7 +91,7 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     float x_sum[MT], grid_term[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-        const uint32_t keep = sample_base + m < a.samples ? 0xffffffffu : 0u;
+        const uint32_t keep = in_row && sample_base + m < a.samples ? 0xffffffffu : 0u;
 #pragma unroll
         for (int i = 0; i < 16; ++i) x[m].r[i] &= keep;
         x_sum[m] = chunk_sum<MK_F16>(x[m]);
@@ -141,7 +145,7 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
 template <int MT>
 void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
-    const dim3 block(a.width / 32);
+    const dim3 block(mk_cdiv(a.width, 2048) * 64);
     if (a.zeros)
         hipLaunchKernelGGL((stream4_kernel<MT, true>), grid, block, 0, stream, a);
     else
@@ -151,7 +155,7 @@ void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
 }  // namespace
 
 bool stream4_accepts(int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform) {
-    return bits == 4 && uniform && x_dtype == MK_F16 && scale_dtype == MK_F16 && width % 2048 == 0 &&
+    return bits == 4 && uniform && x_dtype == MK_F16 && scale_dtype == MK_F16 && width % kChunkCodes == 0 &&
            width <= 16384 && (group % kChunkCodes == 0 || group >= width);
 }
 

@@ -150,10 +150,16 @@ def structured_transform(value: Tensor, *, inverse: bool = False) -> Tensor:
     return rotate(value, inverse=inverse)
 
 
-def random_signs(width: int, seed: int, device: torch.device | str, dtype: torch.dtype = torch.float32) -> Tensor:
-    """The +-1 vector ``randomized_transform`` draws for ``seed`` on ``device``."""
+@functools.lru_cache(maxsize=256)
+def _cached_signs(width: int, seed: int, device: torch.device) -> Tensor:
     generator = torch.Generator(device=device).manual_seed(seed)
-    return torch.randint(2, (width,), generator=generator, device=device).to(dtype) * 2 - 1
+    return torch.randint(2, (width,), generator=generator, device=device).float() * 2 - 1
+
+
+def random_signs(width: int, seed: int, device: torch.device | str, dtype: torch.dtype = torch.float32) -> Tensor:
+    """The +-1 vector ``randomized_transform`` draws for ``seed`` on ``device`` (drawn once per
+    width, seed and device: an online rotation reuses it on every call)."""
+    return _cached_signs(width, seed, torch.device(device)).to(dtype)
 
 
 def randomized_transform(value: Tensor, *, seed: int = 0, inverse: bool = False) -> Tensor:

@@ -160,3 +160,35 @@ def test_rejects_layouts_that_split_a_word():
         1, 16, 250, 50, 3, 1, 0.0, 1.0, None)
     assert status == native.MK_ERR_UNSUPPORTED
     assert "packing word" in native.last_error()
+
+
+@pytest.mark.parametrize("name,values,bits,integer", [
+    ("int2", scaling.int_values(2), 2, True), ("int3", scaling.int_values(3), 3, True),
+    ("nf4", scaling.NF4_VALUES, 4, False), ("e2m1", np.array([-6, -4, -3, -2, -1.5, -1, -.5, 0, .5, 1, 1.5, 2, 3, 4, 6],
+                                                             dtype=np.float32), 4, False),
+    ("codebook7", np.array([-1, -.5, -.25, 0, .25, .5, 1], dtype=np.float32), 3, False),
+])
+@pytest.mark.parametrize("group", [32, 128, 2048])
+def test_pair_table_kernel_offsets_bias_and_ragged_rows(name, values, bits, integer, group, width=2048):
+    """fp16 activations and scales at K = 2048: the LDS pair-table kernel covers rows 0..31 and
+    the word kernel rows 32..39; asymmetric offsets, bias and every sample tile."""
+    weight = helpers.normal_weight(40, 2048, seed=16, student_t=True)
+    for asym in (False, True):
+        layer = helpers.quantised_layer(weight, values, bits=bits, group=group, integer=integer, asym=asym)
+        for samples in (1, 2, 3, 8, 11):
+            x = helpers.activations(samples, 2048, seed=17 + samples)
+            bias = helpers.activations(1, 40, seed=18)[0]
+            check(run_matvec(layer, x, bias=bias), layer, x, bias)
+
+
+@pytest.mark.parametrize("width", [32, 896, 2080, 4864])
+@pytest.mark.parametrize("bits,values,integer", [(4, INT4, True), (3, scaling.int_values(3), True),
+                                                 (4, scaling.NF4_VALUES, False)])
+def test_streaming_kernels_on_rows_that_do_not_fill_a_wavefront(width, bits, values, integer):
+    """K a multiple of 32 but not of 2048: the trailing lanes of the last wavefront idle."""
+    weight = helpers.normal_weight(50, width, seed=19, student_t=True)
+    for asym in (False, True):
+        layer = helpers.quantised_layer(weight, values, bits=bits, group=32, integer=integer, asym=asym)
+        for samples in (1, 4, 8):
+            x = helpers.activations(samples, width, seed=20 + samples)
+            check(run_matvec(layer, x), layer, x)
