@@ -155,6 +155,42 @@ def _time(function, repeats=20, warmup=3):
     return begin.elapsed_time(end) / repeats
 
 
+def gptq_layer(device: torch.device, generator: torch.Generator) -> dict:
+    """GPTQ, INT4 g128, 4096 x 11008, refit = block = 128; the Hessian product and the Cholesky
+    factorisation (outside the kernels of this repository) are timed apart."""
+    import mlkit_amd as mk
+    from mlkit_amd.quantization.core import Ctx
+
+    rows, width = 4096, 11008
+    target = (torch.randn((rows, width), device=device, generator=generator) * 0.02).half().float()
+    inputs = torch.randn((16384, width), device=device, generator=generator).half()
+    hot = torch.randperm(width, device=device, generator=generator)[: width // 100]
+    inputs[:, hot] *= 30
+    hessian = (inputs.float().T @ inputs.float()) / inputs.shape[0]
+    del inputs
+    mk.feedback_coefficients(hessian.clone(), 1)
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    mk.feedback_coefficients(hessian.clone(), 1)
+    torch.cuda.synchronize()
+    factor_ms = (time.perf_counter() - started) * 1e3
+    quantizer = mk.gptq(mk.int(4, group=128))
+    quantizer(target, Ctx("warmup", H=hessian))
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    result = quantizer(target, Ctx("down_proj", H=hessian))
+    torch.cuda.synchronize()
+    total_ms = (time.perf_counter() - started) * 1e3
+    update_flops = sum(2 * rows * 128 * (width - stop) for stop in range(128, width, 128))
+    rtn = mk.int(4, group=128)(target)
+    return {
+        "total_ms": total_ms, "coefficients_ms": factor_ms, "sweep_and_update_ms": total_ms - factor_ms,
+        "columns_per_s": width / ((total_ms - factor_ms) / 1e3), "trailing_update_flops": update_flops,
+        "proxy_loss": float(mk.proxy_loss(target, result.w, hessian)),
+        "rtn_proxy_loss": float(mk.proxy_loss(target, rtn.w, hessian)),
+    }
+
+
 def other_kernels(device: torch.device) -> dict:
     """Timings of the other kernels of the path at the shapes of the benchmark configurations
     (`--kernels`); each entry carries its algorithmic bytes or flops and the rate they give."""
@@ -244,34 +280,7 @@ def other_kernels(device: torch.device) -> dict:
     matvec(151936, 896, 128, 4, values, True, False, "int4 g128 (tied head)")
     del weight, rotated, dense, codes
 
-    # GPTQ, INT4 g128, 4096 x 11008, refit = block = 128 (Hessian and Cholesky timed apart)
-    rows, width = 4096, 11008
-    target = (torch.randn((rows, width), device=device, generator=generator) * 0.02).half().float()
-    inputs = torch.randn((16384, width), device=device, generator=generator).half()
-    hot = torch.randperm(width, device=device, generator=generator)[: width // 100]
-    inputs[:, hot] *= 30
-    hessian = (inputs.float().T @ inputs.float()) / inputs.shape[0]
-    del inputs
-    torch.cuda.synchronize()
-    started = time.perf_counter()
-    mk.feedback_coefficients(hessian.clone(), 1)
-    torch.cuda.synchronize()
-    factor_ms = (time.perf_counter() - started) * 1e3
-    quantizer = mk.gptq(mk.int(4, group=128))
-    quantizer(target, Ctx("warmup", H=hessian))
-    torch.cuda.synchronize()
-    started = time.perf_counter()
-    result = quantizer(target, Ctx("down_proj", H=hessian))
-    torch.cuda.synchronize()
-    total_ms = (time.perf_counter() - started) * 1e3
-    update_flops = sum(2 * rows * 128 * (width - stop) for stop in range(128, width, 128))
-    rtn = mk.int(4, group=128)(target)
-    out["gptq int4 g128 4096x11008"] = {
-        "total_ms": total_ms, "coefficients_ms": factor_ms, "sweep_and_update_ms": total_ms - factor_ms,
-        "columns_per_s": width / ((total_ms - factor_ms) / 1e3), "trailing_update_flops": update_flops,
-        "proxy_loss": float(mk.proxy_loss(target, result.w, hessian)),
-        "rtn_proxy_loss": float(mk.proxy_loss(target, rtn.w, hessian)),
-    }
+    out["gptq int4 g128 4096x11008"] = gptq_layer(device, generator)
     return out
 
 
@@ -285,6 +294,8 @@ def main() -> None:
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--kernels", action="store_true",
                         help="also time the other kernels of the path (adds a `kernels` object to the line)")
+    parser.add_argument("--profile-gptq", action="store_true",
+                        help="for rocprofv3: only run the GPTQ layer (4096 x 11008) and print its timings")
     parser.add_argument("--profile-launches", type=int, default=0,
                         help="for rocprofv3: only launch the M=1 matvec this many times, plus three "
                              "256 MiB device copies whose counters calibrate FETCH_SIZE / WRITE_SIZE")
@@ -299,6 +310,9 @@ def main() -> None:
     copies = make_copies(options.copies, device)
     generator = torch.Generator(device=device).manual_seed(5)
 
+    if options.profile_gptq:
+        print(json.dumps(gptq_layer(device, generator)))
+        return
     if options.profile_launches:
         x = torch.randn((1, WIDTH), device=device, generator=generator).half()
         y = torch.empty((1, ROWS), device=device, dtype=torch.float16)

@@ -171,6 +171,17 @@ int mk_feedback_block_update(float *feedback, const float *original, const float
                              const float *coeff, int rows, int width, int tile_start, int tile_stop,
                              void *stream);
 
+/* The same update for `chains` consecutive tiles of chain_width columns starting at
+ * first_column, restricted to columns [column_begin, column_end) of feedback (which must
+ * follow the last chain): f = (((f + S_0) + S_1) ...), every S_i a sum from zero over the k of
+ * tile i.  The result equals applying mk_feedback_block_update tile after tile, which lets a
+ * sweep defer the update of far columns and touch them once per several tiles.
+ * Replaces: the same addmm_ (quantization/algorithms/error_feedback.py:366-370), batched. */
+int mk_feedback_block_update_range(float *feedback, const float *original, const float *output,
+                                   const float *coeff, int rows, int width, int first_column,
+                                   int chain_width, int chains, int column_begin, int column_end,
+                                   void *stream);
+
 #ifdef __cplusplus
 }
 #endif

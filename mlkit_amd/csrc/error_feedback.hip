@@ -203,71 +203,190 @@ int launch_sweep(const SweepArgs &a, hipStream_t stream) {
 }
 
 // ---- trailing block update on the fp32 matrix cores ------------------------------------
+//
+// feedback[:, c0:c1] receives, chain after chain, the product of one tile's deviations with
+// its coefficient rows:  f = (...((f + S_0) + S_1)...) , S_i = sum over the k of chain i,
+// started from zero.  Several deferred tiles (chains) can therefore be applied in one pass
+// over feedback with exactly the roundings of applying them one launch at a time.
+//
+// A workgroup of four wavefronts owns a 128 x 128 tile of feedback; each wavefront keeps a
+// 64 x 64 quarter as 2 x 2 MFMA tiles.  k advances in chunks of 32: the next chunk's global
+// loads are issued before the current chunk's 64 MFMAs and land in the other LDS buffer
+// afterwards, so one barrier per chunk suffices.
 
 typedef float mk_f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kTileRows = 128, kTileColumns = 128, kDepthChunk = 32, kUpdateThreads = 256;
+constexpr int kDeviationLoads = kTileRows * kDepthChunk / 4 / kUpdateThreads;      // float4 per thread
+constexpr int kCoefficientLoads = kDepthChunk * kTileColumns / 4 / kUpdateThreads;
 
 struct UpdateArgs {
     float *feedback;
     const float *original;
     const float *output;
     const float *coeff;
-    int rows, width, tile_start, tile_stop;
+    int rows, width;
+    int first_column;   // first column of chain 0
+    int chain_width;    // columns (= k) per chain
+    int chains;
+    int column_begin, column_end;  // columns of feedback that are updated
 };
 
-__global__ void __launch_bounds__(kUpdateThreads) block_update_kernel(const UpdateArgs a) {
-    __shared__ float deviation_t[kDepthChunk][kTileRows + 1];  // [k][row]
-    __shared__ float coefficient[kDepthChunk][kTileColumns];   // [k][column]
+struct UpdateStage {
+    float4 deviation[kDeviationLoads];
+    float4 coefficient[kCoefficientLoads];
+};
+
+// VEC: rows and tiles start on 16-byte boundaries, so operands load as float4.
+template <bool VEC>
+__device__ __forceinline__ void fetch_stage(const UpdateArgs &a, int row0, int column0, int k_base, int k_limit,
+                                            UpdateStage &stage) {
+#pragma unroll
+    for (int p = 0; p < kDeviationLoads; ++p) {
+        const int flat = p * kUpdateThreads + threadIdx.x;
+        const int r = flat / (kDepthChunk / 4), k = (flat % (kDepthChunk / 4)) * 4;
+        const bool row_ok = row0 + r < a.rows;
+        const size_t base = static_cast<size_t>(row_ok ? row0 + r : 0) * a.width + k_base;
+        float values[4];
+        if (VEC && k + 4 <= k_limit) {
+            const float4 w = *reinterpret_cast<const float4 *>(a.original + base + k);
+            const float4 q = *reinterpret_cast<const float4 *>(a.output + base + k);
+            values[0] = __fsub_rn(w.x, q.x); values[1] = __fsub_rn(w.y, q.y);
+            values[2] = __fsub_rn(w.z, q.z); values[3] = __fsub_rn(w.w, q.w);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool ok = k + i < k_limit;
+                const size_t index = base + (ok ? k + i : 0);
+                const float difference = __fsub_rn(a.original[index], a.output[index]);
+                values[i] = ok ? difference : 0.0f;
+            }
+        }
+        stage.deviation[p] = row_ok ? make_float4(values[0], values[1], values[2], values[3])
+                                    : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+#pragma unroll
+    for (int p = 0; p < kCoefficientLoads; ++p) {
+        const int flat = p * kUpdateThreads + threadIdx.x;
+        const int k = flat / (kTileColumns / 4), c = (flat % (kTileColumns / 4)) * 4;
+        const bool k_ok = k < k_limit;
+        const size_t base = static_cast<size_t>(k_base + (k_ok ? k : 0)) * a.width;
+        float values[4];
+        if (VEC && column0 + c + 4 <= a.column_end) {
+            const float4 v = *reinterpret_cast<const float4 *>(a.coeff + base + column0 + c);
+            values[0] = v.x; values[1] = v.y; values[2] = v.z; values[3] = v.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool ok = column0 + c + i < a.column_end;
+                const float loaded = a.coeff[base + (ok ? column0 + c + i : 0)];
+                values[i] = ok ? loaded : 0.0f;
+            }
+        }
+        stage.coefficient[p] = k_ok ? make_float4(values[0], values[1], values[2], values[3])
+                                    : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+}
+
+__device__ __forceinline__ void keep_stage(float (*deviation_t)[kTileRows + 1], float (*coefficient)[kTileColumns],
+                                           const UpdateStage &stage) {
+#pragma unroll
+    for (int p = 0; p < kDeviationLoads; ++p) {
+        const int flat = p * kUpdateThreads + threadIdx.x;
+        const int r = flat / (kDepthChunk / 4), k = (flat % (kDepthChunk / 4)) * 4;
+        deviation_t[k + 0][r] = stage.deviation[p].x;
+        deviation_t[k + 1][r] = stage.deviation[p].y;
+        deviation_t[k + 2][r] = stage.deviation[p].z;
+        deviation_t[k + 3][r] = stage.deviation[p].w;
+    }
+#pragma unroll
+    for (int p = 0; p < kCoefficientLoads; ++p) {
+        const int flat = p * kUpdateThreads + threadIdx.x;
+        const int k = flat / (kTileColumns / 4), c = (flat % (kTileColumns / 4)) * 4;
+        *reinterpret_cast<float4 *>(&coefficient[k][c]) = stage.coefficient[p];
+    }
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(kUpdateThreads, 2) block_update_kernel(const UpdateArgs a) {
+    __shared__ float deviation_t[2][kDepthChunk][kTileRows + 1];  // [buffer][k][row]
+    __shared__ __attribute__((aligned(16))) float coefficient[2][kDepthChunk][kTileColumns];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int row0 = blockIdx.y * kTileRows;
-    const int column0 = a.tile_stop + blockIdx.x * kTileColumns;
+    const int column0 = a.column_begin + blockIdx.x * kTileColumns;
     const int wave_row = (wave >> 1) * 64, wave_column = (wave & 1) * 64;
-    const int depth = a.tile_stop - a.tile_start;
+    const int chunks_per_chain = (a.chain_width + kDepthChunk - 1) / kDepthChunk;
+    const int steps = a.chains * chunks_per_chain;
 
-    mk_f32x16 sums[2][2];
+    // Running totals start from feedback itself.
+    mk_f32x16 totals[2][2];
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sums[mi][ni][r] = 0.0f;
+            for (int r = 0; r < 16; ++r) {
+                const int row = row0 + wave_row + mi * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                const int column = column0 + wave_column + ni * 32 + (lane & 31);
+                const bool inside = row < a.rows && column < a.column_end;
+                totals[mi][ni][r] = inside ? a.feedback[static_cast<size_t>(row) * a.width + column] : 0.0f;
+            }
 
-    for (int k0 = 0; k0 < depth; k0 += kDepthChunk) {
+    auto k_of = [&](int step, int &k_base, int &k_limit) __attribute__((always_inline)) {
+        const int chain = step / chunks_per_chain, chunk = step - chain * chunks_per_chain;
+        k_base = a.first_column + chain * a.chain_width + chunk * kDepthChunk;
+        k_limit = a.chain_width - chunk * kDepthChunk;
+        if (k_limit > kDepthChunk) k_limit = kDepthChunk;
+    };
+
+    UpdateStage stage;
+    int k_base, k_limit;
+    k_of(0, k_base, k_limit);
+    fetch_stage<VEC>(a, row0, column0, k_base, k_limit, stage);
+    keep_stage(deviation_t[0], coefficient[0], stage);
+    __syncthreads();
+
+    mk_f32x16 sums[2][2];
+    for (int step = 0; step < steps; ++step) {
+        const int buffer = step & 1;
+        const int chunk = step % chunks_per_chain;
+        if (chunk == 0) {
 #pragma unroll
-        for (int p = 0; p < kTileRows * kDepthChunk / kUpdateThreads; ++p) {
-            const int flat = p * kUpdateThreads + threadIdx.x;
-            const int r = flat / kDepthChunk, k = flat % kDepthChunk;
-            const bool wanted = row0 + r < a.rows && k0 + k < depth;
-            const size_t index = static_cast<size_t>(wanted ? row0 + r : 0) * a.width + a.tile_start + (wanted ? k0 + k : 0);
-            const float difference = __fsub_rn(a.original[index], a.output[index]);
-            deviation_t[k][r] = wanted ? difference : 0.0f;
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sums[mi][ni][r] = 0.0f;
         }
-#pragma unroll
-        for (int p = 0; p < kDepthChunk * kTileColumns / kUpdateThreads; ++p) {
-            const int flat = p * kUpdateThreads + threadIdx.x;
-            const int k = flat / kTileColumns, c = flat % kTileColumns;
-            const bool wanted = column0 + c < a.width && k0 + k < depth;
-            const size_t index = static_cast<size_t>(a.tile_start + (wanted ? k0 + k : 0)) * a.width + (wanted ? column0 + c : 0);
-            const float loaded = a.coeff[index];
-            coefficient[k][c] = wanted ? loaded : 0.0f;
+        const bool more = step + 1 < steps;
+        if (more) {
+            k_of(step + 1, k_base, k_limit);
+            fetch_stage<VEC>(a, row0, column0, k_base, k_limit, stage);
         }
-        __syncthreads();
-#pragma unroll
+#pragma unroll 4
         for (int kk = 0; kk < kDepthChunk; kk += 2) {
             const int k = kk + (lane >> 5);
             float left[2], right[2];
 #pragma unroll
-            for (int mi = 0; mi < 2; ++mi) left[mi] = deviation_t[k][wave_row + mi * 32 + (lane & 31)];
+            for (int mi = 0; mi < 2; ++mi) left[mi] = deviation_t[buffer][k][wave_row + mi * 32 + (lane & 31)];
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni) right[ni] = coefficient[k][wave_column + ni * 32 + (lane & 31)];
+            for (int ni = 0; ni < 2; ++ni) right[ni] = coefficient[buffer][k][wave_column + ni * 32 + (lane & 31)];
 #pragma unroll
             for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
                 for (int ni = 0; ni < 2; ++ni)
                     sums[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(left[mi], right[ni], sums[mi][ni], 0, 0, 0);
         }
+        if (chunk == chunks_per_chain - 1) {
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) totals[mi][ni][r] = __fadd_rn(totals[mi][ni][r], sums[mi][ni][r]);
+        }
+        if (more) keep_stage(deviation_t[buffer ^ 1], coefficient[buffer ^ 1], stage);
         __syncthreads();
     }
 
@@ -279,11 +398,22 @@ __global__ void __launch_bounds__(kUpdateThreads) block_update_kernel(const Upda
             for (int r = 0; r < 16; ++r) {
                 const int row = row0 + wave_row + mi * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
                 const int column = column0 + wave_column + ni * 32 + (lane & 31);
-                if (row < a.rows && column < a.width) {
-                    const size_t index = static_cast<size_t>(row) * a.width + column;
-                    a.feedback[index] = __fadd_rn(a.feedback[index], sums[mi][ni][r]);
-                }
+                if (row < a.rows && column < a.column_end)
+                    a.feedback[static_cast<size_t>(row) * a.width + column] = totals[mi][ni][r];
             }
+}
+
+int launch_update(const UpdateArgs &a, hipStream_t stream) {
+    MK_REQUIRE(mk_cdiv(a.rows, kTileRows) <= 65535, MK_ERR_UNSUPPORTED, "mk_feedback_block_update: too many rows");
+    const dim3 grid(mk_cdiv(a.column_end - a.column_begin, kTileColumns), mk_cdiv(a.rows, kTileRows));
+    const auto aligned = [](const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15u) == 0; };
+    const bool vec = a.width % 4 == 0 && a.first_column % 4 == 0 && a.chain_width % 4 == 0 && a.column_begin % 4 == 0 &&
+                     aligned(a.original) && aligned(a.output) && aligned(a.coeff);
+    if (vec)
+        hipLaunchKernelGGL((block_update_kernel<true>), grid, dim3(kUpdateThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((block_update_kernel<false>), grid, dim3(kUpdateThreads), 0, stream, a);
+    return MK_OK;
 }
 
 int check_tile(const char *name, int rows, int width, int tile_start, int tile_width) {
@@ -342,18 +472,31 @@ extern "C" int mk_feedback_pending(const float *feedback, const float *coeff, co
     return MK_OK;
 }
 
-extern "C" int mk_feedback_block_update(float *feedback, const float *original, const float *output,
-                                        const float *coeff, int rows, int width, int tile_start, int tile_stop,
-                                        void *stream_) {
+extern "C" int mk_feedback_block_update_range(float *feedback, const float *original, const float *output,
+                                              const float *coeff, int rows, int width, int first_column,
+                                              int chain_width, int chains, int column_begin, int column_end,
+                                              void *stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MK_REQUIRE(feedback && original && output && coeff, MK_ERR_INVALID, "mk_feedback_block_update: null tensor pointer");
-    MK_REQUIRE(rows >= 1 && width >= 1 && tile_start >= 0 && tile_start < tile_stop && tile_stop <= width,
-               MK_ERR_INVALID, "mk_feedback_block_update: columns [%d, %d) lie outside a row of %d", tile_start, tile_stop, width);
-    if (tile_stop == width) return MK_OK;
-    MK_REQUIRE(mk_cdiv(rows, kTileRows) <= 65535, MK_ERR_UNSUPPORTED, "mk_feedback_block_update: too many rows");
-    UpdateArgs a{feedback, original, output, coeff, rows, width, tile_start, tile_stop};
-    const dim3 grid(mk_cdiv(width - tile_stop, kTileColumns), mk_cdiv(rows, kTileRows));
-    hipLaunchKernelGGL(block_update_kernel, grid, dim3(kUpdateThreads), 0, stream, a);
+    MK_REQUIRE(rows >= 1 && width >= 1 && first_column >= 0 && chain_width >= 1 && chains >= 1 &&
+                   first_column + static_cast<long long>(chain_width) * chains <= width,
+               MK_ERR_INVALID, "mk_feedback_block_update: %d chains of %d columns from column %d lie outside a row of %d",
+               chains, chain_width, first_column, width);
+    MK_REQUIRE(column_begin >= first_column + chain_width * chains && column_end <= width, MK_ERR_INVALID,
+               "mk_feedback_block_update: updated columns [%d, %d) must follow the chains and lie inside the row",
+               column_begin, column_end);
+    if (column_begin >= column_end) return MK_OK;
+    UpdateArgs a{feedback, original, output, coeff, rows, width, first_column, chain_width, chains, column_begin, column_end};
+    if (int status = launch_update(a, stream)) return status;
     MK_LAUNCH_CHECK("mk_feedback_block_update");
     return MK_OK;
+}
+
+extern "C" int mk_feedback_block_update(float *feedback, const float *original, const float *output,
+                                        const float *coeff, int rows, int width, int tile_start, int tile_stop,
+                                        void *stream) {
+    MK_REQUIRE(tile_start >= 0 && tile_start < tile_stop && tile_stop <= width, MK_ERR_INVALID,
+               "mk_feedback_block_update: columns [%d, %d) lie outside a row of %d", tile_start, tile_stop, width);
+    return mk_feedback_block_update_range(feedback, original, output, coeff, rows, width, tile_start,
+                                          tile_stop - tile_start, 1, tile_stop, width, stream);
 }

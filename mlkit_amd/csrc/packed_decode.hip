@@ -3,13 +3,14 @@
 // out[n, k] = (uniform ? grid_min + code*grid_step : values[code]) * scale[n, k/group]
 //             (+ zero[n, k/group]),  every operation a separate fp32 operation.
 //
-// One thread decodes one packing word (the fewest whole bytes holding whole codes), so
-// consecutive threads read consecutive bytes and write consecutive elements.
+// Rows that are whole multiples of 32 codes are decoded a chunk of 32 codes (BITS dwords)
+// per thread: a few wide loads, 32 values from registers, wide stores.  Other layouts take
+// the word kernel: one thread per packing word (the fewest whole bytes holding whole codes).
 //
 // Replaces the reference's Triton kernel `decode_rows`
 // (kernels/packed_linear.py:229-276 in /root/reference/src/mlkit).
 
-#include "mk_common.h"
+#include "packed_matvec_impl.h"
 
 namespace {
 
@@ -21,7 +22,7 @@ struct DecodeArgs {
     void *out;
     int rows, width, group, groups;
     int scale_dtype, out_dtype;
-    int bits, bytes_per_word, codes_per_word, uniform;
+    int bits, bytes_per_word, codes_per_word, uniform, n_values;
     float grid_min, grid_step;
 };
 
@@ -54,6 +55,78 @@ __global__ void packed_decode_kernel(const DecodeArgs a) {
     }
 }
 
+
+// One thread per chunk of 32 codes.  The value table is staged in LDS.
+template <int BITS>
+__global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeArgs a) {
+    __shared__ float table[1 << BITS];
+    if (!a.uniform) {
+        for (int i = threadIdx.x; i < (1 << BITS); i += blockDim.x) table[i] = i < a.n_values ? a.values[i] : 0.0f;
+        __syncthreads();
+    }
+    const int row_chunks = a.width / mk_matvec::kChunkCodes;
+    const size_t total = static_cast<size_t>(a.rows) * row_chunks;
+    const bool one_slot = a.group % mk_matvec::kChunkCodes == 0 || a.group >= a.width;
+    for (size_t chunk = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; chunk < total;
+         chunk += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const size_t row = chunk / row_chunks;
+        const int first = static_cast<int>(chunk - row * row_chunks) * mk_matvec::kChunkCodes;
+        mk_matvec::CodeChunk<BITS> codes;
+        mk_matvec::load_codes<BITS>(codes, a.packed + chunk * (4 * BITS));
+        size_t slot = row * a.groups + first / a.group;
+        float scale = mk_load_as_float(a.scales, slot, a.scale_dtype);
+        float zero = a.zeros ? mk_load_as_float(a.zeros, slot, a.scale_dtype) : 0.0f;
+        float out[32];
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+            if (!one_slot) {
+                slot = row * a.groups + (first + k) / a.group;
+                scale = mk_load_as_float(a.scales, slot, a.scale_dtype);
+                if (a.zeros) zero = mk_load_as_float(a.zeros, slot, a.scale_dtype);
+            }
+            const uint32_t code = mk_matvec::code_at<BITS>(codes, k);
+            float weight = a.uniform ? __fadd_rn(a.grid_min, __fmul_rn(static_cast<float>(code), a.grid_step))
+                                     : table[code];
+            weight = __fmul_rn(weight, scale);
+            if (a.zeros) weight = __fadd_rn(weight, zero);
+            out[k] = weight;
+        }
+        const size_t base = row * a.width + first;
+        if (a.out_dtype == MK_F32) {
+            float4 *target = reinterpret_cast<float4 *>(static_cast<float *>(a.out) + base);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) target[q] = make_float4(out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]);
+        } else {
+            mk_u32x4 *target = reinterpret_cast<mk_u32x4 *>(static_cast<uint16_t *>(a.out) + base);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                mk_u32x4 packed4;
+#pragma unroll
+                for (int h = 0; h < 4; ++h) {
+                    const float low = out[8 * q + 2 * h], high = out[8 * q + 2 * h + 1];
+                    uint32_t pair;
+                    if (a.out_dtype == MK_F16) {
+                        const mk_h2 halves = {static_cast<_Float16>(low), static_cast<_Float16>(high)};
+                        pair = __builtin_bit_cast(uint32_t, halves);
+                    } else {
+                        pair = static_cast<uint32_t>(mk_float_to_bf16(low)) | (static_cast<uint32_t>(mk_float_to_bf16(high)) << 16);
+                    }
+                    packed4[h] = pair;
+                }
+                target[q] = packed4;
+            }
+        }
+    }
+}
+
+template <int BITS>
+void launch_chunks(const DecodeArgs &a, hipStream_t stream) {
+    const size_t chunks = static_cast<size_t>(a.rows) * (a.width / mk_matvec::kChunkCodes);
+    size_t blocks = (chunks + 255) / 256;
+    if (blocks > 256u * 64u) blocks = 256u * 64u;
+    hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+}
+
 }  // namespace
 
 extern "C" int mk_packed_decode(const uint8_t *packed, const void *scales, int scale_dtype,
@@ -79,6 +152,22 @@ extern "C" int mk_packed_decode(const uint8_t *packed, const void *scales, int s
     const int divisor = mk_gcd(bits, 8);
     a.bytes_per_word = bits / divisor; a.codes_per_word = 8 / divisor; a.uniform = uniform;
     a.grid_min = grid_min; a.grid_step = grid_step;
+    a.n_values = n_values;
+    const bool wide = input_width % mk_matvec::kChunkCodes == 0 && (reinterpret_cast<uintptr_t>(packed) & 3u) == 0 &&
+                      (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && bits >= 2;
+    if (wide) {
+        switch (bits) {
+            case 2: launch_chunks<2>(a, stream); break;
+            case 3: launch_chunks<3>(a, stream); break;
+            case 4: launch_chunks<4>(a, stream); break;
+            case 5: launch_chunks<5>(a, stream); break;
+            case 6: launch_chunks<6>(a, stream); break;
+            case 7: launch_chunks<7>(a, stream); break;
+            default: launch_chunks<8>(a, stream); break;
+        }
+        MK_LAUNCH_CHECK("mk_packed_decode");
+        return MK_OK;
+    }
     const size_t words = static_cast<size_t>(output_width) * (input_width / a.codes_per_word);
     size_t blocks = (words + 255) / 256;
     if (blocks > 256u * 32u) blocks = 256u * 32u;

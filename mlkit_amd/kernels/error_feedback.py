@@ -104,3 +104,28 @@ def block_update(
         feedback.data_ptr(), original.data_ptr(), output.data_ptr(), coefficients.data_ptr(), rows, width,
         tile_start, tile_stop, native.current_stream(device),
     ))
+
+
+def block_update_range(
+    feedback: Tensor,
+    original: Tensor,
+    output: Tensor,
+    coefficients: Tensor,
+    first_column: int,
+    chain_width: int,
+    chains: int,
+    column_begin: int,
+    column_end: int,
+) -> None:
+    """The updates of ``chains`` consecutive tiles applied to columns ``[column_begin,
+    column_end)`` in one pass, with the roundings of applying them tile after tile."""
+    device = native.require_device(feedback, original, output, coefficients)
+    rows, width = original.shape
+    _check("original", original)
+    _check("feedback", feedback, (rows, width))
+    _check("output", output, (rows, width))
+    _check("coefficients", coefficients, (width, width))
+    native.check(native.library().mk_feedback_block_update_range(
+        feedback.data_ptr(), original.data_ptr(), output.data_ptr(), coefficients.data_ptr(), rows, width,
+        first_column, chain_width, chains, column_begin, column_end, native.current_stream(device),
+    ))

@@ -28,6 +28,7 @@ FUSED_VECTOR_DIMENSIONS = {2, 4, 8, 16}
 FUSED_VECTOR_CODEBOOK_LIMIT = 65536
 UPPER_FACTORIZATION_WIDTH = 4096
 MAXIMUM_FUSED_TILE = 1024
+DEFERRED_TILES = 4  # tiles whose far-column updates are applied in one pass on the device
 
 
 def feedback_coefficients(hessian: Tensor, step: int, *, damp: float = 0.01,
@@ -250,8 +251,32 @@ class ErrorFeedback(Quantizer):
         on_device = w.is_cuda
         if on_device:
             from mlkit_amd.kernels import error_feedback as kernel
+        # On the device the update of far columns is deferred: after a tile, only columns up to
+        # `limit` are updated at once; the tiles in `deferred` reach the columns beyond it in
+        # one pass when the super-block ends (or when a region needs those columns).  Every
+        # column still receives the tiles' sums one by one in tile order, so nothing changes
+        # in the result.
+        deferred: list[tuple[int, int]] = []
+        limit = 0
+
+        def flush() -> None:
+            index = 0
+            while index < len(deferred):  # runs of equally wide consecutive tiles
+                run = index + 1
+                chain = deferred[index][1] - deferred[index][0]
+                while run < len(deferred) and deferred[run][1] - deferred[run][0] == chain:
+                    run += 1
+                kernel.block_update_range(feedback, original, output, coefficients, deferred[index][0], chain,
+                                          run - index, limit, width)
+                index = run
+            deferred.clear()
+
         for region_start in range(0, width, refit_width):
             region_stop = min(width, region_start + refit_width)
+            if deferred and region_stop > limit:
+                flush()
+            if not deferred:
+                limit = min(width, max(region_start + DEFERRED_TILES * self.block_size, region_stop))
             targets = original[:, region_start:region_stop]
             if region_start:
                 if on_device and region_stop - region_start <= MAXIMUM_FUSED_TILE:
@@ -277,12 +302,19 @@ class ErrorFeedback(Quantizer):
                 else:
                     self._round_tile_by_blocks(rounder, original, feedback, coefficients, output, collected,
                                                region_start, tile_start, tile_stop)
-                if tile_stop < width:
-                    if on_device:
-                        kernel.block_update(feedback, original, output, coefficients, tile_start, tile_stop)
-                    else:
-                        deviations = original[:, tile_start:tile_stop] - output[:, tile_start:tile_stop]
-                        feedback[:, tile_stop:].addmm_(deviations, coefficients[tile_start:tile_stop, tile_stop:])
+                if tile_stop >= width:
+                    continue
+                if not on_device:
+                    deviations = original[:, tile_start:tile_stop] - output[:, tile_start:tile_stop]
+                    feedback[:, tile_stop:].addmm_(deviations, coefficients[tile_start:tile_stop, tile_stop:])
+                    continue
+                if tile_stop < limit:
+                    kernel.block_update_range(feedback, original, output, coefficients, tile_start,
+                                              tile_stop - tile_start, 1, tile_stop, limit)
+                if limit < width:
+                    deferred.append((tile_start, tile_stop))
+                    if tile_stop >= limit:
+                        flush()
         return collected.result(output, permutation, refit_width, ctx)
 
 

@@ -106,3 +106,27 @@ def test_block_update_matches_fma_chain(rows, width, start, stop):
     exact = feedback[:, stop:].astype(np.float64) + (weight - output)[:, start:stop].astype(np.float64) @ coeff[start:stop, stop:].astype(np.float64)
     np.testing.assert_allclose(host(updated)[:, stop:], exact, rtol=1e-4, atol=1e-6)
     np.testing.assert_array_equal(host(updated)[:, :stop], feedback[:, :stop])
+
+
+@pytest.mark.parametrize("rows,width,first,chain,chains,begin,end", [
+    (130, 1024, 0, 128, 4, 512, 1024),     # a deferred super-block reaching the far columns
+    (64, 700, 64, 96, 3, 352, 700),        # ragged widths, unaligned end
+    (64, 640, 128, 128, 1, 256, 384),      # the narrow update inside a super-block
+    (33, 333, 10, 50, 2, 111, 333),        # nothing aligned: scalar loads
+])
+def test_chained_block_update_equals_tile_after_tile(rows, width, first, chain, chains, begin, end):
+    from mlkit_amd.kernels import error_feedback
+
+    weight, coeff, _ = problem(rows, width, seed=width + chains)
+    rng = np.random.default_rng(4)
+    output = (weight + rng.standard_normal(weight.shape).astype(F32) * 0.003).astype(F32)
+    feedback = (rng.standard_normal(weight.shape) * 0.01).astype(F32)
+    expected = feedback.copy()
+    for index in range(chains):   # the oracle applies one tile at a time to every later column
+        start = first + index * chain
+        scratch = expected.copy()
+        oracle_feedback.block_update(scratch, weight, output, coeff, start, start + chain, mode=0)
+        expected[:, begin:end] = scratch[:, begin:end]
+    updated = dev(feedback)
+    error_feedback.block_update_range(updated, dev(weight), dev(output), dev(coeff), first, chain, chains, begin, end)
+    np.testing.assert_array_equal(host(updated), expected)

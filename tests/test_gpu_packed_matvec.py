@@ -192,3 +192,50 @@ def test_streaming_kernels_on_rows_that_do_not_fill_a_wavefront(width, bits, val
         for samples in (1, 4, 8):
             x = helpers.activations(samples, width, seed=20 + samples)
             check(run_matvec(layer, x), layer, x)
+
+
+@pytest.mark.parametrize("name", WIDTHS)
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("width", [256, 288, 264])
+def test_packed_decode_is_exact(name, out_dtype, width):
+    """packed -> dense: fp32 output equals the oracle's decode bit for bit, half-precision
+    outputs equal its rounding (multiply and add kept separate); 256/288 take the chunk
+    kernel, 264 the word kernel."""
+    from mlkit_amd.kernels import packed_linear
+
+    values, bits, group, integer = WIDTHS[name]
+    if width % group and group != 48:
+        group = 8 if bits in (4, 8, 2) else 24 if bits in (3, 6) else 8 * bits if width % (8 * bits) == 0 else group
+    layout = packed_linear.layout_for(bits, width, group)
+    if layout is None:
+        pytest.skip("no fused layout for this combination")
+    weight = helpers.normal_weight(21, width, seed=30, scale=1.0)
+    for asym in (False, True):
+        layer = helpers.quantised_layer(weight, values, bits=bits, group=group, integer=integer, asym=asym)
+        tensors = helpers.to_device(layer)
+        uniform, minimum, step = helpers.uniform_grid(layer["values"])
+        dense = torch.empty((21, width), dtype=out_dtype, device="cuda")
+        packed_linear.decode(tensors["packed"], tensors["scales"], tensors["values"], tensors["zeros"], dense,
+                             layer["group"], layout, uniform, minimum, step)
+        torch.cuda.synchronize()
+        expected = torch.from_numpy(layer["dense"]).to(out_dtype)
+        assert torch.equal(dense.cpu(), expected)
+
+
+def test_packed_decode_full_layer_matches_matvec_input():
+    """4096 x 14336 INT4-g128 -> fp16: spot rows against the oracle, and the dense product
+    agrees with the fused matvec."""
+    from mlkit_amd.kernels import packed_linear
+
+    weight = helpers.normal_weight(4096, 14336, seed=31)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
+    tensors = helpers.to_device(layer)
+    dense = torch.empty((4096, 14336), dtype=torch.float16, device="cuda")
+    packed_linear.decode(tensors["packed"], tensors["scales"], tensors["values"], None, dense, 128,
+                         packed_linear.layout_for(4, 14336, 128), True, -8.0, 1.0)
+    torch.cuda.synchronize()
+    rows = [0, 1, 777, 4095]
+    assert torch.equal(dense[rows].cpu(), torch.from_numpy(layer["dense"][rows]).half())
+    x = helpers.activations(2, 14336, seed=32)
+    fused = run_matvec(layer, x)
+    np.testing.assert_allclose((x.cuda().float() @ dense.float().T).cpu().numpy(), fused, rtol=2e-3, atol=2e-3)
