@@ -43,7 +43,7 @@ struct FwhtArgs {
 __host__ __device__ __forceinline__ int padded(int index) { return index + (index >> 4); }
 
 // E values per thread; stage group `g` covers index bits [base, base + log2 E).
-template <int E>
+template <int E, bool VEC>
 __global__ void __launch_bounds__(kMaxThreads) fwht_kernel(const FwhtArgs a) {
     extern __shared__ float tile[];
     constexpr int kLogE = E == 1 ? 0 : E == 2 ? 1 : E == 4 ? 2 : E == 8 ? 3 : E == 16 ? 4 : 5;
@@ -56,14 +56,58 @@ __global__ void __launch_bounds__(kMaxThreads) fwht_kernel(const FwhtArgs a) {
     const size_t row_base = static_cast<size_t>(active ? row : 0) * a.width;
     const int sign_base = a.sign_period ? static_cast<int>(row_base % static_cast<size_t>(a.sign_period)) : 0;
 
-    // HBM -> LDS, consecutive lanes read consecutive elements.
+    // HBM -> LDS.  All loads of a thread are issued before any is used; with VEC a thread
+    // reads groups of four adjacent elements (16 bytes of fp32, 8 of fp16 / bf16).
     if (active) {
+        float staged[E];
+        if constexpr (VEC) {
+            constexpr int kQuads = E / 4;
+            if (a.source_dtype == MK_F32) {
+                const float4 *source = reinterpret_cast<const float4 *>(static_cast<const float *>(a.source) + row_base);
+                float4 loaded[kQuads];
 #pragma unroll
-        for (int j = 0; j < E; ++j) {
-            const int index = j * threads_per_row + t;
-            float value = mk_load_as_float(a.source, row_base + index, a.source_dtype);
-            if (a.signs_before) value *= a.signs_before[sign_base + index];
-            mine[padded(index)] = value;
+                for (int q = 0; q < kQuads; ++q) loaded[q] = source[q * threads_per_row + t];
+#pragma unroll
+                for (int q = 0; q < kQuads; ++q) {
+                    staged[4 * q] = loaded[q].x; staged[4 * q + 1] = loaded[q].y;
+                    staged[4 * q + 2] = loaded[q].z; staged[4 * q + 3] = loaded[q].w;
+                }
+            } else {
+                const mk_u32x2 *source = reinterpret_cast<const mk_u32x2 *>(static_cast<const uint16_t *>(a.source) + row_base);
+                mk_u32x2 loaded[kQuads];
+#pragma unroll
+                for (int q = 0; q < kQuads; ++q) loaded[q] = source[q * threads_per_row + t];
+#pragma unroll
+                for (int q = 0; q < kQuads; ++q)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t word = i < 2 ? loaded[q].x : loaded[q].y;
+                        const uint16_t raw = static_cast<uint16_t>((i & 1) ? word >> 16 : word);
+                        staged[4 * q + i] = a.source_dtype == MK_F16 ? static_cast<float>(__builtin_bit_cast(_Float16, raw))
+                                                                     : mk_bf16_to_float(raw);
+                    }
+            }
+            if (a.signs_before) {
+                const float4 *signs = reinterpret_cast<const float4 *>(a.signs_before + sign_base);
+#pragma unroll
+                for (int q = 0; q < kQuads; ++q) {
+                    const float4 sign = signs[q * threads_per_row + t];
+                    staged[4 * q] *= sign.x; staged[4 * q + 1] *= sign.y;
+                    staged[4 * q + 2] *= sign.z; staged[4 * q + 3] *= sign.w;
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < kQuads; ++q)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) mine[padded((q * threads_per_row + t) * 4 + i)] = staged[4 * q + i];
+        } else {
+#pragma unroll
+            for (int j = 0; j < E; ++j) {
+                const int index = j * threads_per_row + t;
+                float value = mk_load_as_float(a.source, row_base + index, a.source_dtype);
+                if (a.signs_before) value *= a.signs_before[sign_base + index];
+                mine[padded(index)] = value;
+            }
         }
     }
     __syncthreads();
@@ -111,6 +155,21 @@ __global__ void __launch_bounds__(kMaxThreads) fwht_kernel(const FwhtArgs a) {
     }
 }
 
+template <int E, bool VEC>
+int launch_fwht_as(const FwhtArgs &a, int threads, size_t lds, hipStream_t stream) {
+    static size_t allowed = 48 * 1024;  // raised once per instantiation when a row needs more
+    if (lds > allowed) {
+        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwht_kernel<E, VEC>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (status != hipSuccess)
+            return mk_fail(MK_ERR_HIP, "mk_fwht: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(status));
+        allowed = 160 * 1024;
+    }
+    const long long blocks = (a.rows + a.rows_per_block - 1) / a.rows_per_block;
+    hipLaunchKernelGGL((fwht_kernel<E, VEC>), dim3(static_cast<unsigned>(blocks)), dim3(threads), lds, stream, a);
+    return MK_OK;
+}
+
 template <int E>
 int launch_fwht(FwhtArgs a, hipStream_t stream) {
     a.threads_per_row = a.width / E;
@@ -118,17 +177,11 @@ int launch_fwht(FwhtArgs a, hipStream_t stream) {
     if (a.rows_per_block > a.rows) a.rows_per_block = static_cast<int>(a.rows);
     const int threads = a.rows_per_block * a.threads_per_row;
     const size_t lds = static_cast<size_t>(a.rows_per_block) * padded(a.width) * sizeof(float);
-    static size_t allowed = 48 * 1024;  // raised once per instantiation when a row needs more
-    if (lds > allowed) {
-        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwht_kernel<E>),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (status != hipSuccess)
-            return mk_fail(MK_ERR_HIP, "mk_fwht: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(status));
-        allowed = 160 * 1024;
+    if constexpr (E % 4 == 0) {
+        const auto aligned = [](const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15u) == 0; };
+        if (aligned(a.source) && aligned(a.signs_before)) return launch_fwht_as<E, true>(a, threads, lds, stream);
     }
-    const long long blocks = (a.rows + a.rows_per_block - 1) / a.rows_per_block;
-    hipLaunchKernelGGL((fwht_kernel<E>), dim3(static_cast<unsigned>(blocks)), dim3(threads), lds, stream, a);
-    return MK_OK;
+    return launch_fwht_as<E, false>(a, threads, lds, stream);
 }
 
 struct MixArgs {
@@ -167,6 +220,77 @@ __global__ void __launch_bounds__(256) basis_mix_kernel(const MixArgs a) {
             a.target[base + static_cast<size_t>(out) * a.power] = sum;
         }
     }
+}
+
+// The same product on the fp32 matrix cores for bases of up to 96 rows.  One wavefront
+// owns 32 adjacent columns p of one row r: the basis (zero-padded to TILES x 32 rows) is
+// the left operand, kept in registers; the right operand comes straight from global memory,
+// lanes 0..31 reading 32 adjacent p of block f and lanes 32..63 of block f + 1, so no LDS is
+// involved.  v_mfma_f32_32x32x2_f32 accumulates over ascending f from zero, which equals
+// the fused multiply-add chain of basis_mix_kernel bit for bit.
+typedef float mk_mix16 __attribute__((ext_vector_type(16)));
+
+template <int TILES>
+__global__ void __launch_bounds__(256) basis_mix_mfma_kernel(const MixArgs a) {
+    constexpr int kMaxPairs = TILES * 16;  // k-pairs of a basis padded to TILES * 32
+    const int lane = threadIdx.x & 63;
+    const int half = lane >> 5, within = lane & 31;
+    const int pairs = (a.order + 1) >> 1;
+    // left[t][q]: mix[32 t + within][2 q + half]
+    float left[TILES][kMaxPairs];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int q = 0; q < kMaxPairs; ++q) {
+            const int out = 32 * t + within, in = 2 * q + half;
+            const bool inside = out < a.order && in < a.order;
+            const int index = a.transpose ? in * a.order + out : out * a.order + in;
+            left[t][q] = inside ? a.basis[inside ? index : 0] : 0.0f;
+        }
+    const int tiles_per_row = (a.power + 31) >> 5;
+    const long long total = a.rows * tiles_per_row;
+    const long long first = static_cast<long long>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const long long stride = static_cast<long long>(gridDim.x) * (blockDim.x >> 6);
+    for (long long tile = first; tile < total; tile += stride) {
+        const long long row = tile / tiles_per_row;
+        const int p = static_cast<int>(tile - row * tiles_per_row) * 32 + within;
+        const bool column_ok = p < a.power;
+        const size_t base = static_cast<size_t>(row) * a.order * a.power + (column_ok ? p : 0);
+        float right[kMaxPairs];
+#pragma unroll
+        for (int q = 0; q < kMaxPairs; ++q) {
+            const int in = 2 * q + half;
+            const bool inside = q < pairs && in < a.order && column_ok;
+            const float loaded = a.source[base + static_cast<size_t>(inside ? in : 0) * a.power];
+            right[q] = inside ? loaded : 0.0f;
+        }
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            mk_mix16 sums;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sums[r] = 0.0f;
+#pragma unroll
+            for (int q = 0; q < kMaxPairs; ++q)
+                if (q < pairs) sums = __builtin_amdgcn_mfma_f32_32x32x2f32(left[t][q], right[q], sums, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int out = 32 * t + (r >> 2) * 8 + half * 4 + (r & 3);
+                if (out < a.order && column_ok) {
+                    float value = sums[r];
+                    if (a.signs_after) value *= a.signs_after[out * a.power + p];
+                    a.target[base + static_cast<size_t>(out) * a.power] = value;
+                }
+            }
+        }
+    }
+}
+
+template <int TILES>
+void launch_mix_mfma(const MixArgs &a, hipStream_t stream) {
+    const long long tiles = a.rows * ((a.power + 31) / 32);
+    long long blocks = (tiles + 3) / 4;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    hipLaunchKernelGGL((basis_mix_mfma_kernel<TILES>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
 }
 
 }  // namespace
@@ -213,12 +337,20 @@ extern "C" int mk_basis_mix(const float *source, float *target, const float *bas
     MK_REQUIRE(source && target && basis, MK_ERR_INVALID, "mk_basis_mix: null tensor pointer");
     MK_REQUIRE(source != target, MK_ERR_INVALID, "mk_basis_mix: source and target must not alias");
     MixArgs a{source, target, basis, signs_after, rows, order, power, transpose};
-    // One LDS column of `order` floats per thread: fewer threads for larger bases (64 KB).
-    const int threads = order <= 64 ? 256 : order <= 128 ? 128 : 64;
-    long long blocks = (rows * power + threads - 1) / threads;
-    if (blocks > 256 * 64) blocks = 256 * 64;
-    hipLaunchKernelGGL(basis_mix_kernel, dim3(static_cast<unsigned>(blocks)), dim3(threads),
-                       static_cast<size_t>(order) * threads * sizeof(float), stream, a);
+    if (order <= 32) {
+        launch_mix_mfma<1>(a, stream);
+    } else if (order <= 64) {
+        launch_mix_mfma<2>(a, stream);
+    } else if (order <= 96) {
+        launch_mix_mfma<3>(a, stream);
+    } else {
+        // One LDS column of `order` floats per thread: fewer threads for larger bases (64 KB).
+        const int threads = order <= 128 ? 128 : 64;
+        long long blocks = (rows * power + threads - 1) / threads;
+        if (blocks > 256 * 64) blocks = 256 * 64;
+        hipLaunchKernelGGL(basis_mix_kernel, dim3(static_cast<unsigned>(blocks)), dim3(threads),
+                           static_cast<size_t>(order) * threads * sizeof(float), stream, a);
+    }
     MK_LAUNCH_CHECK("mk_basis_mix");
     return MK_OK;
 }
