@@ -182,6 +182,23 @@ int mk_feedback_block_update_range(float *feedback, const float *original, const
                                    int chain_width, int chains, int column_begin, int column_end,
                                    void *stream);
 
+/* The whole natural-order error-feedback sweep of a layer with per-region absmax / minmax
+ * scale fits, enqueued in one call: for every region of `refit` columns the pending
+ * continuation (into workspace, [rows, refit] fp32; may be NULL when refit >= width), the
+ * scale fit on those targets (scales rounded to scale_format, zeros stored as rounded
+ * magnitude with sign), then per tile of `block` columns mk_feedback_round_tile and the
+ * trailing updates, far columns deferred by up to deferred_tiles tiles
+ * (mk_feedback_block_update_range).  scales / zeros: [rows, G] fp32, G = sum over regions of
+ * ceil(region width / min(group, region width)), region after region.  Results equal those
+ * of issuing the separate entry points region by region.
+ * Replaces: the host loop of quantization/algorithms/error_feedback.py:296-370. */
+int mk_feedback_sweep(const float *original, float *feedback, float *output, uint8_t *encoded,
+                      const float *coeff, float *scales, float *zeros, float *workspace,
+                      const float *values, int n_values, int rows, int width, int group, int refit,
+                      int block, int integer_grid, float code_min, float code_max, int asym,
+                      float reciprocal, float value_minimum, int scale_format, int deferred_tiles,
+                      void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -500,3 +500,113 @@ extern "C" int mk_feedback_block_update(float *feedback, const float *original, 
     return mk_feedback_block_update_range(feedback, original, output, coeff, rows, width, tile_start,
                                           tile_stop - tile_start, 1, tile_stop, width, stream);
 }
+
+// The whole natural-order sweep of a layer, enqueued from here so that a region costs a few
+// kernel launches and no host round trips: per region the pending-continuation solve into
+// `workspace`, the scale fit on those targets, then per tile the column sweep and the
+// (deferred, chained) trailing updates.
+extern "C" int mk_feedback_sweep(const float *original, float *feedback, float *output, uint8_t *encoded,
+                                 const float *coeff, float *scales, float *zeros, float *workspace,
+                                 const float *values, int n_values, int rows, int width, int group, int refit,
+                                 int block, int integer_grid, float code_min, float code_max, int asym,
+                                 float reciprocal, float value_minimum, int scale_format, int deferred_tiles,
+                                 void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(original && feedback && output && encoded && coeff && scales && (!asym || zeros), MK_ERR_INVALID,
+               "mk_feedback_sweep: null tensor pointer");
+    MK_REQUIRE(rows >= 1 && width >= 1 && group >= 1 && block >= 1 && block <= 1024 && refit >= 1 && deferred_tiles >= 1,
+               MK_ERR_INVALID, "mk_feedback_sweep: sizes must be positive and tiles at most 1024 columns wide");
+    MK_REQUIRE(refit >= width || (refit <= 1024 && workspace), MK_ERR_INVALID,
+               "mk_feedback_sweep: regions of %d columns need a workspace and at most 1024 columns", refit);
+    if (integer_grid) {
+        MK_REQUIRE(code_max >= code_min && code_max - code_min <= 255.0f, MK_ERR_INVALID,
+                   "mk_feedback_sweep: integer grid must span at most 256 codes");
+    } else {
+        MK_REQUIRE(values && n_values >= 1 && n_values <= 256, MK_ERR_INVALID,
+                   "mk_feedback_sweep: a value table of 1..256 entries is required");
+    }
+    const int region_width = refit < width ? refit : width;
+    long long total_groups = 0;
+    for (int start = 0; start < width; start += region_width) {
+        const int span = width - start < region_width ? width - start : region_width;
+        total_groups += mk_cdiv(span, group < span ? group : span);
+    }
+    MK_REQUIRE(total_groups < (1ll << 31) / rows, MK_ERR_INVALID, "mk_feedback_sweep: too many scale groups");
+
+    struct Tile { int start, stop; };
+    Tile deferred[64];
+    int deferred_count = 0, limit = 0;
+    auto update = [&](int first, int chain, int chains, int begin, int end) -> int {
+        if (begin >= end) return MK_OK;
+        UpdateArgs u{feedback, original, output, coeff, rows, width, first, chain, chains, begin, end};
+        return launch_update(u, stream);
+    };
+    auto flush = [&]() -> int {
+        int index = 0;
+        while (index < deferred_count) {
+            const int chain = deferred[index].stop - deferred[index].start;
+            int run = index + 1;
+            while (run < deferred_count && deferred[run].stop - deferred[run].start == chain) ++run;
+            if (int status = update(deferred[index].start, chain, run - index, limit, width)) return status;
+            index = run;
+        }
+        deferred_count = 0;
+        return MK_OK;
+    };
+
+    long long group_offset = 0;
+    for (int region_start = 0; region_start < width; region_start += region_width) {
+        const int region_stop = region_start + region_width < width ? region_start + region_width : width;
+        const int span = region_stop - region_start;
+        const int fitted_group = group < span ? group : span;
+        const int region_groups = mk_cdiv(span, fitted_group);
+        if (deferred_count && region_stop > limit)
+            if (int status = flush()) return status;
+        if (!deferred_count) {
+            limit = region_start + deferred_tiles * block;
+            if (limit < region_stop) limit = region_stop;
+            if (limit > width) limit = width;
+        }
+        float *region_scales = scales + group_offset;
+        float *region_zeros = asym ? zeros + group_offset : nullptr;
+        if (region_start == 0) {
+            if (int status = mk_fit_scales_strided(original, width, region_scales, region_zeros, total_groups, rows, span,
+                                                   fitted_group, asym, reciprocal, value_minimum, scale_format, 1, stream))
+                return status;
+        } else {
+            SweepArgs solve{};
+            solve.original = original; solve.feedback = feedback; solve.coeff = coeff; solve.output = workspace;
+            solve.rows = rows; solve.width = width; solve.region_start = region_start; solve.tile_start = region_start;
+            solve.tile_width = span; solve.group = 1;
+            launch_sweep<kModeSolve>(solve, stream);
+            if (int status = mk_fit_scales_strided(workspace, span, region_scales, region_zeros, total_groups, rows, span,
+                                                   fitted_group, asym, reciprocal, value_minimum, scale_format, 1, stream))
+                return status;
+        }
+        for (int tile_start = region_start; tile_start < region_stop; tile_start += block) {
+            const int tile_stop = tile_start + block < region_stop ? tile_start + block : region_stop;
+            SweepArgs a{};
+            a.original = original; a.feedback = feedback; a.coeff = coeff; a.scales = region_scales;
+            a.zeros = region_zeros; a.values = values; a.output = output; a.encoded = encoded; a.rows = rows;
+            a.width = width; a.region_start = region_start; a.tile_start = tile_start;
+            a.tile_width = tile_stop - tile_start; a.group = fitted_group;
+            a.groups_per_row = static_cast<int>(total_groups); a.n_values = n_values;
+            a.code_min = code_min; a.code_max = code_max;
+            if (integer_grid) launch_sweep<kModeInteger>(a, stream);
+            else launch_sweep<kModeCodebook>(a, stream);
+            if (tile_stop >= width) continue;
+            if (tile_stop < limit)
+                if (int status = update(tile_start, tile_stop - tile_start, 1, tile_stop, limit)) return status;
+            if (limit < width) {
+                deferred[deferred_count].start = tile_start;
+                deferred[deferred_count].stop = tile_stop;
+                ++deferred_count;
+                if (tile_stop >= limit || deferred_count == 64)
+                    if (int status = flush()) return status;
+            }
+        }
+        group_offset += region_groups;
+    }
+    MK_LAUNCH_CHECK("mk_feedback_sweep");
+    return MK_OK;
+}

@@ -35,6 +35,11 @@ static inline int mk_gcd(int a, int b) {
     return a;
 }
 
+// Defined in scalar_codec.hip, also used by the error-feedback sweep (error_feedback.hip).
+int mk_fit_scales_strided(const float *value, long long row_stride, float *scales, float *zeros,
+                          long long out_row_stride, int rows, int span, int group, int asym, float reciprocal,
+                          float value_minimum, int scale_format, int store_zero, hipStream_t stream);
+
 #ifdef __HIPCC__
 
 typedef uint32_t mk_u32x2 __attribute__((ext_vector_type(2)));

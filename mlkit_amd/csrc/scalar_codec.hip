@@ -265,7 +265,7 @@ struct FitArgs {
     const float *value;
     float *scales;
     float *zeros;
-    long long row_stride;
+    long long row_stride, out_row_stride;
     int rows, span, group, groups_per_row, total_groups;
     int asym, format, store_zero;
     float reciprocal, value_minimum;
@@ -299,9 +299,10 @@ __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
             finite = __shfl_xor(static_cast<int>(finite), offset, 64) && finite;
         }
         if (lane_in_team != 0 || wanted >= a.total_groups) continue;
+        const size_t slot = static_cast<size_t>(row) * a.out_row_stride + (identifier - row * a.groups_per_row);
         if (!finite) {  // fminf/fmaxf drop NaNs: report them as the tensor reductions would
-            a.scales[identifier] = __builtin_nanf("");
-            if (a.zeros) a.zeros[identifier] = __builtin_nanf("");
+            a.scales[slot] = __builtin_nanf("");
+            if (a.zeros) a.zeros[slot] = __builtin_nanf("");
             continue;
         }
         float scale, zero = 0.0f;
@@ -311,13 +312,13 @@ __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
         } else {
             scale = __fmul_rn(fmaxf(fmaxf(high, -low), 1e-12f), a.reciprocal);
         }
-        a.scales[identifier] = rounded_scale(scale, a.format);
+        a.scales[slot] = rounded_scale(scale, a.format);
         if (a.zeros) {
             if (a.store_zero) {
                 const float magnitude = rounded_scale(fmaxf(fabsf(zero), 1e-12f), a.format);
                 zero = zero > 0.0f ? magnitude : (zero < 0.0f ? -magnitude : 0.0f);
             }
-            a.zeros[identifier] = zero;
+            a.zeros[slot] = zero;
         }
     }
 }
@@ -455,19 +456,21 @@ extern "C" int mk_snap(const float *value, const float *values, int n_values, fl
     return MK_OK;
 }
 
-extern "C" int mk_fit_scales(const float *value, long long row_stride, float *scales, float *zeros, int rows,
-                             int span, int group, int asym, float reciprocal, float value_minimum,
-                             int scale_format, int store_zero, void *stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+// Shared with the error-feedback sweep: scales of row r land at scales[r * out_row_stride + g].
+int mk_fit_scales_strided(const float *value, long long row_stride, float *scales, float *zeros,
+                          long long out_row_stride, int rows, int span, int group, int asym, float reciprocal,
+                          float value_minimum, int scale_format, int store_zero, hipStream_t stream) {
     MK_REQUIRE(value && scales && (!asym || zeros), MK_ERR_INVALID, "mk_fit_scales: null tensor pointer");
     MK_REQUIRE(rows >= 1 && span >= 1 && group >= 1 && row_stride >= span, MK_ERR_INVALID,
                "mk_fit_scales: sizes must be positive and rows at least `span` apart");
     MK_REQUIRE(scale_format >= 0 && scale_format <= 4, MK_ERR_INVALID, "mk_fit_scales: unknown scale format code");
     const int groups_per_row = mk_cdiv(span, group);
+    MK_REQUIRE(out_row_stride >= groups_per_row, MK_ERR_INVALID, "mk_fit_scales: output rows overlap");
     MK_REQUIRE(static_cast<long long>(rows) * groups_per_row < (1ll << 31), MK_ERR_INVALID,
                "mk_fit_scales: too many scale groups");
     FitArgs a{};
     a.value = value; a.scales = scales; a.zeros = asym ? zeros : nullptr; a.row_stride = row_stride;
+    a.out_row_stride = out_row_stride;
     a.rows = rows; a.span = span; a.group = group; a.groups_per_row = groups_per_row;
     a.total_groups = rows * groups_per_row; a.asym = asym; a.format = scale_format; a.store_zero = store_zero;
     a.reciprocal = reciprocal; a.value_minimum = value_minimum;
@@ -479,4 +482,12 @@ extern "C" int mk_fit_scales(const float *value, long long row_stride, float *sc
     else launch_fit<4>(a, stream);
     MK_LAUNCH_CHECK("mk_fit_scales");
     return MK_OK;
+}
+
+extern "C" int mk_fit_scales(const float *value, long long row_stride, float *scales, float *zeros, int rows,
+                             int span, int group, int asym, float reciprocal, float value_minimum,
+                             int scale_format, int store_zero, void *stream) {
+    const int groups = group >= 1 ? mk_cdiv(span, group) : 0;
+    return mk_fit_scales_strided(value, row_stride, scales, zeros, groups, rows, span, group, asym, reciprocal,
+                                 value_minimum, scale_format, store_zero, static_cast<hipStream_t>(stream));
 }

@@ -129,3 +129,52 @@ def block_update_range(
         feedback.data_ptr(), original.data_ptr(), output.data_ptr(), coefficients.data_ptr(), rows, width,
         first_column, chain_width, chains, column_begin, column_end, native.current_stream(device),
     ))
+
+
+def sweep(
+    original: Tensor,
+    feedback: Tensor,
+    output: Tensor,
+    encoded: Tensor,
+    coefficients: Tensor,
+    *,
+    values: Tensor,
+    group: int,
+    refit: int,
+    block: int,
+    integer_grid: bool,
+    code_minimum: float,
+    code_maximum: float,
+    asym: bool,
+    reciprocal: float,
+    value_minimum: float,
+    scale_format: str,
+    deferred_tiles: int = 4,
+) -> tuple[Tensor, Tensor | None]:
+    """The whole natural-order sweep in one call; returns the regions' scales (and offsets)
+    side by side, ``[rows, total groups]``."""
+    device = native.require_device(original, feedback, output, encoded, coefficients, values)
+    rows, width = original.shape
+    _check("original", original)
+    _check("feedback", feedback, (rows, width))
+    _check("output", output, (rows, width))
+    _check("coefficients", coefficients, (width, width))
+    if encoded.dtype != torch.uint8 or tuple(encoded.shape) != (rows, width) or not encoded.is_contiguous():
+        raise ValueError("encoded must be a contiguous uint8 tensor shaped like the weight")
+    region = min(refit, width)
+    groups = 0
+    for start in range(0, width, region):
+        span = min(region, width - start)
+        groups += -(-span // min(group, span))
+    scales = torch.empty((rows, groups), device=device, dtype=torch.float32)
+    zeros = torch.empty_like(scales) if asym else None
+    workspace = torch.empty((rows, region), device=device, dtype=torch.float32) if region < width else None
+    values = values.to(torch.float32).contiguous()
+    native.check(native.library().mk_feedback_sweep(
+        original.data_ptr(), feedback.data_ptr(), output.data_ptr(), encoded.data_ptr(), coefficients.data_ptr(),
+        scales.data_ptr(), native.pointer(zeros), native.pointer(workspace), values.data_ptr(), values.numel(),
+        rows, width, group, refit, block, int(integer_grid), float(code_minimum), float(code_maximum), int(asym),
+        float(reciprocal), float(value_minimum), native.SCALE_FORMAT_CODES[scale_format], deferred_tiles,
+        native.current_stream(device),
+    ))
+    return scales, zeros

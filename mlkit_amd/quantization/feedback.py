@@ -190,6 +190,45 @@ class ErrorFeedback(Quantizer):
             raise ValueError("fused error feedback requires a HIP device and a native scalar rounder with step=1")
         return None
 
+    def _whole_sweep(self, original: Tensor, feedback: Tensor, output: Tensor, coefficients: Tensor,
+                     collected: "_Collected") -> bool:
+        """Run every region in one call into the library when the inner format is a scaled
+        scalar grid with range-fitted scales (no search, no user scale rule)."""
+        from mlkit_amd.quantization.scaled import SCALE_FORMAT_BITS, Scaled
+
+        inner = self.inner
+        rows, width = original.shape
+        refit = width if self.refit is None else self.refit
+        usable = (type(inner) is Scaled and self.step == 1 and self.backend != "torch" and inner.scale == "absmax"
+                  and isinstance(inner.scale_fmt, str) and inner.scale_fmt in SCALE_FORMAT_BITS
+                  and inner.grid.values is not None and inner.grid.bits <= 8
+                  and inner.grid.values.numel() <= FUSED_CODEBOOK_LIMIT and self.block_size <= MAXIMUM_FUSED_TILE
+                  and (refit >= width or refit <= MAXIMUM_FUSED_TILE))
+        if not usable:
+            return False
+        from mlkit_amd.kernels import error_feedback as kernel
+
+        group = width if inner.group is None else inner.group
+        values = inner.values_on(original.device)
+        encoded = torch.empty((rows, width), dtype=torch.uint8, device=original.device)
+        scales, zeros = kernel.sweep(
+            original, feedback, output, encoded, coefficients, values=values, group=group, refit=refit,
+            block=self.block_size, integer_grid=inner.grid.integer, code_minimum=inner._value_minimum,
+            code_maximum=inner._value_maximum, asym=inner.asym,
+            reciprocal=inner._range_reciprocal if inner.asym else inner._magnitude_reciprocal,
+            value_minimum=inner._value_minimum, scale_format=inner.scale_fmt, deferred_tiles=DEFERRED_TILES)
+        if not bool(torch.isfinite(scales).all()):
+            raise ValueError("scaled requires a finite floating-point weight matrix")
+        collected.codes = encoded
+        collected.shared = {"values": values, "group": min(group, min(refit, width))}
+        collected.metadata = {"code_bits": inner.grid.bits, "scale_fmt": inner.scale_fmt,
+                              "trainable": ["scales"] + (["zero"] if inner.asym else [])}
+        collected.scales = [scales]
+        collected.zeros = [] if zeros is None else [zeros]
+        side_bits = scales.numel() * SCALE_FORMAT_BITS[inner.scale_fmt] * (2 if inner.asym else 1)
+        collected.count(inner.grid.bits * rows * width + side_bits)
+        return True
+
     @staticmethod
     def _pending_continuation(feedback: Tensor, coefficients: Tensor, start: int, stop: int) -> Tensor:
         """The adjustment the region's columns would take if nothing more were rounded:
@@ -256,6 +295,9 @@ class ErrorFeedback(Quantizer):
         # one pass when the super-block ends (or when a region needs those columns).  Every
         # column still receives the tiles' sums one by one in tile order, so nothing changes
         # in the result.
+        fused = self._whole_sweep(original, feedback, output, coefficients, collected) if on_device else False
+        if fused:
+            return collected.result(output, permutation, refit_width, ctx)
         deferred: list[tuple[int, int]] = []
         limit = 0
 

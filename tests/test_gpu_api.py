@@ -342,3 +342,29 @@ def test_capabilities_on_device():
     assert report.packed_inference == "fused kernel" and report.online_activations == "fused kernel"
     assert mk.capabilities(mk.gptq(mk.int(4))).packed_inference == "fused kernel"
     assert mk.capabilities(mk.int(3, group=50), shape=(16, 250)).packed_inference.startswith("packed storage with dense")
+
+
+def test_whole_sweep_entry_point_equals_the_region_by_region_loop(rng):
+    """`mk_feedback_sweep` (one call) against the same kernels issued region by region from
+    Python (a subclass of Scaled is not eligible for the single call)."""
+    from mlkit_amd.quantization.scaled import Scaled
+
+    class Plain(Scaled):
+        pass
+
+    rows, width = 70, 1000   # ragged last region and tile
+    weight = dev(helpers.normal_weight(rows, width, seed=50))
+    inputs = rng.standard_normal((2048, width)).astype(F32)
+    inputs[:, ::11] *= 4
+    hessian = dev((inputs.T @ inputs / 2048).astype(F32))
+    for asym, refit, block in ((False, 128, 128), (True, 256, 64), (False, None, 128), (True, 96, 128)):
+        single = mk.gptq(Scaled(mk.grid.int(4), 32, asym=asym), refit=refit, block_size=block)(weight, Ctx(H=hessian))
+        looped = mk.gptq(Plain(mk.grid.int(4), 32, asym=asym), refit=refit, block_size=block)(weight, Ctx(H=hessian))
+        assert torch.equal(single.codes, looped.codes)
+        assert torch.equal(single.params["scales"], looped.params["scales"])
+        assert (single.params["zero"] is None) == (looped.params["zero"] is None)
+        if asym:
+            assert torch.equal(single.params["zero"], looped.params["zero"])
+        assert single.bits == looped.bits and single.params["group"] == looped.params["group"]
+        assert single.params["refit"] == looped.params["refit"] and single.metadata == looped.metadata
+        assert torch.equal(single.w, looped.w)
