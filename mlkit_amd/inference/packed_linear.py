@@ -15,7 +15,7 @@ import torch.nn.functional as functional
 from torch import Tensor, nn
 
 from mlkit_amd import native
-from mlkit_amd.kernels.packed_linear import MAXIMUM_CODE_BITS, decode, layout_for
+from mlkit_amd.kernels.packed_linear import MAXIMUM_CODE_BITS, decode, layout_for, packed_matvec_op
 from mlkit_amd.quantization.bitstream import pack, unpack
 from mlkit_amd.quantization.codecs import decode_scaled
 from mlkit_amd.quantization.core import Q
@@ -120,8 +120,13 @@ class PackedLinear(nn.Module):
         flat = inputs.reshape(rows, width)
         if not flat.is_contiguous():
             flat = flat.contiguous()
-        output = inputs.new_empty((rows, self.out_features))
-        self._matvec(flat, output, rows)
+        if torch.compiler.is_compiling():
+            output = packed_matvec_op(flat, self.packed, self.scales, self.values, self.zeros, self.bias,
+                                      self.out_features, self.group, self.code_bits, self.uniform_grid,
+                                      self.grid_minimum, self.grid_step)
+        else:
+            output = inputs.new_empty((rows, self.out_features))
+            self._matvec(flat, output, rows)
         return output.view(shape[:-1] + (self.out_features,))
 
     def _matvec(self, inputs: Tensor, output: Tensor, rows: int) -> None:

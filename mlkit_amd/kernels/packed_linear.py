@@ -132,3 +132,41 @@ def decode(
         native.current_stream(device),
     )
     native.check(status)
+
+
+@torch.library.custom_op("mlkit_amd::packed_matvec", mutates_args=())
+def packed_matvec_op(
+    inputs: Tensor,
+    packed: Tensor,
+    scales: Tensor,
+    values: Tensor,
+    zeros: Tensor | None,
+    bias: Tensor | None,
+    output_width: int,
+    group: int,
+    bits: int,
+    uniform_grid: bool,
+    grid_minimum: float,
+    grid_step: float,
+) -> Tensor:
+    """The fused matvec as a traceable operator: what a compiled graph holds in place of the
+    ``ctypes`` call (the reference lets the compiler capture its Triton launch instead,
+    inference/packed_linear.py:161-176).  It only enqueues on the current stream, so
+    ``mode="reduce-overhead"`` can capture it into a HIP graph."""
+    device = native.require_device(inputs, packed, scales, values, zeros, bias)
+    output = inputs.new_empty((inputs.shape[0], output_width))
+    status = native.library().mk_packed_matvec(
+        inputs.data_ptr(), native.dtype_code(inputs), packed.data_ptr(), scales.data_ptr(),
+        native.dtype_code(scales), values.data_ptr(), values.numel(), native.pointer(zeros),
+        native.pointer(bias), 0 if bias is None else native.dtype_code(bias), output.data_ptr(),
+        inputs.shape[0], output_width, inputs.shape[1], group, bits, int(uniform_grid), grid_minimum, grid_step,
+        native.current_stream(device),
+    )
+    native.check(status)
+    return output
+
+
+@packed_matvec_op.register_fake
+def _packed_matvec_shape(inputs, packed, scales, values, zeros, bias, output_width, group, bits, uniform_grid,
+                         grid_minimum, grid_step):
+    return inputs.new_empty((inputs.shape[0], output_width))

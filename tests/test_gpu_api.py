@@ -368,3 +368,32 @@ def test_whole_sweep_entry_point_equals_the_region_by_region_loop(rng):
         assert single.bits == looped.bits and single.params["group"] == looped.params["group"]
         assert single.params["refit"] == looped.params["refit"] and single.metadata == looped.metadata
         assert torch.equal(single.w, looped.w)
+
+
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+def test_packed_linear_under_torch_compile(backend):
+    """A compiled module holds the fused matvec as the operator `mlkit_amd::packed_matvec`."""
+    packed, converted = packed_and_reference(mk.int(4, group=64), dtype=torch.float16)
+    inputs = torch.randn(2, 256, dtype=torch.float16, device="cuda")
+    with torch.inference_mode():
+        expected = packed.module(inputs)
+        compiled = torch.compile(packed.module, backend=backend)
+        for _ in range(3):
+            torch.testing.assert_close(compiled(inputs), expected, rtol=0, atol=0)
+
+
+def test_optimize_with_compilation_replays_correctly():
+    """`mk.optimize(compile=True)` (mode "reduce-overhead": HIP graphs): every replay, with
+    eager work between replays, matches the eager packed model."""
+    torch.manual_seed(44)
+    module = nn.Sequential(nn.Linear(256, 96, dtype=torch.float16), nn.Linear(96, 64, dtype=torch.float16))
+    converted = mk.quantize(module, mk.int(4, group=32), calib=None)
+    eager = mk.optimize(converted, backend="packed")
+    compiled = mk.optimize(converted, backend="packed", compile=True)
+    assert compiled.execution_backend == "packed:2+compiled"
+    with torch.inference_mode():
+        for step in range(5):
+            inputs = torch.randn(1, 256, dtype=torch.float16, device="cuda") * (step + 1)
+            expected = eager(inputs).clone()
+            torch.cuda.synchronize()
+            torch.testing.assert_close(compiled(inputs).clone(), expected, rtol=0, atol=0)
