@@ -10,6 +10,7 @@ raises if that library is missing.
 """
 
 from mlkit_amd.checkpoints import load_checkpoint, save
+from mlkit_amd.conversion import Rotate, install_transform, rotate
 from mlkit_amd.evaluation.capabilities import Capabilities, capabilities
 from mlkit_amd.inference.optimization import optimize
 from mlkit_amd.inference.packed_linear import PackedEmbedding, PackedLinear, packed_compatible
@@ -34,8 +35,8 @@ def rtn(w, ctx=None, *, fmt=None):
 
 __all__ = [
     "Capabilities", "Ctx", "Grid", "Model", "NF4_VALUES", "PackedEmbedding", "PackedLinear", "Q", "QModel",
-    "Quantizer", "Scaled", "capabilities", "codec", "concatenate_rows", "deterministic_signs",
-    "feedback_coefficients", "gptq", "grid", "hadamard", "int", "layer_seed", "ldlq", "load_checkpoint", "mxfp4",
+    "Quantizer", "Rotate", "Scaled", "capabilities", "codec", "concatenate_rows", "deterministic_signs",
+    "feedback_coefficients", "gptq", "grid", "hadamard", "install_transform", "int", "layer_seed", "ldlq", "load_checkpoint", "mxfp4",
     "nf4", "optimize", "pack", "packed_compatible", "paley_matrix", "proxy_loss", "quantize", "quantizer", "rht",
-    "rtn", "save", "scaled", "snap", "store_scale", "structured_transform", "transform_factor", "unpack",
+    "rotate", "rtn", "save", "scaled", "snap", "store_scale", "structured_transform", "transform_factor", "unpack",
 ]

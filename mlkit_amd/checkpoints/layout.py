@@ -187,9 +187,13 @@ def load_checkpoint(path: "str | Path", *, model: "nn.Module | Callable[[], nn.M
     tied = manifest.get("tied_weights", {})
     for parameter_name, layer_name in tied.items():
         state[parameter_name] = state[_weight_name(layer_name)]
+    from mlkit_amd.conversion import install_transform, record_transform
+
+    for descriptor in manifest.get("transforms", []):
+        install_transform(module, descriptor)
+        record_transform(module, descriptor)
     module.load_state_dict(state, strict=True)
     converted = QModel(module.eval(), None, name=manifest["name"])
     converted.quantized = restored
     converted.tied_weights = dict(tied)
-    converted.transforms = list(manifest.get("transforms", []))
     return converted

@@ -1,0 +1,66 @@
+"""Online input rotations of linear layers: the part of the reference's ``rotate`` pass that
+sits on the packed-inference path.
+
+Mirrors /root/reference/src/mlkit/conversion/model_transforms.py:116-128 (the online branch of
+``Rotate``: every ``o_proj`` / ``down_proj`` gets its weight columns rotated offline with a
+per-layer seed and a forward pre-hook that rotates its inputs) and :179-209
+(``record_transform``, ``install_transform``; descriptor ``{"kind": "rotation", "name", "seed"}``,
+persisted in the checkpoint manifest and re-installed on load).  The residual-stream rotation
+of the same pass needs the architecture adapters and norm fusion, which are outside this
+package's path.
+"""
+
+from dataclasses import dataclass
+from typing import Any
+
+import torch
+from torch import nn
+
+from mlkit_amd.models import Model
+from mlkit_amd.quantization.core import layer_seed
+from mlkit_amd.quantization.transforms import rht
+
+ROTATED_LAYER_NAMES = ("o_proj", "down_proj")
+
+
+def record_transform(model: nn.Module, descriptor: dict[str, Any]) -> None:
+    descriptors = getattr(model, "_mlkit_transforms", [])
+    descriptors.append(descriptor)
+    model.__dict__["_mlkit_transforms"] = descriptors
+
+
+def install_transform(model: nn.Module, descriptor: dict[str, Any]) -> None:
+    """Attach the online half of a recorded transform to the layer it names."""
+    if descriptor["kind"] != "rotation":
+        raise ValueError(f"unknown model transform {descriptor['kind']!r}")
+    seed = descriptor["seed"]
+
+    def rotate_inputs(layer: nn.Module, arguments: tuple) -> tuple:
+        # fp16 / bf16 inputs are transformed in fp32 inside the kernel and rounded once
+        return (rht(arguments[0], seed=seed), *arguments[1:])
+
+    model.get_submodule(descriptor["name"]).register_forward_pre_hook(rotate_inputs)
+
+
+@dataclass
+class Rotate:
+    """``Rotate(seed)(model)``: rotate the input side of every selected linear layer."""
+
+    seed: int = 0
+    names: tuple[str, ...] = ROTATED_LAYER_NAMES
+
+    def __call__(self, model: "Model | nn.Module", calib: Any = None) -> None:
+        module = model.module if isinstance(model, Model) else model
+        with torch.no_grad():
+            for name, layer in module.named_modules():
+                if not isinstance(layer, nn.Linear) or name.split(".")[-1] not in self.names:
+                    continue
+                seed = layer_seed(name, self.seed)
+                layer.weight.copy_(rht(layer.weight.float(), seed=seed).to(layer.weight.dtype))
+                descriptor = {"kind": "rotation", "name": name, "seed": seed}
+                install_transform(module, descriptor)
+                record_transform(module, descriptor)
+
+
+def rotate(seed: int = 0, names: tuple[str, ...] = ROTATED_LAYER_NAMES) -> Rotate:
+    return Rotate(seed, tuple(names))

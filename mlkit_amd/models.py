@@ -49,7 +49,11 @@ class QModel(Model):
         super().__init__(*args, **kwargs)
         self.quantized: dict[str, Q] = {}
         self.tied_weights: dict[str, str] = {}
-        self.transforms: list[dict[str, Any]] = []
+
+    @property
+    def transforms(self) -> list[dict[str, Any]]:
+        """Descriptors of the online transforms installed on the module (rotations)."""
+        return list(getattr(self.module, "_mlkit_transforms", []))
 
     @property
     def bpw(self) -> float | None:

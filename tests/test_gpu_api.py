@@ -397,3 +397,38 @@ def test_optimize_with_compilation_replays_correctly():
             expected = eager(inputs).clone()
             torch.cuda.synchronize()
             torch.testing.assert_close(compiled(inputs).clone(), expected, rtol=0, atol=0)
+
+
+class Block(nn.Module):
+    def __init__(self, width=896, hidden=4864):
+        super().__init__()
+        self.up_proj = nn.Linear(width, hidden, bias=False)
+        self.down_proj = nn.Linear(hidden, width, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(torch.relu(self.up_proj(x)))
+
+
+def test_online_rotation_survives_quantization_packing_and_checkpoints(tmp_path):
+    """Rotated down projection (4864 = 76 x 64, Paley order 76): same function before
+    quantization; after quantization the packed model keeps the input hook, and a checkpoint
+    restores both the codes and the rotation."""
+    torch.manual_seed(45)
+    module = Block().cuda()
+    inputs = torch.randn(3, 896, device="cuda")
+    expected = module(inputs)
+    mk.rotate(seed=7)(module)
+    assert module._mlkit_transforms == [{"kind": "rotation", "name": "down_proj",
+                                         "seed": mk.layer_seed("down_proj", 7)}]
+    torch.testing.assert_close(module(inputs), expected, rtol=1e-4, atol=1e-4)
+    converted = mk.quantize(module, mk.int(4, group=64), calib=None)
+    assert converted.transforms == module._mlkit_transforms
+    quantized_output = converted(inputs)
+    packed = mk.optimize(converted, backend="packed")
+    assert isinstance(packed.module.down_proj, mk.PackedLinear) and len(packed.module.down_proj._forward_pre_hooks) == 1
+    with torch.inference_mode():
+        torch.testing.assert_close(packed(inputs), quantized_output, rtol=1e-4, atol=1e-4)
+    mk.save(converted, tmp_path / "rotated")
+    restored = mk.load_checkpoint(tmp_path / "rotated", model=Block)
+    assert restored.transforms == converted.transforms
+    torch.testing.assert_close(restored(inputs), quantized_output, rtol=0, atol=0)
