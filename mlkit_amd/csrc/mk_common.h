@@ -46,6 +46,7 @@ typedef uint32_t mk_u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t mk_u32x3 __attribute__((ext_vector_type(3)));
 typedef uint32_t mk_u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 mk_h2 __attribute__((ext_vector_type(2)));
+typedef __bf16 mk_bf2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float mk_bf16_to_float(uint16_t bits) {
     return __uint_as_float(static_cast<uint32_t>(bits) << 16);

@@ -211,6 +211,7 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
         s4.samples = samples; s4.rows = output_width; s4.width = input_width; s4.group = group;
         s4.groups = groups; s4.bias_dtype = bias_dtype; s4.grid_min = grid_min; s4.grid_step = grid_step;
         s4.values = values; s4.n_values = n_values; s4.uniform = uniform; s4.bits = bits;
+        s4.x_dtype = x_dtype; s4.scale_dtype = scale_dtype;
         done_rows = mk_matvec::pairs_launch(s4, stream);
         if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
     } else if (aligned && plan_chunked(samples, output_width, input_width, group, groups, bits, x_dtype,

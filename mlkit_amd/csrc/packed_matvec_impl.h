@@ -65,6 +65,7 @@ struct Stream4Args {
     float grid_min, grid_step;
     const float *values;  // fp32 table (pair-table kernel, when uniform == 0)
     int n_values, uniform, bits;
+    int x_dtype, scale_dtype;  // pair-table kernel: MK_F16 or MK_BF16 each
 };
 // Pair-table kernel (packed_matvec_pairs.hip): 2-, 3- and 4-bit codes of any scalar grid.
 bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype);

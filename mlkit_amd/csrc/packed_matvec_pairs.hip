@@ -1,11 +1,11 @@
 // Packed matvec for 2-, 3- and 4-bit codes of any scalar grid (integer grids, NF4, small
-// codebooks) with fp16 activations and fp16 scales, rows of K = 32 ... 16384 codes (K % 32 == 0).
+// codebooks) with fp16 or bf16 activations and 16-bit scales, rows of K = 32 ... 16384 codes (K % 32 == 0).
 //
-// Two adjacent codes index a table of fp16 pairs (value[low], value[high]) held in LDS, so
-// one LDS read decodes two weights and one v_dot2_f32_f16 multiplies them with the
-// matching pair of activations, accumulating in fp32.  Table entries are the grid values
-// rounded to fp16 (exact for integer grids and minifloats; NF4-like tables lose at most
-// 2^-11 relative per weight, inside the fp16 output's own rounding).  Entries of different
+// Two adjacent codes index a table of 16-bit pairs (value[low], value[high]) held in LDS, so
+// one LDS read decodes two weights and one v_dot2_f32_f16 (v_dot2_f32_bf16) multiplies them
+// with the matching pair of activations, accumulating in fp32.  Table entries are the grid
+// values rounded to the activations' type (exact for integer grids and minifloats; NF4-like
+// tables lose at most half an ulp of that type per weight, as the activations themselves do).  Entries of different
 // pairs fall in different LDS banks except by coincidence, so the lookups mostly proceed
 // at full rate.  Work split, load order and the reduction are those of the 4-bit streaming
 // kernel: a workgroup of ceil(K/2048) wavefronts owns 16 rows; lane t owns codes [32t, 32t + 32)
@@ -23,6 +23,13 @@ namespace {
 
 constexpr int kPairRows = 16;
 constexpr int kPairAhead = 8;
+
+// A 16-bit scale or offset (fp16 or bf16, uniform per launch) as fp32.
+__device__ __forceinline__ float side_value(uint16_t raw, int dtype) {
+    const float from_half = static_cast<float>(__builtin_bit_cast(_Float16, raw));
+    const float from_brain = __uint_as_float(static_cast<uint32_t>(raw) << 16);
+    return dtype == MK_F16 ? from_half : from_brain;
+}
 
 template <int MT>
 constexpr int pair_reduce_rows() {
@@ -44,10 +51,10 @@ __device__ __forceinline__ uint32_t pair_offset(const CodeChunk<BITS> &c, int i)
     return (__builtin_amdgcn_alignbit(c.w[(word + 1) % BITS], c.w[word], shift) << 2) & mask;
 }
 
-template <int BITS, int MT, bool HAS_ZERO>
+template <int BITS, int MT, bool HAS_ZERO, int XT>
 __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
     constexpr int kEntries = 1 << (2 * BITS);
-    __shared__ uint32_t table[kEntries];  // fp16 pairs
+    __shared__ uint32_t table[kEntries];  // fp16 (or bf16) pairs
     __shared__ float partials[64 * 8];    // [row sum][wavefront]
     constexpr int kReduceRows = pair_reduce_rows<MT>();
     constexpr int kSums = kReduceRows * MT;
@@ -76,17 +83,21 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
             first = low < a.n_values ? a.values[low] : 0.0f;
             second = high < a.n_values ? a.values[high] : 0.0f;
         }
-        const mk_h2 pair = {static_cast<_Float16>(first), static_cast<_Float16>(second)};
-        table[entry] = __builtin_bit_cast(uint32_t, pair);
+        if constexpr (XT == MK_F16) {
+            const mk_h2 pair = {static_cast<_Float16>(first), static_cast<_Float16>(second)};
+            table[entry] = __builtin_bit_cast(uint32_t, pair);
+        } else {
+            table[entry] = static_cast<uint32_t>(mk_float_to_bf16(first)) | (static_cast<uint32_t>(mk_float_to_bf16(second)) << 16);
+        }
     }
     // Also aligns the wavefronts, so that nobody's small loads queue behind another's codes.
     __syncthreads();
 
-    XChunk<MK_F16> x[MT];
+    XChunk<XT> x[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int sample = sample_base + m < a.samples ? sample_base + m : a.samples - 1;
-        load_x_chunk<MK_F16>(x[m], a.x, static_cast<size_t>(sample) * a.width + static_cast<size_t>(chunk) * kChunkCodes);
+        load_x_chunk<XT>(x[m], a.x, static_cast<size_t>(sample) * a.width + static_cast<size_t>(chunk) * kChunkCodes);
     }
     const uint32_t group_offset = ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
@@ -115,7 +126,7 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
         const uint32_t keep = in_row && sample_base + m < a.samples ? 0xffffffffu : 0u;
 #pragma unroll
         for (int i = 0; i < 16; ++i) x[m].r[i] &= keep;
-        x_sum[m] = HAS_ZERO ? chunk_sum<MK_F16>(x[m]) : 0.0f;
+        x_sum[m] = HAS_ZERO ? chunk_sum<XT>(x[m]) : 0.0f;
     }
 
     const uint8_t *table_bytes = reinterpret_cast<const uint8_t *>(table);
@@ -131,20 +142,24 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const uint32_t entry = *reinterpret_cast<const uint32_t *>(table_bytes + pair_offset<BITS>(codes[r], i));
-                const mk_h2 weights = __builtin_bit_cast(mk_h2, entry);
 #pragma unroll
-                for (int m = 0; m < MT; ++m)
-                    dot[m] = __builtin_amdgcn_fdot2(weights, __builtin_bit_cast(mk_h2, x[m].r[i]), dot[m], false);
+                for (int m = 0; m < MT; ++m) {
+                    if constexpr (XT == MK_F16)
+                        dot[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(mk_h2, entry),
+                                                        __builtin_bit_cast(mk_h2, x[m].r[i]), dot[m], false);
+                    else
+                        dot[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mk_bf2, entry),
+                                                                 __builtin_bit_cast(mk_bf2, x[m].r[i]), dot[m], false);
+                }
             }
             if (r + kPairAhead < kPairRows)
                 load_codes<BITS>(codes[r + kPairAhead],
                                  codes_base + static_cast<size_t>(r + kPairAhead) * row_bytes + code_offset);
-            const float scale = static_cast<float>(__builtin_bit_cast(_Float16, scale_raw[r]));
+            const float scale = side_value(scale_raw[r], a.scale_dtype);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 float value = scale * dot[m];
-                if constexpr (HAS_ZERO)
-                    value = __builtin_fmaf(static_cast<float>(__builtin_bit_cast(_Float16, zero_raw[r])), x_sum[m], value);
+                if constexpr (HAS_ZERO) value = __builtin_fmaf(side_value(zero_raw[r], a.scale_dtype), x_sum[m], value);
                 sums[j * MT + m] = value;
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -163,20 +178,30 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
             const int sample = sample_base + m;
             if (sample < a.samples) {
                 if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
-                static_cast<_Float16 *>(a.y)[static_cast<size_t>(sample) * a.rows + row] = static_cast<_Float16>(total);
+                const size_t index = static_cast<size_t>(sample) * a.rows + row;
+                if constexpr (XT == MK_F16)
+                    static_cast<_Float16 *>(a.y)[index] = static_cast<_Float16>(total);
+                else
+                    static_cast<uint16_t *>(a.y)[index] = mk_float_to_bf16(total);
             }
         }
     }
 }
 
-template <int BITS, int MT>
-void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
+template <int BITS, int MT, int XT>
+void launch_tile_as(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     if (a.zeros)
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT>), grid, block, 0, stream, a);
+}
+
+template <int BITS, int MT>
+void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
+    if (a.x_dtype == MK_F16) launch_tile_as<BITS, MT, MK_F16>(a, tiles, stream);
+    else launch_tile_as<BITS, MT, MK_BF16>(a, tiles, stream);
 }
 
 template <int BITS>
@@ -194,7 +219,7 @@ void launch_bits(const Stream4Args &a, int tiles, hipStream_t stream) {
 }  // namespace
 
 bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype) {
-    return bits >= 2 && bits <= 4 && x_dtype == MK_F16 && scale_dtype == MK_F16 && width % kChunkCodes == 0 &&
+    return bits >= 2 && bits <= 4 && x_dtype != MK_F32 && scale_dtype != MK_F32 && width % kChunkCodes == 0 &&
            width <= 16384 && (group % kChunkCodes == 0 || group >= width);
 }
 

@@ -24,8 +24,14 @@ namespace mk_matvec {
 
 namespace {
 
-constexpr int kStreamRows = 16;   // rows per workgroup
-constexpr int kStreamAhead = 8;   // rows of codes in flight per wavefront
+#ifndef MK_S4_ROWS
+#define MK_S4_ROWS 16
+#endif
+#ifndef MK_S4_AHEAD
+#define MK_S4_AHEAD 8
+#endif
+constexpr int kStreamRows = MK_S4_ROWS;    // rows per workgroup
+constexpr int kStreamAhead = MK_S4_AHEAD;  // rows of codes in flight per wavefront
 
 // Rows per transposed reduction: all 16 when that is at most 64 sums per lane (measured
 // faster than splitting the reduction to hide part of it behind the stream).

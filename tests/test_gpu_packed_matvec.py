@@ -239,3 +239,18 @@ def test_packed_decode_full_layer_matches_matvec_input():
     x = helpers.activations(2, 14336, seed=32)
     fused = run_matvec(layer, x)
     np.testing.assert_allclose((x.cuda().float() @ dense.float().T).cpu().numpy(), fused, rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("bits,values,integer", [(4, INT4, True), (2, scaling.int_values(2), True),
+                                                 (3, scaling.int_values(3), True), (4, scaling.NF4_VALUES, False)])
+@pytest.mark.parametrize("scale_dtype", [torch.float16, torch.bfloat16])
+def test_bf16_activations_use_the_pair_table_kernel(bits, values, integer, scale_dtype):
+    """bf16 activations (bf16 outputs) with fp16 or bf16 scales; integer grids are exact in the
+    bf16 table, so the error is the bf16 rounding of inputs and outputs only."""
+    weight = helpers.normal_weight(48, 4096, seed=21, student_t=True)
+    for asym in (False, True):
+        layer = helpers.quantised_layer(weight, values, bits=bits, group=128, integer=integer, asym=asym,
+                                        fmt="fp16" if scale_dtype == torch.float16 else "bf16")
+        for samples in (1, 8):
+            x = helpers.activations(samples, 4096, seed=22 + samples, dtype=torch.bfloat16)
+            check(run_matvec(layer, x, scale_dtype=scale_dtype), layer, x, relative=8e-3)
