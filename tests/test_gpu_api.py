@@ -432,3 +432,40 @@ def test_online_rotation_survives_quantization_packing_and_checkpoints(tmp_path)
     restored = mk.load_checkpoint(tmp_path / "rotated", model=Block)
     assert restored.transforms == converted.transforms
     torch.testing.assert_close(restored(inputs), quantized_output, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("rows,width", [(4096, 14336), (14336, 4096)])
+def test_config5_rotated_int4_layer_end_to_end(rows, width):
+    """Offline rotation of the weight columns (14336 -> 28 x 512 Paley blocks, 4096 -> one
+    FWHT), INT4-g128 quantization, online rotation of fp16 activations and the fused matvec:
+    against the oracle's rotated path at matvec tolerance, and against the unrotated fp32
+    product within quantization error."""
+    from mlkit_amd.quantization.transforms import random_signs
+    from oracle import matvec as oracle_matvec
+
+    torch.manual_seed(46)
+    layer = nn.Linear(width, rows, bias=False, dtype=torch.float16)
+    with torch.no_grad():
+        layer.weight.normal_(0, 0.02)
+    module = nn.ModuleDict({"down_proj": layer}).cuda()
+    plain = layer.weight.detach().float().clone()
+    mk.rotate(seed=3)(module)
+    seed = mk.layer_seed("down_proj", 3)
+    converted = mk.quantize(module, mk.int(4, group=128), calib=None)
+    packed = mk.optimize(converted, backend="packed", inplace=True)
+    fused = packed.module["down_proj"]
+    assert isinstance(fused, mk.PackedLinear) and fused.layout is not None
+    q = converted.quantized["down_proj"]
+    signs = host(random_signs(width, seed, "cuda"))
+    dense = scaling.decode_grouped(host(q.codes), host(q.params["scales"]), scaling.int_values(4), 128)
+    for samples in (1, 8):
+        x = torch.randn(samples, width, device="cuda").half()
+        with torch.inference_mode():
+            y = fused(x)
+        rotated = oracle_transforms.randomized(host(x.float()), signs).astype(np.float16).astype(F32)
+        expected = oracle_matvec.reconstruct_then_matmul_f64(rotated, dense)
+        error = np.abs(host(y.float()) - expected).max() / np.abs(expected).max()
+        assert error <= 2e-3, error
+        exact = host(x.float() @ plain.T)
+        relative = np.linalg.norm(host(y.float()) - exact) / np.linalg.norm(exact)
+        assert relative < 0.15, relative   # 4-bit rounding noise of a Gaussian layer
