@@ -1,9 +1,10 @@
 // Packed matvec for 2-, 3- and 4-bit codes of any scalar grid (integer grids, NF4, small
 // codebooks) with fp16 or bf16 activations and 16-bit scales, rows of K = 32 ... 16384 codes (K % 32 == 0).
 //
-// Two adjacent codes index a table of 16-bit pairs (value[low], value[high]) held in LDS, so
-// one LDS read decodes two weights and one v_dot2_f32_f16 (v_dot2_f32_bf16) multiplies them
-// with the matching pair of activations, accumulating in fp32.  Table entries are the grid
+// Adjacent codes (two 4-bit codes, four 2- or 3-bit codes) index a table of 16-bit value
+// pairs held in LDS, so one LDS read decodes two or four weights and one v_dot2_f32_f16
+// (v_dot2_f32_bf16) per pair multiplies them with the matching activations, accumulating
+// in fp32.  Table entries are the grid
 // values rounded to the activations' type (exact for integer grids and minifloats; NF4-like
 // tables lose at most half an ulp of that type per weight, as the activations themselves do).  Entries of different
 // pairs fall in different LDS banks except by coincidence, so the lookups mostly proceed
@@ -36,25 +37,37 @@ constexpr int pair_reduce_rows() {
     return kPairRows * MT <= 64 ? kPairRows : 64 / MT;
 }
 
-// Field i (0..15) of 2*BITS bits out of a chunk of BITS dwords, times four (a byte offset
-// into the table).  i is a compile-time constant after unrolling.
-template <int BITS>
-__device__ __forceinline__ uint32_t pair_offset(const CodeChunk<BITS> &c, int i) {
-    constexpr int kField = 2 * BITS;
-    constexpr uint32_t mask = ((1u << kField) - 1u) << 2;
+// Codes decoded per table lookup: two (an entry is one 16-bit pair), or four for 2-bit codes
+// and for 3-bit codes of long rows (entries of two pairs; the 4096-entry 3-bit table only pays
+// for itself when a workgroup has enough threads to fill it quickly).
+template <int BITS, bool QUAD>
+constexpr int lookup_codes() {
+    return QUAD ? 4 : 2;
+}
+
+// Byte offset into the table of field i of a chunk of BITS dwords; a field holds
+// lookup_codes() adjacent codes and an entry two bytes per code.  i is a compile-time
+// constant after unrolling.
+template <int BITS, bool QUAD>
+__device__ __forceinline__ uint32_t lookup_offset(const CodeChunk<BITS> &c, int i) {
+    constexpr int kField = lookup_codes<BITS, QUAD>() * BITS;
+    constexpr int kEntryShift = QUAD ? 3 : 2;
+    constexpr uint32_t mask = ((1u << kField) - 1u) << kEntryShift;
     const int bit = i * kField;
     const int word = bit >> 5, shift = bit & 31;
     if (shift + kField <= 32) {
-        if (shift >= 2) return (c.w[word] >> (shift - 2)) & mask;
-        return (c.w[word] << (2 - shift)) & mask;
+        if (shift >= kEntryShift) return (c.w[word] >> (shift - kEntryShift)) & mask;
+        return (c.w[word] << (kEntryShift - shift)) & mask;
     }
-    return (__builtin_amdgcn_alignbit(c.w[(word + 1) % BITS], c.w[word], shift) << 2) & mask;
+    return (__builtin_amdgcn_alignbit(c.w[(word + 1) % BITS], c.w[word], shift) << kEntryShift) & mask;
 }
 
-template <int BITS, int MT, bool HAS_ZERO, int XT>
+template <int BITS, int MT, bool HAS_ZERO, int XT, bool QUAD>
 __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
-    constexpr int kEntries = 1 << (2 * BITS);
-    __shared__ uint32_t table[kEntries];  // fp16 (or bf16) pairs
+    constexpr int kLookup = lookup_codes<BITS, QUAD>();
+    constexpr int kEntries = 1 << (kLookup * BITS);
+    constexpr int kEntryWords = kLookup / 2;
+    __shared__ __attribute__((aligned(8))) uint32_t table[kEntries * kEntryWords];  // 16-bit pairs
     __shared__ float partials[64 * 8];    // [row sum][wavefront]
     constexpr int kReduceRows = pair_reduce_rows<MT>();
     constexpr int kSums = kReduceRows * MT;
@@ -73,21 +86,24 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
     const int chunk = in_row ? tid : 0;
     const uint32_t code_offset = static_cast<uint32_t>(chunk) * (4u * BITS);
 
-    for (int entry = tid; entry < kEntries; entry += blockDim.x) {
-        const int low = entry & ((1 << BITS) - 1), high = entry >> BITS;
-        float first, second;
-        if (a.uniform) {
-            first = __builtin_fmaf(static_cast<float>(low), a.grid_step, a.grid_min);
-            second = __builtin_fmaf(static_cast<float>(high), a.grid_step, a.grid_min);
-        } else {
-            first = low < a.n_values ? a.values[low] : 0.0f;
-            second = high < a.n_values ? a.values[high] : 0.0f;
-        }
+    // The grid's values first (one global load per value), then every table entry from them.
+    __shared__ float grid_values[1 << BITS];
+    if (tid < (1 << BITS)) {
+        float value = 0.0f;
+        if (a.uniform) value = __builtin_fmaf(static_cast<float>(tid), a.grid_step, a.grid_min);
+        else if (tid < a.n_values) value = a.values[tid];
+        grid_values[tid] = value;
+    }
+    __syncthreads();
+    for (int word = tid; word < kEntries * kEntryWords; word += blockDim.x) {
+        const int entry = word / kEntryWords, half = word - entry * kEntryWords;
+        const float first = grid_values[(entry >> (2 * half * BITS)) & ((1 << BITS) - 1)];
+        const float second = grid_values[(entry >> ((2 * half + 1) * BITS)) & ((1 << BITS) - 1)];
         if constexpr (XT == MK_F16) {
             const mk_h2 pair = {static_cast<_Float16>(first), static_cast<_Float16>(second)};
-            table[entry] = __builtin_bit_cast(uint32_t, pair);
+            table[word] = __builtin_bit_cast(uint32_t, pair);
         } else {
-            table[entry] = static_cast<uint32_t>(mk_float_to_bf16(first)) | (static_cast<uint32_t>(mk_float_to_bf16(second)) << 16);
+            table[word] = static_cast<uint32_t>(mk_float_to_bf16(first)) | (static_cast<uint32_t>(mk_float_to_bf16(second)) << 16);
         }
     }
     // Also aligns the wavefronts, so that nobody's small loads queue behind another's codes.
@@ -140,17 +156,27 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
 #pragma unroll
             for (int m = 0; m < MT; ++m) dot[m] = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const uint32_t entry = *reinterpret_cast<const uint32_t *>(table_bytes + pair_offset<BITS>(codes[r], i));
-#pragma unroll
-                for (int m = 0; m < MT; ++m) {
-                    if constexpr (XT == MK_F16)
-                        dot[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(mk_h2, entry),
-                                                        __builtin_bit_cast(mk_h2, x[m].r[i]), dot[m], false);
-                    else
-                        dot[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mk_bf2, entry),
-                                                                 __builtin_bit_cast(mk_bf2, x[m].r[i]), dot[m], false);
+            for (int i = 0; i < 32 / kLookup; ++i) {
+                uint32_t entry[kEntryWords];
+                if constexpr (kEntryWords == 2) {
+                    const mk_u32x2 both = *reinterpret_cast<const mk_u32x2 *>(table_bytes + lookup_offset<BITS, QUAD>(codes[r], i));
+                    entry[0] = both.x;
+                    entry[1] = both.y;
+                } else {
+                    entry[0] = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, QUAD>(codes[r], i));
                 }
+#pragma unroll
+                for (int h = 0; h < kEntryWords; ++h)
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) {
+                        const uint32_t inputs = x[m].r[kEntryWords * i + h];
+                        if constexpr (XT == MK_F16)
+                            dot[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(mk_h2, entry[h]),
+                                                            __builtin_bit_cast(mk_h2, inputs), dot[m], false);
+                        else
+                            dot[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mk_bf2, entry[h]),
+                                                                     __builtin_bit_cast(mk_bf2, inputs), dot[m], false);
+                    }
             }
             if (r + kPairAhead < kPairRows)
                 load_codes<BITS>(codes[r + kPairAhead],
@@ -188,14 +214,26 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
     }
 }
 
-template <int BITS, int MT, int XT>
-void launch_tile_as(const Stream4Args &a, int tiles, hipStream_t stream) {
+template <int BITS, int MT, int XT, bool QUAD>
+void launch_tile_with(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     if (a.zeros)
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, QUAD>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, QUAD>), grid, block, 0, stream, a);
+}
+
+template <int BITS, int MT, int XT>
+void launch_tile_as(const Stream4Args &a, int tiles, hipStream_t stream) {
+    if constexpr (BITS == 2) {
+        launch_tile_with<BITS, MT, XT, true>(a, tiles, stream);
+    } else if constexpr (BITS == 3) {
+        if (a.width >= 8192) launch_tile_with<BITS, MT, XT, true>(a, tiles, stream);
+        else launch_tile_with<BITS, MT, XT, false>(a, tiles, stream);
+    } else {
+        launch_tile_with<BITS, MT, XT, false>(a, tiles, stream);
+    }
 }
 
 template <int BITS, int MT>

@@ -286,11 +286,22 @@ __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
         const float *row_value = a.value + static_cast<size_t>(row) * a.row_stride;
         float low = __builtin_inff(), high = -__builtin_inff();
         bool finite = true;
-        for (int column = start + lane_in_team; column < stop; column += LANES) {
-            const float v = row_value[column];
-            finite = finite && v - v == 0.0f;
-            low = fminf(low, v);
-            high = fmaxf(high, v);
+        // Four adjacent values per lane and step where the group allows 16-byte loads.
+        const bool wide = ((reinterpret_cast<uintptr_t>(row_value + start) & 15u) == 0) && ((stop - start) & 3) == 0;
+        if (wide) {
+            for (int column = start + 4 * lane_in_team; column < stop; column += 4 * LANES) {
+                const float4 v = *reinterpret_cast<const float4 *>(row_value + column);
+                finite = finite && (v.x - v.x == 0.0f) && (v.y - v.y == 0.0f) && (v.z - v.z == 0.0f) && (v.w - v.w == 0.0f);
+                low = fminf(fminf(low, fminf(v.x, v.y)), fminf(v.z, v.w));
+                high = fmaxf(fmaxf(high, fmaxf(v.x, v.y)), fmaxf(v.z, v.w));
+            }
+        } else {
+            for (int column = start + lane_in_team; column < stop; column += LANES) {
+                const float v = row_value[column];
+                finite = finite && v - v == 0.0f;
+                low = fminf(low, v);
+                high = fmaxf(high, v);
+            }
         }
 #pragma unroll
         for (int offset = 1; offset < LANES; offset <<= 1) {
@@ -474,7 +485,9 @@ int mk_fit_scales_strided(const float *value, long long row_stride, float *scale
     a.rows = rows; a.span = span; a.group = group; a.groups_per_row = groups_per_row;
     a.total_groups = rows * groups_per_row; a.asym = asym; a.format = scale_format; a.store_zero = store_zero;
     a.reciprocal = reciprocal; a.value_minimum = value_minimum;
-    const int reach = group < span ? group : span;
+    int reach = group < span ? group : span;
+    const bool wide = row_stride % 4 == 0 && group % 4 == 0 && span % 4 == 0 && (reinterpret_cast<uintptr_t>(value) & 15u) == 0;
+    if (wide) reach /= 4;  // lanes read four values at a time
     if (reach >= 64) launch_fit<64>(a, stream);
     else if (reach >= 32) launch_fit<32>(a, stream);
     else if (reach >= 16) launch_fit<16>(a, stream);
