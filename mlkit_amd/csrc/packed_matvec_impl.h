@@ -129,14 +129,16 @@ __device__ __forceinline__ float chunk_sum(const XChunk<XT> &x) {
 
 // (x0,x1)(x2,x3)(x4,x5)(x6,x7) -> (x0,x4) (x1,x5)/16 (x2,x6) (x3,x7)/16 for every eight
 // codes: the pair order and scaling the 4-bit extraction of chunk_dot expects.  Returns
-// what that extraction accumulates for all-zero codes, 1024 * sum(stored values).
-__device__ __forceinline__ float pair_for_nibbles(XChunk<MK_F16> &x) {
+// what that extraction accumulates for all-zero codes, 1024 * sum(stored values); with
+// `stored_sum`, also the sum of the activations as the dot products see them.
+__device__ __forceinline__ float pair_for_nibbles(XChunk<MK_F16> &x, float *stored_sum = nullptr) {
     const mk_h2 sixteenth = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
-    const mk_h2 base = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+    const mk_h2 ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
     auto scaled = [&](uint32_t pair) __attribute__((always_inline)) {
         return __builtin_bit_cast(uint32_t, __builtin_bit_cast(mk_h2, pair) * sixteenth);
     };
-    float offset = 0.0f;
+    // plain: sum of the activations kept as they are; reduced: sum of those kept at 1/16.
+    float plain = 0.0f, reduced = 0.0f;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         const uint32_t p0 = x.r[4 * g + 0], p1 = x.r[4 * g + 1];
@@ -145,11 +147,14 @@ __device__ __forceinline__ float pair_for_nibbles(XChunk<MK_F16> &x) {
         x.r[4 * g + 1] = scaled(__builtin_amdgcn_perm(p2, p0, 0x07060302u));
         x.r[4 * g + 2] = __builtin_amdgcn_perm(p3, p1, 0x05040100u);
         x.r[4 * g + 3] = scaled(__builtin_amdgcn_perm(p3, p1, 0x07060302u));
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            offset = __builtin_amdgcn_fdot2(base, __builtin_bit_cast(mk_h2, x.r[4 * g + j]), offset, false);
+        plain = __builtin_amdgcn_fdot2(ones, __builtin_bit_cast(mk_h2, x.r[4 * g + 0]), plain, false);
+        reduced = __builtin_amdgcn_fdot2(ones, __builtin_bit_cast(mk_h2, x.r[4 * g + 1]), reduced, false);
+        plain = __builtin_amdgcn_fdot2(ones, __builtin_bit_cast(mk_h2, x.r[4 * g + 2]), plain, false);
+        reduced = __builtin_amdgcn_fdot2(ones, __builtin_bit_cast(mk_h2, x.r[4 * g + 3]), reduced, false);
     }
-    return offset;
+    // The sum the dot products effectively see: the 1/16 activations count sixteen-fold.
+    if (stored_sum) *stored_sum = __builtin_fmaf(16.0f, reduced, plain);
+    return 1024.0f * (plain + reduced);
 }
 
 // ---------------------------------------------------------------------------------

@@ -100,8 +100,7 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
         const uint32_t keep = in_row && sample_base + m < a.samples ? 0xffffffffu : 0u;
 #pragma unroll
         for (int i = 0; i < 16; ++i) x[m].r[i] &= keep;
-        x_sum[m] = chunk_sum<MK_F16>(x[m]);
-        const float code_free = pair_for_nibbles(x[m]);
+        const float code_free = pair_for_nibbles(x[m], &x_sum[m]);
         grid_term[m] = a.grid_min * x_sum[m] - a.grid_step * code_free;
     }
 
