@@ -303,7 +303,7 @@ class TiedHead(nn.Module):
 
 def test_embedding_tied_to_a_packed_head_reads_the_packed_rows():
     torch.manual_seed(42)
-    converted = mk.quantize(TiedHead(), mk.int(4, group=64), calib=None)
+    converted = mk.quantize(TiedHead(), mk.int(4, group=64), calib=None, head=mk.int(4, group=64))
     assert converted.tied_weights == {"embed.weight": "head"}
     packed = mk.optimize(converted, backend="packed")
     assert isinstance(packed.module.embed, mk.PackedEmbedding) and isinstance(packed.module.head, mk.PackedLinear)
@@ -469,3 +469,81 @@ def test_config5_rotated_int4_layer_end_to_end(rows, width):
         exact = host(x.float() @ plain.T)
         relative = np.linalg.norm(host(y.float()) - exact) / np.linalg.norm(exact)
         assert relative < 0.15, relative   # 4-bit rounding noise of a Gaussian layer
+
+
+def test_checkpoint_mirrors_of_the_reference_tests(tmp_path):
+    import json
+
+    def create_model():
+        return nn.Sequential(nn.Linear(32, 16), nn.ReLU(), nn.Linear(16, 8))
+
+    torch.manual_seed(47)
+    source = create_model()
+    before = source[0].weight.detach().clone()
+    converted = mk.quantize(source, mk.int(4, group=8), calib=None)
+    assert torch.equal(source[0].weight, before)          # the source model is left alone
+    directory = tmp_path / "checkpoint"
+    converted.save(directory)
+    restored = mk.load_checkpoint(directory, model=create_model)
+    inputs = torch.randn(4, 32)
+    torch.testing.assert_close(restored(inputs), converted(inputs), rtol=0, atol=0)
+    assert restored.bpw == converted.bpw
+    manifest = json.loads((directory / "mlkit.json").read_text())
+    assert manifest["tensor_bytes"] < sum(v.numel() * v.element_size() for v in converted.module.state_dict().values())
+    converted.save(directory, overwrite=True)
+    restored.save(tmp_path / "restored")
+    assert json.loads((tmp_path / "restored" / "mlkit.json").read_text())["tensor_bytes"] == manifest["tensor_bytes"]
+
+    custom = mk.quantize(nn.Sequential(nn.Linear(8, 4)), lambda w, ctx: w.round(), calib=None)
+    custom.save(tmp_path / "custom")
+    reloaded = mk.load_checkpoint(tmp_path / "custom", model=lambda: nn.Sequential(nn.Linear(8, 4)))
+    assert reloaded.bpw is None
+    torch.testing.assert_close(custom.module[0].weight, reloaded.module[0].weight)
+
+    root = mk.quantize(nn.Linear(32, 16, bias=False), mk.int(4, group=8), calib=None)
+    root.save(tmp_path / "root")
+    again = mk.load_checkpoint(tmp_path / "root", model=lambda: nn.Linear(32, 16, bias=False))
+    sample = torch.randn(3, 32)
+    torch.testing.assert_close(again(sample), root(sample), rtol=0, atol=0)
+    packed = mk.optimize(again, inplace=True)
+    assert isinstance(packed.module, mk.PackedLinear)
+    torch.testing.assert_close(packed(sample), root(sample), rtol=1e-5, atol=1e-6)
+
+
+def test_checkpoint_stores_tied_weights_and_shared_parameters_once(tmp_path):
+    import json
+
+    class TiedLanguageModel(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.embedding = nn.Embedding(32, 16)
+            self.projections = nn.Sequential(nn.Linear(16, 16), nn.Linear(16, 16))
+            self.lm_head = nn.Linear(16, 32, bias=False)
+            self.lm_head.weight = self.embedding.weight
+
+        def forward(self, tokens):
+            return self.lm_head(self.projections(self.embedding(tokens)))
+
+    converted = mk.quantize(TiedLanguageModel(), mk.int(4, group=8), calib=None)
+    converted.save(tmp_path / "shared")
+    manifest = json.loads((tmp_path / "shared" / "mlkit.json").read_text())
+    assert manifest["state_aliases"] == {"lm_head.weight": "embedding.weight"}
+    first = manifest["layers"]["projections.0"]["params"]["values"]["tensor"]
+    assert first == manifest["layers"]["projections.1"]["params"]["values"]["tensor"]
+    restored = mk.load_checkpoint(tmp_path / "shared", model=TiedLanguageModel)
+    tokens = torch.randint(32, (2, 7))
+    torch.testing.assert_close(restored(tokens), converted(tokens), rtol=0, atol=0)
+    assert restored.module.embedding.weight is restored.module.lm_head.weight
+
+
+def test_row_chunked_conversion_of_a_wide_head_equals_whole_conversion(monkeypatch):
+    import mlkit_amd.models as models
+
+    torch.manual_seed(48)
+    layer = nn.Linear(256, 1000, bias=False)
+    whole = mk.quantize(layer, mk.int(4, group=64), calib=None).quantized[""]
+    monkeypatch.setattr(models, "CHUNKED_CONVERSION_ELEMENTS", 1000)
+    monkeypatch.setattr(models, "ROW_CHUNK_ELEMENTS", 256 * 96)
+    chunked = mk.quantize(layer, mk.int(4, group=64), calib=None).quantized[""]
+    assert torch.equal(chunked.codes, whole.codes) and torch.equal(chunked.params["scales"], whole.params["scales"])
+    assert chunked.bits == whole.bits and chunked.codec == "scaled"
