@@ -123,6 +123,16 @@ int mk_fit_scales(const float *value, long long row_stride, float *scales, float
                   int span, int group, int asym, float reciprocal, float value_minimum,
                   int scale_format, int store_zero, void *stream);
 
+/* output = quantize-dequantize of `inputs` ([rows, width], fp32 / fp16 / bf16; output has the
+ * same dtype and may alias) with per-group scales fitted on the fly: the result equals
+ * mk_fit_scales (zeros stored rounded) + mk_scalar_encode + mk_scalar_decode on the fp32
+ * values, rounded to the input dtype.  `group` is clipped to width.
+ * Replaces: kernels/activation_reconstruction.py:76-103 (reconstruct). */
+int mk_reconstruct_activations(const void *inputs, int dtype, void *output, const float *values,
+                               int n_values, int rows, int width, int group, int scale_format,
+                               int asym, int integer, float minimum, float maximum, float reciprocal,
+                               void *stream);
+
 /* Walsh-Hadamard transform of `rows` rows of `width` = 2^S values: radix-2 butterflies in
  * ascending stride in fp32, then one multiplication by `scale`.  Input and output may be
  * fp32, fp16 or bf16 and may alias.  signs_before / signs_after (NULL or fp32 vectors of

@@ -341,6 +341,72 @@ void launch_fit(const FitArgs &a, hipStream_t stream) {
     hipLaunchKernelGGL((fit_kernel<LANES>), dim3(blocks), dim3(kThreads), 0, stream, a);
 }
 
+struct ReconstructArgs {
+    const void *inputs;
+    void *output;
+    const float *values;
+    int rows, width, group, groups_per_row, total_groups;
+    int dtype, n_values, format, asym, integer;
+    float reciprocal, minimum, maximum;
+};
+
+// Online quantize-dequantize of activations: a team of LANES lanes owns one (row, group);
+// it finds the group's range, derives the stored scale (and offset) exactly as fit_kernel
+// does, then rounds every element to the grid and writes scale * value (+ offset) in the
+// input's dtype.  The second pass re-reads the group from cache.
+template <int LANES>
+__global__ void __launch_bounds__(kThreads) reconstruct_kernel(const ReconstructArgs a) {
+    __shared__ float table[kMaxTable];
+    if (!a.integer) stage_table(table, a.values, a.n_values);
+    const int steps = bisection_steps(a.n_values);
+    constexpr int kTeams = kThreads / LANES;
+    const int lane_in_team = threadIdx.x % LANES;
+    for (int first = blockIdx.x * kTeams; first < a.total_groups; first += gridDim.x * kTeams) {
+        const int wanted = first + threadIdx.x / LANES;
+        const int identifier = wanted < a.total_groups ? wanted : a.total_groups - 1;
+        const int row = identifier / a.groups_per_row;
+        const int start = (identifier - row * a.groups_per_row) * a.group;
+        const int stop = start + a.group < a.width ? start + a.group : a.width;
+        const size_t base = static_cast<size_t>(row) * a.width;
+        float low = __builtin_inff(), high = -__builtin_inff();
+        for (int column = start + lane_in_team; column < stop; column += LANES) {
+            const float v = mk_load_as_float(a.inputs, base + column, a.dtype);
+            low = fminf(low, v);
+            high = fmaxf(high, v);
+        }
+#pragma unroll
+        for (int offset = 1; offset < LANES; offset <<= 1) {
+            low = fminf(low, __shfl_xor(low, offset, 64));
+            high = fmaxf(high, __shfl_xor(high, offset, 64));
+        }
+        float scale, zero = 0.0f;
+        if (a.asym) {
+            const float raw = __fmul_rn(fmaxf(__fsub_rn(high, low), 1e-12f), a.reciprocal);
+            zero = __fsub_rn(low, __fmul_rn(a.minimum, raw));
+            scale = rounded_scale(raw, a.format);
+            const float magnitude = rounded_scale(fmaxf(fabsf(zero), 1e-12f), a.format);
+            zero = zero > 0.0f ? magnitude : (zero < 0.0f ? -magnitude : 0.0f);
+        } else {
+            scale = rounded_scale(__fmul_rn(fmaxf(fmaxf(high, -low), 1e-12f), a.reciprocal), a.format);
+        }
+        if (wanted >= a.total_groups) continue;
+        for (int column = start + lane_in_team; column < stop; column += LANES) {
+            const float v = mk_load_as_float(a.inputs, base + column, a.dtype);
+            const float normalized = __fdiv_rn(__fsub_rn(v, zero), scale);
+            const float rounded = a.integer ? nearest_integer(normalized, a.minimum, a.maximum)
+                                            : table[nearest_entry(normalized, table, a.n_values, steps)];
+            mk_store_from_float(a.output, base + column, a.dtype, __fadd_rn(__fmul_rn(rounded, scale), zero));
+        }
+    }
+}
+
+template <int LANES>
+void launch_reconstruct(const ReconstructArgs &a, hipStream_t stream) {
+    int blocks = mk_cdiv(a.total_groups, kThreads / LANES);
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    hipLaunchKernelGGL((reconstruct_kernel<LANES>), dim3(blocks), dim3(kThreads), 0, stream, a);
+}
+
 int check_table(const char *name, const float *values, int n_values) {
     MK_REQUIRE(values && n_values >= 1 && n_values <= kMaxTable, MK_ERR_INVALID,
                "%s: a value table of 1..256 entries is required", name);
@@ -503,4 +569,33 @@ extern "C" int mk_fit_scales(const float *value, long long row_stride, float *sc
     const int groups = group >= 1 ? mk_cdiv(span, group) : 0;
     return mk_fit_scales_strided(value, row_stride, scales, zeros, groups, rows, span, group, asym, reciprocal,
                                  value_minimum, scale_format, store_zero, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mk_reconstruct_activations(const void *inputs, int dtype, void *output, const float *values,
+                                          int n_values, int rows, int width, int group, int scale_format,
+                                          int asym, int integer, float minimum, float maximum, float reciprocal,
+                                          void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(rows >= 0 && width >= 1 && group >= 1, MK_ERR_INVALID, "mk_reconstruct_activations: sizes must be positive");
+    if (rows == 0) return MK_OK;
+    MK_REQUIRE(inputs && output, MK_ERR_INVALID, "mk_reconstruct_activations: null tensor pointer");
+    MK_REQUIRE(mk_dtype_valid(dtype), MK_ERR_INVALID, "mk_reconstruct_activations: unknown dtype code");
+    MK_REQUIRE(scale_format >= 0 && scale_format <= 4, MK_ERR_INVALID, "mk_reconstruct_activations: unknown scale format code");
+    if (!integer)
+        if (int status = check_table("mk_reconstruct_activations", values, n_values)) return status;
+    if (group > width) group = width;
+    const int groups_per_row = mk_cdiv(width, group);
+    MK_REQUIRE(static_cast<long long>(rows) * groups_per_row < (1ll << 31), MK_ERR_INVALID,
+               "mk_reconstruct_activations: too many scale groups");
+    ReconstructArgs a{};
+    a.inputs = inputs; a.output = output; a.values = values; a.rows = rows; a.width = width; a.group = group;
+    a.groups_per_row = groups_per_row; a.total_groups = rows * groups_per_row; a.dtype = dtype;
+    a.n_values = integer ? 1 : n_values; a.format = scale_format; a.asym = asym; a.integer = integer;
+    a.reciprocal = reciprocal; a.minimum = minimum; a.maximum = maximum;
+    if (group >= 64) launch_reconstruct<64>(a, stream);
+    else if (group >= 32) launch_reconstruct<32>(a, stream);
+    else if (group >= 16) launch_reconstruct<16>(a, stream);
+    else launch_reconstruct<8>(a, stream);
+    MK_LAUNCH_CHECK("mk_reconstruct_activations");
+    return MK_OK;
 }

@@ -147,3 +147,31 @@ def fit_scales(
         int(store_zero), native.current_stream(device),
     ))
     return scales, zeros
+
+
+def reconstruct(
+    inputs: Tensor,
+    values: Tensor,
+    group: int,
+    scale_format: str,
+    asymmetric: bool,
+    integer: bool,
+    minimum: float,
+    maximum: float,
+    scale_reciprocal: float,
+) -> Tensor:
+    """Round ``inputs`` (two-dimensional, fp32 / fp16 / bf16) to a scaled scalar grid with scales
+    fitted per group on the fly; same signature as the reference's
+    kernels/activation_reconstruction.py:76-103."""
+    device = native.require_device(inputs, values)
+    if inputs.dim() != 2 or not inputs.is_contiguous():
+        raise ValueError("reconstruct requires a contiguous two-dimensional tensor")
+    output = torch.empty_like(inputs)
+    values = values.to(torch.float32).contiguous()
+    native.check(native.library().mk_reconstruct_activations(
+        inputs.data_ptr(), native.dtype_code(inputs), output.data_ptr(), values.data_ptr(), values.numel(),
+        inputs.shape[0], inputs.shape[1], min(group, inputs.shape[1]), native.SCALE_FORMAT_CODES[scale_format],
+        int(asymmetric), int(integer), float(minimum), float(maximum), float(scale_reciprocal),
+        native.current_stream(device),
+    ))
+    return output

@@ -58,6 +58,10 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
         _c_void_p, _c_longlong, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_float,
         _c_float, _c_int, _c_int, _c_void_p,
     ]),
+    "mk_reconstruct_activations": (_c_int, [
+        _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+        _c_float, _c_float, _c_float, _c_void_p,
+    ]),
     "mk_fwht": (_c_int, [
         _c_void_p, _c_int, _c_void_p, _c_int, _c_longlong, _c_int, _c_void_p, _c_void_p, _c_int,
         _c_float, _c_void_p,

@@ -130,25 +130,19 @@ class Scaled(Quantizer):
 
     def reconstruct_activations(self, value: Tensor) -> Tensor:
         """Quantize-dequantize a two-dimensional activation tensor online (no codec state kept):
-        scale fit, encode and decode kernels on a HIP device, the rounder itself otherwise."""
-        fused = (value.is_cuda and value.dim() == 2 and self.grid.values is not None and self.scale == "absmax"
+        one fused kernel on a HIP device, the rounder itself otherwise."""
+        fused = (value.is_cuda and value.dim() == 2 and value.dtype in (torch.float32, torch.float16, torch.bfloat16) and self.grid.values is not None and self.scale == "absmax"
                  and isinstance(self.scale_fmt, str) and self.scale_fmt in SCALE_FORMAT_BITS
                  and self.grid.values.numel() <= FUSED_CODEBOOK_LIMIT and self.grid.bits <= 8)
         if not fused:
             return self(value.float()).w.to(value.dtype)
-        from mlkit_amd.kernels import scalar_decode, scalar_encode
+        from mlkit_amd.kernels import scalar_encode
 
         assert isinstance(self.scale_fmt, str)
-        table = self.values_on(value.device)
-        samples = value.float().contiguous()
-        group = min(self.group or samples.shape[1], samples.shape[1])
-        scales, zero = scalar_encode.fit_scales(
-            samples, group, asym=self.asym,
-            reciprocal=self._range_reciprocal if self.asym else self._magnitude_reciprocal,
-            value_minimum=self._value_minimum, scale_format=self.scale_fmt, store_zero=True)
-        codes = scalar_encode.encode(samples, scales, zero, table, group, None, integer=self.grid.integer,
-                                     minimum=self._value_minimum, maximum=self._value_maximum)
-        return scalar_decode.decode(codes, scales, table, zero, group).to(value.dtype)
+        return scalar_encode.reconstruct(
+            value.contiguous(), self.values_on(value.device), self.group or value.shape[1], self.scale_fmt,
+            self.asym, self.grid.integer, self._value_minimum, self._value_maximum,
+            self._range_reciprocal if self.asym else self._magnitude_reciprocal)
 
     def logical_bits(self, shape: tuple[int, int]) -> float:
         rows, width = shape

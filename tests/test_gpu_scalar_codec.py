@@ -186,3 +186,50 @@ def test_large_layer_round_trip_properties():
     assert bool(((weight - decoded).abs() <= bound * 1.0001)[inside].all())
     again = scalar_encode.encode(decoded, scales, None, values, 128, None, integer=True, minimum=-8.0, maximum=7.0)
     assert torch.equal(again, codes)
+
+
+def _activation_formats():
+    import mlkit_amd as mk
+
+    return {
+        "int3-g32": mk.int(3, group=32),
+        "int4-row": mk.int(4, group=None),
+        "int4-fp32": mk.int(4, group=32, scale_fmt="fp32"),
+        "nf4-g64": mk.nf4(group=64),
+        "mxfp4": mk.mxfp4(),
+        "int4-asymmetric": mk.int(4, group=32, asym=True),
+        "int4-asymmetric-fp32": mk.int(4, group=32, asym=True, scale_fmt="fp32"),
+        "int4-bf16": mk.int(4, group=32, scale_fmt="bf16"),
+        "int4-fp8": mk.int(4, group=32, scale_fmt="fp8"),
+        "e2m1-fp16": mk.scaled(mk.grid.fp("e2m1"), group=32),
+    }
+
+
+@pytest.mark.parametrize("name", ["int3-g32", "int4-row", "int4-fp32", "nf4-g64", "mxfp4", "int4-asymmetric",
+                                  "int4-asymmetric-fp32", "int4-bf16", "int4-fp8", "e2m1-fp16"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+def test_fused_activation_reconstruction_is_exact_on_rounding_ties(name, dtype):
+    """The reference's own test (tests/kernels/test_activation_reconstruction.py:20-40): half
+    precision inputs land on exact rounding ties; the fused kernel must equal the fitted
+    format (itself checked against the oracle above) on every element."""
+    fmt = _activation_formats()[name]
+    generator = torch.Generator(device="cuda").manual_seed(97)
+    inputs = torch.randn(512, 2050, dtype=dtype, device="cuda", generator=generator)
+    inputs *= torch.rand(512, 1, device="cuda", generator=generator) * 20 + 0.01
+    expected = fmt(inputs.float()).w.to(dtype)
+    result = fmt.reconstruct_activations(inputs)
+    assert result.dtype == dtype
+    mismatched = int((result != expected).sum())
+    assert mismatched == 0, f"{mismatched} of {result.numel()} elements differ"
+    small = torch.randn(7, 130, dtype=dtype, device="cuda", generator=generator)
+    torch.testing.assert_close(fmt.reconstruct_activations(small), fmt(small.float()).w.to(dtype), rtol=0, atol=0)
+
+
+def test_activation_reconstruction_matches_oracle_directly():
+    import mlkit_amd as mk
+
+    value = helpers.normal_weight(33, 512, seed=40, scale=1.0)
+    expected = scaling.quantize(value, INT4, group=64, integer=True, asym=True)
+    dense = scaling.decode_grouped(expected["codes"], expected["scales"], INT4, 64, expected["zero"])
+    result = mk.int(4, group=64, asym=True).reconstruct_activations(dev(value))
+    np.testing.assert_array_equal(host(result), dense)
