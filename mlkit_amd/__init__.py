@@ -20,6 +20,7 @@ from mlkit_amd.quantization.codecs import codec, concatenate_rows, deterministic
 from mlkit_amd.quantization.core import Ctx, Q, Quantizer, layer_seed, quantizer
 from mlkit_amd.quantization.feedback import feedback_coefficients, gptq, ldlq, proxy_loss
 from mlkit_amd.quantization.grids import NF4_VALUES, Grid, grid
+from mlkit_amd.quantization.incoherence import Incoherent, incoherent
 from mlkit_amd.quantization.scaled import Scaled, int, mxfp4, nf4, scaled, store_scale  # noqa: A004
 from mlkit_amd.quantization.search import snap
 from mlkit_amd.quantization.transforms import hadamard, paley_matrix, rht, structured_transform, transform_factor
@@ -36,7 +37,7 @@ def rtn(w, ctx=None, *, fmt=None):
 __all__ = [
     "Capabilities", "Ctx", "Grid", "Model", "NF4_VALUES", "PackedEmbedding", "PackedLinear", "Q", "QModel",
     "Quantizer", "Rotate", "Scaled", "capabilities", "codec", "concatenate_rows", "deterministic_signs",
-    "feedback_coefficients", "gptq", "grid", "hadamard", "install_transform", "int", "layer_seed", "ldlq", "load_checkpoint", "mxfp4",
+    "feedback_coefficients", "gptq", "grid", "hadamard", "incoherent", "install_transform", "int", "layer_seed", "ldlq", "load_checkpoint", "mxfp4",
     "nf4", "optimize", "pack", "packed_compatible", "paley_matrix", "proxy_loss", "quantize", "quantizer", "rht",
     "rotate", "rtn", "save", "scaled", "snap", "store_scale", "structured_transform", "transform_factor", "unpack",
 ]

@@ -4,12 +4,14 @@ Mirrors, in /root/reference/src/mlkit/quantization/codecs:
   registry.py:1-46        codec, decoder, registered, row_parameters
   scaled.py:19-101        decode_grouped, decode_scaled ("scaled"), decode_feedback ("feedback")
   composition.py:14-20    deterministic_signs
+  composition.py:23-47    decode_basis ("basis")      composition.py:61-84   compose
   composition.py:87-116   concatenate_rows
 Decoding uint8 codes with FP32 parameters on a HIP device runs ``mk_scalar_decode``; tensors
 that track gradients, or live on the host, use the same expression in tensor operations.
 """
 
 from collections.abc import Callable, Sequence
+from typing import Any
 
 import torch
 from torch import Tensor
@@ -113,6 +115,42 @@ def deterministic_signs(width: int, seed: int, device: torch.device | str) -> Te
         v = ((v ^ (v >> 16)) * 0x45D9F3B) & 0xFFFFFFFF
     v = v ^ (v >> 16)
     return (v & 1).float() * 2 - 1
+
+
+@codec("basis")
+def decode_basis(codes: Tensor, *, inner_codec: str, shape: "tuple[int, int] | list[int]", left_seed: int | None,
+                 right_seed: int | None, left_signs: Tensor | None, right_signs: Tensor | None,
+                 **parameters: Any) -> Tensor:
+    """Codes of a matrix quantized in a rotated basis: the inner decoder's reconstruction is
+    rotated back, input side (columns) first, then output side (rows)."""
+    from mlkit_amd.quantization.transforms import rotate
+
+    inner = {key.removeprefix("inner_"): value for key, value in parameters.items()}
+    restored = decoder(inner_codec)(codes, **inner)
+    if right_seed is not None:
+        signs = right_signs if right_signs is not None else deterministic_signs(shape[1], right_seed, codes.device)
+        restored = rotate(restored, inverse=True, signs=signs)
+    if left_seed is not None:
+        signs = left_signs if left_signs is not None else deterministic_signs(shape[0], left_seed, codes.device)
+        restored = rotate(restored.T.contiguous(), inverse=True, signs=signs).T
+    return restored
+
+
+def compose(quantized: Q, name: str, parameters: dict[str, Any]) -> Q:
+    """Wrap a portable inner representation in the decoder ``name``; the inner codec's
+    parameters travel with an ``inner_`` prefix."""
+    if quantized.codes is None or quantized.codec is None or not registered(quantized.codec):
+        raise ValueError("portable composition requires a registered inner codec")
+    metadata = dict(quantized.metadata)
+    metadata["trainable"] = [f"inner_{key}" for key in metadata.get("trainable", [])]
+    formats = dict(metadata.get("parameter_formats", {}))
+    if quantized.codec in {"scaled", "feedback"}:
+        formats["scales"] = formats["zero"] = metadata.get("scale_fmt", "fp32")
+    metadata["parameter_formats"] = {f"inner_{key}": value for key, value in formats.items()}
+    metadata["parameter_bits"] = {f"inner_{key}": value for key, value in metadata.get("parameter_bits", {}).items()}
+    inner = {f"inner_{key}": value for key, value in quantized.params.items()}
+    return Q(codes=quantized.codes, params={**inner, "inner_codec": quantized.codec, **parameters},
+             decode=decoder(name), codec=name, bits=quantized.bits, metadata=metadata)
 
 
 def concatenate_rows(parts: Sequence[Q]) -> Q:

@@ -547,3 +547,27 @@ def test_row_chunked_conversion_of_a_wide_head_equals_whole_conversion(monkeypat
     chunked = mk.quantize(layer, mk.int(4, group=64), calib=None).quantized[""]
     assert torch.equal(chunked.codes, whole.codes) and torch.equal(chunked.params["scales"], whole.params["scales"])
     assert chunked.bits == whole.bits and chunked.codec == "scaled"
+
+
+def test_incoherent_quantization_on_device_and_checkpoint(tmp_path):
+    """Two-sided rotation (896 = 28 x 32 Paley rows, 4864 = 76 x 64 columns) around INT4: the
+    basis codec decodes on the device, beats plain INT4 on a layer with outlier columns, and
+    survives a checkpoint bit for bit."""
+    torch.manual_seed(49)
+    layer = nn.Linear(4864, 896, bias=False)
+    with torch.no_grad():
+        layer.weight.normal_(0, 0.02)
+        layer.weight[:, ::97] *= 15
+    identity = mk.incoherent(lambda w, ctx: mk.Q(w, bits=32 * w.numel()))(layer.weight.detach().cuda())
+    torch.testing.assert_close(identity.w, layer.weight.detach().cuda(), rtol=1e-4, atol=1e-5)
+    converted = mk.quantize(layer, mk.incoherent(mk.int(4, group=64)), calib=None)
+    q = converted.quantized[""]
+    assert q.codec == "basis" and q.params["inner_codec"] == "scaled" and q.codes.dtype == torch.uint8
+    original = layer.weight.detach().cuda()
+    plain = mk.int(4, group=64)(original).w
+    assert float((q.w - original).norm()) < 0.8 * float((plain - original).norm())
+    assert not mk.packed_compatible(q)
+    converted.save(tmp_path / "basis")
+    restored = mk.load_checkpoint(tmp_path / "basis", model=lambda: nn.Linear(4864, 896, bias=False))
+    torch.testing.assert_close(restored.module.weight, converted.module.weight, rtol=0, atol=0)
+    assert restored.quantized[""].params["right_seed"] == q.params["right_seed"]

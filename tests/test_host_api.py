@@ -311,3 +311,25 @@ def test_function_quantizers_bind_parameters():
     with pytest.raises(TypeError):
         clipped(unknown=3)
     assert isinstance(nn.Linear(2, 2), nn.Module)
+
+
+@pytest.mark.parametrize("shape", [(32, 64), (28, 96), (12, 20)])
+def test_incoherent_identity_and_basis_codec(shape):
+    torch.manual_seed(3)
+    weights = torch.randn(*shape)
+    identity = mk.incoherent(lambda w, ctx: mk.Q(w, bits=32 * w.numel()))(weights)
+    torch.testing.assert_close(identity.w, weights, rtol=1e-5, atol=1e-5)
+    coded = mk.incoherent(mk.int(8, group=None))(weights, Ctx("layer.0"))
+    assert coded.codec == "basis" and coded.params["inner_codec"] == "scaled"
+    assert coded.params["right_seed"] == (coded.params["left_seed"] + 1) % 2**32
+    assert coded.metadata["trainable"] == ["inner_scales"] and coded.metadata["parameter_formats"]["inner_scales"] == "fp16"
+    assert float((coded.w - weights).abs().max()) < 0.08 * float(weights.abs().max())
+    # one-sided and calibrated variants
+    right_only = mk.incoherent(mk.int(8, group=None), left=None)(weights)
+    assert right_only.params["left_seed"] is None
+    inputs = torch.randn(4 * shape[1], shape[1])
+    with_feedback = mk.incoherent(mk.gptq(mk.int(4, group=None), refit=None))(weights, Ctx("l", X=inputs))
+    assert with_feedback.codec == "basis" and with_feedback.params["inner_codec"] == "feedback"
+    assert torch.isfinite(with_feedback.w).all()
+    with pytest.raises(ValueError, match="rht or None"):
+        mk.incoherent(mk.int(4), left="dct")
