@@ -1,10 +1,9 @@
-// Packed matvec for 2-, 3- and 4-bit codes of any scalar grid (integer grids, NF4, small
+// Packed matvec for 2- to 8-bit codes of any scalar grid (integer grids, NF4, small
 // codebooks) with fp16 or bf16 activations and 16-bit scales, rows of K = 32 ... 16384 codes (K % 32 == 0).
 //
-// Adjacent codes (two 4-bit codes, four 2- or 3-bit codes) index a table of 16-bit value
-// pairs held in LDS, so one LDS read decodes two or four weights and one v_dot2_f32_f16
-// (v_dot2_f32_bf16) per pair multiplies them with the matching activations, accumulating
-// in fp32.  Table entries are the grid
+// Adjacent codes (one, two or four, by code width) index a table of 16-bit values held in
+// LDS, so one LDS read decodes up to four weights and one v_dot2_f32_f16 (v_dot2_f32_bf16)
+// per pair multiplies them with the matching activations, accumulating in fp32.  Table entries are the grid
 // values rounded to the activations' type (exact for integer grids and minifloats; NF4-like
 // tables lose at most half an ulp of that type per weight, as the activations themselves do).  Entries of different
 // pairs fall in different LDS banks except by coincidence, so the lookups mostly proceed
@@ -23,7 +22,12 @@ namespace mk_matvec {
 namespace {
 
 constexpr int kPairRows = 16;
-constexpr int kPairAhead = 8;
+// Rows of codes in flight per wavefront: eight rows of 16 bytes per lane, or as many wider
+// rows as hold the same number of bytes.
+template <int BITS>
+constexpr int rows_in_flight() {
+    return BITS <= 4 ? 8 : 32 / BITS;
+}
 
 // A 16-bit scale or offset (fp16 or bf16, uniform per launch) as fp32.
 __device__ __forceinline__ float side_value(uint16_t raw, int dtype) {
@@ -37,21 +41,16 @@ constexpr int pair_reduce_rows() {
     return kPairRows * MT <= 64 ? kPairRows : 64 / MT;
 }
 
-// Codes decoded per table lookup: two (an entry is one 16-bit pair), or four for 2-bit codes
-// and for 3-bit codes of long rows (entries of two pairs; the 4096-entry 3-bit table only pays
-// for itself when a workgroup has enough threads to fill it quickly).
-template <int BITS, bool QUAD>
-constexpr int lookup_codes() {
-    return QUAD ? 4 : 2;
-}
-
-// Byte offset into the table of field i of a chunk of BITS dwords; a field holds
-// lookup_codes() adjacent codes and an entry two bytes per code.  i is a compile-time
+// LOOKUP = codes decoded per table read: 1 (an entry is one 16-bit value; two reads make a
+// pair), 2 (an entry is one pair) or 4 (two pairs).  Wider fields mean fewer reads but a
+// table of 2^(LOOKUP * BITS) entries that every workgroup has to fill first.
+//
+// Byte offset into the table of field i of a chunk of BITS dwords.  i is a compile-time
 // constant after unrolling.
-template <int BITS, bool QUAD>
+template <int BITS, int LOOKUP>
 __device__ __forceinline__ uint32_t lookup_offset(const CodeChunk<BITS> &c, int i) {
-    constexpr int kField = lookup_codes<BITS, QUAD>() * BITS;
-    constexpr int kEntryShift = QUAD ? 3 : 2;
+    constexpr int kField = LOOKUP * BITS;
+    constexpr int kEntryShift = LOOKUP == 4 ? 3 : LOOKUP == 2 ? 2 : 1;
     constexpr uint32_t mask = ((1u << kField) - 1u) << kEntryShift;
     const int bit = i * kField;
     const int word = bit >> 5, shift = bit & 31;
@@ -62,12 +61,14 @@ __device__ __forceinline__ uint32_t lookup_offset(const CodeChunk<BITS> &c, int 
     return (__builtin_amdgcn_alignbit(c.w[(word + 1) % BITS], c.w[word], shift) << kEntryShift) & mask;
 }
 
-template <int BITS, int MT, bool HAS_ZERO, int XT, bool QUAD>
+template <int BITS, int MT, bool HAS_ZERO, int XT, int LOOKUP>
 __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
-    constexpr int kLookup = lookup_codes<BITS, QUAD>();
+    constexpr int kLookup = LOOKUP;
+    constexpr int kPairAhead = rows_in_flight<BITS>();
     constexpr int kEntries = 1 << (kLookup * BITS);
-    constexpr int kEntryWords = kLookup / 2;
-    __shared__ __attribute__((aligned(8))) uint32_t table[kEntries * kEntryWords];  // 16-bit pairs
+    constexpr int kTableWords = kEntries * kLookup / 2;
+    constexpr int kEntryWords = kLookup >= 2 ? kLookup / 2 : 1;
+    __shared__ __attribute__((aligned(8))) uint32_t table[kTableWords];  // 16-bit values, pairs or double pairs
     __shared__ float partials[64 * 8];    // [row sum][wavefront]
     constexpr int kReduceRows = pair_reduce_rows<MT>();
     constexpr int kSums = kReduceRows * MT;
@@ -88,17 +89,25 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
 
     // The grid's values first (one global load per value), then every table entry from them.
     __shared__ float grid_values[1 << BITS];
-    if (tid < (1 << BITS)) {
+    for (int code = tid; code < (1 << BITS); code += blockDim.x) {
         float value = 0.0f;
-        if (a.uniform) value = __builtin_fmaf(static_cast<float>(tid), a.grid_step, a.grid_min);
-        else if (tid < a.n_values) value = a.values[tid];
-        grid_values[tid] = value;
+        if (a.uniform) value = __builtin_fmaf(static_cast<float>(code), a.grid_step, a.grid_min);
+        else if (code < a.n_values) value = a.values[code];
+        grid_values[code] = value;
     }
     __syncthreads();
-    for (int word = tid; word < kEntries * kEntryWords; word += blockDim.x) {
-        const int entry = word / kEntryWords, half = word - entry * kEntryWords;
-        const float first = grid_values[(entry >> (2 * half * BITS)) & ((1 << BITS) - 1)];
-        const float second = grid_values[(entry >> ((2 * half + 1) * BITS)) & ((1 << BITS) - 1)];
+    for (int word = tid; word < kTableWords; word += blockDim.x) {
+        int low, high;  // the codes whose values share this dword
+        if constexpr (kLookup == 1) {
+            low = 2 * word;
+            high = 2 * word + 1;
+        } else {
+            const int entry = word / kEntryWords, half = word - entry * kEntryWords;
+            low = (entry >> (2 * half * BITS)) & ((1 << BITS) - 1);
+            high = (entry >> ((2 * half + 1) * BITS)) & ((1 << BITS) - 1);
+        }
+        const float first = grid_values[low];
+        const float second = grid_values[high];
         if constexpr (XT == MK_F16) {
             const mk_h2 pair = {static_cast<_Float16>(first), static_cast<_Float16>(second)};
             table[word] = __builtin_bit_cast(uint32_t, pair);
@@ -156,14 +165,18 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
 #pragma unroll
             for (int m = 0; m < MT; ++m) dot[m] = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 32 / kLookup; ++i) {
+            for (int i = 0; i < (kLookup == 1 ? 16 : 32 / kLookup); ++i) {
                 uint32_t entry[kEntryWords];
-                if constexpr (kEntryWords == 2) {
-                    const mk_u32x2 both = *reinterpret_cast<const mk_u32x2 *>(table_bytes + lookup_offset<BITS, QUAD>(codes[r], i));
+                if constexpr (kLookup == 4) {
+                    const mk_u32x2 both = *reinterpret_cast<const mk_u32x2 *>(table_bytes + lookup_offset<BITS, 4>(codes[r], i));
                     entry[0] = both.x;
                     entry[1] = both.y;
+                } else if constexpr (kLookup == 2) {
+                    entry[0] = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, 2>(codes[r], i));
                 } else {
-                    entry[0] = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, QUAD>(codes[r], i));
+                    const uint32_t even = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[r], 2 * i));
+                    const uint32_t odd = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[r], 2 * i + 1));
+                    entry[0] = even | (odd << 16);
                 }
 #pragma unroll
                 for (int h = 0; h < kEntryWords; ++h)
@@ -214,25 +227,31 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
     }
 }
 
-template <int BITS, int MT, int XT, bool QUAD>
+template <int BITS, int MT, int XT, int LOOKUP>
 void launch_tile_with(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     if (a.zeros)
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, QUAD>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, QUAD>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, LOOKUP>), grid, block, 0, stream, a);
 }
 
+// Field width per code width: the widest whose table a workgroup fills quickly.
 template <int BITS, int MT, int XT>
 void launch_tile_as(const Stream4Args &a, int tiles, hipStream_t stream) {
     if constexpr (BITS == 2) {
-        launch_tile_with<BITS, MT, XT, true>(a, tiles, stream);
+        launch_tile_with<BITS, MT, XT, 4>(a, tiles, stream);                                   // 256 entries
     } else if constexpr (BITS == 3) {
-        if (a.width >= 8192) launch_tile_with<BITS, MT, XT, true>(a, tiles, stream);
-        else launch_tile_with<BITS, MT, XT, false>(a, tiles, stream);
+        if (a.width >= 8192) launch_tile_with<BITS, MT, XT, 4>(a, tiles, stream);              // 4096 entries
+        else launch_tile_with<BITS, MT, XT, 2>(a, tiles, stream);                              // 64
+    } else if constexpr (BITS <= 5) {
+        launch_tile_with<BITS, MT, XT, 2>(a, tiles, stream);                                   // 256 / 1024
+    } else if constexpr (BITS == 6) {
+        if (a.width >= 4096) launch_tile_with<BITS, MT, XT, 2>(a, tiles, stream);              // 4096
+        else launch_tile_with<BITS, MT, XT, 1>(a, tiles, stream);                              // 64
     } else {
-        launch_tile_with<BITS, MT, XT, false>(a, tiles, stream);
+        launch_tile_with<BITS, MT, XT, 1>(a, tiles, stream);                                   // 128 / 256
     }
 }
 
@@ -257,7 +276,7 @@ void launch_bits(const Stream4Args &a, int tiles, hipStream_t stream) {
 }  // namespace
 
 bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype) {
-    return bits >= 2 && bits <= 4 && x_dtype != MK_F32 && scale_dtype != MK_F32 && width % kChunkCodes == 0 &&
+    return bits >= 2 && bits <= 8 && x_dtype != MK_F32 && scale_dtype != MK_F32 && width % kChunkCodes == 0 &&
            width <= 16384 && (group % kChunkCodes == 0 || group >= width);
 }
 
@@ -268,7 +287,11 @@ int pairs_launch(const Stream4Args &a, hipStream_t stream) {
     switch (a.bits) {
         case 2: launch_bits<2>(a, tiles, stream); break;
         case 3: launch_bits<3>(a, tiles, stream); break;
-        default: launch_bits<4>(a, tiles, stream); break;
+        case 4: launch_bits<4>(a, tiles, stream); break;
+        case 5: launch_bits<5>(a, tiles, stream); break;
+        case 6: launch_bits<6>(a, tiles, stream); break;
+        case 7: launch_bits<7>(a, tiles, stream); break;
+        default: launch_bits<8>(a, tiles, stream); break;
     }
     return tiles * kPairRows;
 }

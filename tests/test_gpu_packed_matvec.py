@@ -254,3 +254,25 @@ def test_bf16_activations_use_the_pair_table_kernel(bits, values, integer, scale
         for samples in (1, 8):
             x = helpers.activations(samples, 4096, seed=22 + samples, dtype=torch.bfloat16)
             check(run_matvec(layer, x, scale_dtype=scale_dtype), layer, x, relative=8e-3)
+
+
+E4M3 = np.array(sorted({s * (m / 8 * 2.0 ** -6 if e == 0 else (1 + m / 8) * 2.0 ** (e - 7))
+                        for s in (-1, 1) for e in range(15) for m in range(8)}), dtype=np.float32)
+
+
+@pytest.mark.parametrize("name,values,bits,integer", [
+    ("int5", scaling.int_values(5), 5, True), ("int6", scaling.int_values(6), 6, True),
+    ("int7", scaling.int_values(7), 7, True), ("int8", scaling.int_values(8), 8, True),
+    ("e4m3", E4M3, 8, False),
+])
+@pytest.mark.parametrize("width", [2048, 4096, 896])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_wide_codes_on_the_table_kernel(name, values, bits, integer, width, dtype):
+    """5- to 8-bit codes with 16-bit activations: single-value or pair tables by width."""
+    weight = helpers.normal_weight(40, width, seed=23, student_t=True)
+    tolerance = 1e-3 if dtype == torch.float16 else 8e-3
+    for asym in (False, True):
+        layer = helpers.quantised_layer(weight, values, bits=bits, group=32, integer=integer, asym=asym)
+        for samples in (1, 8):
+            x = helpers.activations(samples, width, seed=24 + samples, dtype=dtype)
+            check(run_matvec(layer, x), layer, x, relative=tolerance)
