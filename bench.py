@@ -278,6 +278,9 @@ def other_kernels(device: torch.device) -> dict:
     matvec(ROWS, WIDTH, 64, 4, nf4, False, False, "nf4 g64")
     matvec(ROWS, WIDTH, 64, 3, seven, False, False, "codebook7 g64")
     matvec(151936, 896, 128, 4, values, True, False, "int4 g128 (tied head)")
+    matvec(ROWS, WIDTH, 128, 8, torch.arange(-128, 128, dtype=torch.float32, device=device), True, False, "int8 g128")
+    for rows, width in ((896, 896), (128, 896), (4864, 896), (896, 4864)):
+        matvec(rows, width, 128, 4, values, True, False, "int4 g128 (decoder layer)")
     del weight, rotated, dense, codes
 
     out["gptq int4 g128 4096x11008"] = gptq_layer(device, generator)
