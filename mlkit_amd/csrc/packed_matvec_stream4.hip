@@ -24,26 +24,29 @@ namespace mk_matvec {
 
 namespace {
 
-#ifndef MK_S4_ROWS
-#define MK_S4_ROWS 16
-#endif
-#ifndef MK_S4_AHEAD
-#define MK_S4_AHEAD 8
-#endif
-constexpr int kStreamRows = MK_S4_ROWS;    // rows per workgroup
-constexpr int kStreamAhead = MK_S4_AHEAD;  // rows of codes in flight per wavefront
+// Rows per workgroup: 16 when that still gives every compute unit a workgroup, 4 for
+// layers with fewer rows (more, shorter workgroups).  Up to 8 rows of codes are in flight
+// per wavefront (both values swept on the GPU together with 8 / 32 rows and 4 - 16 ahead).
+constexpr int kWideRows = 16, kNarrowRows = 4;
+
+template <int ROWS>
+constexpr int rows_ahead_of() {
+    return ROWS < 8 ? ROWS : 8;
+}
 
 // Rows per transposed reduction: all 16 when that is at most 64 sums per lane (measured
 // faster than splitting the reduction to hide part of it behind the stream).
-template <int MT>
+template <int MT, int ROWS>
 constexpr int reduce_rows() {
-    return kStreamRows * MT <= 64 ? kStreamRows : 64 / MT;
+    return ROWS * MT <= 64 ? ROWS : 64 / MT;
 }
 
-template <int MT, bool HAS_ZERO>
+template <int MT, bool HAS_ZERO, int ROWS>
 __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     __shared__ float partials[64 * 8];  // [row sum][wavefront]
-    constexpr int kReduceRows = reduce_rows<MT>();
+    constexpr int kStreamRows = ROWS;
+    constexpr int kStreamAhead = rows_ahead_of<ROWS>();
+    constexpr int kReduceRows = reduce_rows<MT, ROWS>();
     constexpr int kSums = kReduceRows * MT;
 
     const int tid = threadIdx.x;
@@ -147,14 +150,29 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     }
 }
 
-template <int MT>
+template <int MT, int ROWS>
 void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     if (a.zeros)
-        hipLaunchKernelGGL((stream4_kernel<MT, true>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((stream4_kernel<MT, false>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS>), grid, block, 0, stream, a);
+}
+
+template <int ROWS>
+int launch_rows(const Stream4Args &a, hipStream_t stream) {
+    const int tiles = a.rows / ROWS;
+    if (tiles == 0) return 0;
+    int tile = 1;
+    while (tile < a.samples && tile < 8) tile <<= 1;
+    switch (tile) {
+        case 1: launch_tile<1, ROWS>(a, tiles, stream); break;
+        case 2: launch_tile<2, ROWS>(a, tiles, stream); break;
+        case 4: launch_tile<4, ROWS>(a, tiles, stream); break;
+        default: launch_tile<8, ROWS>(a, tiles, stream); break;
+    }
+    return tiles * ROWS;
 }
 
 }  // namespace
@@ -164,19 +182,11 @@ bool stream4_accepts(int width, int group, int bits, int x_dtype, int scale_dtyp
            width <= 16384 && (group % kChunkCodes == 0 || group >= width);
 }
 
-// Multiplies rows [0, 16 * tiles); returns the number of rows covered.
+// Multiplies the leading whole tiles of rows; returns the number of rows covered.
 int stream4_launch(const Stream4Args &a, hipStream_t stream) {
-    const int tiles = a.rows / kStreamRows;
-    if (tiles == 0) return 0;
-    int tile = 1;
-    while (tile < a.samples && tile < 8) tile <<= 1;
-    switch (tile) {
-        case 1: launch_tile<1>(a, tiles, stream); break;
-        case 2: launch_tile<2>(a, tiles, stream); break;
-        case 4: launch_tile<4>(a, tiles, stream); break;
-        default: launch_tile<8>(a, tiles, stream); break;
-    }
-    return tiles * kStreamRows;
+    constexpr int kComputeUnits = 256;
+    if (a.rows / kWideRows >= kComputeUnits) return launch_rows<kWideRows>(a, stream);
+    return launch_rows<kNarrowRows>(a, stream);
 }
 
 }  // namespace mk_matvec
