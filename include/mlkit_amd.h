@@ -199,12 +199,15 @@ int mk_feedback_block_update_range(float *feedback, const float *original, const
  * magnitude with sign), then per tile of `block` columns mk_feedback_round_tile and the
  * trailing updates, far columns deferred by up to deferred_tiles tiles
  * (mk_feedback_block_update_range).  scales / zeros: [rows, G] fp32, G = sum over regions of
- * ceil(region width / min(group, region width)), region after region.  Results equal those
- * of issuing the separate entry points region by region.
+ * ceil(region width / min(group, region width)), region after region.  deviations: NULL, or
+ * [width, rows] fp32 scratch in which the sweep leaves original - reconstruction column by
+ * column for the trailing updates to read (faster; same results).  Results equal those of
+ * issuing the separate entry points region by region.
  * Replaces: the host loop of quantization/algorithms/error_feedback.py:296-370. */
 int mk_feedback_sweep(const float *original, float *feedback, float *output, uint8_t *encoded,
                       const float *coeff, float *scales, float *zeros, float *workspace,
-                      const float *values, int n_values, int rows, int width, int group, int refit,
+                      float *deviations, const float *values, int n_values, int rows, int width,
+                      int group, int refit,
                       int block, int integer_grid, float code_min, float code_max, int asym,
                       float reciprocal, float value_minimum, int scale_format, int deferred_tiles,
                       void *stream);

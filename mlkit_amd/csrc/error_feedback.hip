@@ -36,6 +36,7 @@ struct SweepArgs {
     const float *values;
     float *output;     // reconstruction [rows, width]; solve: [rows, span]
     uint8_t *encoded;  // [rows, width]
+    float *deviation_t;  // null, or [width, rows]: original - reconstruction, column-major
     int rows, width;
     int region_start, tile_start, tile_width;
     int group, groups_per_row, n_values;
@@ -186,6 +187,8 @@ __global__ void __launch_bounds__(kSweepThreads) sweep_kernel(const SweepArgs a)
         } else {
             a.output[row_base + a.tile_start + c] = finished[s];
             a.encoded[row_base + a.tile_start + c] = static_cast<uint8_t>(code[s]);
+            if (a.deviation_t)
+                a.deviation_t[static_cast<size_t>(a.tile_start + c) * a.rows + row] = __fsub_rn(weight[s], finished[s]);
         }
     }
 }
@@ -230,6 +233,7 @@ struct UpdateArgs {
     int chain_width;    // columns (= k) per chain
     int chains;
     int column_begin, column_end;  // columns of feedback that are updated
+    const float *deviation_t;      // null, or [width, rows] deviations written by the sweep
 };
 
 struct UpdateStage {
@@ -403,13 +407,144 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_kernel(const U
             }
 }
 
+// The same update with the deviations read from the column-major buffer the sweep kernel
+// fills, for launches made of whole tiles only (rows and updated columns in multiples of
+// 128, chains in multiples of 32 columns): the left operand loads and lands in LDS as whole
+// float4s along the rows (no subtraction, no transposing stores), nothing is masked, and
+// every address that does not depend on k is computed once.
+constexpr int kDeviationStride = kTileRows + 4;  // floats per k row in LDS, keeps 16-byte alignment
+
+__global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviations_kernel(const UpdateArgs a) {
+    __shared__ __attribute__((aligned(16))) float deviation_t[2][kDepthChunk][kDeviationStride];  // [buffer][k][row]
+    __shared__ __attribute__((aligned(16))) float coefficient[2][kDepthChunk][kTileColumns];      // [buffer][k][column]
+    // Addresses are a wavefront-uniform 64-bit base plus a 32-bit per-lane offset, so that
+    // the compiler keeps the bases in scalar registers.
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int row0 = blockIdx.y * kTileRows;
+    const int column0 = a.column_begin + blockIdx.x * kTileColumns;
+    const int wave_row = (wave >> 1) * 64, wave_column = (wave & 1) * 64;
+    const int chunks_per_chain = a.chain_width / kDepthChunk;
+    const int steps = a.chains * chunks_per_chain;
+
+    // Per chunk a thread loads four float4 of deviations and four of coefficients (both
+    // tiles are 32 x 128): k = thread / 32 + 8 p, elements 4 (thread % 32) ... + 3.
+    const int lead_k = threadIdx.x / (kTileRows / 4);
+    const int lead_four = (threadIdx.x % (kTileRows / 4)) * 4;
+    const uint32_t left_lane = static_cast<uint32_t>(lead_k) * a.rows + lead_four;
+    const uint32_t right_lane = static_cast<uint32_t>(lead_k) * a.width + lead_four;
+    const float *left_tile = a.deviation_t + row0;     // + k * rows
+    const float *right_tile = a.coeff + column0;       // + k * width
+    const uint32_t left_lds = lead_k * kDeviationStride + lead_four;
+    const uint32_t right_lds = lead_k * kTileColumns + lead_four;
+
+    // This lane's cell of every 32 x 32 MFMA tile: rows (lane / 32) * 4 + ..., column lane % 32.
+    const uint32_t cell_lane = static_cast<uint32_t>((lane >> 5) * 4) * a.width + (lane & 31);
+    float *quarter = a.feedback + static_cast<size_t>(row0 + wave_row) * a.width + column0 + wave_column;
+    auto cell = [&](int mi, int ni, int r) __attribute__((always_inline)) -> float * {
+        return quarter + static_cast<size_t>(mi * 32 + (r >> 2) * 8 + (r & 3)) * a.width + ni * 32 + cell_lane;
+    };
+    mk_f32x16 totals[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) totals[mi][ni][r] = *cell(mi, ni, r);
+
+    float4 l0, l1, l2, l3, r0, r1, r2, r3;  // the next chunk's operands on their way to LDS
+    auto fetch = [&](int step) __attribute__((always_inline)) {
+        const int chain = step / chunks_per_chain, chunk = step - chain * chunks_per_chain;
+        const size_t k_base = static_cast<size_t>(a.first_column + chain * a.chain_width + chunk * kDepthChunk);
+        const float *left = left_tile + k_base * a.rows;
+        const float *right = right_tile + k_base * a.width;
+        const size_t left_step = static_cast<size_t>(8) * a.rows, right_step = static_cast<size_t>(8) * a.width;
+        l0 = *reinterpret_cast<const float4 *>(left + left_lane);
+        l1 = *reinterpret_cast<const float4 *>(left + left_step + left_lane);
+        l2 = *reinterpret_cast<const float4 *>(left + 2 * left_step + left_lane);
+        l3 = *reinterpret_cast<const float4 *>(left + 3 * left_step + left_lane);
+        r0 = *reinterpret_cast<const float4 *>(right + right_lane);
+        r1 = *reinterpret_cast<const float4 *>(right + right_step + right_lane);
+        r2 = *reinterpret_cast<const float4 *>(right + 2 * right_step + right_lane);
+        r3 = *reinterpret_cast<const float4 *>(right + 3 * right_step + right_lane);
+    };
+    auto keep = [&](int buffer) __attribute__((always_inline)) {
+        float *left_target = &deviation_t[buffer][0][0] + left_lds;
+        float *right_target = &coefficient[buffer][0][0] + right_lds;
+        *reinterpret_cast<float4 *>(left_target) = l0;
+        *reinterpret_cast<float4 *>(left_target + 8 * kDeviationStride) = l1;
+        *reinterpret_cast<float4 *>(left_target + 16 * kDeviationStride) = l2;
+        *reinterpret_cast<float4 *>(left_target + 24 * kDeviationStride) = l3;
+        *reinterpret_cast<float4 *>(right_target) = r0;
+        *reinterpret_cast<float4 *>(right_target + 8 * kTileColumns) = r1;
+        *reinterpret_cast<float4 *>(right_target + 16 * kTileColumns) = r2;
+        *reinterpret_cast<float4 *>(right_target + 24 * kTileColumns) = r3;
+    };
+
+    fetch(0);
+    keep(0);
+    __syncthreads();
+
+    const uint32_t left_read = (lane >> 5) * kDeviationStride + wave_row + (lane & 31);
+    const uint32_t right_read = (lane >> 5) * kTileColumns + wave_column + (lane & 31);
+    mk_f32x16 sums[2][2];
+    for (int step = 0; step < steps; ++step) {
+        const int buffer = step & 1;
+        const int chunk = step % chunks_per_chain;
+        if (chunk == 0) {
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sums[mi][ni][r] = 0.0f;
+        }
+        const bool more = step + 1 < steps;
+        if (more) fetch(step + 1);
+        const float *left_rows = &deviation_t[buffer][0][0] + left_read;
+        const float *right_rows = &coefficient[buffer][0][0] + right_read;
+#pragma unroll 4
+        for (int kk = 0; kk < kDepthChunk; kk += 2) {
+            const float left0 = left_rows[kk * kDeviationStride], left1 = left_rows[kk * kDeviationStride + 32];
+            const float right0 = right_rows[kk * kTileColumns], right1 = right_rows[kk * kTileColumns + 32];
+            sums[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(left0, right0, sums[0][0], 0, 0, 0);
+            sums[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(left0, right1, sums[0][1], 0, 0, 0);
+            sums[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(left1, right0, sums[1][0], 0, 0, 0);
+            sums[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(left1, right1, sums[1][1], 0, 0, 0);
+        }
+        if (chunk == chunks_per_chain - 1) {
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) totals[mi][ni][r] = __fadd_rn(totals[mi][ni][r], sums[mi][ni][r]);
+        }
+        if (more) keep(buffer ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) *cell(mi, ni, r) = totals[mi][ni][r];
+}
+
 int launch_update(const UpdateArgs &a, hipStream_t stream) {
     MK_REQUIRE(mk_cdiv(a.rows, kTileRows) <= 65535, MK_ERR_UNSUPPORTED, "mk_feedback_block_update: too many rows");
     const dim3 grid(mk_cdiv(a.column_end - a.column_begin, kTileColumns), mk_cdiv(a.rows, kTileRows));
     const auto aligned = [](const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15u) == 0; };
     const bool vec = a.width % 4 == 0 && a.first_column % 4 == 0 && a.chain_width % 4 == 0 && a.column_begin % 4 == 0 &&
                      aligned(a.original) && aligned(a.output) && aligned(a.coeff);
-    if (vec)
+    // The deviation buffer path handles whole tiles only.
+    const bool staged = a.deviation_t && aligned(a.deviation_t) && aligned(a.coeff) && a.rows % kTileRows == 0 &&
+                        a.width % 4 == 0 && a.column_begin % 4 == 0 &&
+                        (a.column_end - a.column_begin) % kTileColumns == 0 && a.chain_width % kDepthChunk == 0;
+    if (staged)
+        hipLaunchKernelGGL(block_update_from_deviations_kernel, grid, dim3(kUpdateThreads), 0, stream, a);
+    else if (vec)
         hipLaunchKernelGGL((block_update_kernel<true>), grid, dim3(kUpdateThreads), 0, stream, a);
     else
         hipLaunchKernelGGL((block_update_kernel<false>), grid, dim3(kUpdateThreads), 0, stream, a);
@@ -486,7 +621,7 @@ extern "C" int mk_feedback_block_update_range(float *feedback, const float *orig
                "mk_feedback_block_update: updated columns [%d, %d) must follow the chains and lie inside the row",
                column_begin, column_end);
     if (column_begin >= column_end) return MK_OK;
-    UpdateArgs a{feedback, original, output, coeff, rows, width, first_column, chain_width, chains, column_begin, column_end};
+    UpdateArgs a{feedback, original, output, coeff, rows, width, first_column, chain_width, chains, column_begin, column_end, nullptr};
     if (int status = launch_update(a, stream)) return status;
     MK_LAUNCH_CHECK("mk_feedback_block_update");
     return MK_OK;
@@ -507,7 +642,8 @@ extern "C" int mk_feedback_block_update(float *feedback, const float *original, 
 // (deferred, chained) trailing updates.
 extern "C" int mk_feedback_sweep(const float *original, float *feedback, float *output, uint8_t *encoded,
                                  const float *coeff, float *scales, float *zeros, float *workspace,
-                                 const float *values, int n_values, int rows, int width, int group, int refit,
+                                 float *deviations, const float *values, int n_values, int rows, int width,
+                                 int group, int refit,
                                  int block, int integer_grid, float code_min, float code_max, int asym,
                                  float reciprocal, float value_minimum, int scale_format, int deferred_tiles,
                                  void *stream_) {
@@ -538,7 +674,7 @@ extern "C" int mk_feedback_sweep(const float *original, float *feedback, float *
     int deferred_count = 0, limit = 0;
     auto update = [&](int first, int chain, int chains, int begin, int end) -> int {
         if (begin >= end) return MK_OK;
-        UpdateArgs u{feedback, original, output, coeff, rows, width, first, chain, chains, begin, end};
+        UpdateArgs u{feedback, original, output, coeff, rows, width, first, chain, chains, begin, end, deviations};
         return launch_update(u, stream);
     };
     auto flush = [&]() -> int {
@@ -591,7 +727,7 @@ extern "C" int mk_feedback_sweep(const float *original, float *feedback, float *
             a.width = width; a.region_start = region_start; a.tile_start = tile_start;
             a.tile_width = tile_stop - tile_start; a.group = fitted_group;
             a.groups_per_row = static_cast<int>(total_groups); a.n_values = n_values;
-            a.code_min = code_min; a.code_max = code_max;
+            a.code_min = code_min; a.code_max = code_max; a.deviation_t = deviations;
             if (integer_grid) launch_sweep<kModeInteger>(a, stream);
             else launch_sweep<kModeCodebook>(a, stream);
             if (tile_stop >= width) continue;

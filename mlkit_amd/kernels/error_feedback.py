@@ -169,10 +169,13 @@ def sweep(
     scales = torch.empty((rows, groups), device=device, dtype=torch.float32)
     zeros = torch.empty_like(scales) if asym else None
     workspace = torch.empty((rows, region), device=device, dtype=torch.float32) if region < width else None
+    # column-major deviations of finished columns: what the trailing updates multiply
+    deviations = torch.empty((width, rows), device=device, dtype=torch.float32) if rows % 4 == 0 and width % 4 == 0 else None
     values = values.to(torch.float32).contiguous()
     native.check(native.library().mk_feedback_sweep(
         original.data_ptr(), feedback.data_ptr(), output.data_ptr(), encoded.data_ptr(), coefficients.data_ptr(),
-        scales.data_ptr(), native.pointer(zeros), native.pointer(workspace), values.data_ptr(), values.numel(),
+        scales.data_ptr(), native.pointer(zeros), native.pointer(workspace), native.pointer(deviations),
+        values.data_ptr(), values.numel(),
         rows, width, group, refit, block, int(integer_grid), float(code_minimum), float(code_maximum), int(asym),
         float(reciprocal), float(value_minimum), native.SCALE_FORMAT_CODES[scale_format], deferred_tiles,
         native.current_stream(device),

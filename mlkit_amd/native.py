@@ -82,7 +82,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     ]),
     "mk_feedback_sweep": (_c_int, [
         _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_float,
+        _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_float,
         _c_float, _c_int, _c_int, _c_void_p,
     ]),
     "mk_feedback_block_update_range": (_c_int, [

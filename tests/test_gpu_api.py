@@ -344,16 +344,17 @@ def test_capabilities_on_device():
     assert mk.capabilities(mk.int(3, group=50), shape=(16, 250)).packed_inference.startswith("packed storage with dense")
 
 
-def test_whole_sweep_entry_point_equals_the_region_by_region_loop(rng):
+@pytest.mark.parametrize("rows,width", [(70, 1000), (256, 1024)])
+def test_whole_sweep_entry_point_equals_the_region_by_region_loop(rows, width, rng):
     """`mk_feedback_sweep` (one call) against the same kernels issued region by region from
-    Python (a subclass of Scaled is not eligible for the single call)."""
+    Python (a subclass of Scaled is not eligible for the single call). The second shape is
+    whole 128 x 128 tiles, where the single call updates from the deviations its sweep kept."""
     from mlkit_amd.quantization.scaled import Scaled
 
     class Plain(Scaled):
         pass
 
-    rows, width = 70, 1000   # ragged last region and tile
-    weight = dev(helpers.normal_weight(rows, width, seed=50))
+    weight = dev(helpers.normal_weight(rows, width, seed=50))   # (70, 1000): ragged last region and tile
     inputs = rng.standard_normal((2048, width)).astype(F32)
     inputs[:, ::11] *= 4
     hessian = dev((inputs.T @ inputs / 2048).astype(F32))
