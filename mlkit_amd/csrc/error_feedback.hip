@@ -22,6 +22,8 @@
 
 #include "mk_common.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int kSweepThreads = 256;  // four wavefronts = four rows
@@ -412,11 +414,15 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_kernel(const U
 // 128, chains in multiples of 32 columns): the left operand loads and lands in LDS as whole
 // float4s along the rows (no subtraction, no transposing stores), nothing is masked, and
 // every address that does not depend on k is computed once.
-constexpr int kDeviationStride = kTileRows + 4;  // floats per k row in LDS, keeps 16-byte alignment
+constexpr int kDeviationStride = kTileRows;  // floats per k row in LDS
 
 __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviations_kernel(const UpdateArgs a) {
-    __shared__ __attribute__((aligned(16))) float deviation_t[2][kDepthChunk][kDeviationStride];  // [buffer][k][row]
-    __shared__ __attribute__((aligned(16))) float coefficient[2][kDepthChunk][kTileColumns];      // [buffer][k][column]
+    // Two buffers per operand, each a variable of its own: the compiler then sees that the
+    // transfer into one buffer cannot touch the buffer being read, and does not wait for it.
+    __shared__ __attribute__((aligned(16))) float deviation_even[kDepthChunk][kDeviationStride];  // [k][row]
+    __shared__ __attribute__((aligned(16))) float deviation_odd[kDepthChunk][kDeviationStride];
+    __shared__ __attribute__((aligned(16))) float coefficient_even[kDepthChunk][kTileColumns];    // [k][column]
+    __shared__ __attribute__((aligned(16))) float coefficient_odd[kDepthChunk][kTileColumns];
     // Addresses are a wavefront-uniform 64-bit base plus a 32-bit per-lane offset, so that
     // the compiler keeps the bases in scalar registers.
     const int lane = threadIdx.x & 63;
@@ -427,16 +433,14 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviation
     const int chunks_per_chain = a.chain_width / kDepthChunk;
     const int steps = a.chains * chunks_per_chain;
 
-    // Per chunk a thread loads four float4 of deviations and four of coefficients (both
-    // tiles are 32 x 128): k = thread / 32 + 8 p, elements 4 (thread % 32) ... + 3.
-    const int lead_k = threadIdx.x / (kTileRows / 4);
-    const int lead_four = (threadIdx.x % (kTileRows / 4)) * 4;
-    const uint32_t left_lane = static_cast<uint32_t>(lead_k) * a.rows + lead_four;
-    const uint32_t right_lane = static_cast<uint32_t>(lead_k) * a.width + lead_four;
+    // Operands go from global memory straight into LDS: one wavefront instruction moves two
+    // consecutive k rows of a tile (2 x 128 floats = 64 lanes x 16 bytes, lane l's bytes at
+    // 16 l from the wavefront-uniform LDS address). Per chunk a wavefront moves k rows
+    // 8 wave ... 8 wave + 7 of both tiles.
+    const uint32_t left_lane = static_cast<uint32_t>(lane >> 5) * a.rows + (lane & 31) * 4;
+    const uint32_t right_lane = static_cast<uint32_t>(lane >> 5) * a.width + (lane & 31) * 4;
     const float *left_tile = a.deviation_t + row0;     // + k * rows
     const float *right_tile = a.coeff + column0;       // + k * width
-    const uint32_t left_lds = lead_k * kDeviationStride + lead_four;
-    const uint32_t right_lds = lead_k * kTileColumns + lead_four;
 
     // This lane's cell of every 32 x 32 MFMA tile: rows (lane / 32) * 4 + ..., column lane % 32.
     const uint32_t cell_lane = static_cast<uint32_t>((lane >> 5) * 4) * a.width + (lane & 31);
@@ -444,52 +448,43 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviation
     auto cell = [&](int mi, int ni, int r) __attribute__((always_inline)) -> float * {
         return quarter + static_cast<size_t>(mi * 32 + (r >> 2) * 8 + (r & 3)) * a.width + ni * 32 + cell_lane;
     };
+    // feedback's own values: one 32 x 32 quarter is requested in each of the first four steps,
+    // behind that step's operand loads, so that no step waits for the whole tile.
     mk_f32x16 totals[2][2];
-#pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) totals[mi][ni][r] = *cell(mi, ni, r);
 
-    float4 l0, l1, l2, l3, r0, r1, r2, r3;  // the next chunk's operands on their way to LDS
-    auto fetch = [&](int step) __attribute__((always_inline)) {
+    auto fetch = [&](int step, auto odd) __attribute__((always_inline)) {
         const int chain = step / chunks_per_chain, chunk = step - chain * chunks_per_chain;
-        const size_t k_base = static_cast<size_t>(a.first_column + chain * a.chain_width + chunk * kDepthChunk);
+        const size_t k_base = static_cast<size_t>(a.first_column + chain * a.chain_width + chunk * kDepthChunk + wave * 8);
         const float *left = left_tile + k_base * a.rows;
         const float *right = right_tile + k_base * a.width;
-        const size_t left_step = static_cast<size_t>(8) * a.rows, right_step = static_cast<size_t>(8) * a.width;
-        l0 = *reinterpret_cast<const float4 *>(left + left_lane);
-        l1 = *reinterpret_cast<const float4 *>(left + left_step + left_lane);
-        l2 = *reinterpret_cast<const float4 *>(left + 2 * left_step + left_lane);
-        l3 = *reinterpret_cast<const float4 *>(left + 3 * left_step + left_lane);
-        r0 = *reinterpret_cast<const float4 *>(right + right_lane);
-        r1 = *reinterpret_cast<const float4 *>(right + right_step + right_lane);
-        r2 = *reinterpret_cast<const float4 *>(right + 2 * right_step + right_lane);
-        r3 = *reinterpret_cast<const float4 *>(right + 3 * right_step + right_lane);
+#pragma unroll
+        for (int pair = 0; pair < 4; ++pair) {
+            const float *left_source = left + static_cast<size_t>(2 * pair) * a.rows + left_lane;
+            const float *right_source = right + static_cast<size_t>(2 * pair) * a.width + right_lane;
+            const int k = wave * 8 + 2 * pair;
+            if constexpr (odd.value) {
+                __builtin_amdgcn_global_load_lds(left_source, &deviation_odd[k][0], 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(right_source, &coefficient_odd[k][0], 16, 0, 0);
+            } else {
+                __builtin_amdgcn_global_load_lds(left_source, &deviation_even[k][0], 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(right_source, &coefficient_even[k][0], 16, 0, 0);
+            }
+        }
     };
-    auto keep = [&](int buffer) __attribute__((always_inline)) {
-        float *left_target = &deviation_t[buffer][0][0] + left_lds;
-        float *right_target = &coefficient[buffer][0][0] + right_lds;
-        *reinterpret_cast<float4 *>(left_target) = l0;
-        *reinterpret_cast<float4 *>(left_target + 8 * kDeviationStride) = l1;
-        *reinterpret_cast<float4 *>(left_target + 16 * kDeviationStride) = l2;
-        *reinterpret_cast<float4 *>(left_target + 24 * kDeviationStride) = l3;
-        *reinterpret_cast<float4 *>(right_target) = r0;
-        *reinterpret_cast<float4 *>(right_target + 8 * kTileColumns) = r1;
-        *reinterpret_cast<float4 *>(right_target + 16 * kTileColumns) = r2;
-        *reinterpret_cast<float4 *>(right_target + 24 * kTileColumns) = r3;
+    // A wavefront's own transfers have landed once its vector memory counter reads zero; the
+    // barrier that follows extends that to the whole workgroup.
+    auto landed = [&]() __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), other counters untouched
+        __syncthreads();
     };
 
-    fetch(0);
-    keep(0);
-    __syncthreads();
+    fetch(0, std::false_type{});
+    landed();
 
     const uint32_t left_read = (lane >> 5) * kDeviationStride + wave_row + (lane & 31);
     const uint32_t right_read = (lane >> 5) * kTileColumns + wave_column + (lane & 31);
     mk_f32x16 sums[2][2];
-    for (int step = 0; step < steps; ++step) {
-        const int buffer = step & 1;
+    auto advance = [&](int step, auto quarter, auto odd) __attribute__((always_inline)) {
         const int chunk = step % chunks_per_chain;
         if (chunk == 0) {
 #pragma unroll
@@ -500,19 +495,36 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviation
                     for (int r = 0; r < 16; ++r) sums[mi][ni][r] = 0.0f;
         }
         const bool more = step + 1 < steps;
-        if (more) fetch(step + 1);
-        const float *left_rows = &deviation_t[buffer][0][0] + left_read;
-        const float *right_rows = &coefficient[buffer][0][0] + right_read;
-#pragma unroll 4
+        if (more) fetch(step + 1, std::bool_constant<!odd.value>{});
+        if constexpr (quarter.value >= 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                totals[quarter.value >> 1][quarter.value & 1][r] = *cell(quarter.value >> 1, quarter.value & 1, r);
+        }
+        const float *left_rows = (odd.value ? &deviation_odd[0][0] : &deviation_even[0][0]) + left_read;
+        const float *right_rows = (odd.value ? &coefficient_odd[0][0] : &coefficient_even[0][0]) + right_read;
+        // The operands of the next pair of depth steps are read from LDS before this pair's
+        // MFMAs are issued: both waves of a SIMD otherwise wait for LDS at the same time.
+        float left0 = left_rows[0], left1 = left_rows[32];
+        float right0 = right_rows[0], right1 = right_rows[32];
+#pragma unroll
         for (int kk = 0; kk < kDepthChunk; kk += 2) {
-            const float left0 = left_rows[kk * kDeviationStride], left1 = left_rows[kk * kDeviationStride + 32];
-            const float right0 = right_rows[kk * kTileColumns], right1 = right_rows[kk * kTileColumns + 32];
+            float next_left0 = 0.0f, next_left1 = 0.0f, next_right0 = 0.0f, next_right1 = 0.0f;
+            if (kk + 2 < kDepthChunk) {
+                next_left0 = left_rows[(kk + 2) * kDeviationStride];
+                next_left1 = left_rows[(kk + 2) * kDeviationStride + 32];
+                next_right0 = right_rows[(kk + 2) * kTileColumns];
+                next_right1 = right_rows[(kk + 2) * kTileColumns + 32];
+            }
+            __builtin_amdgcn_sched_barrier(0);
             sums[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(left0, right0, sums[0][0], 0, 0, 0);
             sums[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(left0, right1, sums[0][1], 0, 0, 0);
             sums[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(left1, right0, sums[1][0], 0, 0, 0);
             sums[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(left1, right1, sums[1][1], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            left0 = next_left0, left1 = next_left1, right0 = next_right0, right1 = next_right1;
         }
-        if (chunk == chunks_per_chain - 1) {
+        if ((quarter.value < 0 || quarter.value == 3) && chunk == chunks_per_chain - 1) {
 #pragma unroll
             for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
@@ -520,9 +532,19 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviation
 #pragma unroll
                     for (int r = 0; r < 16; ++r) totals[mi][ni][r] = __fadd_rn(totals[mi][ni][r], sums[mi][ni][r]);
         }
-        if (more) keep(buffer ^ 1);
-        __syncthreads();
+        landed();
+    };
+    using None = std::integral_constant<int, -1>;
+    advance(0, std::integral_constant<int, 0>{}, std::false_type{});   // the launcher guarantees chains of four steps or more
+    advance(1, std::integral_constant<int, 1>{}, std::true_type{});
+    advance(2, std::integral_constant<int, 2>{}, std::false_type{});
+    advance(3, std::integral_constant<int, 3>{}, std::true_type{});
+    int step = 4;
+    for (; step + 1 < steps; step += 2) {
+        advance(step, None{}, std::false_type{});
+        advance(step + 1, None{}, std::true_type{});
     }
+    if (step < steps) advance(step, None{}, std::false_type{});
 
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi)
@@ -541,7 +563,8 @@ int launch_update(const UpdateArgs &a, hipStream_t stream) {
     // The deviation buffer path handles whole tiles only.
     const bool staged = a.deviation_t && aligned(a.deviation_t) && aligned(a.coeff) && a.rows % kTileRows == 0 &&
                         a.width % 4 == 0 && a.column_begin % 4 == 0 &&
-                        (a.column_end - a.column_begin) % kTileColumns == 0 && a.chain_width % kDepthChunk == 0;
+                        (a.column_end - a.column_begin) % kTileColumns == 0 && a.chain_width % kDepthChunk == 0 &&
+                        a.chain_width / kDepthChunk >= 4;   // the first chain spans the four steps that read feedback
     if (staged)
         hipLaunchKernelGGL(block_update_from_deviations_kernel, grid, dim3(kUpdateThreads), 0, stream, a);
     else if (vec)
