@@ -45,6 +45,17 @@ struct SweepArgs {
     float code_min, code_max;
 };
 
+// 16 bytes per lane from global memory straight into LDS: lane l's bytes land at
+// `target` + 16 l (`target` is wavefront-uniform).  Completion counts as a vector memory load.
+__device__ __forceinline__ void rows_to_lds(const float *source, float *target) {
+    __builtin_amdgcn_global_load_lds(source, target, 16, 0, 0);
+}
+
+// Waits until this wavefront's vector memory loads, LDS transfers included, are complete.
+__device__ __forceinline__ void wait_for_loads() {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), other counters untouched
+}
+
 template <int S>
 struct SweepShape {
     static constexpr int kWidth = 64 * S;                      // padded tile width
@@ -52,25 +63,35 @@ struct SweepShape {
     static constexpr int kPerThread = kChunk * kWidth / kSweepThreads;
 };
 
+// Coefficients outside the strict upper triangle of the tile count as zero.  fetch_chunk
+// only issues the loads; keep_chunk, a chunk of steps later, is the first to look at them.
+template <int S>
+__device__ __forceinline__ bool chunk_wanted(const SweepArgs &a, int first, int p, int *j, int *c) {
+    const int flat = p * kSweepThreads + threadIdx.x;
+    *j = first + flat / SweepShape<S>::kWidth;
+    *c = flat % SweepShape<S>::kWidth;
+    return *j < a.tile_width && *c > *j && *c < a.tile_width;
+}
+
 template <int S>
 __device__ __forceinline__ void fetch_chunk(const SweepArgs &a, int first, float (&held)[SweepShape<S>::kPerThread]) {
-    using Shape = SweepShape<S>;
 #pragma unroll
-    for (int p = 0; p < Shape::kPerThread; ++p) {
-        const int flat = p * kSweepThreads + threadIdx.x;
-        const int j = first + flat / Shape::kWidth;
-        const int c = flat % Shape::kWidth;
-        const bool wanted = j < a.tile_width && c > j && c < a.tile_width;
-        const size_t index = static_cast<size_t>(a.tile_start + (wanted ? j : 0)) * a.width + a.tile_start + (wanted ? c : 0);
-        const float loaded = a.coeff[index];
-        held[p] = wanted ? loaded : 0.0f;
+    for (int p = 0; p < SweepShape<S>::kPerThread; ++p) {
+        int j, c;
+        const bool wanted = chunk_wanted<S>(a, first, p, &j, &c);
+        held[p] = a.coeff[static_cast<size_t>(a.tile_start + (wanted ? j : 0)) * a.width + a.tile_start + (wanted ? c : 0)];
     }
 }
 
 template <int S>
-__device__ __forceinline__ void keep_chunk(float *buffer, const float (&held)[SweepShape<S>::kPerThread]) {
+__device__ __forceinline__ void keep_chunk(const SweepArgs &a, int first, float *buffer,
+                                           const float (&held)[SweepShape<S>::kPerThread]) {
 #pragma unroll
-    for (int p = 0; p < SweepShape<S>::kPerThread; ++p) buffer[p * kSweepThreads + threadIdx.x] = held[p];
+    for (int p = 0; p < SweepShape<S>::kPerThread; ++p) {
+        int j, c;
+        const bool wanted = chunk_wanted<S>(a, first, p, &j, &c);
+        buffer[p * kSweepThreads + threadIdx.x] = wanted ? held[p] : 0.0f;
+    }
 }
 
 __device__ __forceinline__ float lane_value(float value, int lane) {
@@ -129,7 +150,7 @@ __global__ void __launch_bounds__(kSweepThreads) sweep_kernel(const SweepArgs a)
             if (a.zeros) zero[s] = inside ? a.zeros[slot] : 0.0f;
         }
     }
-    keep_chunk<S>(chunks[0], held);
+    keep_chunk<S>(a, 0, chunks[0], held);
     __syncthreads();
 
     int chunk_index = 0;
@@ -169,7 +190,7 @@ __global__ void __launch_bounds__(kSweepThreads) sweep_kernel(const SweepArgs a)
                 for (int later = s; later < S; ++later)
                     running[later] = __fadd_rn(running[later], __fmul_rn(pushed, coefficient_row[64 * later]));
             }
-            if (more) keep_chunk<S>(chunks[(chunk_index + 1) & 1], held);
+            if (more) keep_chunk<S>(a, first + Shape::kChunk, chunks[(chunk_index + 1) & 1], held);
             __syncthreads();
             ++chunk_index;
         }
@@ -195,9 +216,241 @@ __global__ void __launch_bounds__(kSweepThreads) sweep_kernel(const SweepArgs a)
     }
 }
 
+// ---- tiles of at most 128 columns: sixteen lanes per row ----------------------------------
+//
+// The sweep is one dependent chain per row (round column j, push its deviation into the
+// later columns), so its time is (instructions per step) x (steps) x (wavefronts per SIMD).
+// Here a wavefront sweeps four rows at once: lane 16 g + p owns columns p, 16 + p, ... ,
+// 112 + p of row g (eight slots).  A step rounds one column in every lane's current slot,
+// hands the owner's deviation to the sixteen lanes of its row (four `v_readlane` and a
+// select) and updates at most eight columns per lane.  4096 rows are 1024 wavefronts, one
+// per SIMD, each with a quarter of the per-step work of the one-row-per-wavefront kernel.
+//
+// Coefficient rows reach LDS sixteen at a time, which is one slot of steps; the layout
+// [row in chunk][p][slot] lets a lane read its eight coefficients as two float4.
+
+constexpr int kRowLanes = 16, kSlots = 8, kNarrowTile = kRowLanes * kSlots;  // 128 columns
+constexpr int kNarrowRows = kSweepThreads / kRowLanes;                       // 16 rows per workgroup
+constexpr int kNarrowHeld = kRowLanes * kNarrowTile / kSweepThreads;         // 8 coefficients per thread and chunk
+
+// Coefficients outside the strict upper triangle of the tile count as zero.  The loads are
+// issued here and first looked at in keep_slot, a slot of steps later.
+__device__ __forceinline__ bool slot_wanted(const SweepArgs &a, int slot, int q, int *j, int *c) {
+    const int flat = q * kSweepThreads + threadIdx.x;
+    *j = slot * kRowLanes + flat / kNarrowTile;
+    *c = flat % kNarrowTile;
+    return *j < a.tile_width && *c > *j && *c < a.tile_width;
+}
+
+__device__ __forceinline__ void fetch_slot(const SweepArgs &a, int slot, float (&held)[kNarrowHeld]) {
+#pragma unroll
+    for (int q = 0; q < kNarrowHeld; ++q) {
+        int j, c;
+        const bool wanted = slot_wanted(a, slot, q, &j, &c);
+        held[q] = a.coeff[static_cast<size_t>(a.tile_start + (wanted ? j : 0)) * a.width + a.tile_start + (wanted ? c : 0)];
+    }
+}
+
+__device__ __forceinline__ void keep_slot(const SweepArgs &a, int slot, float *buffer, const float (&held)[kNarrowHeld]) {
+#pragma unroll
+    for (int q = 0; q < kNarrowHeld; ++q) {
+        int j, c;
+        const bool wanted = slot_wanted(a, slot, q, &j, &c);
+        const int i = j - slot * kRowLanes;
+        buffer[i * kNarrowTile + (c % kRowLanes) * kSlots + c / kRowLanes] = wanted ? held[q] : 0.0f;
+    }
+}
+
+// The value lane 16 g + owner holds, in all sixteen lanes of row g.
+__device__ __forceinline__ float row_value(float value, int owner, int row_in_wave) {
+    const uint32_t bits = __float_as_uint(value);
+    const uint32_t v0 = __builtin_amdgcn_readlane(bits, owner);
+    const uint32_t v1 = __builtin_amdgcn_readlane(bits, owner + 16);
+    const uint32_t v2 = __builtin_amdgcn_readlane(bits, owner + 32);
+    const uint32_t v3 = __builtin_amdgcn_readlane(bits, owner + 48);
+    uint32_t chosen = v3;
+    chosen = row_in_wave == 2 ? v2 : chosen;
+    chosen = row_in_wave == 1 ? v1 : chosen;
+    chosen = row_in_wave == 0 ? v0 : chosen;
+    return __uint_as_float(chosen);
+}
+
+// The same for an owner known at compile time: a DPP row broadcast, which the compiler
+// folds into the multiplications that use the value.
+template <int OWNER>
+__device__ __forceinline__ float row_value(float value, std::integral_constant<int, OWNER>, int) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(value), 0x150 + OWNER, 0xf, 0xf, false));
+}
+
+// WHOLE: the tile is exactly 128 columns.  All 128 steps are unrolled, so owners, register
+// slots and LDS offsets are constants, and the tile's 128 x 128 coefficients go from global
+// memory straight into LDS before the first step (row-major; one memory latency for the
+// whole kernel instead of one per slot).  Otherwise the sixteen steps of a slot are a loop
+// over coefficient rows staged slot by slot.
+template <int MODE, bool WHOLE>
+__global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const SweepArgs a) {
+    static_assert(MODE == kModeInteger || MODE == kModeSolve, "codebooks use the one-row-per-wavefront kernel");
+    constexpr int kStaged = WHOLE ? kNarrowTile * kNarrowTile : 2 * kRowLanes * kNarrowTile;
+    __shared__ __attribute__((aligned(16))) float staged[kStaged];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int row_in_wave = lane >> 4, p = lane & (kRowLanes - 1);
+    const int wanted_row = blockIdx.x * kNarrowRows + wave * 4 + row_in_wave;
+    const bool active = wanted_row < a.rows;
+    const int row = active ? wanted_row : a.rows - 1;
+    const size_t row_base = static_cast<size_t>(row) * a.width;
+
+    float held[kNarrowHeld];
+    if constexpr (WHOLE) {
+        // One wavefront instruction moves two coefficient rows of the tile (2 x 128 floats,
+        // lane l's 16 bytes at 16 l from the uniform LDS address); a wavefront moves rows
+        // 32 wave ... 32 wave + 31.
+        const float *corner = a.coeff + static_cast<size_t>(a.tile_start) * a.width + a.tile_start;
+        const uint32_t lane_offset = static_cast<uint32_t>(lane >> 5) * a.width + (lane & 31) * 4;
+#pragma unroll
+        for (int pair = 0; pair < 16; ++pair) {
+            const int j = wave * 32 + 2 * pair;
+            rows_to_lds(corner + static_cast<size_t>(j) * a.width + lane_offset, &staged[j * kNarrowTile]);
+        }
+    } else {
+        fetch_slot(a, 0, held);
+    }
+
+    float weight[kSlots], running[kSlots], scale[kSlots], zero[kSlots], finished[kSlots], base[kSlots];
+    uint32_t code[kSlots];
+#pragma unroll
+    for (int t = 0; t < kSlots; ++t) {
+        const int c = kRowLanes * t + p;
+        const bool inside = c < a.tile_width;
+        const int position = a.tile_start + (inside ? c : 0);
+        running[t] = inside ? a.feedback[row_base + position] : 0.0f;
+        weight[t] = 0.0f; scale[t] = 1.0f; zero[t] = 0.0f; finished[t] = 0.0f; code[t] = 0; base[t] = 0.0f;
+        if constexpr (MODE != kModeSolve) {
+            weight[t] = inside ? a.original[row_base + position] : 0.0f;
+            const int slot = row * a.groups_per_row + (position - a.region_start) / a.group;
+            scale[t] = inside ? a.scales[slot] : 1.0f;
+            if (a.zeros) zero[t] = inside ? a.zeros[slot] : 0.0f;
+        } else {
+            if (a.original) base[t] = a.original[row_base + position];  // added to the solved adjustment at the end
+        }
+    }
+    if constexpr (WHOLE) {
+        wait_for_loads();
+    } else {
+        keep_slot(a, 0, staged, held);
+    }
+    __syncthreads();
+
+    // One step: round column 16 t + owner of every row, push its deviation into the later
+    // columns.  `owner` is an int or a std::integral_constant.  `coefficients` is row
+    // 16 t + owner of the tile as this lane reads it.
+    auto advance = [&](auto slot, auto owner, const float *coefficients) __attribute__((always_inline)) {
+        constexpr int t = decltype(slot)::value;
+        float pushed;
+        if constexpr (MODE == kModeSolve) {
+            pushed = -row_value(running[t], owner, row_in_wave);
+        } else {
+            const float target = __fadd_rn(weight[t], running[t]);
+            const float normalized = __fdiv_rn(__fsub_rn(target, zero[t]), scale[t]);
+            const float chosen = fminf(fmaxf(rintf(normalized), a.code_min), a.code_max);
+            const uint32_t index = static_cast<uint32_t>(static_cast<int>(__fsub_rn(chosen, a.code_min)));
+            const float reconstruction = __fadd_rn(__fmul_rn(chosen, scale[t]), zero[t]);
+            const bool mine = p == static_cast<int>(owner);
+            finished[t] = mine ? reconstruction : finished[t];
+            code[t] = mine ? index : code[t];
+            pushed = row_value(__fsub_rn(weight[t], reconstruction), owner, row_in_wave);
+        }
+        float row_of[kSlots];
+        if constexpr (WHOLE) {
+            // Row-major row: this lane's columns are 16 floats apart.  Columns up to the
+            // owner's hold whatever the matrix has there; only the solve still reads its
+            // running values of such columns afterwards, so it masks them.
+#pragma unroll
+            for (int later = t; later < kSlots; ++later) row_of[later] = coefficients[kRowLanes * later];
+            if constexpr (MODE == kModeSolve) row_of[t] = p > static_cast<int>(owner) ? row_of[t] : 0.0f;
+        } else {
+            float4 low = {0.0f, 0.0f, 0.0f, 0.0f};
+            if constexpr (t < 4) low = *reinterpret_cast<const float4 *>(coefficients);
+            const float4 high = *reinterpret_cast<const float4 *>(coefficients + 4);
+            row_of[0] = low.x, row_of[1] = low.y, row_of[2] = low.z, row_of[3] = low.w;
+            row_of[4] = high.x, row_of[5] = high.y, row_of[6] = high.z, row_of[7] = high.w;
+        }
+#pragma unroll
+        for (int later = t; later < kSlots; ++later)
+            running[later] = __fadd_rn(running[later], __fmul_rn(pushed, row_of[later]));
+    };
+    auto step_of_whole = [&](auto slot, auto owner) __attribute__((always_inline)) {
+        advance(slot, owner, staged + (kRowLanes * decltype(slot)::value + decltype(owner)::value) * kNarrowTile + p);
+    };
+    auto slot_of_steps = [&](auto slot) __attribute__((always_inline)) {
+        constexpr int t = decltype(slot)::value;
+        if constexpr (WHOLE) {
+            step_of_whole(slot, std::integral_constant<int, 0>{});
+            step_of_whole(slot, std::integral_constant<int, 1>{});
+            step_of_whole(slot, std::integral_constant<int, 2>{});
+            step_of_whole(slot, std::integral_constant<int, 3>{});
+            step_of_whole(slot, std::integral_constant<int, 4>{});
+            step_of_whole(slot, std::integral_constant<int, 5>{});
+            step_of_whole(slot, std::integral_constant<int, 6>{});
+            step_of_whole(slot, std::integral_constant<int, 7>{});
+            step_of_whole(slot, std::integral_constant<int, 8>{});
+            step_of_whole(slot, std::integral_constant<int, 9>{});
+            step_of_whole(slot, std::integral_constant<int, 10>{});
+            step_of_whole(slot, std::integral_constant<int, 11>{});
+            step_of_whole(slot, std::integral_constant<int, 12>{});
+            step_of_whole(slot, std::integral_constant<int, 13>{});
+            step_of_whole(slot, std::integral_constant<int, 14>{});
+            step_of_whole(slot, std::integral_constant<int, 15>{});
+        } else if (kRowLanes * t < a.tile_width) {  // uniform
+            const bool more = kRowLanes * (t + 1) < a.tile_width;
+            if (more) fetch_slot(a, t + 1, held);
+            const float *mine_in_chunk = staged + (t & 1) * kRowLanes * kNarrowTile + p * kSlots;
+            const int owners = min(kRowLanes, a.tile_width - kRowLanes * t);
+            for (int owner = 0; owner < owners; ++owner) advance(slot, owner, mine_in_chunk + owner * kNarrowTile);
+            if (more) keep_slot(a, t + 1, staged + ((t + 1) & 1) * kRowLanes * kNarrowTile, held);
+            __syncthreads();
+        }
+    };
+    slot_of_steps(std::integral_constant<int, 0>{});
+    slot_of_steps(std::integral_constant<int, 1>{});
+    slot_of_steps(std::integral_constant<int, 2>{});
+    slot_of_steps(std::integral_constant<int, 3>{});
+    slot_of_steps(std::integral_constant<int, 4>{});
+    slot_of_steps(std::integral_constant<int, 5>{});
+    slot_of_steps(std::integral_constant<int, 6>{});
+    slot_of_steps(std::integral_constant<int, 7>{});
+
+    if (!active) return;
+#pragma unroll
+    for (int t = 0; t < kSlots; ++t) {
+        const int c = kRowLanes * t + p;
+        if (c >= a.tile_width) continue;
+        if constexpr (MODE == kModeSolve) {
+            // a.output is [rows, tile_width]; with `original` given the solved adjustment is
+            // added to the region's weights (the targets a region's scales are fitted to).
+            a.output[static_cast<size_t>(row) * a.tile_width + c] = a.original ? __fadd_rn(base[t], running[t]) : running[t];
+        } else {
+            a.output[row_base + a.tile_start + c] = finished[t];
+            a.encoded[row_base + a.tile_start + c] = static_cast<uint8_t>(code[t]);
+            if (a.deviation_t)
+                a.deviation_t[static_cast<size_t>(a.tile_start + c) * a.rows + row] = __fsub_rn(weight[t], finished[t]);
+        }
+    }
+}
+
 template <int MODE>
 int launch_sweep(const SweepArgs &a, hipStream_t stream) {
     const dim3 grid(mk_cdiv(a.rows, kSweepThreads / 64)), block(kSweepThreads);
+    if constexpr (MODE != kModeCodebook) {
+        if (a.tile_width <= kNarrowTile) {
+            const dim3 narrow_grid(mk_cdiv(a.rows, kNarrowRows));
+            if (a.tile_width == kNarrowTile)
+                hipLaunchKernelGGL((narrow_sweep_kernel<MODE, true>), narrow_grid, block, 0, stream, a);
+            else
+                hipLaunchKernelGGL((narrow_sweep_kernel<MODE, false>), narrow_grid, block, 0, stream, a);
+            return MK_OK;
+        }
+    }
     if (a.tile_width <= 128)
         hipLaunchKernelGGL((sweep_kernel<2, MODE>), grid, block, 0, stream, a);
     else if (a.tile_width <= 256)
@@ -463,18 +716,18 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviation
             const float *right_source = right + static_cast<size_t>(2 * pair) * a.width + right_lane;
             const int k = wave * 8 + 2 * pair;
             if constexpr (odd.value) {
-                __builtin_amdgcn_global_load_lds(left_source, &deviation_odd[k][0], 16, 0, 0);
-                __builtin_amdgcn_global_load_lds(right_source, &coefficient_odd[k][0], 16, 0, 0);
+                rows_to_lds(left_source, &deviation_odd[k][0]);
+                rows_to_lds(right_source, &coefficient_odd[k][0]);
             } else {
-                __builtin_amdgcn_global_load_lds(left_source, &deviation_even[k][0], 16, 0, 0);
-                __builtin_amdgcn_global_load_lds(right_source, &coefficient_even[k][0], 16, 0, 0);
+                rows_to_lds(left_source, &deviation_even[k][0]);
+                rows_to_lds(right_source, &coefficient_even[k][0]);
             }
         }
     };
     // A wavefront's own transfers have landed once its vector memory counter reads zero; the
     // barrier that follows extends that to the whole workgroup.
     auto landed = [&]() __attribute__((always_inline)) {
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), other counters untouched
+        wait_for_loads();
         __syncthreads();
     };
 
