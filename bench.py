@@ -302,6 +302,8 @@ def main() -> None:
     parser.add_argument("--profile-launches", type=int, default=0,
                         help="for rocprofv3: only launch the M=1 matvec this many times, plus three "
                              "256 MiB device copies whose counters calibrate FETCH_SIZE / WRITE_SIZE")
+    parser.add_argument("--profile-rows", type=int, default=1,
+                        help="activation rows M of the --profile-launches launches")
     options = parser.parse_args()
     if options.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -317,8 +319,8 @@ def main() -> None:
         print(json.dumps(gptq_layer(device, generator)))
         return
     if options.profile_launches:
-        x = torch.randn((1, WIDTH), device=device, generator=generator).half()
-        y = torch.empty((1, ROWS), device=device, dtype=torch.float16)
+        x = torch.randn((options.profile_rows, WIDTH), device=device, generator=generator).half()
+        y = torch.empty((options.profile_rows, ROWS), device=device, dtype=torch.float16)
         launchers = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
         raw = torch.cuda.current_stream().cuda_stream
         for step in range(options.profile_launches):
