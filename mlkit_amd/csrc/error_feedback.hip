@@ -27,7 +27,7 @@
 namespace {
 
 constexpr int kSweepThreads = 256;  // four wavefronts = four rows
-constexpr int kModeInteger = 0, kModeCodebook = 1, kModeSolve = 2;
+constexpr int kModeInteger = 0, kModeCodebook = 1, kModeSolve = 2, kModeRegion = 3;
 
 struct SweepArgs {
     const float *original;
@@ -43,6 +43,11 @@ struct SweepArgs {
     int region_start, tile_start, tile_width;
     int group, groups_per_row, n_values;
     float code_min, code_max;
+    // kModeRegion only: the region's scales (and offsets) are fitted inside the kernel and
+    // written to fit_scales / fit_zeros (same indexing as scales / zeros).
+    float *fit_scales, *fit_zeros;
+    int solve_first, asym, scale_format;
+    float reciprocal, value_minimum;
 };
 
 // 16 bytes per lane from global memory straight into LDS: lane l's bytes land at
@@ -289,7 +294,8 @@ __device__ __forceinline__ float row_value(float value, std::integral_constant<i
 // over coefficient rows staged slot by slot.
 template <int MODE, bool WHOLE>
 __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const SweepArgs a) {
-    static_assert(MODE == kModeInteger || MODE == kModeSolve, "codebooks use the one-row-per-wavefront kernel");
+    static_assert(MODE == kModeInteger || MODE == kModeSolve || (MODE == kModeRegion && WHOLE),
+                  "codebooks use the one-row-per-wavefront kernel; a fused region is one whole tile");
     constexpr int kStaged = WHOLE ? kNarrowTile * kNarrowTile : 2 * kRowLanes * kNarrowTile;
     __shared__ __attribute__((aligned(16))) float staged[kStaged];
     const int lane = threadIdx.x & 63;
@@ -325,7 +331,9 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
         const int position = a.tile_start + (inside ? c : 0);
         running[t] = inside ? a.feedback[row_base + position] : 0.0f;
         weight[t] = 0.0f; scale[t] = 1.0f; zero[t] = 0.0f; finished[t] = 0.0f; code[t] = 0; base[t] = 0.0f;
-        if constexpr (MODE != kModeSolve) {
+        if constexpr (MODE == kModeRegion) {
+            weight[t] = a.original[row_base + position];
+        } else if constexpr (MODE != kModeSolve) {
             weight[t] = inside ? a.original[row_base + position] : 0.0f;
             const int slot = row * a.groups_per_row + (position - a.region_start) / a.group;
             scale[t] = inside ? a.scales[slot] : 1.0f;
@@ -344,10 +352,11 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
     // One step: round column 16 t + owner of every row, push its deviation into the later
     // columns.  `owner` is an int or a std::integral_constant.  `coefficients` is row
     // 16 t + owner of the tile as this lane reads it.
-    auto advance = [&](auto slot, auto owner, const float *coefficients) __attribute__((always_inline)) {
+    auto advance = [&](auto slot, auto owner, const float *coefficients, auto solving) __attribute__((always_inline)) {
         constexpr int t = decltype(slot)::value;
+        constexpr bool kSolving = decltype(solving)::value;
         float pushed;
-        if constexpr (MODE == kModeSolve) {
+        if constexpr (kSolving) {
             pushed = -row_value(running[t], owner, row_in_wave);
         } else {
             const float target = __fadd_rn(weight[t], running[t]);
@@ -367,7 +376,7 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
             // running values of such columns afterwards, so it masks them.
 #pragma unroll
             for (int later = t; later < kSlots; ++later) row_of[later] = coefficients[kRowLanes * later];
-            if constexpr (MODE == kModeSolve) row_of[t] = p > static_cast<int>(owner) ? row_of[t] : 0.0f;
+            if constexpr (kSolving) row_of[t] = p > static_cast<int>(owner) ? row_of[t] : 0.0f;
         } else {
             float4 low = {0.0f, 0.0f, 0.0f, 0.0f};
             if constexpr (t < 4) low = *reinterpret_cast<const float4 *>(coefficients);
@@ -379,46 +388,116 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
         for (int later = t; later < kSlots; ++later)
             running[later] = __fadd_rn(running[later], __fmul_rn(pushed, row_of[later]));
     };
-    auto step_of_whole = [&](auto slot, auto owner) __attribute__((always_inline)) {
-        advance(slot, owner, staged + (kRowLanes * decltype(slot)::value + decltype(owner)::value) * kNarrowTile + p);
+    auto step_of_whole = [&](auto slot, auto owner, auto solving) __attribute__((always_inline)) {
+        advance(slot, owner, staged + (kRowLanes * decltype(slot)::value + decltype(owner)::value) * kNarrowTile + p, solving);
     };
-    auto slot_of_steps = [&](auto slot) __attribute__((always_inline)) {
+    auto slot_of_steps = [&](auto slot, auto solving) __attribute__((always_inline)) {
         constexpr int t = decltype(slot)::value;
         if constexpr (WHOLE) {
-            step_of_whole(slot, std::integral_constant<int, 0>{});
-            step_of_whole(slot, std::integral_constant<int, 1>{});
-            step_of_whole(slot, std::integral_constant<int, 2>{});
-            step_of_whole(slot, std::integral_constant<int, 3>{});
-            step_of_whole(slot, std::integral_constant<int, 4>{});
-            step_of_whole(slot, std::integral_constant<int, 5>{});
-            step_of_whole(slot, std::integral_constant<int, 6>{});
-            step_of_whole(slot, std::integral_constant<int, 7>{});
-            step_of_whole(slot, std::integral_constant<int, 8>{});
-            step_of_whole(slot, std::integral_constant<int, 9>{});
-            step_of_whole(slot, std::integral_constant<int, 10>{});
-            step_of_whole(slot, std::integral_constant<int, 11>{});
-            step_of_whole(slot, std::integral_constant<int, 12>{});
-            step_of_whole(slot, std::integral_constant<int, 13>{});
-            step_of_whole(slot, std::integral_constant<int, 14>{});
-            step_of_whole(slot, std::integral_constant<int, 15>{});
+            step_of_whole(slot, std::integral_constant<int, 0>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 1>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 2>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 3>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 4>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 5>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 6>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 7>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 8>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 9>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 10>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 11>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 12>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 13>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 14>{}, solving);
+            step_of_whole(slot, std::integral_constant<int, 15>{}, solving);
         } else if (kRowLanes * t < a.tile_width) {  // uniform
             const bool more = kRowLanes * (t + 1) < a.tile_width;
             if (more) fetch_slot(a, t + 1, held);
             const float *mine_in_chunk = staged + (t & 1) * kRowLanes * kNarrowTile + p * kSlots;
             const int owners = min(kRowLanes, a.tile_width - kRowLanes * t);
-            for (int owner = 0; owner < owners; ++owner) advance(slot, owner, mine_in_chunk + owner * kNarrowTile);
+            for (int owner = 0; owner < owners; ++owner) advance(slot, owner, mine_in_chunk + owner * kNarrowTile, solving);
             if (more) keep_slot(a, t + 1, staged + ((t + 1) & 1) * kRowLanes * kNarrowTile, held);
             __syncthreads();
         }
     };
-    slot_of_steps(std::integral_constant<int, 0>{});
-    slot_of_steps(std::integral_constant<int, 1>{});
-    slot_of_steps(std::integral_constant<int, 2>{});
-    slot_of_steps(std::integral_constant<int, 3>{});
-    slot_of_steps(std::integral_constant<int, 4>{});
-    slot_of_steps(std::integral_constant<int, 5>{});
-    slot_of_steps(std::integral_constant<int, 6>{});
-    slot_of_steps(std::integral_constant<int, 7>{});
+    auto all_slots = [&](auto solving) __attribute__((always_inline)) {
+        slot_of_steps(std::integral_constant<int, 0>{}, solving);
+        slot_of_steps(std::integral_constant<int, 1>{}, solving);
+        slot_of_steps(std::integral_constant<int, 2>{}, solving);
+        slot_of_steps(std::integral_constant<int, 3>{}, solving);
+        slot_of_steps(std::integral_constant<int, 4>{}, solving);
+        slot_of_steps(std::integral_constant<int, 5>{}, solving);
+        slot_of_steps(std::integral_constant<int, 6>{}, solving);
+        slot_of_steps(std::integral_constant<int, 7>{}, solving);
+    };
+    if constexpr (MODE == kModeRegion) {
+        // The region's scales are fitted to original + x, where x U = feedback over the
+        // region's own columns (U: the unit upper coefficient tile); then the same columns
+        // are rounded with those scales.  Both passes read the coefficient tile from LDS.
+        float fed[kSlots];
+#pragma unroll
+        for (int t = 0; t < kSlots; ++t) fed[t] = running[t];
+        if (a.solve_first) all_slots(std::true_type{});   // uniform
+        float fitted[kSlots];
+#pragma unroll
+        for (int t = 0; t < kSlots; ++t) {
+            fitted[t] = a.solve_first ? __fadd_rn(weight[t], running[t]) : weight[t];
+            running[t] = fed[t];
+        }
+        // A scale group is `a.group` columns: group / 16 adjacent slots of all sixteen lanes.
+        const int slots_per_group = a.group / kRowLanes;
+        auto fit_groups = [&](auto span) __attribute__((always_inline)) {
+            constexpr int kSpan = decltype(span)::value;
+#pragma unroll
+            for (int first = 0; first < kSlots; first += kSpan) {
+                float low = fitted[first], high = fitted[first];
+                bool all_finite = true;
+#pragma unroll
+                for (int t = first; t < first + kSpan; ++t) {
+                    low = fminf(low, fitted[t]);
+                    high = fmaxf(high, fitted[t]);
+                    all_finite = all_finite && (fitted[t] - fitted[t] == 0.0f);
+                }
+#pragma unroll
+                for (int offset = 1; offset < kRowLanes; offset <<= 1) {
+                    low = fminf(low, __shfl_xor(low, offset, 64));
+                    high = fmaxf(high, __shfl_xor(high, offset, 64));
+                    all_finite = __shfl_xor(static_cast<int>(all_finite), offset, 64) && all_finite;
+                }
+                float group_scale, group_zero = 0.0f;
+                if (a.asym) {
+                    group_scale = __fmul_rn(fmaxf(__fsub_rn(high, low), 1e-12f), a.reciprocal);
+                    group_zero = __fsub_rn(low, __fmul_rn(a.value_minimum, group_scale));
+                    const float magnitude = mk_rounded_scale(fmaxf(fabsf(group_zero), 1e-12f), a.scale_format);
+                    group_zero = group_zero > 0.0f ? magnitude : (group_zero < 0.0f ? -magnitude : 0.0f);
+                } else {
+                    group_scale = __fmul_rn(fmaxf(fmaxf(high, -low), 1e-12f), a.reciprocal);
+                }
+                group_scale = mk_rounded_scale(group_scale, a.scale_format);
+                if (!all_finite) {  // fminf / fmaxf drop NaNs: report them as the tensor reductions would
+                    group_scale = __builtin_nanf("");
+                    group_zero = __builtin_nanf("");
+                }
+#pragma unroll
+                for (int t = first; t < first + kSpan; ++t) {
+                    scale[t] = group_scale;
+                    zero[t] = group_zero;
+                }
+                if (active && p == 0) {
+                    const int slot = row * a.groups_per_row + first / kSpan;
+                    a.fit_scales[slot] = group_scale;
+                    if (a.fit_zeros) a.fit_zeros[slot] = group_zero;
+                }
+            }
+        };
+        if (slots_per_group == 8) fit_groups(std::integral_constant<int, 8>{});
+        else if (slots_per_group == 4) fit_groups(std::integral_constant<int, 4>{});
+        else if (slots_per_group == 2) fit_groups(std::integral_constant<int, 2>{});
+        else fit_groups(std::integral_constant<int, 1>{});
+        all_slots(std::false_type{});
+    } else {
+        all_slots(std::bool_constant<MODE == kModeSolve>{});
+    }
 
     if (!active) return;
 #pragma unroll
@@ -436,6 +515,19 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
                 a.deviation_t[static_cast<size_t>(a.tile_start + c) * a.rows + row] = __fsub_rn(weight[t], finished[t]);
         }
     }
+}
+
+// One kernel for a region that is a single whole tile of an integer grid: pending solve,
+// scale fit and column sweep.
+bool region_fusable(int span, int block, int fitted_group, bool integer_grid) {
+    return integer_grid && span == kNarrowTile && block >= kNarrowTile && fitted_group % kRowLanes == 0 &&
+           kNarrowTile % fitted_group == 0;
+}
+
+int launch_region(const SweepArgs &a, hipStream_t stream) {
+    hipLaunchKernelGGL((narrow_sweep_kernel<kModeRegion, true>), dim3(mk_cdiv(a.rows, kNarrowRows)), dim3(kSweepThreads), 0,
+                       stream, a);
+    return MK_OK;
 }
 
 template <int MODE>
@@ -981,7 +1073,11 @@ extern "C" int mk_feedback_sweep(const float *original, float *feedback, float *
         }
         float *region_scales = scales + group_offset;
         float *region_zeros = asym ? zeros + group_offset : nullptr;
-        if (region_start == 0) {
+        const bool fused = region_fusable(span, block, fitted_group, integer_grid != 0) && scale_format >= 0 &&
+                           scale_format <= 4;
+        if (fused) {
+            // fitted inside the sweep kernel below
+        } else if (region_start == 0) {
             if (int status = mk_fit_scales_strided(original, width, region_scales, region_zeros, total_groups, rows, span,
                                                    fitted_group, asym, reciprocal, value_minimum, scale_format, 1, stream))
                 return status;
@@ -1004,7 +1100,11 @@ extern "C" int mk_feedback_sweep(const float *original, float *feedback, float *
             a.tile_width = tile_stop - tile_start; a.group = fitted_group;
             a.groups_per_row = static_cast<int>(total_groups); a.n_values = n_values;
             a.code_min = code_min; a.code_max = code_max; a.deviation_t = deviations;
-            if (integer_grid) launch_sweep<kModeInteger>(a, stream);
+            if (fused) {
+                a.fit_scales = region_scales; a.fit_zeros = region_zeros; a.solve_first = region_start != 0;
+                a.asym = asym; a.scale_format = scale_format; a.reciprocal = reciprocal; a.value_minimum = value_minimum;
+                launch_region(a, stream);
+            } else if (integer_grid) launch_sweep<kModeInteger>(a, stream);
             else launch_sweep<kModeCodebook>(a, stream);
             if (tile_stop >= width) continue;
             if (tile_stop < limit)

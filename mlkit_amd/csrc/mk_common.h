@@ -116,4 +116,34 @@ __device__ __forceinline__ float mk_segment_sum(float value) {
     return value;
 }
 
+// Storage rounding of a positive scale; format codes: 0 fp32, 1 fp16, 2 bf16, 3 fp8 e4m3,
+// 4 e8m0 (power of two).
+__device__ __forceinline__ float mk_rounded_scale(float value, int format) {
+    if (format == 1) {
+        const float clamped = fminf(fmaxf(value, 0x1p-24f), 65504.0f);
+        return static_cast<float>(static_cast<_Float16>(clamped));
+    }
+    if (format == 2) return mk_bf16_to_float(mk_float_to_bf16(value));
+    if (format == 3) {
+        const float clamped = fminf(fmaxf(value, 0x1p-9f), 448.0f);
+        const int exponent = static_cast<int>((__float_as_uint(clamped) >> 23) & 255u) - 127;
+        const int quantum_exponent = (exponent > -6 ? exponent : -6) - 3;
+        const float quantum = __uint_as_float(static_cast<uint32_t>(quantum_exponent + 127) << 23);
+        const float reciprocal = __uint_as_float(static_cast<uint32_t>(127 - quantum_exponent) << 23);
+        return __fmul_rn(rintf(__fmul_rn(clamped, reciprocal)), quantum);
+    }
+    if (format == 4) {
+        // 2^round(log2 v) exactly: the mantissa m in [1, 2) rounds up iff m^2 > 2.
+        const float clamped = fmaxf(value, 0x1p-126f);
+        const uint32_t bits = __float_as_uint(clamped);
+        int exponent = static_cast<int>((bits >> 23) & 255u) - 127;
+        const uint64_t mantissa = (bits & 0x7fffffu) | 0x800000u;
+        if (mantissa * mantissa > (2ull << 46)) ++exponent;
+        if (value < 0x1p-126f) exponent = value > 0x1.6a09e6p-127f ? -126 : -127;
+        exponent = exponent > 127 ? 127 : exponent;
+        return ldexpf(1.0f, exponent);
+    }
+    return value;
+}
+
 #endif  // __HIPCC__

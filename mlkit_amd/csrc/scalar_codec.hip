@@ -52,36 +52,6 @@ __device__ __forceinline__ void stage_table(float *shared, const float *values, 
     __syncthreads();
 }
 
-// Storage rounding of a positive scale; format codes: 0 fp32, 1 fp16, 2 bf16, 3 fp8 e4m3,
-// 4 e8m0 (power of two).
-__device__ __forceinline__ float rounded_scale(float value, int format) {
-    if (format == 1) {
-        const float clamped = fminf(fmaxf(value, 0x1p-24f), 65504.0f);
-        return static_cast<float>(static_cast<_Float16>(clamped));
-    }
-    if (format == 2) return mk_bf16_to_float(mk_float_to_bf16(value));
-    if (format == 3) {
-        const float clamped = fminf(fmaxf(value, 0x1p-9f), 448.0f);
-        const int exponent = static_cast<int>((__float_as_uint(clamped) >> 23) & 255u) - 127;
-        const int quantum_exponent = (exponent > -6 ? exponent : -6) - 3;
-        const float quantum = __uint_as_float(static_cast<uint32_t>(quantum_exponent + 127) << 23);
-        const float reciprocal = __uint_as_float(static_cast<uint32_t>(127 - quantum_exponent) << 23);
-        return __fmul_rn(rintf(__fmul_rn(clamped, reciprocal)), quantum);
-    }
-    if (format == 4) {
-        // 2^round(log2 v) exactly: the mantissa m in [1, 2) rounds up iff m^2 > 2.
-        const float clamped = fmaxf(value, 0x1p-126f);
-        const uint32_t bits = __float_as_uint(clamped);
-        int exponent = static_cast<int>((bits >> 23) & 255u) - 127;
-        const uint64_t mantissa = (bits & 0x7fffffu) | 0x800000u;
-        if (mantissa * mantissa > (2ull << 46)) ++exponent;
-        if (value < 0x1p-126f) exponent = value > 0x1.6a09e6p-127f ? -126 : -127;
-        exponent = exponent > 127 ? 127 : exponent;
-        return ldexpf(1.0f, exponent);
-    }
-    return value;
-}
-
 struct CodecArgs {
     const float *value;
     const float *scales;
@@ -243,7 +213,7 @@ __global__ void __launch_bounds__(kThreads) search_kernel(const SearchArgs a) {
         float best_scale = base;
         float best_error = team_error<LANES>(a, table, steps, row_value, group_start, lane_in_team, base, zero);
         for (int c = 0; c < a.n_fractions; ++c) {
-            const float scale = rounded_scale(__fmul_rn(base, fraction[c]), a.format);
+            const float scale = mk_rounded_scale(__fmul_rn(base, fraction[c]), a.format);
             const float error = team_error<LANES>(a, table, steps, row_value, group_start, lane_in_team, scale, zero);
             const bool improved = error < best_error;
             best_scale = improved ? scale : best_scale;
@@ -323,10 +293,10 @@ __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
         } else {
             scale = __fmul_rn(fmaxf(fmaxf(high, -low), 1e-12f), a.reciprocal);
         }
-        a.scales[slot] = rounded_scale(scale, a.format);
+        a.scales[slot] = mk_rounded_scale(scale, a.format);
         if (a.zeros) {
             if (a.store_zero) {
-                const float magnitude = rounded_scale(fmaxf(fabsf(zero), 1e-12f), a.format);
+                const float magnitude = mk_rounded_scale(fmaxf(fabsf(zero), 1e-12f), a.format);
                 zero = zero > 0.0f ? magnitude : (zero < 0.0f ? -magnitude : 0.0f);
             }
             a.zeros[slot] = zero;
@@ -383,11 +353,11 @@ __global__ void __launch_bounds__(kThreads) reconstruct_kernel(const Reconstruct
         if (a.asym) {
             const float raw = __fmul_rn(fmaxf(__fsub_rn(high, low), 1e-12f), a.reciprocal);
             zero = __fsub_rn(low, __fmul_rn(a.minimum, raw));
-            scale = rounded_scale(raw, a.format);
-            const float magnitude = rounded_scale(fmaxf(fabsf(zero), 1e-12f), a.format);
+            scale = mk_rounded_scale(raw, a.format);
+            const float magnitude = mk_rounded_scale(fmaxf(fabsf(zero), 1e-12f), a.format);
             zero = zero > 0.0f ? magnitude : (zero < 0.0f ? -magnitude : 0.0f);
         } else {
-            scale = rounded_scale(__fmul_rn(fmaxf(fmaxf(high, -low), 1e-12f), a.reciprocal), a.format);
+            scale = mk_rounded_scale(__fmul_rn(fmaxf(fmaxf(high, -low), 1e-12f), a.reciprocal), a.format);
         }
         if (wanted >= a.total_groups) continue;
         for (int column = start + lane_in_team; column < stop; column += LANES) {

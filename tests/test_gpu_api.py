@@ -358,7 +358,7 @@ def test_whole_sweep_entry_point_equals_the_region_by_region_loop(rows, width, r
     inputs = rng.standard_normal((2048, width)).astype(F32)
     inputs[:, ::11] *= 4
     hessian = dev((inputs.T @ inputs / 2048).astype(F32))
-    for asym, refit, block in ((False, 128, 128), (True, 256, 64), (False, None, 128), (True, 96, 128)):
+    for asym, refit, block in ((False, 128, 128), (True, 128, 128), (True, 256, 64), (False, None, 128), (True, 96, 128)):
         single = mk.gptq(Scaled(mk.grid.int(4), 32, asym=asym), refit=refit, block_size=block)(weight, Ctx(H=hessian))
         looped = mk.gptq(Plain(mk.grid.int(4), 32, asym=asym), refit=refit, block_size=block)(weight, Ctx(H=hessian))
         assert torch.equal(single.codes, looped.codes)
