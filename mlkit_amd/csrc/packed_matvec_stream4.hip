@@ -82,7 +82,10 @@ __device__ __forceinline__ void chunk_from_slice(XChunk<MK_F16> &x, const uint32
 template <int MT, bool HAS_ZERO, int ROWS>
 __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     __shared__ float partials[64 * 8];  // [row sum][wavefront]
-    __shared__ __attribute__((aligned(16))) uint32_t x_slices[8][kSliceWords];
+    // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
+    // must not hold LDS for eight).
+    extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
+    uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
     constexpr int kStreamRows = ROWS;
     constexpr int kStreamAhead = rows_ahead_of<ROWS>();
     constexpr int kReduceRows = reduce_rows<MT, ROWS>();
@@ -142,8 +145,8 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) park_piece(x_slices[wave], i, lane, pieces[m][i]);
-        chunk_from_slice(x[m], x_slices[wave], lane);
+        for (int i = 0; i < 4; ++i) park_piece(x_slice, i, lane, pieces[m][i]);
+        chunk_from_slice(x[m], x_slice, lane);
     }
 
     // sum_k (min + step c_k) x_k = step * dot + min * sum(x) - step * (code-free part of dot).
@@ -233,7 +236,10 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     constexpr int kAhead = kSteps < 8 ? kSteps : 8;
     constexpr int kSums = ROWS;                     // per set and lane before the reduction
     __shared__ float partials[SETS * ROWS * 4 * 8];  // [set][row][sample in set][wavefront]
-    __shared__ __attribute__((aligned(16))) uint32_t x_slices[8][kSliceWords];
+    // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
+    // must not hold LDS for eight).
+    extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
+    uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -281,10 +287,10 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) park_piece(x_slices[wave], i, lane, pieces[j][i]);
+            for (int i = 0; i < 4; ++i) park_piece(x_slice, i, lane, pieces[j][i]);
             if (t == j) {
 #pragma unroll
-                for (int s = 0; s < kSlices; ++s) chunk_from_slice(x[set][s], x_slices[wave], s * 16 + block);
+                for (int s = 0; s < kSlices; ++s) chunk_from_slice(x[set][s], x_slice, s * 16 + block);
             }
         }
     }
@@ -409,20 +415,22 @@ template <int SETS, int ROWS>
 void launch_blocks(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
+    const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
     if (a.zeros)
-        hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS>), grid, block, slices, stream, a);
     else
-        hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS>), grid, block, slices, stream, a);
 }
 
 template <int MT, int ROWS>
 void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
+    const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
     if (a.zeros)
-        hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS>), grid, block, slices, stream, a);
     else
-        hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS>), grid, block, slices, stream, a);
 }
 
 template <int ROWS>
