@@ -152,6 +152,20 @@ int mk_fwht(const void *source, int source_dtype, void *target, int target_dtype
 int mk_basis_mix(const float *source, float *target, const float *basis, long long rows, int order,
                  int power, int transpose, const float *signs_after, void *stream);
 
+/* The blocked transform of a width order * power (power a power of two) in one launch:
+ * every row [order, power] of `source` is multiplied by signs_before (NULL or
+ * [order * power] floats), each block goes through the Walsh-Hadamard stages of mk_fwht
+ * and is multiplied by `scale`, the blocks are mixed as in mk_basis_mix, and the result
+ * times signs_after is written to `target` in target_dtype.  Results equal mk_fwht
+ * followed by mk_basis_mix bit for bit.  Returns MK_ERR_UNSUPPORTED when order * power
+ * values do not fit one workgroup (order > 96, power < 32, or more than 160 KB of LDS);
+ * callers then use the two calls.
+ * Replaces: quantization/operations/orthogonal_transforms.py:87-109 (structured_transform)
+ * and the rotate_inputs hook of conversion/model_transforms.py:116-128 for blocked widths. */
+int mk_rotate_blocks(const void *source, int source_dtype, void *target, int target_dtype, long long rows,
+                     int order, int power, const float *basis, int transpose, const float *signs_before,
+                     const float *signs_after, float scale, void *stream);
+
 /* Error-feedback sweep over columns [tile_start, tile_start + tile_width) of every row:
  * target = original + correction; the nearest grid value (as in mk_scalar_encode, with the
  * table's nearest entry taken as the lowest index of the least distance) times scale plus

@@ -38,20 +38,33 @@ struct FwhtArgs {
     int sign_period;  // signs repeat every sign_period elements of the flattened tensor
     int rows_per_block, threads_per_row;
     float scale;
+    // Blocked transform in one launch: `rows` counts blocks of `width` values, every `order`
+    // of them form one outer row, which a workgroup transforms and then mixes with `basis`.
+    const float *basis;  // [order, order] row-major, or null
+    int order, transpose;
 };
+
+typedef float mk_mix16 __attribute__((ext_vector_type(16)));
 
 __host__ __device__ __forceinline__ int padded(int index) { return index + (index >> 4); }
 
 // E values per thread; stage group `g` covers index bits [base, base + log2 E).
-template <int E, bool VEC>
+// TILES > 0: the workgroup's rows are the `order` blocks of one outer row; after the last
+// stage they stay in LDS and are multiplied by the basis (padded to TILES x 32 rows) on the
+// fp32 matrix cores, exactly as basis_mix_mfma_kernel does from global memory.  The
+// workgroup is then a whole number of wavefronts; threads beyond the rows' share only take
+// part in that product.
+template <int E, bool VEC, int TILES>
 __global__ void __launch_bounds__(kMaxThreads) fwht_kernel(const FwhtArgs a) {
     extern __shared__ float tile[];
     constexpr int kLogE = E == 1 ? 0 : E == 2 ? 1 : E == 4 ? 2 : E == 8 ? 3 : E == 16 ? 4 : 5;
     const int threads_per_row = a.threads_per_row;
-    const int local_row = threadIdx.x / threads_per_row;
-    const int t = threadIdx.x - local_row * threads_per_row;
+    const int wanted_row = threadIdx.x / threads_per_row;
+    const bool working = wanted_row < a.rows_per_block;
+    const int local_row = working ? wanted_row : 0;
+    const int t = threadIdx.x - wanted_row * threads_per_row;
     const long long row = static_cast<long long>(blockIdx.x) * a.rows_per_block + local_row;
-    const bool active = row < a.rows;
+    const bool active = working && row < a.rows;
     float *mine = tile + local_row * padded(a.width);
     const size_t row_base = static_cast<size_t>(active ? row : 0) * a.width;
     const int sign_base = a.sign_period ? static_cast<int>(row_base % static_cast<size_t>(a.sign_period)) : 0;
@@ -138,7 +151,12 @@ __global__ void __launch_bounds__(kMaxThreads) fwht_kernel(const FwhtArgs a) {
         }
         done = base + kLogE;
         if (done >= a.log_width) {
-            if (active) {
+            if constexpr (TILES > 0) {
+                if (working) {
+#pragma unroll
+                    for (int j = 0; j < E; ++j) mine[padded(origin | (j << base))] = v[j] * a.scale;
+                }
+            } else if (active) {
 #pragma unroll
                 for (int j = 0; j < E; ++j) {
                     const int index = origin | (j << base);
@@ -149,25 +167,92 @@ __global__ void __launch_bounds__(kMaxThreads) fwht_kernel(const FwhtArgs a) {
             }
             break;
         }
+        if (working) {
 #pragma unroll
-        for (int j = 0; j < E; ++j) mine[padded(origin | (j << base))] = v[j];
+            for (int j = 0; j < E; ++j) mine[padded(origin | (j << base))] = v[j];
+        }
         __syncthreads();
+    }
+
+    if constexpr (TILES > 0) {
+        // target[f', p] = sum_f mix[f', f] * block f [p] over ascending f from zero; a wavefront
+        // owns 32 adjacent p at a time, lanes 0..31 reading block f and lanes 32..63 block f + 1.
+        __syncthreads();
+        constexpr int kMaxPairs = TILES * 16;
+        const int lane = threadIdx.x & 63;
+        const int half = lane >> 5, within = lane & 31;
+        const int pairs = (a.order + 1) >> 1;
+        float left[TILES][kMaxPairs];  // left[tile][q]: mix[32 tile + within][2 q + half]
+#pragma unroll
+        for (int o = 0; o < TILES; ++o)
+#pragma unroll
+            for (int q = 0; q < kMaxPairs; ++q) {
+                const int out = 32 * o + within, in = 2 * q + half;
+                const bool inside = out < a.order && in < a.order;
+                const int index = a.transpose ? in * a.order + out : out * a.order + in;
+                left[o][q] = inside ? a.basis[inside ? index : 0] : 0.0f;
+            }
+        const int row_words = padded(a.width);
+        const size_t outer_base = static_cast<size_t>(blockIdx.x) * a.order * a.width;
+        for (int first = (threadIdx.x >> 6) * 32; first < a.width; first += (blockDim.x >> 6) * 32) {
+            const int p = first + within;
+            float right[kMaxPairs];
+#pragma unroll
+            for (int q = 0; q < kMaxPairs; ++q) {
+                const int in = 2 * q + half;
+                const bool inside = q < pairs && in < a.order;
+                const float held = tile[(inside ? in : 0) * row_words + padded(p)];
+                right[q] = inside ? held : 0.0f;
+            }
+#pragma unroll
+            for (int o = 0; o < TILES; ++o) {
+                mk_mix16 sums;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sums[r] = 0.0f;
+#pragma unroll
+                for (int q = 0; q < kMaxPairs; ++q)
+                    if (q < pairs) sums = __builtin_amdgcn_mfma_f32_32x32x2f32(left[o][q], right[q], sums, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int out = 32 * o + (r >> 2) * 8 + half * 4 + (r & 3);
+                    if (out < a.order) {
+                        float value = sums[r];
+                        if (a.signs_after) value *= a.signs_after[out * a.width + p];
+                        mk_store_from_float(a.target, outer_base + static_cast<size_t>(out) * a.width + p, a.target_dtype, value);
+                    }
+                }
+            }
+        }
     }
 }
 
-template <int E, bool VEC>
+template <int E, bool VEC, int TILES = 0>
 int launch_fwht_as(const FwhtArgs &a, int threads, size_t lds, hipStream_t stream) {
     static size_t allowed = 48 * 1024;  // raised once per instantiation when a row needs more
     if (lds > allowed) {
-        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwht_kernel<E, VEC>),
+        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwht_kernel<E, VEC, TILES>),
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (status != hipSuccess)
             return mk_fail(MK_ERR_HIP, "mk_fwht: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(status));
         allowed = 160 * 1024;
     }
     const long long blocks = (a.rows + a.rows_per_block - 1) / a.rows_per_block;
-    hipLaunchKernelGGL((fwht_kernel<E, VEC>), dim3(static_cast<unsigned>(blocks)), dim3(threads), lds, stream, a);
+    hipLaunchKernelGGL((fwht_kernel<E, VEC, TILES>), dim3(static_cast<unsigned>(blocks)), dim3(threads), lds, stream, a);
     return MK_OK;
+}
+
+// The blocked transform in one launch: a workgroup per outer row.  Returns MK_OK after a
+// launch, -1 when the shape does not fit one workgroup (the caller then uses two launches).
+template <int E, int TILES>
+int launch_blocked(FwhtArgs a, hipStream_t stream) {
+    a.threads_per_row = a.width / E;
+    a.rows_per_block = a.order;
+    const int threads = (a.order * a.threads_per_row + 63) / 64 * 64;
+    const size_t lds = static_cast<size_t>(a.order) * padded(a.width) * sizeof(float);
+    if (threads > kMaxThreads || lds > 160 * 1024) return -1;
+    const auto aligned = [](const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15u) == 0; };
+    if (aligned(a.source) && aligned(a.signs_before)) return launch_fwht_as<E, true, TILES>(a, threads, lds, stream);
+    return launch_fwht_as<E, false, TILES>(a, threads, lds, stream);
 }
 
 template <int E>
@@ -228,8 +313,6 @@ __global__ void __launch_bounds__(256) basis_mix_kernel(const MixArgs a) {
 // lanes 0..31 reading 32 adjacent p of block f and lanes 32..63 of block f + 1, so no LDS is
 // involved.  v_mfma_f32_32x32x2_f32 accumulates over ascending f from zero, which equals
 // the fused multiply-add chain of basis_mix_kernel bit for bit.
-typedef float mk_mix16 __attribute__((ext_vector_type(16)));
-
 template <int TILES>
 __global__ void __launch_bounds__(256) basis_mix_mfma_kernel(const MixArgs a) {
     constexpr int kMaxPairs = TILES * 16;  // k-pairs of a basis padded to TILES * 32
@@ -325,6 +408,43 @@ extern "C" int mk_fwht(const void *source, int source_dtype, void *target, int t
     else status = launch_fwht<1>(a, stream);
     if (status) return status;
     MK_LAUNCH_CHECK("mk_fwht");
+    return MK_OK;
+}
+
+extern "C" int mk_rotate_blocks(const void *source, int source_dtype, void *target, int target_dtype, long long rows,
+                                int order, int power, const float *basis, int transpose, const float *signs_before,
+                                const float *signs_after, float scale, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(rows >= 0 && order >= 1, MK_ERR_INVALID, "mk_rotate_blocks: sizes must be positive");
+    MK_REQUIRE(power >= 1 && (power & (power - 1)) == 0, MK_ERR_INVALID,
+               "mk_rotate_blocks: the block width must be a power of two (got %d)", power);
+    MK_REQUIRE(order <= 96 && power >= 32 && power <= 32768, MK_ERR_UNSUPPORTED,
+               "mk_rotate_blocks: %d blocks of %d values do not fit one workgroup", order, power);
+    if (rows == 0) return MK_OK;
+    MK_REQUIRE(source && target && basis, MK_ERR_INVALID, "mk_rotate_blocks: null tensor pointer");
+    MK_REQUIRE(source != target, MK_ERR_INVALID, "mk_rotate_blocks: source and target must not alias");
+    MK_REQUIRE(mk_dtype_valid(source_dtype) && mk_dtype_valid(target_dtype), MK_ERR_INVALID,
+               "mk_rotate_blocks: unknown dtype code");
+    MK_REQUIRE(rows < (1ll << 31) / order, MK_ERR_INVALID, "mk_rotate_blocks: too many rows");
+    FwhtArgs a{};
+    a.source = source; a.target = target; a.signs_before = signs_before; a.signs_after = signs_after;
+    a.rows = rows * order; a.width = power; a.source_dtype = source_dtype; a.target_dtype = target_dtype;
+    a.sign_period = (signs_before || signs_after) ? order * power : 0; a.scale = scale;
+    a.basis = basis; a.order = order; a.transpose = transpose;
+    a.log_width = 0;
+    while ((1 << a.log_width) < power) ++a.log_width;
+    int status = -1;
+    if (order * (power / 16) <= kMaxThreads) {
+        status = order <= 32 ? launch_blocked<16, 1>(a, stream)
+                             : order <= 64 ? launch_blocked<16, 2>(a, stream) : launch_blocked<16, 3>(a, stream);
+    } else if (order * (power / 32) <= kMaxThreads) {
+        status = order <= 32 ? launch_blocked<32, 1>(a, stream)
+                             : order <= 64 ? launch_blocked<32, 2>(a, stream) : launch_blocked<32, 3>(a, stream);
+    }
+    if (status < 0)
+        return mk_fail(MK_ERR_UNSUPPORTED, "mk_rotate_blocks: %d blocks of %d values do not fit one workgroup", order, power);
+    if (status) return status;
+    MK_LAUNCH_CHECK("mk_rotate_blocks");
     return MK_OK;
 }
 

@@ -76,3 +76,48 @@ def mix_blocks(value: Tensor, basis: Tensor, *, transpose: bool, signs_after: Te
         native.pointer(signs_after), native.current_stream(device),
     ))
     return output
+
+
+MAXIMUM_FUSED_ORDER = 96      # basis rows the one-launch blocked transform handles
+MAXIMUM_FUSED_LDS = 160 * 1024
+
+
+def fits_one_launch(order: int, power: int) -> bool:
+    """Whether ``rotate_blocks`` takes ``order`` blocks of ``power`` values (one workgroup holds them)."""
+    if order > MAXIMUM_FUSED_ORDER or power < 32 or power & (power - 1):
+        return False
+    padded = power + (power >> 4)
+    if order * padded * 4 > MAXIMUM_FUSED_LDS:
+        return False
+    return order * (power // 16) <= 1024 or order * (power // 32) <= 1024
+
+
+def rotate_blocks(
+    value: Tensor,
+    basis: Tensor,
+    *,
+    transpose: bool,
+    signs_before: Tensor | None = None,
+    signs_after: Tensor | None = None,
+    normalize: bool = True,
+) -> Tensor:
+    """``transform`` of every block of a ``[..., order, power]`` tensor followed by ``mix_blocks``,
+    in one launch and in ``value``'s dtype; bit-identical to the two calls."""
+    device = native.require_device(value, basis, signs_before, signs_after)
+    if value.dim() < 2 or not value.is_contiguous():
+        raise ValueError("rotate_blocks requires a contiguous tensor [..., order, power]")
+    order, power = value.shape[-2], value.shape[-1]
+    if basis.shape != (order, order) or basis.dtype != torch.float32 or not basis.is_contiguous():
+        raise ValueError("basis must be a contiguous FP32 [order, order] matrix")
+    for signs in (signs_before, signs_after):
+        if signs is not None and (signs.dtype != torch.float32 or not signs.is_contiguous()
+                                  or signs.numel() != order * power):
+            raise ValueError("sign vectors must be contiguous FP32 with order * power entries")
+    output = torch.empty_like(value)
+    rows = value.numel() // (order * power)
+    native.check(native.library().mk_rotate_blocks(
+        value.data_ptr(), native.dtype_code(value), output.data_ptr(), native.dtype_code(output), rows,
+        order, power, basis.data_ptr(), int(transpose), native.pointer(signs_before),
+        native.pointer(signs_after), normaliser(power) if normalize else 1.0, native.current_stream(device),
+    ))
+    return output

@@ -104,6 +104,40 @@ def test_blocked_transform_matches_oracle(width):
     np.testing.assert_allclose(host(back), transforms.randomized(expected, signs, inverse=True), rtol=1e-5, atol=2e-5)
 
 
+@pytest.mark.parametrize("width", [896, 4864, 11008, 14336])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_one_launch_blocked_transform_equals_the_two_calls(width, dtype):
+    """`mk_rotate_blocks` against `mk_fwht` + `mk_basis_mix` (+ the cast), bit for bit, forward
+    with the signs in front and inverse with the signs behind; 5 rows and 1 row."""
+    from mlkit_amd.kernels import hadamard
+
+    order, power, basis = transforms.transform_factor(width)
+    assert hadamard.fits_one_launch(order, power)
+    generator = torch.Generator(device="cuda").manual_seed(width)
+    signs = dev(transforms.deterministic_signs(width, seed=9))
+    for rows in (5, 1):
+        value = torch.randn((rows, order, power), device="cuda", generator=generator).to(dtype)
+        for inverse in (False, True):
+            before, after = (None, signs) if inverse else (signs, None)
+            staged = torch.empty(value.shape, device="cuda", dtype=torch.float32)
+            hadamard.transform(value, signs_before=before, out=staged)
+            expected = hadamard.mix_blocks(staged, dev(basis), transpose=inverse, signs_after=after).to(dtype)
+            result = hadamard.rotate_blocks(value, dev(basis), transpose=inverse, signs_before=before, signs_after=after)
+            assert result.dtype == dtype
+            assert torch.equal(result, expected)
+
+
+def test_one_launch_blocked_transform_declines_what_does_not_fit():
+    from mlkit_amd.kernels import hadamard
+
+    assert not hadamard.fits_one_launch(7, 16)       # blocks narrower than an MFMA tile
+    assert not hadamard.fits_one_launch(97, 64)      # basis beyond three MFMA row tiles
+    assert not hadamard.fits_one_launch(3, 32768)    # more than 160 KB of LDS
+    value = torch.zeros((2, 7, 16), device="cuda")
+    with pytest.raises(Exception, match="do not fit one workgroup"):
+        hadamard.rotate_blocks(value, torch.eye(7, device="cuda"), transpose=False)
+
+
 def test_weight_sized_rotation_keeps_norms():
     """4096 x 14336 fp32 along K as 7 x 2048 blocks (the literal blocked FWHT) and along
     4096: row norms are preserved and the transform is its own inverse."""
