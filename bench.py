@@ -196,6 +196,7 @@ def other_kernels(device: torch.device) -> dict:
     (`--kernels`); each entry carries its algorithmic bytes or flops and the rate they give."""
     import mlkit_amd as mk
     from mlkit_amd.kernels import hadamard, packed_linear, scalar_decode, scalar_encode
+    from mlkit_amd.quantization.transforms import OnlineRotation
     from mlkit_amd.quantization.core import Ctx
 
     out = {}
@@ -251,6 +252,8 @@ def other_kernels(device: torch.device) -> dict:
         for width in (4096, 14336):
             x = torch.randn((samples, width), device=device, generator=generator).half()
             out[f"rht activations M={samples} K={width} fp16"] = {"us": _time(lambda: mk.rht(x, seed=3), 50) * 1e3}
+            hook = OnlineRotation(3)
+            out[f"online rotation hook M={samples} K={width} fp16"] = {"us": _time(lambda: hook(x), 50) * 1e3}
 
     # other matvec shapes and codecs, M = 1 and 8: HIP-graph launches through the C ABI over
     # enough distinct weight copies (> 512 MB) that the Infinity Cache cannot serve them

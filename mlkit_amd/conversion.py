@@ -18,7 +18,7 @@ from torch import nn
 
 from mlkit_amd.models import Model
 from mlkit_amd.quantization.core import layer_seed
-from mlkit_amd.quantization.transforms import rht
+from mlkit_amd.quantization.transforms import OnlineRotation, rht
 
 ROTATED_LAYER_NAMES = ("o_proj", "down_proj")
 
@@ -33,11 +33,11 @@ def install_transform(model: nn.Module, descriptor: dict[str, Any]) -> None:
     """Attach the online half of a recorded transform to the layer it names."""
     if descriptor["kind"] != "rotation":
         raise ValueError(f"unknown model transform {descriptor['kind']!r}")
-    seed = descriptor["seed"]
+    rotation = OnlineRotation(descriptor["seed"])
 
     def rotate_inputs(layer: nn.Module, arguments: tuple) -> tuple:
         # fp16 / bf16 inputs are transformed in fp32 inside the kernel and rounded once
-        return (rht(arguments[0], seed=seed), *arguments[1:])
+        return (rotation(arguments[0]), *arguments[1:])
 
     model.get_submodule(descriptor["name"]).register_forward_pre_hook(rotate_inputs)
 

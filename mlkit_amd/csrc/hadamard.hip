@@ -69,6 +69,12 @@ __global__ void __launch_bounds__(kMaxThreads) fwht_kernel(const FwhtArgs a) {
     const size_t row_base = static_cast<size_t>(active ? row : 0) * a.width;
     const int sign_base = a.sign_period ? static_cast<int>(row_base % static_cast<size_t>(a.sign_period)) : 0;
 
+    // The basis goes to LDS behind the rows (read back as the left MFMA operand).
+    float *basis_tile = tile + a.rows_per_block * padded(a.width);
+    if constexpr (TILES > 0) {
+        for (int i = threadIdx.x; i < a.order * a.order; i += blockDim.x) basis_tile[i] = a.basis[i];
+    }
+
     // HBM -> LDS.  All loads of a thread are issued before any is used; with VEC a thread
     // reads groups of four adjacent elements (16 bytes of fp32, 8 of fp16 / bf16).
     if (active) {
@@ -190,7 +196,8 @@ __global__ void __launch_bounds__(kMaxThreads) fwht_kernel(const FwhtArgs a) {
                 const int out = 32 * o + within, in = 2 * q + half;
                 const bool inside = out < a.order && in < a.order;
                 const int index = a.transpose ? in * a.order + out : out * a.order + in;
-                left[o][q] = inside ? a.basis[inside ? index : 0] : 0.0f;
+                const float held = basis_tile[inside ? index : 0];
+                left[o][q] = inside ? held : 0.0f;
             }
         const int row_words = padded(a.width);
         const size_t outer_base = static_cast<size_t>(blockIdx.x) * a.order * a.width;
@@ -248,7 +255,7 @@ int launch_blocked(FwhtArgs a, hipStream_t stream) {
     a.threads_per_row = a.width / E;
     a.rows_per_block = a.order;
     const int threads = (a.order * a.threads_per_row + 63) / 64 * 64;
-    const size_t lds = static_cast<size_t>(a.order) * padded(a.width) * sizeof(float);
+    const size_t lds = (static_cast<size_t>(a.order) * padded(a.width) + static_cast<size_t>(a.order) * a.order) * sizeof(float);
     if (threads > kMaxThreads || lds > 160 * 1024) return -1;
     const auto aligned = [](const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15u) == 0; };
     if (aligned(a.source) && aligned(a.signs_before)) return launch_fwht_as<E, true, TILES>(a, threads, lds, stream);

@@ -87,7 +87,7 @@ def fits_one_launch(order: int, power: int) -> bool:
     if order > MAXIMUM_FUSED_ORDER or power < 32 or power & (power - 1):
         return False
     padded = power + (power >> 4)
-    if order * padded * 4 > MAXIMUM_FUSED_LDS:
+    if (order * padded + order * order) * 4 > MAXIMUM_FUSED_LDS:
         return False
     return order * (power // 16) <= 1024 or order * (power // 32) <= 1024
 

@@ -172,8 +172,81 @@ def random_signs(width: int, seed: int, device: torch.device | str, dtype: torch
 
 
 def randomized_transform(value: Tensor, *, seed: int = 0, inverse: bool = False) -> Tensor:
-    signs = random_signs(value.shape[-1], seed, value.device, value.dtype)
+    # the cached FP32 vector itself: +-1 is exact in every dtype and the kernels take FP32 signs
+    signs = _cached_signs(value.shape[-1], seed, value.device)
+    if not _on_kernel(value):
+        signs = signs.to(value.dtype)
     return rotate(value, inverse=inverse, signs=signs)
+
+
+class OnlineRotation:
+    """``rht(value, seed=seed)`` for the forward pre-hook of a rotated layer: the same result
+    with the per-call work reduced to one allocation and one library call (the launch
+    arguments of a width, device and dtype are prepared once)."""
+
+    def __init__(self, seed: int):
+        self.seed = seed
+        self._plans: dict = {}
+
+    def __call__(self, value: Tensor) -> Tensor:
+        key = (value.shape[-1], value.device, value.dtype)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = self._plans[key] = self._prepare(value)
+        return plan(value)
+
+    def _prepare(self, value: Tensor):
+        seed = self.seed
+        width = value.shape[-1]
+        order, power, basis = transform_factor(width)
+
+        def general(tensor: Tensor) -> Tensor:
+            return randomized_transform(tensor, seed=seed)
+
+        if not (_on_kernel(value) and power <= MAXIMUM_KERNEL_WIDTH and order <= MAXIMUM_KERNEL_ORDER):
+            return general
+        from mlkit_amd import native
+        from mlkit_amd.kernels import hadamard as kernel
+
+        device = value.device
+        signs = _cached_signs(width, seed, device)
+        library = native.library()
+        code = native.dtype_code(value)
+        sign_pointer = signs.data_ptr()
+        if basis is None:
+            scale = kernel.normaliser(width)
+            launch = library.mk_fwht
+
+            def whole(tensor: Tensor) -> Tensor:
+                if not tensor.is_contiguous():
+                    tensor = tensor.contiguous()
+                output = torch.empty_like(tensor)
+                native.check(launch(tensor.data_ptr(), code, output.data_ptr(), code, tensor.numel() // width, width,
+                                    sign_pointer, None, width, scale, torch.cuda.current_stream(device).cuda_stream))
+                return output
+
+            whole.keeps = (signs,)
+            return whole
+        if not kernel.fits_one_launch(order, power):
+            return general
+        basis_on_device = _basis_on(width, device)
+        basis_pointer = basis_on_device.data_ptr()
+        scale = kernel.normaliser(power)
+        launch = library.mk_rotate_blocks
+
+        def blocked(tensor: Tensor) -> Tensor:
+            rows = tensor.numel() // width
+            if rows > ONE_LAUNCH_ROWS:
+                return general(tensor)
+            if not tensor.is_contiguous():
+                tensor = tensor.contiguous()
+            output = torch.empty_like(tensor)
+            native.check(launch(tensor.data_ptr(), code, output.data_ptr(), code, rows, order, power, basis_pointer, 0,
+                                sign_pointer, None, scale, torch.cuda.current_stream(device).cuda_stream))
+            return output
+
+        blocked.keeps = (signs, basis_on_device)
+        return blocked
 
 
 def rht(value: Tensor, *, seed: int = 0, inverse: bool = False) -> Tensor:

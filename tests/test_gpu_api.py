@@ -572,3 +572,24 @@ def test_incoherent_quantization_on_device_and_checkpoint(tmp_path):
     restored = mk.load_checkpoint(tmp_path / "basis", model=lambda: nn.Linear(4864, 896, bias=False))
     torch.testing.assert_close(restored.module.weight, converted.module.weight, rtol=0, atol=0)
     assert restored.quantized[""].params["right_seed"] == q.params["right_seed"]
+
+
+@pytest.mark.parametrize("width", [4096, 14336, 896, 12])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_online_rotation_hook_equals_rht(width, dtype):
+    """The prepared launch of the forward pre-hook against ``mk.rht`` on the same input:
+    equal bit for bit, for one row, a batch, more rows than the one-launch kernel takes,
+    and a non-contiguous view."""
+    from mlkit_amd.quantization.transforms import OnlineRotation
+
+    rotation = OnlineRotation(seed=11)
+    generator = torch.Generator(device="cuda").manual_seed(width)
+    for rows in (1, 8, 300):
+        value = torch.randn((rows, width), device="cuda", generator=generator).to(dtype)
+        assert torch.equal(rotation(value), mk.rht(value, seed=11))
+    wide = torch.randn((4, 2 * width), device="cuda", generator=generator).to(dtype)
+    view = wide[:, :width]
+    assert torch.equal(rotation(view), mk.rht(view, seed=11))
+    batched = torch.randn((2, 3, width), device="cuda", generator=generator).to(dtype)
+    assert torch.equal(rotation(batched), mk.rht(batched, seed=11))
+    assert rotation(batched).shape == batched.shape
