@@ -25,7 +25,7 @@ WEIGHT_BYTES = CODE_BYTES + SCALE_BYTES
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
 # profiles/packed_matvec_stream4_int4_g128_4096x14336_m1.md), M=1.
-MEASURED_TRAFFIC_BYTES = 30_635_000
+MEASURED_TRAFFIC_BYTES = 30_641_000
 
 
 def algorithmic_bytes(samples: int) -> int:

@@ -57,18 +57,32 @@ __global__ void packed_decode_kernel(const DecodeArgs a) {
 
 
 // One thread per chunk of 32 codes.  The value table is staged in LDS.
-template <int BITS>
+//
+// A lane's 32 outputs are 64 bytes (128 of fp32): stored directly, a wavefront instruction
+// would write 16 bytes at a stride of 64 and touch 64 cache lines.  The lanes of a
+// wavefront therefore exchange their 16-byte pieces through LDS (each chunk's pieces one
+// piece apart from the next chunk's, so both directions avoid bank conflicts) and every
+// store instruction writes 1 KB of adjacent bytes.  A wavefront's 64 chunks are adjacent
+// in the row-major output because rows are whole chunks.
+template <int BITS, int PIECES>
 __global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeArgs a) {
     __shared__ float table[1 << BITS];
+    __shared__ mk_u32x4 exchange[4][64 * (PIECES + 1)];
     if (!a.uniform) {
         for (int i = threadIdx.x; i < (1 << BITS); i += blockDim.x) table[i] = i < a.n_values ? a.values[i] : 0.0f;
         __syncthreads();
     }
+    const int lane = threadIdx.x & 63;
+    mk_u32x4 *mine = exchange[threadIdx.x >> 6];
     const int row_chunks = a.width / mk_matvec::kChunkCodes;
     const size_t total = static_cast<size_t>(a.rows) * row_chunks;
     const bool one_slot = a.group % mk_matvec::kChunkCodes == 0 || a.group >= a.width;
-    for (size_t chunk = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; chunk < total;
-         chunk += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    // The trip count is uniform within a wavefront: lanes past the end repeat the last chunk
+    // and store nothing.
+    for (size_t first_chunk = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) & ~static_cast<size_t>(63);
+         first_chunk < total; first_chunk += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const size_t wanted = first_chunk + lane;
+        const size_t chunk = wanted < total ? wanted : total - 1;
         const size_t row = chunk / row_chunks;
         const int first = static_cast<int>(chunk - row * row_chunks) * mk_matvec::kChunkCodes;
         mk_matvec::CodeChunk<BITS> codes;
@@ -91,30 +105,34 @@ __global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeA
             if (a.zeros) weight = __fadd_rn(weight, zero);
             out[k] = weight;
         }
-        const size_t base = row * a.width + first;
-        if (a.out_dtype == MK_F32) {
-            float4 *target = reinterpret_cast<float4 *>(static_cast<float *>(a.out) + base);
 #pragma unroll
-            for (int q = 0; q < 8; ++q) target[q] = make_float4(out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]);
-        } else {
-            mk_u32x4 *target = reinterpret_cast<mk_u32x4 *>(static_cast<uint16_t *>(a.out) + base);
+        for (int q = 0; q < PIECES; ++q) {
+            mk_u32x4 piece;
+            if constexpr (PIECES == 8) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                mk_u32x4 packed4;
+                for (int h = 0; h < 4; ++h) piece[h] = __float_as_uint(out[4 * q + h]);
+            } else {
 #pragma unroll
                 for (int h = 0; h < 4; ++h) {
                     const float low = out[8 * q + 2 * h], high = out[8 * q + 2 * h + 1];
-                    uint32_t pair;
                     if (a.out_dtype == MK_F16) {
                         const mk_h2 halves = {static_cast<_Float16>(low), static_cast<_Float16>(high)};
-                        pair = __builtin_bit_cast(uint32_t, halves);
+                        piece[h] = __builtin_bit_cast(uint32_t, halves);
                     } else {
-                        pair = static_cast<uint32_t>(mk_float_to_bf16(low)) | (static_cast<uint32_t>(mk_float_to_bf16(high)) << 16);
+                        piece[h] = static_cast<uint32_t>(mk_float_to_bf16(low)) | (static_cast<uint32_t>(mk_float_to_bf16(high)) << 16);
                     }
-                    packed4[h] = pair;
                 }
-                target[q] = packed4;
             }
+            mine[lane * (PIECES + 1) + q] = piece;
+        }
+        // LDS operations of a wavefront complete in order: no barrier between the two loops.
+        mk_u32x4 *target = static_cast<mk_u32x4 *>(a.out) + first_chunk * PIECES;
+        const size_t pieces_left = (total - first_chunk) * PIECES;
+#pragma unroll
+        for (int q = 0; q < PIECES; ++q) {
+            const int index = q * 64 + lane;
+            const mk_u32x4 piece = mine[(index / PIECES) * (PIECES + 1) + index % PIECES];
+            if (static_cast<size_t>(index) < pieces_left) target[index] = piece;
         }
     }
 }
@@ -124,7 +142,10 @@ void launch_chunks(const DecodeArgs &a, hipStream_t stream) {
     const size_t chunks = static_cast<size_t>(a.rows) * (a.width / mk_matvec::kChunkCodes);
     size_t blocks = (chunks + 255) / 256;
     if (blocks > 256u * 64u) blocks = 256u * 64u;
-    hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+    if (a.out_dtype == MK_F32)
+        hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS, 8>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+    else
+        hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS, 4>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
 }
 
 }  // namespace
