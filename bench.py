@@ -54,7 +54,7 @@ class Launcher:
         self.function = native.library().mk_packed_matvec
         self.keep = (x, packed, scales, values, y, zeros)
         self.arguments = (
-            x.data_ptr(), native.MK_F16, packed.data_ptr(), scales.data_ptr(), native.MK_F16,
+            x.data_ptr(), native.dtype_code(x), packed.data_ptr(), scales.data_ptr(), native.dtype_code(scales),
             values.data_ptr(), values.numel(), None if zeros is None else zeros.data_ptr(), None, 0,
             y.data_ptr(), x.shape[0], rows, width, group, bits, int(uniform), grid_min, grid_step,
         )
@@ -257,7 +257,7 @@ def other_kernels(device: torch.device) -> dict:
 
     # other matvec shapes and codecs, M = 1 and 8: HIP-graph launches through the C ABI over
     # enough distinct weight copies (> 512 MB) that the Infinity Cache cannot serve them
-    def matvec(rows, width, group, bits, table, uniform, asym, label):
+    def matvec(rows, width, group, bits, table, uniform, asym, label, dtype=torch.float16):
         code_bytes = rows * width * bits // 8
         count = max(2, min(40, -(-(512 * 2**20) // code_bytes)))
         streams = [torch.randint(0, 256, (code_bytes,), dtype=torch.uint8, device=device, generator=generator)
@@ -265,8 +265,8 @@ def other_kernels(device: torch.device) -> dict:
         side = (torch.rand((rows, width // group), device=device, generator=generator) * 0.004 + 0.005).half()
         zeros = side.clone() if asym else None
         for samples in (1, 8):
-            x = torch.randn((samples, width), device=device, generator=generator).half()
-            y = torch.empty((samples, rows), device=device, dtype=torch.float16)
+            x = torch.randn((samples, width), device=device, generator=generator).to(dtype)
+            y = torch.empty((samples, rows), device=device, dtype=dtype)
             launchers = [Launcher(x, stream, side, table, y, zeros=zeros, rows=rows, width=width, group=group,
                                   bits=bits, uniform=uniform, grid_min=float(table[0]),
                                   grid_step=float(table[1] - table[0])) for stream in streams]
@@ -276,6 +276,7 @@ def other_kernels(device: torch.device) -> dict:
 
     nf4 = mk.NF4_VALUES.to(device)
     matvec(4096, 4096, 128, 4, values, True, True, "int4 asym g128")
+    matvec(ROWS, WIDTH, 128, 4, values, True, False, "int4 g128, bf16 activations", dtype=torch.bfloat16)
     matvec(ROWS, WIDTH, 64, 2, torch.arange(-2, 2, dtype=torch.float32, device=device), True, False, "int2 g64")
     matvec(ROWS, WIDTH, 64, 3, torch.arange(-4, 4, dtype=torch.float32, device=device), True, False, "int3 g64")
     matvec(ROWS, WIDTH, 64, 4, nf4, False, False, "nf4 g64")

@@ -70,7 +70,7 @@ struct Stream4Args {
 // Pair-table kernel (packed_matvec_pairs.hip): 2-, 3- and 4-bit codes of any scalar grid.
 bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype);
 int pairs_launch(const Stream4Args &a, hipStream_t stream);
-bool stream4_accepts(int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
+bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
 
 // ---------------------------------------------------------------------------------

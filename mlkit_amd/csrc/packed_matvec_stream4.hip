@@ -68,7 +68,8 @@ __device__ __forceinline__ void park_piece(uint32_t *slice, int i, int lane, mk_
     *reinterpret_cast<mk_u32x4 *>(slice + (16 * i + (lane >> 2)) * kChunkStrideWords + (lane & 3) * 4) = piece;
 }
 
-__device__ __forceinline__ void chunk_from_slice(XChunk<MK_F16> &x, const uint32_t *slice, int chunk_in_slice) {
+template <int XT>
+__device__ __forceinline__ void chunk_from_slice(XChunk<XT> &x, const uint32_t *slice, int chunk_in_slice) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const mk_u32x4 v = *reinterpret_cast<const mk_u32x4 *>(slice + chunk_in_slice * kChunkStrideWords + 4 * i);
@@ -79,7 +80,72 @@ __device__ __forceinline__ void chunk_from_slice(XChunk<MK_F16> &x, const uint32
     }
 }
 
-template <int MT, bool HAS_ZERO, int ROWS>
+// ---- bf16 activations ----------------------------------------------------------------------
+//
+// bf16 has seven mantissa bits, so only the low nibble of each half fits the magic-number
+// insertion (128 + c); every pair of codes needs its own shift: 3 shifts, 4 v_bfi and 4
+// v_dot2_f32_bf16 per eight codes, against 1 + 4 + 4 for fp16.  Pairs are (x0,x4) (x1,x5)
+// (x2,x6) (x3,x7) of every eight codes, unscaled.
+
+// Re-pairs a chunk in place; returns the sum of its activations.
+__device__ __forceinline__ float pair_for_nibbles_bf16(XChunk<MK_BF16> &x) {
+    const uint32_t ones = 0x3f803f80u;
+    float total = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const uint32_t p0 = x.r[4 * g + 0], p1 = x.r[4 * g + 1];
+        const uint32_t p2 = x.r[4 * g + 2], p3 = x.r[4 * g + 3];
+        x.r[4 * g + 0] = __builtin_amdgcn_perm(p2, p0, 0x05040100u);
+        x.r[4 * g + 1] = __builtin_amdgcn_perm(p2, p0, 0x07060302u);
+        x.r[4 * g + 2] = __builtin_amdgcn_perm(p3, p1, 0x05040100u);
+        x.r[4 * g + 3] = __builtin_amdgcn_perm(p3, p1, 0x07060302u);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            total = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mk_bf2, ones), __builtin_bit_cast(mk_bf2, x.r[4 * g + i]), total, false);
+    }
+    return total;
+}
+
+// sum over the chunk of (128 + code_k) x_k for MT samples.
+template <int MT>
+__device__ __forceinline__ void chunk_dot_bf16(const CodeChunk<4> &codes, const XChunk<MK_BF16> (&x)[MT], float (&dot)[MT]) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) dot[m] = 0.0f;
+    uint32_t magic = 0x43004300u;
+    asm volatile("" : "+v"(magic));
+    auto insert = [&](uint32_t word) __attribute__((always_inline)) {
+        return __builtin_bit_cast(mk_bf2, (word & 0x000f000fu) | (magic & ~0x000f000fu));
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w = codes.w[i];
+        const mk_bf2 h0 = insert(w), h1 = insert(w >> 4), h2 = insert(w >> 8), h3 = insert(w >> 12);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            float d = dot[m];
+            d = __builtin_amdgcn_fdot2_f32_bf16(h0, __builtin_bit_cast(mk_bf2, x[m].r[4 * i + 0]), d, false);
+            d = __builtin_amdgcn_fdot2_f32_bf16(h1, __builtin_bit_cast(mk_bf2, x[m].r[4 * i + 1]), d, false);
+            d = __builtin_amdgcn_fdot2_f32_bf16(h2, __builtin_bit_cast(mk_bf2, x[m].r[4 * i + 2]), d, false);
+            d = __builtin_amdgcn_fdot2_f32_bf16(h3, __builtin_bit_cast(mk_bf2, x[m].r[4 * i + 3]), d, false);
+            dot[m] = d;
+        }
+    }
+}
+
+// A 16-bit scale or offset as fp32; `dtype` (MK_F16 or MK_BF16) is uniform per launch.
+__device__ __forceinline__ float side_as_float(uint16_t raw, int dtype) {
+    const float from_half = static_cast<float>(__builtin_bit_cast(_Float16, raw));
+    const float from_brain = __uint_as_float(static_cast<uint32_t>(raw) << 16);
+    return dtype == MK_F16 ? from_half : from_brain;
+}
+
+template <int XT>
+__device__ __forceinline__ void store_output(void *y, size_t index, float value) {
+    if constexpr (XT == MK_F16) static_cast<_Float16 *>(y)[index] = static_cast<_Float16>(value);
+    else static_cast<uint16_t *>(y)[index] = mk_float_to_bf16(value);
+}
+
+template <int MT, bool HAS_ZERO, int ROWS, int XT>
 __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     __shared__ float partials[64 * 8];  // [row sum][wavefront]
     // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
@@ -141,7 +207,7 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
 
     // Each lane's chunk of every sample, through the wavefront's LDS buffer (LDS operations
     // of a wavefront complete in order, so no barrier is needed).
-    XChunk<MK_F16> x[MT];
+    XChunk<XT> x[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
 #pragma unroll
@@ -156,7 +222,13 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
         const uint32_t keep = in_row && sample_base + m < a.samples ? 0xffffffffu : 0u;
 #pragma unroll
         for (int i = 0; i < 16; ++i) x[m].r[i] &= keep;
-        const float code_free = pair_for_nibbles(x[m], &x_sum[m]);
+        float code_free;
+        if constexpr (XT == MK_F16) {
+            code_free = pair_for_nibbles(x[m], &x_sum[m]);
+        } else {
+            x_sum[m] = pair_for_nibbles_bf16(x[m]);
+            code_free = 128.0f * x_sum[m];
+        }
         grid_term[m] = a.grid_min * x_sum[m] - a.grid_step * code_free;
     }
 
@@ -167,16 +239,17 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
         for (int j = 0; j < kReduceRows; ++j) {
             const int r = pass * kReduceRows + j;
             float dot[MT];
-            chunk_dot<4, MK_F16, MT, true>(codes[r], x, nullptr, dot);
+            if constexpr (XT == MK_F16) chunk_dot<4, MK_F16, MT, true>(codes[r], x, nullptr, dot);
+            else chunk_dot_bf16<MT>(codes[r], x, dot);
             if (r + kStreamAhead < kStreamRows)
                 load_codes<4>(codes[r + kStreamAhead],
                               codes_base + static_cast<size_t>(r + kStreamAhead) * row_bytes + code_offset);
-            const float scale = static_cast<float>(__builtin_bit_cast(_Float16, scale_raw[r]));
+            const float scale = side_as_float(scale_raw[r], a.scale_dtype);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 float value = scale * __builtin_fmaf(a.grid_step, dot[m], grid_term[m]);
                 if constexpr (HAS_ZERO)
-                    value = __builtin_fmaf(static_cast<float>(__builtin_bit_cast(_Float16, zero_raw[r])), x_sum[m], value);
+                    value = __builtin_fmaf(side_as_float(zero_raw[r], a.scale_dtype), x_sum[m], value);
                 sums[j * MT + m] = value;
             }
             // Keeps the rows in arrival order and their temporaries short-lived.
@@ -197,7 +270,7 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
             const int sample = sample_base + m;
             if (sample < a.samples) {
                 if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
-                static_cast<_Float16 *>(a.y)[static_cast<size_t>(sample) * a.rows + row] = static_cast<_Float16>(total);
+                store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
             }
         }
     }
@@ -221,6 +294,7 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
 // and reach the multiply as DPP quad broadcasts.
 
 typedef _Float16 mk_h4 __attribute__((ext_vector_type(4)));
+typedef short mk_s4 __attribute__((ext_vector_type(4)));
 typedef float mk_f4 __attribute__((ext_vector_type(4)));
 
 template <int R>
@@ -228,7 +302,7 @@ __device__ __forceinline__ float quad_value(float value) {
     return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, value), R * 0x55, 0xf, 0xf, true));
 }
 
-template <int SETS, bool HAS_ZERO, int ROWS>
+template <int SETS, bool HAS_ZERO, int ROWS, int XT>
 __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a) {
     constexpr int kQuads = ROWS / 4;
     constexpr int kSlices = 4;                      // sub-slices of sixteen chunks per wavefront
@@ -273,7 +347,7 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     // Activations of sample t (and t + 4) for this lane's four chunks, 16 fp16 pairs each:
     // the wavefront reads each sample's slice coalesced and the four lanes in sixteen whose
     // sample it is pick their chunks out of LDS.
-    XChunk<MK_F16> x[SETS][kSlices];
+    XChunk<XT> x[SETS][kSlices];
 #pragma unroll
     for (int set = 0; set < SETS; ++set) {
         mk_u32x4 pieces[4][4];
@@ -323,7 +397,13 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
             const uint32_t keep = in_row[s] && sample_present ? 0xffffffffu : 0u;
 #pragma unroll
             for (int i = 0; i < 16; ++i) x[set][s].r[i] &= keep;
-            const float code_free = pair_for_nibbles(x[set][s], &x_sum[set][s]);
+            float code_free;
+            if constexpr (XT == MK_F16) {
+                code_free = pair_for_nibbles(x[set][s], &x_sum[set][s]);
+            } else {
+                x_sum[set][s] = pair_for_nibbles_bf16(x[set][s]);
+                code_free = 128.0f * x_sum[set][s];
+            }
             grid_term[set][s] = a.grid_min * x_sum[set][s] - a.grid_step * code_free;
         }
     }
@@ -334,14 +414,18 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
 #pragma unroll
         for (int j = 0; j < kSums; ++j) sums[set][j] = 0.0f;
 
-    uint32_t magic = 0x64006400u;
+    uint32_t magic = XT == MK_F16 ? 0x64006400u : 0x43004300u;
     asm volatile("" : "+v"(magic));
     auto insert = [&](uint32_t mask, uint32_t word) __attribute__((always_inline)) {
         return (word & mask) | (magic & ~mask);
     };
-    auto four = [](uint32_t low, uint32_t high) __attribute__((always_inline)) {
-        const mk_u32x2 both = {low, high};
-        return __builtin_bit_cast(mk_h4, both);
+    // One instruction: sixteen 4 x 4 x 4 blocks, four 16-bit values per lane and operand.
+    auto blocks = [](uint32_t a_low, uint32_t a_high, uint32_t b_low, uint32_t b_high, mk_f4 sum) __attribute__((always_inline)) {
+        const mk_u32x2 left = {a_low, a_high}, right = {b_low, b_high};
+        if constexpr (XT == MK_F16)
+            return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(mk_h4, left), __builtin_bit_cast(mk_h4, right), sum, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(mk_s4, left), __builtin_bit_cast(mk_s4, right), sum, 0, 0, 0);
     };
 
 #pragma unroll
@@ -353,23 +437,29 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t w = codes[step].w[i];
-            const uint32_t w8 = w >> 8;
-            const mk_h4 first = four(insert(0x000f000fu, w), insert(0x00f000f0u, w));     // codes 0, 4, 1, 5
-            const mk_h4 second = four(insert(0x000f000fu, w8), insert(0x00f000f0u, w8));  // codes 2, 6, 3, 7
+            uint32_t pair[4];  // codes (0, 4), (1, 5), (2, 6), (3, 7) as 16-bit floats
+            if constexpr (XT == MK_F16) {
+                const uint32_t w8 = w >> 8;
+                pair[0] = insert(0x000f000fu, w), pair[1] = insert(0x00f000f0u, w);
+                pair[2] = insert(0x000f000fu, w8), pair[3] = insert(0x00f000f0u, w8);
+            } else {
+                pair[0] = insert(0x000f000fu, w), pair[1] = insert(0x000f000fu, w >> 4);
+                pair[2] = insert(0x000f000fu, w >> 8), pair[3] = insert(0x000f000fu, w >> 12);
+            }
 #pragma unroll
             for (int set = 0; set < SETS; ++set) {
-                dot[set] = __builtin_amdgcn_mfma_f32_4x4x4f16(first, four(x[set][s].r[4 * i + 0], x[set][s].r[4 * i + 1]), dot[set], 0, 0, 0);
-                dot[set] = __builtin_amdgcn_mfma_f32_4x4x4f16(second, four(x[set][s].r[4 * i + 2], x[set][s].r[4 * i + 3]), dot[set], 0, 0, 0);
+                dot[set] = blocks(pair[0], pair[1], x[set][s].r[4 * i + 0], x[set][s].r[4 * i + 1], dot[set]);
+                dot[set] = blocks(pair[2], pair[3], x[set][s].r[4 * i + 2], x[set][s].r[4 * i + 3], dot[set]);
             }
         }
         if (step + kAhead < kSteps)
             load_codes<4>(codes[step + kAhead], codes_base + static_cast<size_t>(4 * ((step + kAhead) / kSlices)) * row_bytes +
                                                     code_offset[(step + kAhead) % kSlices]);
         // Row 4 q + r of the block: scale (and offset) come from lane r of the quad.
-        const float scale = static_cast<float>(__builtin_bit_cast(_Float16, scale_raw[step]));
+        const float scale = side_as_float(scale_raw[step], a.scale_dtype);
         const float scaled_step = scale * a.grid_step;
         float zero = 0.0f;
-        if constexpr (HAS_ZERO) zero = static_cast<float>(__builtin_bit_cast(_Float16, zero_raw[step]));
+        if constexpr (HAS_ZERO) zero = side_as_float(zero_raw[step], a.scale_dtype);
         auto add_row = [&](auto r) __attribute__((always_inline)) {
             constexpr int R = decltype(r)::value;
 #pragma unroll
@@ -406,7 +496,7 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
         const int sample = blockIdx.y * 4 * SETS + 4 * set + (index & 3);
         if (sample < a.samples) {
             if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
-            static_cast<_Float16 *>(a.y)[static_cast<size_t>(sample) * a.rows + row] = static_cast<_Float16>(total);
+            store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
         }
     }
 }
@@ -416,10 +506,17 @@ void launch_blocks(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
-    if (a.zeros)
-        hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS>), grid, block, slices, stream, a);
-    else
-        hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS>), grid, block, slices, stream, a);
+    if (a.x_dtype == MK_F16) {
+        if (a.zeros)
+            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS, MK_F16>), grid, block, slices, stream, a);
+        else
+            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS, MK_F16>), grid, block, slices, stream, a);
+    } else {
+        if (a.zeros)
+            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS, MK_BF16>), grid, block, slices, stream, a);
+        else
+            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS, MK_BF16>), grid, block, slices, stream, a);
+    }
 }
 
 template <int MT, int ROWS>
@@ -427,10 +524,17 @@ void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
-    if (a.zeros)
-        hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS>), grid, block, slices, stream, a);
-    else
-        hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS>), grid, block, slices, stream, a);
+    if (a.x_dtype == MK_F16) {
+        if (a.zeros)
+            hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS, MK_F16>), grid, block, slices, stream, a);
+        else
+            hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS, MK_F16>), grid, block, slices, stream, a);
+    } else {
+        if (a.zeros)
+            hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS, MK_BF16>), grid, block, slices, stream, a);
+        else
+            hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS, MK_BF16>), grid, block, slices, stream, a);
+    }
 }
 
 template <int ROWS>
@@ -452,9 +556,12 @@ int launch_rows(const Stream4Args &a, hipStream_t stream) {
 
 }  // namespace
 
-bool stream4_accepts(int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform) {
-    return bits == 4 && uniform && x_dtype == MK_F16 && scale_dtype == MK_F16 && width % kChunkCodes == 0 &&
-           width <= 16384 && (group % kChunkCodes == 0 || group >= width);
+bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform) {
+    const bool sixteen_bit_sides = scale_dtype == MK_F16 || scale_dtype == MK_BF16;
+    (void)samples;
+    const bool activations = x_dtype == MK_F16 || x_dtype == MK_BF16;
+    return bits == 4 && uniform && activations && sixteen_bit_sides && width % kChunkCodes == 0 && width <= 16384 &&
+           (group % kChunkCodes == 0 || group >= width);
 }
 
 // Multiplies the leading whole tiles of rows; returns the number of rows covered.

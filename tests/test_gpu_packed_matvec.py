@@ -103,6 +103,18 @@ def test_metric_shape_int4_g128_4096x14336_all_row_counts():
         check(run_matvec(layer, x), layer, x)
 
 
+@pytest.mark.parametrize("scale_dtype", [torch.float16, torch.bfloat16])
+def test_metric_shape_with_bf16_activations(scale_dtype):
+    """The same layer in a bf16 model: one and two rows take the bf16 variant of the INT4
+    streaming kernel (seven-bit mantissas: one nibble per half and shift), more rows the table kernel."""
+    weight = helpers.normal_weight(4096, 14336, seed=9)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True,
+                                    fmt="fp16" if scale_dtype == torch.float16 else "bf16")
+    for samples in (1, 2, 5):
+        x = helpers.activations(samples, 14336, seed=40 + samples, dtype=torch.bfloat16)
+        check(run_matvec(layer, x, scale_dtype=scale_dtype), layer, x, relative=8e-3)
+
+
 def test_down_projection_14336x4096():
     weight = helpers.normal_weight(14336, 4096, seed=11)
     layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
@@ -244,14 +256,14 @@ def test_packed_decode_full_layer_matches_matvec_input():
 @pytest.mark.parametrize("bits,values,integer", [(4, INT4, True), (2, scaling.int_values(2), True),
                                                  (3, scaling.int_values(3), True), (4, scaling.NF4_VALUES, False)])
 @pytest.mark.parametrize("scale_dtype", [torch.float16, torch.bfloat16])
-def test_bf16_activations_use_the_pair_table_kernel(bits, values, integer, scale_dtype):
+def test_bf16_activations(bits, values, integer, scale_dtype):
     """bf16 activations (bf16 outputs) with fp16 or bf16 scales; integer grids are exact in the
     bf16 table, so the error is the bf16 rounding of inputs and outputs only."""
     weight = helpers.normal_weight(48, 4096, seed=21, student_t=True)
     for asym in (False, True):
         layer = helpers.quantised_layer(weight, values, bits=bits, group=128, integer=integer, asym=asym,
                                         fmt="fp16" if scale_dtype == torch.float16 else "bf16")
-        for samples in (1, 8):
+        for samples in (1, 2, 8):
             x = helpers.activations(samples, 4096, seed=22 + samples, dtype=torch.bfloat16)
             check(run_matvec(layer, x, scale_dtype=scale_dtype), layer, x, relative=8e-3)
 
