@@ -17,6 +17,8 @@
 
 #include "packed_matvec_impl.h"
 
+#include <type_traits>
+
 namespace mk_matvec {
 
 namespace {
@@ -61,33 +63,16 @@ __device__ __forceinline__ uint32_t lookup_offset(const CodeChunk<BITS> &c, int 
     return (__builtin_amdgcn_alignbit(c.w[(word + 1) % BITS], c.w[word], shift) << kEntryShift) & mask;
 }
 
-template <int BITS, int MT, bool HAS_ZERO, int XT, int LOOKUP>
-__global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
+// Fills `table` (kEntries * LOOKUP / 2 dwords) with the grid's values as 16-bit floats: one
+// value, one pair or two pairs per entry.  The grid's values come first (one global load per
+// value), then every entry from them.  Ends before the caller's barrier.
+template <int BITS, int LOOKUP, int XT>
+__device__ __forceinline__ void fill_table(uint32_t *table, const Stream4Args &a) {
     constexpr int kLookup = LOOKUP;
-    constexpr int kPairAhead = rows_in_flight<BITS>();
     constexpr int kEntries = 1 << (kLookup * BITS);
     constexpr int kTableWords = kEntries * kLookup / 2;
     constexpr int kEntryWords = kLookup >= 2 ? kLookup / 2 : 1;
-    __shared__ __attribute__((aligned(8))) uint32_t table[kTableWords];  // 16-bit values, pairs or double pairs
-    __shared__ float partials[64 * 8];    // [row sum][wavefront]
-    constexpr int kReduceRows = pair_reduce_rows<MT>();
-    constexpr int kSums = kReduceRows * MT;
-
     const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int waves = blockDim.x >> 6;
-    const int row_base = blockIdx.x * kPairRows;
-    const int sample_base = blockIdx.y * MT;
-    const uint32_t row_bytes = (static_cast<uint32_t>(a.width) * BITS) >> 3;
-    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
-    // Lanes past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
-    // activations: they add nothing.
-    const bool in_row = tid * kChunkCodes < a.width;
-    const int chunk = in_row ? tid : 0;
-    const uint32_t code_offset = static_cast<uint32_t>(chunk) * (4u * BITS);
-
-    // The grid's values first (one global load per value), then every table entry from them.
     __shared__ float grid_values[1 << BITS];
     for (int code = tid; code < (1 << BITS); code += blockDim.x) {
         float value = 0.0f;
@@ -115,6 +100,35 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
             table[word] = static_cast<uint32_t>(mk_float_to_bf16(first)) | (static_cast<uint32_t>(mk_float_to_bf16(second)) << 16);
         }
     }
+}
+
+template <int BITS, int MT, bool HAS_ZERO, int XT, int LOOKUP>
+__global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
+    constexpr int kLookup = LOOKUP;
+    constexpr int kPairAhead = rows_in_flight<BITS>();
+    constexpr int kEntries = 1 << (kLookup * BITS);
+    constexpr int kTableWords = kEntries * kLookup / 2;
+    constexpr int kEntryWords = kLookup >= 2 ? kLookup / 2 : 1;
+    __shared__ __attribute__((aligned(8))) uint32_t table[kTableWords];  // 16-bit values, pairs or double pairs
+    __shared__ float partials[64 * 8];    // [row sum][wavefront]
+    constexpr int kReduceRows = pair_reduce_rows<MT>();
+    constexpr int kSums = kReduceRows * MT;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int waves = blockDim.x >> 6;
+    const int row_base = blockIdx.x * kPairRows;
+    const int sample_base = blockIdx.y * MT;
+    const uint32_t row_bytes = (static_cast<uint32_t>(a.width) * BITS) >> 3;
+    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
+    // Lanes past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
+    // activations: they add nothing.
+    const bool in_row = tid * kChunkCodes < a.width;
+    const int chunk = in_row ? tid : 0;
+    const uint32_t code_offset = static_cast<uint32_t>(chunk) * (4u * BITS);
+
+    fill_table<BITS, LOOKUP, XT>(table, a);
     // Also aligns the wavefronts, so that nobody's small loads queue behind another's codes.
     __syncthreads();
 
@@ -227,6 +241,208 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
     }
 }
 
+// ---- three to eight samples: the dot products on the matrix cores -------------------------
+//
+// As in the 4-bit streaming kernel: v_mfma_f32_4x4x4_16B_{f16,bf16} multiplies sixteen
+// independent 4 x 4 x 4 blocks, block b being "rows 4 q ... 4 q + 3 of the weight x four
+// samples over four adjacent codes of chunk b".  Lane 4 b + t looks up the values of row t's
+// codes (two table reads per four codes, or one for double-pair tables) and holds sample
+// t's activations for chunk b in their natural order.  A wavefront owns 2048 codes of K as
+// four sub-slices of sixteen chunks; the four row sums of a result lane take their scales
+// from the four lanes of its quad.
+template <int BITS, int SETS, bool HAS_ZERO, int XT, int LOOKUP>
+__global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) {
+    constexpr int kQuads = kPairRows / 4;
+    constexpr int kSlices = 4;
+    constexpr int kSteps = kQuads * kSlices;
+    constexpr int kAhead = rows_in_flight<BITS>();
+    constexpr int kEntries = 1 << (LOOKUP * BITS);
+    constexpr int kTableWords = kEntries * LOOKUP / 2;
+    __shared__ __attribute__((aligned(8))) uint32_t table[kTableWords];
+    __shared__ float partials[SETS * kPairRows * 4 * 8];  // [set][row][sample in set][wavefront]
+    extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int waves = blockDim.x >> 6;
+    const int block = lane >> 2, t = lane & 3;
+    uint32_t *const x_slice = x_slices_storage + wave * kSliceWords;
+    const int row_base = blockIdx.x * kPairRows;
+    const uint32_t row_bytes = (static_cast<uint32_t>(a.width) * BITS) >> 3;
+    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
+    const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
+    const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
+    const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
+                                        : nullptr;
+
+    fill_table<BITS, LOOKUP, XT>(table, a);
+
+    // Chunks past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
+    // activations: they add nothing.
+    bool in_row[kSlices];
+    uint32_t code_offset[kSlices], group_offset[kSlices];
+#pragma unroll
+    for (int s = 0; s < kSlices; ++s) {
+        const int wanted = wave * 64 + s * 16 + block;
+        in_row[s] = wanted * kChunkCodes < a.width;
+        const int chunk = in_row[s] ? wanted : 0;
+        code_offset[s] = static_cast<uint32_t>(t) * row_bytes + static_cast<uint32_t>(chunk) * (4u * BITS);
+        group_offset[s] = static_cast<uint32_t>(t) * scale_row_bytes +
+                          ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
+    }
+    __syncthreads();  // the table is complete; also aligns the wavefronts before their loads
+
+    // Activations of sample t (and t + 4) for this lane's four chunks: each sample's slice is
+    // read coalesced and the four lanes in sixteen whose sample it is pick their chunks.
+    XChunk<XT> x[SETS][kSlices];
+#pragma unroll
+    for (int set = 0; set < SETS; ++set) {
+        mk_u32x4 pieces[4][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int wanted_sample = blockIdx.y * 4 * SETS + 4 * set + j;
+            const int sample = wanted_sample < a.samples ? wanted_sample : a.samples - 1;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pieces[j][i] = request_piece(a, sample, wave * 2048, i, lane);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) park_piece(x_slice, i, lane, pieces[j][i]);
+            if (t == j) {
+#pragma unroll
+                for (int s = 0; s < kSlices; ++s) chunk_from_slice(x[set][s], x_slice, s * 16 + block);
+            }
+        }
+    }
+    uint16_t scale_raw[kSteps], zero_raw[HAS_ZERO ? kSteps : 1];
+#pragma unroll
+    for (int q = 0; q < kQuads; ++q)
+#pragma unroll
+        for (int s = 0; s < kSlices; ++s) {
+            const size_t quad_offset = static_cast<size_t>(4 * q) * scale_row_bytes;
+            scale_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(scale_base + quad_offset + group_offset[s]);
+            if constexpr (HAS_ZERO)
+                zero_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(zero_base + quad_offset + group_offset[s]);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+
+    CodeChunk<BITS> codes[kSteps];
+#pragma unroll
+    for (int step = 0; step < kAhead; ++step) {
+        load_codes<BITS>(codes[step], codes_base + static_cast<size_t>(4 * (step / kSlices)) * row_bytes + code_offset[step % kSlices]);
+        __builtin_amdgcn_sched_barrier(0);  // in order
+    }
+
+    float x_sum[SETS][kSlices];
+#pragma unroll
+    for (int set = 0; set < SETS; ++set) {
+        const bool sample_present = blockIdx.y * 4 * SETS + 4 * set + t < a.samples;
+#pragma unroll
+        for (int s = 0; s < kSlices; ++s) {
+            const uint32_t keep = in_row[s] && sample_present ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) x[set][s].r[i] &= keep;
+            x_sum[set][s] = HAS_ZERO ? chunk_sum<XT>(x[set][s]) : 0.0f;
+        }
+    }
+
+    float sums[SETS][kPairRows];
+#pragma unroll
+    for (int set = 0; set < SETS; ++set)
+#pragma unroll
+        for (int j = 0; j < kPairRows; ++j) sums[set][j] = 0.0f;
+
+    auto blocks = [](uint32_t a_low, uint32_t a_high, uint32_t b_low, uint32_t b_high, mk_f4 sum) __attribute__((always_inline)) {
+        const mk_u32x2 left = {a_low, a_high}, right = {b_low, b_high};
+        if constexpr (XT == MK_F16)
+            return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(mk_h4, left), __builtin_bit_cast(mk_h4, right), sum, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(mk_s4, left), __builtin_bit_cast(mk_s4, right), sum, 0, 0, 0);
+    };
+    const uint8_t *table_bytes = reinterpret_cast<const uint8_t *>(table);
+
+#pragma unroll
+    for (int step = 0; step < kSteps; ++step) {
+        const int q = step / kSlices, s = step % kSlices;
+        mk_f4 dot[SETS];
+#pragma unroll
+        for (int set = 0; set < SETS; ++set) dot[set] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {  // codes 4 i ... 4 i + 3
+            uint32_t low, high;
+            if constexpr (LOOKUP == 4) {
+                const mk_u32x2 both = *reinterpret_cast<const mk_u32x2 *>(table_bytes + lookup_offset<BITS, 4>(codes[step], i));
+                low = both.x, high = both.y;
+            } else if constexpr (LOOKUP == 2) {
+                low = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, 2>(codes[step], 2 * i));
+                high = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, 2>(codes[step], 2 * i + 1));
+            } else {
+                const uint32_t v0 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i));
+                const uint32_t v1 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i + 1));
+                const uint32_t v2 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i + 2));
+                const uint32_t v3 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i + 3));
+                low = v0 | (v1 << 16), high = v2 | (v3 << 16);
+            }
+#pragma unroll
+            for (int set = 0; set < SETS; ++set)
+                dot[set] = blocks(low, high, x[set][s].r[2 * i], x[set][s].r[2 * i + 1], dot[set]);
+        }
+        if (step + kAhead < kSteps)
+            load_codes<BITS>(codes[step + kAhead], codes_base + static_cast<size_t>(4 * ((step + kAhead) / kSlices)) * row_bytes +
+                                                       code_offset[(step + kAhead) % kSlices]);
+        // Row 4 q + r of the block: scale (and offset) come from lane r of the quad.
+        const float scale = side_as_float(scale_raw[step], a.scale_dtype);
+        float zero = 0.0f;
+        if constexpr (HAS_ZERO) zero = side_as_float(zero_raw[step], a.scale_dtype);
+        auto add_row = [&](auto r) __attribute__((always_inline)) {
+            constexpr int R = decltype(r)::value;
+#pragma unroll
+            for (int set = 0; set < SETS; ++set) {
+                float total = __builtin_fmaf(quad_value<R>(scale), dot[set][R], sums[set][4 * q + R]);
+                if constexpr (HAS_ZERO) total = __builtin_fmaf(quad_value<R>(zero), x_sum[set][s], total);
+                sums[set][4 * q + R] = total;
+            }
+        };
+        add_row(std::integral_constant<int, 0>{});
+        add_row(std::integral_constant<int, 1>{});
+        add_row(std::integral_constant<int, 2>{});
+        add_row(std::integral_constant<int, 3>{});
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // Over the sixteen blocks of the wavefront (lane bits 2 - 5), then over the wavefronts.
+#pragma unroll
+    for (int set = 0; set < SETS; ++set) {
+        transposed_wave_sum<kPairRows, 2>(sums[set], lane);
+        partials[((set * kPairRows + transposed_value_of_lane<kPairRows>(lane >> 2)) * 4 + t) * 8 + wave] = sums[set][0];
+    }
+    __syncthreads();
+    for (int index = tid; index < SETS * kPairRows * 4; index += blockDim.x) {  // a workgroup may be one wavefront
+        float total = partials[index * 8];
+#pragma unroll
+        for (int w = 1; w < 8; ++w) total += w < waves ? partials[index * 8 + w] : 0.0f;
+        const int set = index / (kPairRows * 4), row = row_base + (index / 4) % kPairRows;
+        const int sample = blockIdx.y * 4 * SETS + 4 * set + (index & 3);
+        if (sample < a.samples) {
+            if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
+            store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
+        }
+    }
+}
+
+template <int BITS, int SETS, int XT, int LOOKUP>
+void launch_blocks_with(const Stream4Args &a, int tiles, hipStream_t stream) {
+    const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
+    const dim3 block(mk_cdiv(a.width, 2048) * 64);
+    const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
+    if (a.zeros)
+        hipLaunchKernelGGL((pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP>), grid, block, slices, stream, a);
+    else
+        hipLaunchKernelGGL((pairs_blocks_kernel<BITS, SETS, false, XT, LOOKUP>), grid, block, slices, stream, a);
+}
+
 template <int BITS, int MT, int XT, int LOOKUP>
 void launch_tile_with(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
@@ -261,8 +477,37 @@ void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
     else launch_tile_as<BITS, MT, MK_BF16>(a, tiles, stream);
 }
 
+// The same field widths for the matrix-core kernel.
+template <int BITS, int SETS, int XT>
+void launch_blocks_as(const Stream4Args &a, int tiles, hipStream_t stream) {
+    if constexpr (BITS == 2) {
+        launch_blocks_with<BITS, SETS, XT, 4>(a, tiles, stream);
+    } else if constexpr (BITS == 3) {
+        if (a.width >= 8192) launch_blocks_with<BITS, SETS, XT, 4>(a, tiles, stream);
+        else launch_blocks_with<BITS, SETS, XT, 2>(a, tiles, stream);
+    } else if constexpr (BITS <= 5) {
+        launch_blocks_with<BITS, SETS, XT, 2>(a, tiles, stream);
+    } else if constexpr (BITS == 6) {
+        if (a.width >= 4096) launch_blocks_with<BITS, SETS, XT, 2>(a, tiles, stream);
+        else launch_blocks_with<BITS, SETS, XT, 1>(a, tiles, stream);
+    } else {
+        launch_blocks_with<BITS, SETS, XT, 1>(a, tiles, stream);
+    }
+}
+
+template <int BITS, int SETS>
+void launch_blocks(const Stream4Args &a, int tiles, hipStream_t stream) {
+    if (a.x_dtype == MK_F16) launch_blocks_as<BITS, SETS, MK_F16>(a, tiles, stream);
+    else launch_blocks_as<BITS, SETS, MK_BF16>(a, tiles, stream);
+}
+
 template <int BITS>
 void launch_bits(const Stream4Args &a, int tiles, hipStream_t stream) {
+    if (a.samples >= 3) {  // measured against the v_dot2 kernel at 4096 x 14336
+        if (a.samples <= 4) launch_blocks<BITS, 1>(a, tiles, stream);
+        else launch_blocks<BITS, 2>(a, tiles, stream);
+        return;
+    }
     int tile = 1;
     while (tile < a.samples && tile < 8) tile <<= 1;
     switch (tile) {

@@ -43,43 +43,6 @@ constexpr int reduce_rows() {
     return ROWS * MT <= 64 ? ROWS : 64 / MT;
 }
 
-// ---- activations: coalesced loads, then each lane's chunk out of LDS ------------------------
-//
-// A lane needs the 32 activations (64 bytes) of a chunk.  Sixty-four lanes reading 16 bytes
-// at a stride of 64 touch 64 cache lines per instruction, and the compute unit's vector
-// memory path takes them one line per cycle, ahead of the code stream.  Instead a wavefront
-// reads the 4 KB of one sample's 2048-code slice as four 1 KB instructions (lane l: bytes
-// 16 l), parks them in its own LDS buffer and reads chunks back.  Chunks are 80 bytes apart
-// in LDS so that sixteen lanes reading 16 bytes of sixteen chunks hit different banks.
-
-constexpr int kChunkStrideWords = 20;
-constexpr int kSliceWords = 64 * kChunkStrideWords;  // one wavefront's buffer: 5 KB
-
-// Piece i of the slice that starts at element `slice_start` of x's row `sample`: 16 bytes per
-// lane.  Pieces past the end of the row read the start of the row instead (their chunks are
-// zeroed later).
-__device__ __forceinline__ mk_u32x4 request_piece(const Stream4Args &a, int sample, int slice_start, int i, int lane) {
-    const int element = slice_start + (16 * i + (lane >> 2)) * kChunkCodes + (lane & 3) * 8;
-    const size_t offset = static_cast<size_t>(sample) * a.width + (element < a.width ? element : (lane & 3) * 8);
-    return *reinterpret_cast<const mk_u32x4 *>(static_cast<const uint8_t *>(a.x) + offset * 2);
-}
-
-__device__ __forceinline__ void park_piece(uint32_t *slice, int i, int lane, mk_u32x4 piece) {
-    *reinterpret_cast<mk_u32x4 *>(slice + (16 * i + (lane >> 2)) * kChunkStrideWords + (lane & 3) * 4) = piece;
-}
-
-template <int XT>
-__device__ __forceinline__ void chunk_from_slice(XChunk<XT> &x, const uint32_t *slice, int chunk_in_slice) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const mk_u32x4 v = *reinterpret_cast<const mk_u32x4 *>(slice + chunk_in_slice * kChunkStrideWords + 4 * i);
-        x.r[4 * i + 0] = v.x;
-        x.r[4 * i + 1] = v.y;
-        x.r[4 * i + 2] = v.z;
-        x.r[4 * i + 3] = v.w;
-    }
-}
-
 // ---- bf16 activations ----------------------------------------------------------------------
 //
 // bf16 has seven mantissa bits, so only the low nibble of each half fits the magic-number
@@ -130,19 +93,6 @@ __device__ __forceinline__ void chunk_dot_bf16(const CodeChunk<4> &codes, const 
             dot[m] = d;
         }
     }
-}
-
-// A 16-bit scale or offset as fp32; `dtype` (MK_F16 or MK_BF16) is uniform per launch.
-__device__ __forceinline__ float side_as_float(uint16_t raw, int dtype) {
-    const float from_half = static_cast<float>(__builtin_bit_cast(_Float16, raw));
-    const float from_brain = __uint_as_float(static_cast<uint32_t>(raw) << 16);
-    return dtype == MK_F16 ? from_half : from_brain;
-}
-
-template <int XT>
-__device__ __forceinline__ void store_output(void *y, size_t index, float value) {
-    if constexpr (XT == MK_F16) static_cast<_Float16 *>(y)[index] = static_cast<_Float16>(value);
-    else static_cast<uint16_t *>(y)[index] = mk_float_to_bf16(value);
 }
 
 template <int MT, bool HAS_ZERO, int ROWS, int XT>
@@ -292,15 +242,6 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
 // workgroup's rows four at a time.  The result lane holds sums for four rows; their scales
 // sit in the four lanes of its quad (each loaded by the lane that loads that row's codes)
 // and reach the multiply as DPP quad broadcasts.
-
-typedef _Float16 mk_h4 __attribute__((ext_vector_type(4)));
-typedef short mk_s4 __attribute__((ext_vector_type(4)));
-typedef float mk_f4 __attribute__((ext_vector_type(4)));
-
-template <int R>
-__device__ __forceinline__ float quad_value(float value) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, value), R * 0x55, 0xf, 0xf, true));
-}
 
 template <int SETS, bool HAS_ZERO, int ROWS, int XT>
 __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a) {
