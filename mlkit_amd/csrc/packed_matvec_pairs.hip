@@ -250,12 +250,12 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
 // t's activations for chunk b in their natural order.  A wavefront owns 2048 codes of K as
 // four sub-slices of sixteen chunks; the four row sums of a result lane take their scales
 // from the four lanes of its quad.
-template <int BITS, int SETS, bool HAS_ZERO, int XT, int LOOKUP>
+template <int BITS, int SETS, bool HAS_ZERO, int XT, int LOOKUP, int SLICES>
 __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) {
     constexpr int kQuads = kPairRows / 4;
-    constexpr int kSlices = 4;
+    constexpr int kSlices = SLICES;  // sub-slices of sixteen chunks per wavefront (rows of up to 512 / 1024 codes: 1 / 2)
     constexpr int kSteps = kQuads * kSlices;
-    constexpr int kAhead = rows_in_flight<BITS>();
+    constexpr int kAhead = rows_in_flight<BITS>() < kSteps ? rows_in_flight<BITS>() : kSteps;
     constexpr int kEntries = 1 << (LOOKUP * BITS);
     constexpr int kTableWords = kEntries * LOOKUP / 2;
     __shared__ __attribute__((aligned(8))) uint32_t table[kTableWords];
@@ -284,7 +284,7 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
     uint32_t code_offset[kSlices], group_offset[kSlices];
 #pragma unroll
     for (int s = 0; s < kSlices; ++s) {
-        const int wanted = wave * 64 + s * 16 + block;
+        const int wanted = wave * (16 * kSlices) + s * 16 + block;
         in_row[s] = wanted * kChunkCodes < a.width;
         const int chunk = in_row[s] ? wanted : 0;
         code_offset[s] = static_cast<uint32_t>(t) * row_bytes + static_cast<uint32_t>(chunk) * (4u * BITS);
@@ -298,18 +298,18 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
     XChunk<XT> x[SETS][kSlices];
 #pragma unroll
     for (int set = 0; set < SETS; ++set) {
-        mk_u32x4 pieces[4][4];
+        mk_u32x4 pieces[4][kSlices];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int wanted_sample = blockIdx.y * 4 * SETS + 4 * set + j;
             const int sample = wanted_sample < a.samples ? wanted_sample : a.samples - 1;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) pieces[j][i] = request_piece(a, sample, wave * 2048, i, lane);
+            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(a, sample, wave * (512 * kSlices), i, lane);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) park_piece(x_slice, i, lane, pieces[j][i]);
+            for (int i = 0; i < kSlices; ++i) park_piece(x_slice, i, lane, pieces[j][i]);
             if (t == j) {
 #pragma unroll
                 for (int s = 0; s < kSlices; ++s) chunk_from_slice(x[set][s], x_slice, s * 16 + block);
@@ -432,15 +432,22 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
     }
 }
 
-template <int BITS, int SETS, int XT, int LOOKUP>
-void launch_blocks_with(const Stream4Args &a, int tiles, hipStream_t stream) {
+template <int BITS, int SETS, int XT, int LOOKUP, int SLICES>
+void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
-    const dim3 block(mk_cdiv(a.width, 2048) * 64);
+    const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
     if (a.zeros)
-        hipLaunchKernelGGL((pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP>), grid, block, slices, stream, a);
+        hipLaunchKernelGGL((pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP, SLICES>), grid, block, slices, stream, a);
     else
-        hipLaunchKernelGGL((pairs_blocks_kernel<BITS, SETS, false, XT, LOOKUP>), grid, block, slices, stream, a);
+        hipLaunchKernelGGL((pairs_blocks_kernel<BITS, SETS, false, XT, LOOKUP, SLICES>), grid, block, slices, stream, a);
+}
+
+// Short rows get fewer sub-slices per wavefront, so that none lies wholly past the row's end.
+template <int BITS, int SETS, int XT, int LOOKUP>
+void launch_blocks_with(const Stream4Args &a, int tiles, hipStream_t stream) {
+    if (a.width <= 1024) launch_blocks_sliced<BITS, SETS, XT, LOOKUP, 2>(a, tiles, stream);
+    else launch_blocks_sliced<BITS, SETS, XT, LOOKUP, 4>(a, tiles, stream);
 }
 
 template <int BITS, int MT, int XT, int LOOKUP>

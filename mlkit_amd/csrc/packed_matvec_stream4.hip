@@ -243,10 +243,10 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
 // sit in the four lanes of its quad (each loaded by the lane that loads that row's codes)
 // and reach the multiply as DPP quad broadcasts.
 
-template <int SETS, bool HAS_ZERO, int ROWS, int XT>
+template <int SETS, bool HAS_ZERO, int ROWS, int XT, int SLICES>
 __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a) {
     constexpr int kQuads = ROWS / 4;
-    constexpr int kSlices = 4;                      // sub-slices of sixteen chunks per wavefront
+    constexpr int kSlices = SLICES;                 // sub-slices of sixteen chunks per wavefront (rows of up to 512 / 1024 codes: 1 / 2)
     constexpr int kSteps = kQuads * kSlices;        // code loads per lane
     constexpr int kAhead = kSteps < 8 ? kSteps : 8;
     constexpr int kSums = ROWS;                     // per set and lane before the reduction
@@ -275,7 +275,7 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     uint32_t code_offset[kSlices], group_offset[kSlices];
 #pragma unroll
     for (int s = 0; s < kSlices; ++s) {
-        const int wanted = wave * 64 + s * 16 + block;
+        const int wanted = wave * (16 * kSlices) + s * 16 + block;
         in_row[s] = wanted * kChunkCodes < a.width;
         const int chunk = in_row[s] ? wanted : 0;
         code_offset[s] = static_cast<uint32_t>(t) * row_bytes + static_cast<uint32_t>(chunk) * 16u;
@@ -291,18 +291,18 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     XChunk<XT> x[SETS][kSlices];
 #pragma unroll
     for (int set = 0; set < SETS; ++set) {
-        mk_u32x4 pieces[4][4];
+        mk_u32x4 pieces[4][kSlices];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int wanted_sample = blockIdx.y * 4 * SETS + 4 * set + j;
             const int sample = wanted_sample < a.samples ? wanted_sample : a.samples - 1;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) pieces[j][i] = request_piece(a, sample, wave * 2048, i, lane);
+            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(a, sample, wave * (512 * kSlices), i, lane);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) park_piece(x_slice, i, lane, pieces[j][i]);
+            for (int i = 0; i < kSlices; ++i) park_piece(x_slice, i, lane, pieces[j][i]);
             if (t == j) {
 #pragma unroll
                 for (int s = 0; s < kSlices; ++s) chunk_from_slice(x[set][s], x_slice, s * 16 + block);
@@ -442,22 +442,31 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     }
 }
 
-template <int SETS, int ROWS>
-void launch_blocks(const Stream4Args &a, int tiles, hipStream_t stream) {
+template <int SETS, int ROWS, int SLICES>
+void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
-    const dim3 block(mk_cdiv(a.width, 2048) * 64);
+    const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
     if (a.x_dtype == MK_F16) {
         if (a.zeros)
-            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS, MK_F16>), grid, block, slices, stream, a);
+            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS, MK_F16, SLICES>), grid, block, slices, stream, a);
         else
-            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS, MK_F16>), grid, block, slices, stream, a);
+            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS, MK_F16, SLICES>), grid, block, slices, stream, a);
     } else {
         if (a.zeros)
-            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS, MK_BF16>), grid, block, slices, stream, a);
+            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS, MK_BF16, SLICES>), grid, block, slices, stream, a);
         else
-            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS, MK_BF16>), grid, block, slices, stream, a);
+            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS, MK_BF16, SLICES>), grid, block, slices, stream, a);
     }
+}
+
+// A wavefront covers 512 codes per sub-slice: short rows get fewer sub-slices, so that no
+// sub-slice lies wholly past the end of the row.
+template <int SETS, int ROWS>
+void launch_blocks(const Stream4Args &a, int tiles, hipStream_t stream) {
+    if (a.width <= 512) launch_blocks_sliced<SETS, ROWS, 1>(a, tiles, stream);
+    else if (a.width <= 1024) launch_blocks_sliced<SETS, ROWS, 2>(a, tiles, stream);
+    else launch_blocks_sliced<SETS, ROWS, 4>(a, tiles, stream);
 }
 
 template <int MT, int ROWS>
