@@ -380,9 +380,10 @@ __device__ __forceinline__ float lane_exchange(float value, int lane) {
 // lower half and receives its partner's lower half, the other lane the upper half.  On
 // return v[0] of lane L is the total of value number
 //     sum over s < log2(V) of bit_s(L) * (V >> (s + 1)).
-template <int V, int STAGE = 0>
+// END < 6 sums over groups of 2^END lanes only (lane bits END and above keep apart).
+template <int V, int STAGE = 0, int END = 6>
 __device__ __forceinline__ void transposed_wave_sum(float (&v)[V], int lane) {
-    if constexpr (STAGE < 6) {
+    if constexpr (STAGE < END) {
         if constexpr (V > 1) {
             constexpr int H = V / 2;
             const bool upper = (lane >> STAGE) & 1;
@@ -393,11 +394,11 @@ __device__ __forceinline__ void transposed_wave_sum(float (&v)[V], int lane) {
                 const float send = upper ? v[j] : v[j + H];
                 next[j] = keep + lane_exchange<STAGE>(send, lane);
             }
-            transposed_wave_sum<H, STAGE + 1>(next, lane);
+            transposed_wave_sum<H, STAGE + 1, END>(next, lane);
             v[0] = next[0];
         } else {
             v[0] += lane_exchange<STAGE>(v[0], lane);
-            transposed_wave_sum<1, STAGE + 1>(v, lane);
+            transposed_wave_sum<1, STAGE + 1, END>(v, lane);
         }
     }
 }

@@ -36,13 +36,6 @@ constexpr int rows_ahead_of() {
     return ROWS < 8 ? ROWS : 8;
 }
 
-// Rows per transposed reduction: all 16 when that is at most 64 sums per lane (measured
-// faster than splitting the reduction to hide part of it behind the stream).
-template <int MT, int ROWS>
-constexpr int reduce_rows() {
-    return ROWS * MT <= 64 ? ROWS : 64 / MT;
-}
-
 // ---- bf16 activations ----------------------------------------------------------------------
 //
 // bf16 has seven mantissa bits, so only the low nibble of each half fits the magic-number
@@ -95,31 +88,37 @@ __device__ __forceinline__ void chunk_dot_bf16(const CodeChunk<4> &codes, const 
     }
 }
 
-template <int MT, bool HAS_ZERO, int ROWS, int XT>
+// PARTS = 2: rows of at most 1024 codes, one wavefront per workgroup; lanes 0 - 31 take one
+// row and lanes 32 - 63 the next, so that a step covers two rows instead of leaving half the
+// wavefront without codes.
+template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS>
 __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
+    static_assert(ROWS * MT <= 64 && ROWS % PARTS == 0, "one transposed reduction per workgroup");
     __shared__ float partials[64 * 8];  // [row sum][wavefront]
     // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
     // must not hold LDS for eight).
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
     uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
-    constexpr int kStreamRows = ROWS;
-    constexpr int kStreamAhead = rows_ahead_of<ROWS>();
-    constexpr int kReduceRows = reduce_rows<MT, ROWS>();
-    constexpr int kSums = kReduceRows * MT;
+    constexpr int kStreamRows = ROWS / PARTS;            // steps: PARTS rows each
+    constexpr int kStreamAhead = rows_ahead_of<kStreamRows>();
+    constexpr int kSums = kStreamRows * MT;
+    constexpr int kRowLanes = 64 / PARTS;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int waves = blockDim.x >> 6;
-    const int row_base = blockIdx.x * kStreamRows;
+    const int row_base = blockIdx.x * ROWS;
+    const int part = lane / kRowLanes;                   // this lane's row within a step
+    const int chunk_lane = wave * 64 + (lane & (kRowLanes - 1));
     const int sample_base = blockIdx.y * MT;
     const uint32_t row_bytes = static_cast<uint32_t>(a.width) >> 1;
     const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
     // Lanes past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
     // activations: they add nothing.
-    const bool in_row = tid * kChunkCodes < a.width;
-    const int chunk = in_row ? tid : 0;
-    const uint32_t code_offset = static_cast<uint32_t>(chunk) * 16u;
+    const bool in_row = chunk_lane * kChunkCodes < a.width;
+    const int chunk = in_row ? chunk_lane : 0;
+    const uint32_t code_offset = static_cast<uint32_t>(part) * row_bytes + static_cast<uint32_t>(chunk) * 16u;
 
     // The workgroup is aligned first: a compute unit serves loads first come, first served,
     // and a wavefront that starts late would queue its small loads behind the others' codes.
@@ -134,24 +133,25 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
         for (int i = 0; i < 4; ++i) pieces[m][i] = request_piece(a, sample, wave * 2048, i, lane);
     }
     // The scale (and offset) of this lane's chunk in every row, 2 bytes each.
-    const uint32_t group_offset = ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
+    const uint32_t group_offset = static_cast<uint32_t>(part) * scale_row_bytes +
+                                  ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
     const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
     const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
                                         : nullptr;
     uint16_t scale_raw[kStreamRows], zero_raw[HAS_ZERO ? kStreamRows : 1];
 #pragma unroll
     for (int r = 0; r < kStreamRows; ++r) {
-        scale_raw[r] = *reinterpret_cast<const uint16_t *>(scale_base + static_cast<size_t>(r) * scale_row_bytes + group_offset);
+        scale_raw[r] = *reinterpret_cast<const uint16_t *>(scale_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
         if constexpr (HAS_ZERO)
-            zero_raw[r] = *reinterpret_cast<const uint16_t *>(zero_base + static_cast<size_t>(r) * scale_row_bytes + group_offset);
+            zero_raw[r] = *reinterpret_cast<const uint16_t *>(zero_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
     }
     __builtin_amdgcn_sched_barrier(0);
 
     CodeChunk<4> codes[kStreamRows];
 #pragma unroll
     for (int r = 0; r < kStreamAhead; ++r) {
-        load_codes<4>(codes[r], codes_base + static_cast<size_t>(r) * row_bytes + code_offset);
+        load_codes<4>(codes[r], codes_base + static_cast<size_t>(PARTS * r) * row_bytes + code_offset);
         __builtin_amdgcn_sched_barrier(0);  // in row order
     }
 
@@ -162,7 +162,7 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     for (int m = 0; m < MT; ++m) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) park_piece(x_slice, i, lane, pieces[m][i]);
-        chunk_from_slice(x[m], x_slice, lane);
+        chunk_from_slice(x[m], x_slice, lane & (kRowLanes - 1));
     }
 
     // sum_k (min + step c_k) x_k = step * dot + min * sum(x) - step * (code-free part of dot).
@@ -182,46 +182,43 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
         grid_term[m] = a.grid_min * x_sum[m] - a.grid_step * code_free;
     }
 
+    float sums[kSums];
 #pragma unroll
-    for (int pass = 0; pass < kStreamRows / kReduceRows; ++pass) {
-        float sums[kSums];
+    for (int r = 0; r < kStreamRows; ++r) {
+        float dot[MT];
+        if constexpr (XT == MK_F16) chunk_dot<4, MK_F16, MT, true>(codes[r], x, nullptr, dot);
+        else chunk_dot_bf16<MT>(codes[r], x, dot);
+        if (r + kStreamAhead < kStreamRows)
+            load_codes<4>(codes[r + kStreamAhead],
+                          codes_base + static_cast<size_t>(PARTS * (r + kStreamAhead)) * row_bytes + code_offset);
+        const float scale = side_as_float(scale_raw[r], a.scale_dtype);
 #pragma unroll
-        for (int j = 0; j < kReduceRows; ++j) {
-            const int r = pass * kReduceRows + j;
-            float dot[MT];
-            if constexpr (XT == MK_F16) chunk_dot<4, MK_F16, MT, true>(codes[r], x, nullptr, dot);
-            else chunk_dot_bf16<MT>(codes[r], x, dot);
-            if (r + kStreamAhead < kStreamRows)
-                load_codes<4>(codes[r + kStreamAhead],
-                              codes_base + static_cast<size_t>(r + kStreamAhead) * row_bytes + code_offset);
-            const float scale = side_as_float(scale_raw[r], a.scale_dtype);
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                float value = scale * __builtin_fmaf(a.grid_step, dot[m], grid_term[m]);
-                if constexpr (HAS_ZERO)
-                    value = __builtin_fmaf(side_as_float(zero_raw[r], a.scale_dtype), x_sum[m], value);
-                sums[j * MT + m] = value;
-            }
-            // Keeps the rows in arrival order and their temporaries short-lived.
-            __builtin_amdgcn_sched_barrier(0);
+        for (int m = 0; m < MT; ++m) {
+            float value = scale * __builtin_fmaf(a.grid_step, dot[m], grid_term[m]);
+            if constexpr (HAS_ZERO)
+                value = __builtin_fmaf(side_as_float(zero_raw[r], a.scale_dtype), x_sum[m], value);
+            sums[r * MT + m] = value;
         }
+        // Keeps the rows in arrival order and their temporaries short-lived.
+        __builtin_amdgcn_sched_barrier(0);
+    }
 
-        // All row sums of this pass over the 64 lanes at once, then over the wavefronts.
-        transposed_wave_sum<kSums>(sums, lane);
-        if (pass > 0) __syncthreads();  // the previous pass's readers are done
-        if (lane < kSums) partials[transposed_value_of_lane<kSums>(lane) * 8 + wave] = sums[0];
-        __syncthreads();
-        if (tid < kSums) {
-            float total = partials[tid * 8];
+    // All row sums over the lanes of a row at once, then over the wavefronts.
+    transposed_wave_sum<kSums, 0, PARTS == 1 ? 6 : 5>(sums, lane);
+    const int lane_in_row = lane & (kRowLanes - 1);
+    if (lane_in_row < kSums)
+        partials[(transposed_value_of_lane<kSums>(lane_in_row) * PARTS + part) * 8 + wave] = sums[0];
+    __syncthreads();
+    if (tid < kSums * PARTS) {
+        float total = partials[tid * 8];
 #pragma unroll
-            for (int w = 1; w < 8; ++w) total += w < waves ? partials[tid * 8 + w] : 0.0f;
-            const int j = tid / MT, m = tid - j * MT;
-            const int row = row_base + pass * kReduceRows + j;
-            const int sample = sample_base + m;
-            if (sample < a.samples) {
-                if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
-                store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
-            }
+        for (int w = 1; w < 8; ++w) total += w < waves ? partials[tid * 8 + w] : 0.0f;
+        const int value = tid / PARTS, j = value / MT, m = value - j * MT;
+        const int row = row_base + PARTS * j + (tid - value * PARTS);
+        const int sample = sample_base + m;
+        if (sample < a.samples) {
+            if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
+            store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
         }
     }
 }
@@ -469,22 +466,28 @@ void launch_blocks(const Stream4Args &a, int tiles, hipStream_t stream) {
     else launch_blocks_sliced<SETS, ROWS, 4>(a, tiles, stream);
 }
 
-template <int MT, int ROWS>
-void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
+template <int MT, int ROWS, int PARTS>
+void launch_tile_parts(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
     if (a.x_dtype == MK_F16) {
         if (a.zeros)
-            hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS, MK_F16>), grid, block, slices, stream, a);
+            hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS, MK_F16, PARTS>), grid, block, slices, stream, a);
         else
-            hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS, MK_F16>), grid, block, slices, stream, a);
+            hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS, MK_F16, PARTS>), grid, block, slices, stream, a);
     } else {
         if (a.zeros)
-            hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS, MK_BF16>), grid, block, slices, stream, a);
+            hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS, MK_BF16, PARTS>), grid, block, slices, stream, a);
         else
-            hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS, MK_BF16>), grid, block, slices, stream, a);
+            hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS, MK_BF16, PARTS>), grid, block, slices, stream, a);
     }
+}
+
+template <int MT, int ROWS>
+void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
+    if (a.width <= 1024) launch_tile_parts<MT, ROWS, 2>(a, tiles, stream);
+    else launch_tile_parts<MT, ROWS, 1>(a, tiles, stream);
 }
 
 template <int ROWS>
