@@ -80,6 +80,47 @@ __global__ void __launch_bounds__(kThreads) encode_kernel(const CodecArgs a) {
     const int column = (blockIdx.x * kThreads + threadIdx.x) * VEC;
     if (column >= a.width) return;
     const bool one_slot = a.group % VEC == 0;
+    if constexpr (VEC == 4) {
+        if (one_slot) {
+            // Four rows per trip, all their loads issued before the first is used.
+            constexpr int kRowsPerTrip = 4;
+            const int group_index = column / a.group;
+            for (int first = blockIdx.y; first < a.rows; first += kRowsPerTrip * gridDim.y) {
+                float4 loaded[kRowsPerTrip];
+                float scale[kRowsPerTrip], zero[kRowsPerTrip];
+#pragma unroll
+                for (int u = 0; u < kRowsPerTrip; ++u) {
+                    const int wanted = first + u * static_cast<int>(gridDim.y);
+                    const int row = wanted < a.rows ? wanted : first;
+                    loaded[u] = *reinterpret_cast<const float4 *>(a.value + static_cast<size_t>(row) * a.width + column);
+                    const int slot = row * a.groups_per_row + group_index;
+                    scale[u] = a.scales[slot];
+                    zero[u] = a.zeros ? a.zeros[slot] : 0.0f;
+                }
+#pragma unroll
+                for (int u = 0; u < kRowsPerTrip; ++u) {
+                    const int row = first + u * static_cast<int>(gridDim.y);
+                    const float sample[4] = {loaded[u].x, loaded[u].y, loaded[u].z, loaded[u].w};
+                    uint32_t packed = 0;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float centered = sample[i];
+                        if (a.zeros) centered = __fsub_rn(centered, zero[u]);
+                        const float normalized = __fdiv_rn(centered, scale[u]);
+                        int index;
+                        if (a.integer)
+                            index = static_cast<int>(__fsub_rn(nearest_integer(normalized, a.minimum, a.maximum), a.minimum));
+                        else
+                            index = nearest_entry(normalized, table, a.n_values, steps);
+                        packed |= static_cast<uint32_t>(index & 255) << (8 * i);
+                    }
+                    if (row < a.rows)
+                        *reinterpret_cast<uint32_t *>(a.codes_out + static_cast<size_t>(row) * a.width + column) = packed;
+                }
+            }
+            return;
+        }
+    }
     for (int row = blockIdx.y; row < a.rows; row += gridDim.y) {
         const size_t base = static_cast<size_t>(row) * a.width + column;
         float sample[VEC];
@@ -119,6 +160,41 @@ __global__ void __launch_bounds__(kThreads) decode_kernel(const CodecArgs a) {
     if (column >= a.width) return;
     const bool one_slot = a.refit == 0 && a.group % VEC == 0;
     const int limit = a.n_values - 1;
+    if constexpr (VEC == 4) {
+        if (one_slot) {
+            // Four rows per trip, all their loads issued before the first is used.
+            constexpr int kRowsPerTrip = 4;
+            const int group_index = column / a.group;
+            for (int first = blockIdx.y; first < a.rows; first += kRowsPerTrip * gridDim.y) {
+                uint32_t packed[kRowsPerTrip];
+                float scale[kRowsPerTrip], zero[kRowsPerTrip];
+#pragma unroll
+                for (int u = 0; u < kRowsPerTrip; ++u) {
+                    const int wanted = first + u * static_cast<int>(gridDim.y);
+                    const int row = wanted < a.rows ? wanted : first;
+                    packed[u] = *reinterpret_cast<const uint32_t *>(a.codes_in + static_cast<size_t>(row) * a.width + column);
+                    const int slot = row * a.groups_per_row + group_index;
+                    scale[u] = a.scales[slot];
+                    zero[u] = a.zeros ? a.zeros[slot] : 0.0f;
+                }
+#pragma unroll
+                for (int u = 0; u < kRowsPerTrip; ++u) {
+                    const int row = first + u * static_cast<int>(gridDim.y);
+                    float weight[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int code = static_cast<int>((packed[u] >> (8 * i)) & 255u);
+                        weight[i] = __fmul_rn(table[code < limit ? code : limit], scale[u]);
+                        if (a.zeros) weight[i] = __fadd_rn(weight[i], zero[u]);
+                    }
+                    if (row < a.rows)
+                        *reinterpret_cast<float4 *>(a.out + static_cast<size_t>(row) * a.width + column) =
+                            make_float4(weight[0], weight[1], weight[2], weight[3]);
+                }
+            }
+            return;
+        }
+    }
     for (int row = blockIdx.y; row < a.rows; row += gridDim.y) {
         const size_t base = static_cast<size_t>(row) * a.width + column;
         uint32_t packed;
@@ -243,10 +319,71 @@ struct FitArgs {
 
 // A team of LANES lanes finds one group's extrema (order does not matter for min and max)
 // and lane 0 derives the stored scale and offset from them.
+// Scale and offset of one group from its extrema, written by one lane.
+__device__ __forceinline__ void store_fit(const FitArgs &a, size_t slot, float low, float high, bool finite) {
+    if (!finite) {  // fminf/fmaxf drop NaNs: report them as the tensor reductions would
+        a.scales[slot] = __builtin_nanf("");
+        if (a.zeros) a.zeros[slot] = __builtin_nanf("");
+        return;
+    }
+    float scale, zero = 0.0f;
+    if (a.asym) {
+        scale = __fmul_rn(fmaxf(__fsub_rn(high, low), 1e-12f), a.reciprocal);
+        zero = __fsub_rn(low, __fmul_rn(a.value_minimum, scale));
+    } else {
+        scale = __fmul_rn(fmaxf(fmaxf(high, -low), 1e-12f), a.reciprocal);
+    }
+    a.scales[slot] = mk_rounded_scale(scale, a.format);
+    if (a.zeros) {
+        if (a.store_zero) {
+            const float magnitude = mk_rounded_scale(fmaxf(fabsf(zero), 1e-12f), a.format);
+            zero = zero > 0.0f ? magnitude : (zero < 0.0f ? -magnitude : 0.0f);
+        }
+        a.zeros[slot] = zero;
+    }
+}
+
 template <int LANES>
 __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
     constexpr int kTeams = kThreads / LANES;
     const int lane_in_team = threadIdx.x % LANES;
+    // Whole groups of exactly 4 * LANES values, 16-byte aligned: one float4 per lane and group,
+    // four groups per trip with all four loads issued first.
+    const bool single_load = a.group == 4 * LANES && a.span % a.group == 0 && a.row_stride % 4 == 0 &&
+                             (reinterpret_cast<uintptr_t>(a.value) & 15u) == 0;
+    if (single_load) {
+        constexpr int kPerTrip = 4;
+        const int team = threadIdx.x / LANES;
+        for (int first = (blockIdx.x * kTeams + team) * kPerTrip; first < a.total_groups; first += gridDim.x * kTeams * kPerTrip) {
+            float4 loaded[kPerTrip];
+#pragma unroll
+            for (int u = 0; u < kPerTrip; ++u) {
+                const int identifier = first + u < a.total_groups ? first + u : first;
+                const int row = identifier / a.groups_per_row;
+                const int start = (identifier - row * a.groups_per_row) * a.group;
+                loaded[u] = *reinterpret_cast<const float4 *>(a.value + static_cast<size_t>(row) * a.row_stride + start + 4 * lane_in_team);
+            }
+#pragma unroll
+            for (int u = 0; u < kPerTrip; ++u) {
+                const float4 v = loaded[u];
+                bool finite = (v.x - v.x == 0.0f) && (v.y - v.y == 0.0f) && (v.z - v.z == 0.0f) && (v.w - v.w == 0.0f);
+                float low = fminf(fminf(v.x, v.y), fminf(v.z, v.w));
+                float high = fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w));
+#pragma unroll
+                for (int offset = 1; offset < LANES; offset <<= 1) {
+                    low = fminf(low, __shfl_xor(low, offset, 64));
+                    high = fmaxf(high, __shfl_xor(high, offset, 64));
+                    finite = __shfl_xor(static_cast<int>(finite), offset, 64) && finite;
+                }
+                const int identifier = first + u;
+                if (lane_in_team == 0 && identifier < a.total_groups) {
+                    const int row = identifier / a.groups_per_row;
+                    store_fit(a, static_cast<size_t>(row) * a.out_row_stride + (identifier - row * a.groups_per_row), low, high, finite);
+                }
+            }
+        }
+        return;
+    }
     for (int first = blockIdx.x * kTeams; first < a.total_groups; first += gridDim.x * kTeams) {
         const int wanted = first + threadIdx.x / LANES;
         const int identifier = wanted < a.total_groups ? wanted : a.total_groups - 1;
@@ -280,27 +417,7 @@ __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
             finite = __shfl_xor(static_cast<int>(finite), offset, 64) && finite;
         }
         if (lane_in_team != 0 || wanted >= a.total_groups) continue;
-        const size_t slot = static_cast<size_t>(row) * a.out_row_stride + (identifier - row * a.groups_per_row);
-        if (!finite) {  // fminf/fmaxf drop NaNs: report them as the tensor reductions would
-            a.scales[slot] = __builtin_nanf("");
-            if (a.zeros) a.zeros[slot] = __builtin_nanf("");
-            continue;
-        }
-        float scale, zero = 0.0f;
-        if (a.asym) {
-            scale = __fmul_rn(fmaxf(__fsub_rn(high, low), 1e-12f), a.reciprocal);
-            zero = __fsub_rn(low, __fmul_rn(a.value_minimum, scale));
-        } else {
-            scale = __fmul_rn(fmaxf(fmaxf(high, -low), 1e-12f), a.reciprocal);
-        }
-        a.scales[slot] = mk_rounded_scale(scale, a.format);
-        if (a.zeros) {
-            if (a.store_zero) {
-                const float magnitude = mk_rounded_scale(fmaxf(fabsf(zero), 1e-12f), a.format);
-                zero = zero > 0.0f ? magnitude : (zero < 0.0f ? -magnitude : 0.0f);
-            }
-            a.zeros[slot] = zero;
-        }
+        store_fit(a, static_cast<size_t>(row) * a.out_row_stride + (identifier - row * a.groups_per_row), low, high, finite);
     }
 }
 
