@@ -146,7 +146,7 @@ class PackedLinear(nn.Module):
         _, tensors, constants = launch
         status = native.library().mk_packed_matvec(
             inputs.data_ptr(), native.DTYPE_CODES[inputs.dtype], *tensors, output.data_ptr(), rows, *constants,
-            torch.cuda.current_stream(inputs.device).cuda_stream)
+            native.current_stream(inputs.device))
         if status:
             native.check(status)
 

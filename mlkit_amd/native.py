@@ -149,7 +149,14 @@ def dtype_code(tensor: Tensor) -> int:
         raise ValueError(f"unsupported tensor dtype {tensor.dtype}") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream(device: torch.device) -> int:
+    """The raw handle of the device's current stream (a plain C call where torch offers one:
+    building a ``torch.cuda.Stream`` object costs several microseconds per launch)."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
 
 

@@ -222,7 +222,7 @@ class OnlineRotation:
                     tensor = tensor.contiguous()
                 output = torch.empty_like(tensor)
                 native.check(launch(tensor.data_ptr(), code, output.data_ptr(), code, tensor.numel() // width, width,
-                                    sign_pointer, None, width, scale, torch.cuda.current_stream(device).cuda_stream))
+                                    sign_pointer, None, width, scale, native.current_stream(device)))
                 return output
 
             whole.keeps = (signs,)
@@ -242,7 +242,7 @@ class OnlineRotation:
                 tensor = tensor.contiguous()
             output = torch.empty_like(tensor)
             native.check(launch(tensor.data_ptr(), code, output.data_ptr(), code, rows, order, power, basis_pointer, 0,
-                                sign_pointer, None, scale, torch.cuda.current_stream(device).cuda_stream))
+                                sign_pointer, None, scale, native.current_stream(device)))
             return output
 
         blocked.keeps = (signs, basis_on_device)
