@@ -268,6 +268,29 @@ def test_bf16_activations(bits, values, integer, scale_dtype):
             check(run_matvec(layer, x, scale_dtype=scale_dtype), layer, x, relative=8e-3)
 
 
+@pytest.mark.parametrize("width", [256, 512, 896, 1024, 1056, 4864])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("name,values,bits,integer", [
+    ("int4", INT4, 4, True), ("int2", scaling.int_values(2), 2, True), ("int3", scaling.int_values(3), 3, True),
+    ("nf4", scaling.NF4_VALUES, 4, False),
+])
+def test_short_rows_on_the_streaming_and_block_kernels(width, dtype, name, values, bits, integer):
+    """Rows of at most 512 / 1024 codes change the work split (two rows per wavefront step,
+    one or two sub-slices per wavefront); 1056 and 4864 leave part of the last wavefront
+    empty.  Symmetric and asymmetric, every row count up to eight, 48 and 4112 rows (the
+    four-row and the sixteen-row tiling)."""
+    tolerance = 1e-3 if dtype == torch.float16 else 8e-3
+    for rows in (48, 4112):
+        if rows == 4112 and (width not in (896, 1056) or name not in ("int4", "nf4")):
+            continue
+        weight = helpers.normal_weight(rows, width, seed=50 + width % 97, student_t=True)
+        for asym in (False, True):
+            layer = helpers.quantised_layer(weight, values, bits=bits, group=32, integer=integer, asym=asym)
+            for samples in (1, 2, 3, 4, 7, 8):
+                x = helpers.activations(samples, width, seed=60 + samples, dtype=dtype)
+                check(run_matvec(layer, x), layer, x, relative=tolerance)
+
+
 E4M3 = np.array(sorted({s * (m / 8 * 2.0 ** -6 if e == 0 else (1 + m / 8) * 2.0 ** (e - 7))
                         for s in (-1, 1) for e in range(15) for m in range(8)}), dtype=np.float32)
 
