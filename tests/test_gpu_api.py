@@ -75,6 +75,11 @@ def test_online_activation_reconstruction_equals_quantize_dequantize():
     (scaling.int_values(4), True, True, 64, 128, 64),      # two tiles per region
     (scaling.NF4_VALUES, False, False, 64, 64, 128),
     (scaling.int_values(3), True, False, 32, None, 128),   # one region: no refits
+    # one kernel per 128-column region (pending solve + scale fit + sweep), every group width it takes
+    (scaling.int_values(4), True, True, 64, 128, 128),
+    (scaling.int_values(4), True, False, 16, 128, 128),
+    (scaling.int_values(3), True, True, 32, 128, 256),
+    (scaling.int_values(8), True, True, 128, 128, 128),
 ])
 def test_gptq_on_device_matches_oracle_sweep(values, integer, asym, group, refit, block, rng):
     rows, width = 80, 512
