@@ -1,0 +1,150 @@
+// Diagonal-block step of a blocked Cholesky factorisation on gfx950.
+//
+// The error-feedback coefficients are U blockdiag(U)^-1 for the damped Hessian H = U^T U
+// (K up to 16384).  The library factorisation spends most of its time in its small
+// unblocked panel kernel, so the blocked algorithm is driven from the host with library
+// triangular solves and matrix products for the block rows and the trailing updates, and
+// this file supplies the part that is neither: one workgroup factors a diagonal block of at
+// most 128 x 128 in LDS.
+//
+// Replaces the `torch.linalg.cholesky_ex` call of `feedback_coefficients`
+// (quantization/algorithms/error_feedback.py:37-83 in /root/reference/src/mlkit) for large
+// matrices on the device.
+
+#include "mk_common.h"
+
+#include <type_traits>
+
+namespace {
+
+constexpr int kBlock = 128;
+constexpr int kThreads = 256;
+
+struct BlockArgs {
+    float *matrix;       // the block's top-left element; row-major with `leading` floats per row
+    long long leading;
+    int size;            // rows = columns of the block, 1 ... 128
+    int first_column;    // index of the block's first column in the whole matrix (for status)
+    int *status;         // stays 0, or becomes 1 + the column whose pivot is not positive
+};
+
+constexpr int kTile = kBlock / 16;
+
+// Steps 16 SIXTEEN ... 16 SIXTEEN + 15 of the factorisation below (the pivot rows of these
+// steps sit in register row SIXTEEN of their owners).  False after a pivot that is not
+// positive and finite, which every thread sees in the same step.
+template <int SIXTEEN>
+__device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[kTile][kTile], float (&pivot_row)[2][kBlock],
+                                              int tx, int ty) {
+#pragma unroll 1
+    for (int lane = 0; lane < 16; ++lane) {
+        const int j = 16 * SIXTEEN + lane;
+        const float *row = pivot_row[j & 1];
+        const float pivot = row[j];
+        if (!(pivot > 0.0f) || !(pivot - pivot == 0.0f)) {
+            if (threadIdx.x == 0) *a.status = a.first_column + j + 1;
+            return false;
+        }
+        const float reciprocal = 1.0f / sqrtf(pivot);
+        float along_rows[kTile], along_columns[kTile];
+#pragma unroll
+        for (int u = 0; u < kTile; ++u) {
+            const int i = ty + 16 * u;
+            along_rows[u] = i > j ? row[i] * reciprocal : 0.0f;      // U[j][i]; zero keeps rows <= j as they are
+            along_columns[u] = row[tx + 16 * u] * reciprocal;        // U[j][k]
+        }
+        // The pivot row's owners keep the scaled row (their entries of columns < j are zeros
+        // of the lower triangle and stay zero).
+        if (ty == lane) {
+#pragma unroll
+            for (int v = 0; v < kTile; ++v) mine[SIXTEEN][v] = along_columns[v];
+        }
+#pragma unroll
+        for (int u = 0; u < kTile; ++u)
+#pragma unroll
+            for (int v = 0; v < kTile; ++v) mine[u][v] -= along_rows[u] * along_columns[v];
+        // Row j + 1 is final now: its owners publish it for the next step.
+        float *next = pivot_row[(j + 1) & 1];
+        if (lane < 15) {
+            if (ty == lane + 1) {
+#pragma unroll
+                for (int v = 0; v < kTile; ++v) next[tx + 16 * v] = mine[SIXTEEN][v];
+            }
+        } else if constexpr (SIXTEEN + 1 < kTile) {
+            if (ty == 0) {
+#pragma unroll
+                for (int v = 0; v < kTile; ++v) next[tx + 16 * v] = mine[SIXTEEN + 1][v];
+            }
+        }
+        __syncthreads();
+    }
+    return true;
+}
+
+// In: the upper triangle of a symmetric positive definite block.  Out: U with block = U^T U
+// in the upper triangle, zeros below it.  A pivot that is not positive (or not finite)
+// records its column and leaves the block unspecified.
+//
+// Right-looking, one column per step.  The block lives in registers for the whole
+// factorisation: thread (ty, tx) of a 16 x 16 grid owns entries (ty + 16 u, tx + 16 v),
+// an 8 x 8 sub-block.  Per step only the pivot row travels: the sixteen threads that own it
+// put it (unscaled) into one of two LDS row buffers, one barrier later every thread reads
+// the sixteen entries it needs, scales them by 1 / sqrt(pivot) and subtracts their outer
+// product from its sub-block.  Rows up to the pivot row are masked out of the update by a
+// zero factor, so finished rows keep their values.
+__global__ void __launch_bounds__(kThreads) cholesky_block_kernel(const BlockArgs a) {
+    __shared__ float pivot_row[2][kBlock];
+    __shared__ int failed;
+    const int n = a.size;
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    if (threadIdx.x == 0) failed = *a.status != 0;   // an earlier block already failed: do nothing
+    float mine[kTile][kTile];
+#pragma unroll
+    for (int u = 0; u < kTile; ++u)
+#pragma unroll
+        for (int v = 0; v < kTile; ++v) {
+            const int row = ty + 16 * u, column = tx + 16 * v;
+            const bool inside = row < n && column < n && column >= row;
+            const float loaded = a.matrix[(inside ? row : 0) * a.leading + (inside ? column : 0)];
+            // Outside the block: an identity diagonal keeps every pivot of the padding at one.
+            mine[u][v] = inside ? loaded : (row == column ? 1.0f : 0.0f);
+        }
+    if (ty == 0) {
+#pragma unroll
+        for (int v = 0; v < kTile; ++v) pivot_row[0][tx + 16 * v] = mine[0][v];
+    }
+    __syncthreads();
+    if (failed) return;
+
+    // All 128 steps run (the padding is an identity): no data-dependent exit other than a bad pivot.
+    bool good = sixteen_steps<0>(a, mine, pivot_row, tx, ty);
+    good = good && sixteen_steps<1>(a, mine, pivot_row, tx, ty);
+    good = good && sixteen_steps<2>(a, mine, pivot_row, tx, ty);
+    good = good && sixteen_steps<3>(a, mine, pivot_row, tx, ty);
+    good = good && sixteen_steps<4>(a, mine, pivot_row, tx, ty);
+    good = good && sixteen_steps<5>(a, mine, pivot_row, tx, ty);
+    good = good && sixteen_steps<6>(a, mine, pivot_row, tx, ty);
+    good = good && sixteen_steps<7>(a, mine, pivot_row, tx, ty);
+    if (!good) return;
+#pragma unroll
+    for (int u = 0; u < kTile; ++u)
+#pragma unroll
+        for (int v = 0; v < kTile; ++v) {
+            const int row = ty + 16 * u, column = tx + 16 * v;
+            if (row < n && column < n) a.matrix[row * a.leading + column] = column >= row ? mine[u][v] : 0.0f;
+        }
+}
+
+}  // namespace
+
+extern "C" int mk_cholesky_block(float *matrix, long long leading, int size, int first_column, int *status,
+                                 void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(matrix && status, MK_ERR_INVALID, "mk_cholesky_block: null pointer");
+    MK_REQUIRE(size >= 1 && size <= kBlock, MK_ERR_UNSUPPORTED, "mk_cholesky_block: blocks of 1 to %d rows (got %d)", kBlock, size);
+    MK_REQUIRE(leading >= size && first_column >= 0, MK_ERR_INVALID, "mk_cholesky_block: rows overlap");
+    BlockArgs a{matrix, leading, size, first_column, status};
+    hipLaunchKernelGGL(cholesky_block_kernel, dim3(1), dim3(kThreads), 0, stream, a);
+    MK_LAUNCH_CHECK("mk_cholesky_block");
+    return MK_OK;
+}

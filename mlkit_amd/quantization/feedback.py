@@ -31,6 +31,56 @@ MAXIMUM_FUSED_TILE = 1024
 DEFERRED_TILES = 4  # tiles whose far-column updates are applied in one pass on the device
 
 
+BLOCKED_FACTORIZATION_WIDTH = 1024  # narrower matrices go to the library factorisation
+FACTORIZATION_BLOCK = 128           # one workgroup factors a diagonal block of this size
+FACTORIZATION_PANEL = 512           # rank of the trailing updates of the whole matrix
+TRAILING_BAND = 2048                # rows per product of a trailing update (only the upper triangle is needed)
+
+
+def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
+    """``(U, status)`` with ``matrix = U^T U`` for a symmetric positive definite FP32 matrix on a
+    HIP device, factored in place.  Two levels of right-looking blocking: panels of 512 columns
+    update the rest of the matrix (a rank-512 product reads and writes the trailing matrix a
+    quarter as often as rank-128 ones would); inside a panel's diagonal block the same scheme
+    runs with 128-column blocks, whose diagonal blocks ``mk_cholesky_block`` factors.
+    Block rows are triangular solves.  ``status`` is a device scalar: zero, or one plus the
+    first column whose pivot is not positive (as ``torch.linalg.cholesky_ex`` reports it)."""
+    from mlkit_amd import native
+
+    width = matrix.shape[0]
+    device = matrix.device
+    library = native.library()
+    status = torch.zeros((), dtype=torch.int32, device=device)
+    stream = native.current_stream(device)
+
+    def eliminate(start: int, stop: int, limit: int) -> None:
+        """Rows start:stop hold a factored diagonal block: finish their block row up to
+        column ``limit`` and subtract its outer product from the square below and right."""
+        if stop >= limit:
+            return
+        row_block = matrix[start:stop, stop:limit]
+        solved = torch.linalg.solve_triangular(matrix[start:stop, start:stop].T, row_block, upper=False)
+        row_block.copy_(solved)                                            # U_jr = U_jj^-T A_jr
+        # A_rr -= U_jr^T U_jr on and above the diagonal, in bands of rows (a band's product also
+        # covers the part of its diagonal square below the diagonal, which is never read)
+        for band_start in range(stop, limit, TRAILING_BAND):
+            band_stop = min(limit, band_start + TRAILING_BAND)
+            matrix[band_start:band_stop, band_start:limit].addmm_(
+                matrix[start:stop, band_start:band_stop].T, matrix[start:stop, band_start:limit], alpha=-1.0)
+
+    for panel_start in range(0, width, FACTORIZATION_PANEL):
+        panel_stop = min(width, panel_start + FACTORIZATION_PANEL)
+        for start in range(panel_start, panel_stop, FACTORIZATION_BLOCK):
+            stop = min(panel_stop, start + FACTORIZATION_BLOCK)
+            native.check(library.mk_cholesky_block(matrix[start, start:].data_ptr(), width, stop - start, start,
+                                                   status.data_ptr(), stream))
+            eliminate(start, stop, panel_stop)
+        # the diagonal block's lower triangle holds leftovers of the products above
+        matrix[panel_start:panel_stop, panel_start:panel_stop].triu_()
+        eliminate(panel_start, panel_stop, width)
+    return matrix, status
+
+
 def feedback_coefficients(hessian: Tensor, step: int, *, damp: float = 0.01,
                           permutation: Tensor | None = None) -> tuple[Tensor, int]:
     """``(A, status)``: ``A = R blockdiag(R)^-1`` for the damped ``H = R R^T``, row-major;
@@ -49,7 +99,11 @@ def feedback_coefficients(hessian: Tensor, step: int, *, damp: float = 0.01,
     diagonal = flipped.diagonal()
     diagonal.masked_fill_(diagonal == 0, 1)
     diagonal.add_(damp * diagonal.mean().clamp_min(1e-12))
-    if width >= UPPER_FACTORIZATION_WIDTH:
+    if width >= BLOCKED_FACTORIZATION_WIDTH and flipped.is_cuda and flipped.dtype == torch.float32:
+        flipped = flipped.contiguous()  # a fresh copy (flip / indexing never alias the caller's matrix)
+        factor, status = _blocked_upper_factor(flipped)
+        lower = factor.T
+    elif width >= UPPER_FACTORIZATION_WIDTH:
         # column-major solvers factor the upper triangle faster; its transpose is the lower factor
         factor, status = torch.linalg.cholesky_ex(flipped, upper=True)
         lower = factor.T

@@ -130,3 +130,45 @@ def test_chained_block_update_equals_tile_after_tile(rows, width, first, chain, 
     updated = dev(feedback)
     error_feedback.block_update_range(updated, dev(weight), dev(output), dev(coeff), first, chain, chains, begin, end)
     np.testing.assert_array_equal(host(updated), expected)
+
+
+@pytest.mark.parametrize("width,step", [(1024, 1), (1100, 1), (1536, 8), (2304, 1)])
+def test_blocked_factorisation_matches_the_float64_coefficients(width, step):
+    """`feedback_coefficients` on the device factors matrices of 1024 columns and more block by
+    block (`mk_cholesky_block` plus matrix products).  Against the float64 definition at the
+    reference's tolerance (tests/quantization/test_algorithms.py:142-166, rtol 1e-3 on the
+    upper triangle), and against the library factorisation of the same matrix."""
+    import mlkit_amd as mk
+
+    rng = np.random.default_rng(width)
+    inputs = rng.standard_normal((2 * width, width)).astype(np.float32)
+    inputs[:, ::13] *= 6
+    inputs[:, 5] = 0   # a dead channel
+    hessian = (inputs.T @ inputs / inputs.shape[0]).astype(np.float32)
+    result, status = mk.feedback_coefficients(dev(hessian).clone(), step)
+    assert status == 0
+    expected, expected_status = oracle_feedback.coefficients(hessian) if step == 1 else (None, 0)
+    assert expected_status == 0
+    if step == 1:
+        upper = np.triu(np.ones((width, width), dtype=bool), 1)
+        np.testing.assert_allclose(host(result)[upper], expected[upper], rtol=1e-3, atol=2e-6)
+    library, library_status = mk.feedback_coefficients(torch.from_numpy(hessian).clone(), step)   # CPU: LAPACK
+    assert library_status == 0
+    blocks = np.kron(np.eye(width // step, dtype=bool), np.ones((step, step), dtype=bool))
+    outside = np.triu(np.ones((width, width), dtype=bool), 1) & ~blocks
+    np.testing.assert_allclose(host(result)[outside], library.numpy()[outside], rtol=1e-3, atol=2e-6)
+
+
+def test_blocked_factorisation_reports_an_indefinite_matrix():
+    import mlkit_amd as mk
+
+    width = 1280
+    rng = np.random.default_rng(3)
+    inputs = rng.standard_normal((width // 2, width)).astype(np.float32)   # rank deficient
+    hessian = (inputs.T @ inputs).astype(np.float32)
+    hessian[700, 700] = -5000.0
+    _, status = mk.feedback_coefficients(dev(hessian).clone(), 1, damp=0.0)
+    assert status != 0
+    quantizer = mk.gptq(mk.int(4, group=128))
+    with pytest.raises(ValueError, match="positive definite"):
+        quantizer(dev(np.zeros((8, width), dtype=np.float32)), mk.Ctx("layer", H=dev(hessian)))
