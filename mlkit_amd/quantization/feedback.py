@@ -58,9 +58,11 @@ def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
         column ``limit`` and subtract its outer product from the square below and right."""
         if stop >= limit:
             return
+        # U_jr = U_jj^-T A_jr, solved in place as X U_jj = A_jr^T: the transposed view of the
+        # row-major block row is column-major, the layout the solver works in
         row_block = matrix[start:stop, stop:limit]
-        solved = torch.linalg.solve_triangular(matrix[start:stop, start:stop].T, row_block, upper=False)
-        row_block.copy_(solved)                                            # U_jr = U_jj^-T A_jr
+        torch.linalg.solve_triangular(matrix[start:stop, start:stop], row_block.T, upper=True, left=False,
+                                      out=row_block.T)
         # A_rr -= U_jr^T U_jr on and above the diagonal, in bands of rows (a band's product also
         # covers the part of its diagonal square below the diagonal, which is never read)
         for band_start in range(stop, limit, TRAILING_BAND):
