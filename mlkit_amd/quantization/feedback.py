@@ -35,6 +35,7 @@ BLOCKED_FACTORIZATION_WIDTH = 1024  # narrower matrices go to the library factor
 FACTORIZATION_BLOCK = 128           # one workgroup factors a diagonal block of this size
 FACTORIZATION_PANEL = 512           # rank of the trailing updates of the whole matrix
 TRAILING_BAND = 2048                # rows per product of a trailing update (only the upper triangle is needed)
+LOOK_AHEAD_WIDTH = 8192             # from here on the far part of a trailing update runs on a second stream
 
 
 def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
@@ -43,43 +44,73 @@ def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
     update the rest of the matrix (a rank-512 product reads and writes the trailing matrix a
     quarter as often as rank-128 ones would); inside a panel's diagonal block the same scheme
     runs with 128-column blocks, whose diagonal blocks ``mk_cholesky_block`` factors.
-    Block rows are triangular solves.  ``status`` is a device scalar: zero, or one plus the
-    first column whose pivot is not positive (as ``torch.linalg.cholesky_ex`` reports it)."""
+    Block rows are triangular solves.
+
+    Look-ahead: of a panel's trailing update only the band of rows the next panel consists of
+    runs on the current stream; the rest runs on a second stream while the next panel's
+    diagonal block, a chain of small dependent kernels, is factored.  Events fix the order in
+    which updates reach every entry, so results do not depend on timing.
+
+    ``status`` is a device scalar: zero, or one plus the first column whose pivot is not
+    positive (as ``torch.linalg.cholesky_ex`` reports it)."""
     from mlkit_amd import native
 
     width = matrix.shape[0]
     device = matrix.device
     library = native.library()
     status = torch.zeros((), dtype=torch.int32, device=device)
-    stream = native.current_stream(device)
+    main = torch.cuda.current_stream(device)
+    look_ahead = width >= LOOK_AHEAD_WIDTH   # narrower: the event traffic costs more than it hides
+    side = torch.cuda.Stream(device) if look_ahead else None
 
-    def eliminate(start: int, stop: int, limit: int) -> None:
-        """Rows start:stop hold a factored diagonal block: finish their block row up to
-        column ``limit`` and subtract its outer product from the square below and right."""
-        if stop >= limit:
-            return
+    def solve_block_row(start: int, stop: int, limit: int) -> None:
         # U_jr = U_jj^-T A_jr, solved in place as X U_jj = A_jr^T: the transposed view of the
         # row-major block row is column-major, the layout the solver works in
         row_block = matrix[start:stop, stop:limit]
         torch.linalg.solve_triangular(matrix[start:stop, start:stop], row_block.T, upper=True, left=False,
                                       out=row_block.T)
-        # A_rr -= U_jr^T U_jr on and above the diagonal, in bands of rows (a band's product also
-        # covers the part of its diagonal square below the diagonal, which is never read)
-        for band_start in range(stop, limit, TRAILING_BAND):
-            band_stop = min(limit, band_start + TRAILING_BAND)
+
+    def subtract_outer_product(start: int, stop: int, first_row: int, last_row: int, limit: int) -> None:
+        """A[r, c] -= sum_k U[k, r] U[k, c] for k in start:stop, rows first_row:last_row, columns from
+        the row band's first column to ``limit``: bands of rows, so that little below the diagonal
+        is computed (what is, is never read)."""
+        for band_start in range(first_row, last_row, TRAILING_BAND):
+            band_stop = min(last_row, band_start + TRAILING_BAND)
             matrix[band_start:band_stop, band_start:limit].addmm_(
                 matrix[start:stop, band_start:band_stop].T, matrix[start:stop, band_start:limit], alpha=-1.0)
 
+    side_done = None
     for panel_start in range(0, width, FACTORIZATION_PANEL):
         panel_stop = min(width, panel_start + FACTORIZATION_PANEL)
+        raw_stream = native.current_stream(device)
         for start in range(panel_start, panel_stop, FACTORIZATION_BLOCK):
             stop = min(panel_stop, start + FACTORIZATION_BLOCK)
             native.check(library.mk_cholesky_block(matrix[start, start:].data_ptr(), width, stop - start, start,
-                                                   status.data_ptr(), stream))
-            eliminate(start, stop, panel_stop)
+                                                   status.data_ptr(), raw_stream))
+            if stop < panel_stop:
+                solve_block_row(start, stop, panel_stop)
+                subtract_outer_product(start, stop, stop, panel_stop, panel_stop)
         # the diagonal block's lower triangle holds leftovers of the products above
         matrix[panel_start:panel_stop, panel_start:panel_stop].triu_()
-        eliminate(panel_start, panel_stop, width)
+        if panel_stop == width:
+            break
+        solve_block_row(panel_start, panel_stop, width)
+        if not look_ahead:
+            subtract_outer_product(panel_start, panel_stop, panel_stop, width, width)
+            continue
+        row_ready = main.record_event()
+        # the rows of the next panel: here, after the second stream's earlier update of them
+        next_stop = min(width, panel_stop + FACTORIZATION_PANEL)
+        if side_done is not None:
+            main.wait_event(side_done)
+        subtract_outer_product(panel_start, panel_stop, panel_stop, next_stop, width)
+        if next_stop < width:
+            side.wait_event(row_ready)
+            with torch.cuda.stream(side):
+                subtract_outer_product(panel_start, panel_stop, next_stop, width, width)
+                side_done = side.record_event()
+    if side_done is not None:
+        main.wait_event(side_done)
     return matrix, status
 
 

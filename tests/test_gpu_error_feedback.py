@@ -159,6 +159,29 @@ def test_blocked_factorisation_matches_the_float64_coefficients(width, step):
     np.testing.assert_allclose(host(result)[outside], library.numpy()[outside], rtol=1e-3, atol=2e-6)
 
 
+@pytest.mark.parametrize("width", [1664, 2304])
+def test_look_ahead_factorisation_equals_the_one_stream_order(width, monkeypatch):
+    """From `LOOK_AHEAD_WIDTH` columns on, the far part of every trailing update runs on a second
+    stream; events keep the order in which updates reach an entry, so the coefficients (the
+    entries above the diagonal; below it both leave leftovers) are the same bit for bit.
+    Twice, because a race would not show every time."""
+    import mlkit_amd as mk
+    from mlkit_amd.quantization import feedback
+
+    rng = np.random.default_rng(width + 1)
+    inputs = rng.standard_normal((2 * width, width)).astype(np.float32)
+    inputs[:, ::7] *= 4
+    hessian = dev((inputs.T @ inputs / inputs.shape[0]).astype(np.float32))
+    monkeypatch.setattr(feedback, "LOOK_AHEAD_WIDTH", 1 << 30)
+    expected, status = mk.feedback_coefficients(hessian.clone(), 1)
+    assert status == 0
+    monkeypatch.setattr(feedback, "LOOK_AHEAD_WIDTH", 1024)
+    for _ in range(2):
+        result, status = mk.feedback_coefficients(hessian.clone(), 1)
+        assert status == 0
+        np.testing.assert_array_equal(np.triu(host(result), 1), np.triu(host(expected), 1))
+
+
 def test_blocked_factorisation_reports_an_indefinite_matrix():
     import mlkit_amd as mk
 
