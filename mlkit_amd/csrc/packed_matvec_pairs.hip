@@ -38,9 +38,18 @@ __device__ __forceinline__ float side_value(uint16_t raw, int dtype) {
     return dtype == MK_F16 ? from_half : from_brain;
 }
 
-template <int MT>
+// Rows of a workgroup of the v_dot2 kernel.  A single sample with long rows leaves the
+// wavefronts waiting on table lookups, so its rows are spread over twice as many workgroups
+// (two per CU at 4096 rows); short rows keep sixteen rows per table fill.
+constexpr int kShortTileRows = 8;
+constexpr int kShortTileWidth = 4096;
+inline int tile_rows(const Stream4Args &a) {
+    return a.samples == 1 && a.width >= kShortTileWidth ? kShortTileRows : kPairRows;
+}
+
+template <int MT, int ROWS>
 constexpr int pair_reduce_rows() {
-    return kPairRows * MT <= 64 ? kPairRows : 64 / MT;
+    return ROWS * MT <= 64 ? ROWS : 64 / MT;
 }
 
 // LOOKUP = codes decoded per table read: 1 (an entry is one 16-bit value; two reads make a
@@ -102,16 +111,17 @@ __device__ __forceinline__ void fill_table(uint32_t *table, const Stream4Args &a
     }
 }
 
-template <int BITS, int MT, bool HAS_ZERO, int XT, int LOOKUP>
+template <int BITS, int MT, bool HAS_ZERO, int XT, int LOOKUP, int ROWS>
 __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
     constexpr int kLookup = LOOKUP;
+    constexpr int kPairRows = ROWS;
     constexpr int kPairAhead = rows_in_flight<BITS>();
     constexpr int kEntries = 1 << (kLookup * BITS);
     constexpr int kTableWords = kEntries * kLookup / 2;
     constexpr int kEntryWords = kLookup >= 2 ? kLookup / 2 : 1;
     __shared__ __attribute__((aligned(8))) uint32_t table[kTableWords];  // 16-bit values, pairs or double pairs
     __shared__ float partials[64 * 8];    // [row sum][wavefront]
-    constexpr int kReduceRows = pair_reduce_rows<MT>();
+    constexpr int kReduceRows = pair_reduce_rows<MT, ROWS>();
     constexpr int kSums = kReduceRows * MT;
 
     const int tid = threadIdx.x;
@@ -454,10 +464,19 @@ template <int BITS, int MT, int XT, int LOOKUP>
 void launch_tile_with(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
+    if constexpr (MT == 1) {
+        if (tile_rows(a) == kShortTileRows) {
+            if (a.zeros)
+                hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP, kShortTileRows>), grid, block, 0, stream, a);
+            else
+                hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, LOOKUP, kShortTileRows>), grid, block, 0, stream, a);
+            return;
+        }
+    }
     if (a.zeros)
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP, kPairRows>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, LOOKUP>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, LOOKUP, kPairRows>), grid, block, 0, stream, a);
 }
 
 // Field width per code width: the widest whose table a workgroup fills quickly.
@@ -534,7 +553,8 @@ bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype)
 
 // Multiplies rows [0, 16 * tiles); returns the number of rows covered.
 int pairs_launch(const Stream4Args &a, hipStream_t stream) {
-    const int tiles = a.rows / kPairRows;
+    const int tile = tile_rows(a);
+    const int tiles = a.rows / tile;
     if (tiles == 0) return 0;
     switch (a.bits) {
         case 2: launch_bits<2>(a, tiles, stream); break;
@@ -545,7 +565,7 @@ int pairs_launch(const Stream4Args &a, hipStream_t stream) {
         case 7: launch_bits<7>(a, tiles, stream); break;
         default: launch_bits<8>(a, tiles, stream); break;
     }
-    return tiles * kPairRows;
+    return tiles * tile;
 }
 
 }  // namespace mk_matvec
