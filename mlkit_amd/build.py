@@ -60,13 +60,15 @@ def _compile(unit: tuple[str, pathlib.Path, list[str]]) -> tuple[str, float, str
     return name, time.time() - started, log
 
 
-def build(verbose: bool = True, jobs: int | None = None) -> pathlib.Path:
-    """Compile all units and link the library; returns its path."""
+def build(verbose: bool = True, jobs: int | None = None, only: list[str] | None = None) -> pathlib.Path:
+    """Compile all units (or, while developing, just the units named in ``only``, reusing the
+    other objects of an earlier full build) and link the library; returns its path."""
     OBJECTS.mkdir(exist_ok=True)
     units = translation_units()
+    chosen = [unit for unit in units if not only or unit[0] in only]
     jobs = jobs or min(len(units), os.cpu_count() or 4, 16)
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        for name, seconds, log in pool.map(_compile, units):
+        for name, seconds, log in pool.map(_compile, chosen):
             if verbose:
                 print(f"[mlkit_amd.build] {name}.o  {seconds:6.1f}s", flush=True)
                 if log.strip():
@@ -82,5 +84,5 @@ def build(verbose: bool = True, jobs: int | None = None) -> pathlib.Path:
 
 
 if __name__ == "__main__":
-    build(verbose=True)
+    build(verbose=True, only=sys.argv[1:] or None)   # e.g. `python -m mlkit_amd.build hadamard`
     sys.exit(0)

@@ -194,6 +194,32 @@ __device__ __forceinline__ void chunk_from_slice(XChunk<XT> &x, const uint32_t *
     }
 }
 
+// The matrix-core kernels park the slices of four samples side by side, unpadded: quarter q
+// of chunk c sits at 16-byte granule 4 c + (q ^ ((c >> 2) & 3)), so that sixteen lanes reading
+// one quarter of sixteen adjacent chunks still spread over all banks, and a sample's buffer
+// is four words longer than its slices, which staggers the four samples.
+constexpr int blocks_sample_words(int slices) {
+    return slices * 16 * 16 + 4;
+}
+
+__device__ __forceinline__ void park_piece_swizzled(uint32_t *slice, int i, int lane, mk_u32x4 piece) {
+    const int chunk = 16 * i + (lane >> 2), quarter = (lane & 3) ^ ((lane >> 4) & 3);
+    *reinterpret_cast<mk_u32x4 *>(slice + chunk * 16 + quarter * 4) = piece;
+}
+
+template <int XT>
+__device__ __forceinline__ void chunk_from_swizzled_slice(XChunk<XT> &x, const uint32_t *slice, int chunk_in_slice) {
+    const int turn = (chunk_in_slice >> 2) & 3;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const mk_u32x4 v = *reinterpret_cast<const mk_u32x4 *>(slice + chunk_in_slice * 16 + (i ^ turn) * 4);
+        x.r[4 * i + 0] = v.x;
+        x.r[4 * i + 1] = v.y;
+        x.r[4 * i + 2] = v.z;
+        x.r[4 * i + 3] = v.w;
+    }
+}
+
 // A 16-bit scale or offset as fp32; `dtype` (MK_F16 or MK_BF16) is uniform per launch.
 __device__ __forceinline__ float side_as_float(uint16_t raw, int dtype) {
     const float from_half = static_cast<float>(__builtin_bit_cast(_Float16, raw));

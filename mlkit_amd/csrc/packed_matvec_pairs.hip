@@ -271,13 +271,14 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
     __shared__ __attribute__((aligned(8))) uint32_t table[kTableWords];
     __shared__ float partials[SETS * kPairRows * 4 * 8];  // [set][row][sample in set][wavefront]
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
+    constexpr int kSampleWords = blocks_sample_words(SLICES);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int waves = blockDim.x >> 6;
     const int block = lane >> 2, t = lane & 3;
-    uint32_t *const x_slice = x_slices_storage + wave * kSliceWords;
+    uint32_t *const x_slice = x_slices_storage + wave * (4 * kSampleWords);   // one buffer per sample of a set
     const int row_base = blockIdx.x * kPairRows;
     const uint32_t row_bytes = (static_cast<uint32_t>(a.width) * BITS) >> 3;
     const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
@@ -303,8 +304,8 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
     }
     __syncthreads();  // the table is complete; also aligns the wavefronts before their loads
 
-    // Activations of sample t (and t + 4) for this lane's four chunks: each sample's slice is
-    // read coalesced and the four lanes in sixteen whose sample it is pick their chunks.
+    // Activations of sample t (and t + 4) for this lane's four chunks: the slices of a set's
+    // four samples are read coalesced and parked side by side; every lane picks its sample's chunks.
     XChunk<XT> x[SETS][kSlices];
 #pragma unroll
     for (int set = 0; set < SETS; ++set) {
@@ -317,14 +318,11 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
             for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(a, sample, wave * (512 * kSlices), i, lane);
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i) park_piece(x_slice, i, lane, pieces[j][i]);
-            if (t == j) {
+            for (int i = 0; i < kSlices; ++i) park_piece_swizzled(x_slice + j * kSampleWords, i, lane, pieces[j][i]);
 #pragma unroll
-                for (int s = 0; s < kSlices; ++s) chunk_from_slice(x[set][s], x_slice, s * 16 + block);
-            }
-        }
+        for (int s = 0; s < kSlices; ++s) chunk_from_swizzled_slice(x[set][s], x_slice + t * kSampleWords, s * 16 + block);
     }
     uint16_t scale_raw[kSteps], zero_raw[HAS_ZERO ? kSteps : 1];
 #pragma unroll
@@ -351,9 +349,12 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
         const bool sample_present = blockIdx.y * 4 * SETS + 4 * set + t < a.samples;
 #pragma unroll
         for (int s = 0; s < kSlices; ++s) {
-            const uint32_t keep = in_row[s] && sample_present ? 0xffffffffu : 0u;
+            const bool kept = in_row[s] && sample_present;
+            if (__builtin_amdgcn_ballot_w64(!kept) != 0) {  // uniform; rarely taken
+                const uint32_t keep = kept ? 0xffffffffu : 0u;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) x[set][s].r[i] &= keep;
+                for (int i = 0; i < 16; ++i) x[set][s].r[i] &= keep;
+            }
             x_sum[set][s] = HAS_ZERO ? chunk_sum<XT>(x[set][s]) : 0.0f;
         }
     }
@@ -446,11 +447,20 @@ template <int BITS, int SETS, int XT, int LOOKUP, int SLICES>
 void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
     const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
-    const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
-    if (a.zeros)
-        hipLaunchKernelGGL((pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP, SLICES>), grid, block, slices, stream, a);
-    else
-        hipLaunchKernelGGL((pairs_blocks_kernel<BITS, SETS, false, XT, LOOKUP, SLICES>), grid, block, slices, stream, a);
+    const size_t slices = static_cast<size_t>(block.x / 64) * 4 * blocks_sample_words(SLICES) * sizeof(uint32_t);
+    // More than 64 KB of dynamic LDS has to be allowed per kernel (static LDS counts against
+    // the CU's 160 KB too, so only what this launch needs is asked for).
+    auto launch = [&](auto kernel) {
+        static size_t allowed = 64 * 1024;
+        if (slices > allowed) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(slices));
+            allowed = slices;
+        }
+        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a);
+    };
+    if (a.zeros) launch(pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP, SLICES>);
+    else launch(pairs_blocks_kernel<BITS, SETS, false, XT, LOOKUP, SLICES>);
 }
 
 // Short rows get fewer sub-slices per wavefront, so that none lies wholly past the row's end.
@@ -509,7 +519,8 @@ void launch_blocks_as(const Stream4Args &a, int tiles, hipStream_t stream) {
     if constexpr (BITS == 2) {
         launch_blocks_with<BITS, SETS, XT, 4>(a, tiles, stream);
     } else if constexpr (BITS == 3) {
-        if (a.width >= 8192) launch_blocks_with<BITS, SETS, XT, 4>(a, tiles, stream);
+        // (eight wavefronts' activation buffers leave no room for the 32 KB table)
+        if (a.width >= 8192 && a.width <= 14336) launch_blocks_with<BITS, SETS, XT, 4>(a, tiles, stream);
         else launch_blocks_with<BITS, SETS, XT, 2>(a, tiles, stream);
     } else if constexpr (BITS <= 5) {
         launch_blocks_with<BITS, SETS, XT, 2>(a, tiles, stream);

@@ -248,10 +248,11 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     constexpr int kAhead = kSteps < 8 ? kSteps : 8;
     constexpr int kSums = ROWS;                     // per set and lane before the reduction
     __shared__ float partials[SETS * ROWS * 4 * 8];  // [set][row][sample in set][wavefront]
-    // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
-    // must not hold LDS for eight).
+    // Four activation buffers per wavefront (one per sample of a set), sized at launch (a
+    // workgroup of one wavefront must not hold LDS for eight).
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
-    uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
+    constexpr int kSampleWords = blocks_sample_words(SLICES);
+    uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * (4 * kSampleWords);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -283,8 +284,8 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     __syncthreads();  // aligns the workgroup's wavefronts before their first loads
 
     // Activations of sample t (and t + 4) for this lane's four chunks, 16 fp16 pairs each:
-    // the wavefront reads each sample's slice coalesced and the four lanes in sixteen whose
-    // sample it is pick their chunks out of LDS.
+    // the wavefront reads the slices of a set's four samples coalesced, parks them side by
+    // side in LDS, and every lane picks its sample's chunks.
     XChunk<XT> x[SETS][kSlices];
 #pragma unroll
     for (int set = 0; set < SETS; ++set) {
@@ -297,14 +298,11 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
             for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(a, sample, wave * (512 * kSlices), i, lane);
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i) park_piece(x_slice, i, lane, pieces[j][i]);
-            if (t == j) {
+            for (int i = 0; i < kSlices; ++i) park_piece_swizzled(x_slice + j * kSampleWords, i, lane, pieces[j][i]);
 #pragma unroll
-                for (int s = 0; s < kSlices; ++s) chunk_from_slice(x[set][s], x_slice, s * 16 + block);
-            }
-        }
+        for (int s = 0; s < kSlices; ++s) chunk_from_swizzled_slice(x[set][s], x_slice + t * kSampleWords, s * 16 + block);
     }
     // Scale (and offset) of row 4 q + t at every sub-slice, 2 bytes each.
     uint16_t scale_raw[kSteps], zero_raw[HAS_ZERO ? kSteps : 1];
@@ -332,9 +330,12 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
         const bool sample_present = blockIdx.y * 4 * SETS + 4 * set + t < a.samples;
 #pragma unroll
         for (int s = 0; s < kSlices; ++s) {
-            const uint32_t keep = in_row[s] && sample_present ? 0xffffffffu : 0u;
+            const bool kept = in_row[s] && sample_present;
+            if (__builtin_amdgcn_ballot_w64(!kept) != 0) {  // uniform; rarely taken
+                const uint32_t keep = kept ? 0xffffffffu : 0u;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) x[set][s].r[i] &= keep;
+                for (int i = 0; i < 16; ++i) x[set][s].r[i] &= keep;
+            }
             float code_free;
             if constexpr (XT == MK_F16) {
                 code_free = pair_for_nibbles(x[set][s], &x_sum[set][s]);
@@ -395,7 +396,6 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
                                                     code_offset[(step + kAhead) % kSlices]);
         // Row 4 q + r of the block: scale (and offset) come from lane r of the quad.
         const float scale = side_as_float(scale_raw[step], a.scale_dtype);
-        const float scaled_step = scale * a.grid_step;
         float zero = 0.0f;
         if constexpr (HAS_ZERO) zero = side_as_float(zero_raw[step], a.scale_dtype);
         auto add_row = [&](auto r) __attribute__((always_inline)) {
@@ -403,8 +403,7 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
 #pragma unroll
             for (int set = 0; set < SETS; ++set) {
                 float total = sums[set][4 * q + R];
-                total = __builtin_fmaf(quad_value<R>(scaled_step), dot[set][R], total);
-                total = __builtin_fmaf(quad_value<R>(scale), grid_term[set][s], total);
+                total = __builtin_fmaf(quad_value<R>(scale), __builtin_fmaf(a.grid_step, dot[set][R], grid_term[set][s]), total);
                 if constexpr (HAS_ZERO) total = __builtin_fmaf(quad_value<R>(zero), x_sum[set][s], total);
                 sums[set][4 * q + R] = total;
             }
@@ -443,17 +442,25 @@ template <int SETS, int ROWS, int SLICES>
 void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
     const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
-    const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
+    // at most 8 wavefronts x 4 samples x 4112 bytes = 129 KB of the CU's 160 KB
+    const size_t slices = static_cast<size_t>(block.x / 64) * 4 * blocks_sample_words(SLICES) * sizeof(uint32_t);
+    // More than 64 KB of dynamic LDS has to be allowed per kernel (static LDS counts against
+    // the CU's 160 KB too, so only what this launch needs is asked for).
+    auto launch = [&](auto kernel) {
+        static size_t allowed = 64 * 1024;
+        if (slices > allowed) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(slices));
+            allowed = slices;
+        }
+        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a);
+    };
     if (a.x_dtype == MK_F16) {
-        if (a.zeros)
-            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS, MK_F16, SLICES>), grid, block, slices, stream, a);
-        else
-            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS, MK_F16, SLICES>), grid, block, slices, stream, a);
+        if (a.zeros) launch(stream4_blocks_kernel<SETS, true, ROWS, MK_F16, SLICES>);
+        else launch(stream4_blocks_kernel<SETS, false, ROWS, MK_F16, SLICES>);
     } else {
-        if (a.zeros)
-            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, true, ROWS, MK_BF16, SLICES>), grid, block, slices, stream, a);
-        else
-            hipLaunchKernelGGL((stream4_blocks_kernel<SETS, false, ROWS, MK_BF16, SLICES>), grid, block, slices, stream, a);
+        if (a.zeros) launch(stream4_blocks_kernel<SETS, true, ROWS, MK_BF16, SLICES>);
+        else launch(stream4_blocks_kernel<SETS, false, ROWS, MK_BF16, SLICES>);
     }
 }
 

@@ -311,3 +311,17 @@ def test_wide_codes_on_the_table_kernel(name, values, bits, integer, width, dtyp
         for samples in (1, 8):
             x = helpers.activations(samples, width, seed=24 + samples, dtype=dtype)
             check(run_matvec(layer, x), layer, x, relative=tolerance)
+
+
+@pytest.mark.parametrize("name,values,bits,integer", [
+    ("int4", INT4, 4, True), ("int3", scaling.int_values(3), 3, True), ("nf4", scaling.NF4_VALUES, 4, False),
+    ("int6", scaling.int_values(6), 6, True),
+])
+def test_widest_rows_fill_the_lds_of_the_block_kernels(name, values, bits, integer, width=16384):
+    """K = 16384: eight wavefronts per workgroup, each parking the slices of four samples in
+    LDS beside the value table (the largest LDS footprint the matvec kernels ask for)."""
+    weight = helpers.normal_weight(48, width, seed=31, student_t=True)
+    layer = helpers.quantised_layer(weight, values, bits=bits, group=128, integer=integer, asym=False)
+    for samples in (1, 4, 8):
+        x = helpers.activations(samples, width, seed=32 + samples)
+        check(run_matvec(layer, x), layer, x)
