@@ -24,6 +24,7 @@ struct DecodeArgs {
     int scale_dtype, out_dtype;
     int bits, bytes_per_word, codes_per_word, uniform, n_values;
     float grid_min, grid_step;
+    int chunks_per_group_shift;   // log2(group / 32) when that is a power of two (31: one group per row), else -1
 };
 
 __global__ void packed_decode_kernel(const DecodeArgs a) {
@@ -64,45 +65,60 @@ __global__ void packed_decode_kernel(const DecodeArgs a) {
 // piece apart from the next chunk's, so both directions avoid bank conflicts) and every
 // store instruction writes 1 KB of adjacent bytes.  A wavefront's 64 chunks are adjacent
 // in the row-major output because rows are whole chunks.
-template <int BITS, int PIECES>
+//
+// OUT is the output type (MK_F32: eight 16-byte pieces per chunk, else four).  MODE fixes the
+// launch's uniform choices at compile time, because tested per element they cost more
+// instructions than the decoding: 0 leaves them to run time (scale groups that are not whole
+// chunks); 1 / 2: one scale per chunk, affine grid, without / with offsets; 3 / 4: the same
+// for a value table.
+template <int BITS, int OUT, int MODE>
 __global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeArgs a) {
+    constexpr int PIECES = OUT == MK_F32 ? 8 : 4;
+    constexpr bool kFixed = MODE != 0;
+    const bool uniform = kFixed ? MODE <= 2 : a.uniform != 0;
+    const bool has_zero = kFixed ? MODE % 2 == 0 : a.zeros != nullptr;
     __shared__ float table[1 << BITS];
     __shared__ mk_u32x4 exchange[4][64 * (PIECES + 1)];
-    if (!a.uniform) {
+    if (!uniform) {
         for (int i = threadIdx.x; i < (1 << BITS); i += blockDim.x) table[i] = i < a.n_values ? a.values[i] : 0.0f;
         __syncthreads();
     }
     const int lane = threadIdx.x & 63;
     mk_u32x4 *mine = exchange[threadIdx.x >> 6];
-    const int row_chunks = a.width / mk_matvec::kChunkCodes;
-    const size_t total = static_cast<size_t>(a.rows) * row_chunks;
-    const bool one_slot = a.group % mk_matvec::kChunkCodes == 0 || a.group >= a.width;
+    // Chunk indices fit 32 bits (the launcher checks): a 64-bit division per lane and trip
+    // would cost as much as decoding the chunk.
+    const uint32_t row_chunks = static_cast<uint32_t>(a.width) / mk_matvec::kChunkCodes;
+    const uint32_t total = static_cast<uint32_t>(a.rows) * row_chunks;
+    const bool one_slot = kFixed || a.group % mk_matvec::kChunkCodes == 0 || a.group >= a.width;
     // The trip count is uniform within a wavefront: lanes past the end repeat the last chunk
     // and store nothing.
-    for (size_t first_chunk = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) & ~static_cast<size_t>(63);
-         first_chunk < total; first_chunk += static_cast<size_t>(gridDim.x) * blockDim.x) {
-        const size_t wanted = first_chunk + lane;
-        const size_t chunk = wanted < total ? wanted : total - 1;
-        const size_t row = chunk / row_chunks;
-        const int first = static_cast<int>(chunk - row * row_chunks) * mk_matvec::kChunkCodes;
+    for (uint32_t first_chunk = (blockIdx.x * blockDim.x + threadIdx.x) & ~63u; first_chunk < total;
+         first_chunk += gridDim.x * blockDim.x) {
+        const uint32_t wanted = first_chunk + lane;
+        const uint32_t chunk = wanted < total ? wanted : total - 1;
+        const uint32_t row = chunk / row_chunks;
+        const uint32_t chunk_in_row = chunk - row * row_chunks;
+        const int first = static_cast<int>(chunk_in_row) * mk_matvec::kChunkCodes;
         mk_matvec::CodeChunk<BITS> codes;
-        mk_matvec::load_codes<BITS>(codes, a.packed + chunk * (4 * BITS));
-        size_t slot = row * a.groups + first / a.group;
+        mk_matvec::load_codes<BITS>(codes, a.packed + static_cast<size_t>(chunk) * (4 * BITS));
+        const uint32_t group_in_row = a.chunks_per_group_shift >= 0 ? chunk_in_row >> a.chunks_per_group_shift
+                                                                    : static_cast<uint32_t>(first) / static_cast<uint32_t>(a.group);
+        size_t slot = static_cast<size_t>(row) * a.groups + group_in_row;
         float scale = mk_load_as_float(a.scales, slot, a.scale_dtype);
-        float zero = a.zeros ? mk_load_as_float(a.zeros, slot, a.scale_dtype) : 0.0f;
+        float zero = has_zero ? mk_load_as_float(a.zeros, slot, a.scale_dtype) : 0.0f;
         float out[32];
 #pragma unroll
         for (int k = 0; k < 32; ++k) {
             if (!one_slot) {
-                slot = row * a.groups + (first + k) / a.group;
+                slot = static_cast<size_t>(row) * a.groups + (first + k) / a.group;
                 scale = mk_load_as_float(a.scales, slot, a.scale_dtype);
-                if (a.zeros) zero = mk_load_as_float(a.zeros, slot, a.scale_dtype);
+                if (has_zero) zero = mk_load_as_float(a.zeros, slot, a.scale_dtype);
             }
             const uint32_t code = mk_matvec::code_at<BITS>(codes, k);
-            float weight = a.uniform ? __fadd_rn(a.grid_min, __fmul_rn(static_cast<float>(code), a.grid_step))
-                                     : table[code];
+            float weight = uniform ? __fadd_rn(a.grid_min, __fmul_rn(static_cast<float>(code), a.grid_step))
+                                   : table[code];
             weight = __fmul_rn(weight, scale);
-            if (a.zeros) weight = __fadd_rn(weight, zero);
+            if (has_zero) weight = __fadd_rn(weight, zero);
             out[k] = weight;
         }
 #pragma unroll
@@ -115,7 +131,7 @@ __global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeA
 #pragma unroll
                 for (int h = 0; h < 4; ++h) {
                     const float low = out[8 * q + 2 * h], high = out[8 * q + 2 * h + 1];
-                    if (a.out_dtype == MK_F16) {
+                    if constexpr (OUT == MK_F16) {
                         const mk_h2 halves = {static_cast<_Float16>(low), static_cast<_Float16>(high)};
                         piece[h] = __builtin_bit_cast(uint32_t, halves);
                     } else {
@@ -126,8 +142,8 @@ __global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeA
             mine[lane * (PIECES + 1) + q] = piece;
         }
         // LDS operations of a wavefront complete in order: no barrier between the two loops.
-        mk_u32x4 *target = static_cast<mk_u32x4 *>(a.out) + first_chunk * PIECES;
-        const size_t pieces_left = (total - first_chunk) * PIECES;
+        mk_u32x4 *target = static_cast<mk_u32x4 *>(a.out) + static_cast<size_t>(first_chunk) * PIECES;
+        const size_t pieces_left = static_cast<size_t>(total - first_chunk) * PIECES;
 #pragma unroll
         for (int q = 0; q < PIECES; ++q) {
             const int index = q * 64 + lane;
@@ -137,15 +153,25 @@ __global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeA
     }
 }
 
-template <int BITS>
-void launch_chunks(const DecodeArgs &a, hipStream_t stream) {
+template <int BITS, int OUT>
+void launch_chunks_as(const DecodeArgs &a, hipStream_t stream) {
     const size_t chunks = static_cast<size_t>(a.rows) * (a.width / mk_matvec::kChunkCodes);
     size_t blocks = (chunks + 255) / 256;
     if (blocks > 256u * 64u) blocks = 256u * 64u;
-    if (a.out_dtype == MK_F32)
-        hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS, 8>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
-    else
-        hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS, 4>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+    const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+    const bool one_slot = a.group % mk_matvec::kChunkCodes == 0 || a.group >= a.width;
+    if (!one_slot) hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS, OUT, 0>), grid, block, 0, stream, a);
+    else if (a.uniform && !a.zeros) hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS, OUT, 1>), grid, block, 0, stream, a);
+    else if (a.uniform) hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS, OUT, 2>), grid, block, 0, stream, a);
+    else if (!a.zeros) hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS, OUT, 3>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((packed_decode_chunks_kernel<BITS, OUT, 4>), grid, block, 0, stream, a);
+}
+
+template <int BITS>
+void launch_chunks(const DecodeArgs &a, hipStream_t stream) {
+    if (a.out_dtype == MK_F32) launch_chunks_as<BITS, MK_F32>(a, stream);
+    else if (a.out_dtype == MK_F16) launch_chunks_as<BITS, MK_F16>(a, stream);
+    else launch_chunks_as<BITS, MK_BF16>(a, stream);
 }
 
 }  // namespace
@@ -174,8 +200,19 @@ extern "C" int mk_packed_decode(const uint8_t *packed, const void *scales, int s
     a.bytes_per_word = bits / divisor; a.codes_per_word = 8 / divisor; a.uniform = uniform;
     a.grid_min = grid_min; a.grid_step = grid_step;
     a.n_values = n_values;
+    a.chunks_per_group_shift = -1;
+    if (group >= input_width) {
+        a.chunks_per_group_shift = 31;
+    } else if (group % mk_matvec::kChunkCodes == 0) {
+        const int chunks_per_group = group / mk_matvec::kChunkCodes;
+        if ((chunks_per_group & (chunks_per_group - 1)) == 0) {
+            a.chunks_per_group_shift = 0;
+            while ((1 << a.chunks_per_group_shift) < chunks_per_group) ++a.chunks_per_group_shift;
+        }
+    }
     const bool wide = input_width % mk_matvec::kChunkCodes == 0 && (reinterpret_cast<uintptr_t>(packed) & 3u) == 0 &&
-                      (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && bits >= 2;
+                      (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && bits >= 2 &&
+                      static_cast<long long>(output_width) * (input_width / mk_matvec::kChunkCodes) < (1ll << 31) - (1 << 24);
     if (wide) {
         switch (bits) {
             case 2: launch_chunks<2>(a, stream); break;
