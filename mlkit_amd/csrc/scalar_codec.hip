@@ -13,6 +13,7 @@
 //   scalar_rounding.py:15-73   rounding helpers (device functions below)
 
 #include "mk_common.h"
+#include "packed_matvec_impl.h"   // lane_exchange
 
 namespace {
 
@@ -343,6 +344,28 @@ __device__ __forceinline__ void store_fit(const FitArgs &a, size_t slot, float l
     }
 }
 
+// Minimum, maximum and "all finite" over the LANES adjacent lanes of a team, by vector-ALU
+// lane moves (an LDS permute per step cost more than the loads of the group).
+template <int LANES>
+__device__ __forceinline__ void team_range(float &low, float &high, bool &finite, int lane) {
+    float bad = finite ? 0.0f : 1.0f;
+    auto stage = [&](auto s) __attribute__((always_inline)) {
+        constexpr int S = decltype(s)::value;
+        if constexpr ((1 << S) < LANES) {
+            low = fminf(low, mk_matvec::lane_exchange<S>(low, lane));
+            high = fmaxf(high, mk_matvec::lane_exchange<S>(high, lane));
+            bad = fmaxf(bad, mk_matvec::lane_exchange<S>(bad, lane));
+        }
+    };
+    stage(std::integral_constant<int, 0>{});
+    stage(std::integral_constant<int, 1>{});
+    stage(std::integral_constant<int, 2>{});
+    stage(std::integral_constant<int, 3>{});
+    stage(std::integral_constant<int, 4>{});
+    stage(std::integral_constant<int, 5>{});
+    finite = bad == 0.0f;
+}
+
 template <int LANES>
 __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
     constexpr int kTeams = kThreads / LANES;
@@ -354,14 +377,25 @@ __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
     if (single_load) {
         constexpr int kPerTrip = 4;
         const int team = threadIdx.x / LANES;
+        const int lane = threadIdx.x & 63;
         for (int first = (blockIdx.x * kTeams + team) * kPerTrip; first < a.total_groups; first += gridDim.x * kTeams * kPerTrip) {
+            // One division per trip: the trip's groups are adjacent, so their rows follow by
+            // stepping (a division per group cost more than the group's arithmetic).
+            int row[kPerTrip], in_row[kPerTrip];
+            row[0] = first / a.groups_per_row;
+            in_row[0] = first - row[0] * a.groups_per_row;
+#pragma unroll
+            for (int u = 1; u < kPerTrip; ++u) {
+                const bool wraps = in_row[u - 1] + 1 == a.groups_per_row;
+                row[u] = wraps ? row[u - 1] + 1 : row[u - 1];
+                in_row[u] = wraps ? 0 : in_row[u - 1] + 1;
+            }
             float4 loaded[kPerTrip];
 #pragma unroll
             for (int u = 0; u < kPerTrip; ++u) {
-                const int identifier = first + u < a.total_groups ? first + u : first;
-                const int row = identifier / a.groups_per_row;
-                const int start = (identifier - row * a.groups_per_row) * a.group;
-                loaded[u] = *reinterpret_cast<const float4 *>(a.value + static_cast<size_t>(row) * a.row_stride + start + 4 * lane_in_team);
+                const bool present = first + u < a.total_groups;
+                loaded[u] = *reinterpret_cast<const float4 *>(a.value + static_cast<size_t>(present ? row[u] : row[0]) * a.row_stride +
+                                                              (present ? in_row[u] : in_row[0]) * a.group + 4 * lane_in_team);
             }
 #pragma unroll
             for (int u = 0; u < kPerTrip; ++u) {
@@ -369,17 +403,9 @@ __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
                 bool finite = (v.x - v.x == 0.0f) && (v.y - v.y == 0.0f) && (v.z - v.z == 0.0f) && (v.w - v.w == 0.0f);
                 float low = fminf(fminf(v.x, v.y), fminf(v.z, v.w));
                 float high = fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w));
-#pragma unroll
-                for (int offset = 1; offset < LANES; offset <<= 1) {
-                    low = fminf(low, __shfl_xor(low, offset, 64));
-                    high = fmaxf(high, __shfl_xor(high, offset, 64));
-                    finite = __shfl_xor(static_cast<int>(finite), offset, 64) && finite;
-                }
-                const int identifier = first + u;
-                if (lane_in_team == 0 && identifier < a.total_groups) {
-                    const int row = identifier / a.groups_per_row;
-                    store_fit(a, static_cast<size_t>(row) * a.out_row_stride + (identifier - row * a.groups_per_row), low, high, finite);
-                }
+                team_range<LANES>(low, high, finite, lane);
+                if (lane_in_team == 0 && first + u < a.total_groups)
+                    store_fit(a, static_cast<size_t>(row[u]) * a.out_row_stride + in_row[u], low, high, finite);
             }
         }
         return;
@@ -410,12 +436,7 @@ __global__ void __launch_bounds__(kThreads) fit_kernel(const FitArgs a) {
                 high = fmaxf(high, v);
             }
         }
-#pragma unroll
-        for (int offset = 1; offset < LANES; offset <<= 1) {
-            low = fminf(low, __shfl_xor(low, offset, 64));
-            high = fmaxf(high, __shfl_xor(high, offset, 64));
-            finite = __shfl_xor(static_cast<int>(finite), offset, 64) && finite;
-        }
+        team_range<LANES>(low, high, finite, threadIdx.x & 63);
         if (lane_in_team != 0 || wanted >= a.total_groups) continue;
         store_fit(a, static_cast<size_t>(row) * a.out_row_stride + (identifier - row * a.groups_per_row), low, high, finite);
     }
