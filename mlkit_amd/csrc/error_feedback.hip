@@ -899,6 +899,59 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviation
             for (int r = 0; r < 16; ++r) *cell(mi, ni, r) = totals[mi][ni][r];
 }
 
+// One chain of exactly 128 columns over a few tiles (the update of a super-block's own later
+// tiles right after a tile's sweep): at most 96 of the 128 x 128 tiles above, each a
+// wavefront-serial chain of 256 MFMAs (16 K cycles), on a GPU with 1024 SIMDs.  Here a
+// workgroup owns a 64 x 64 tile and a wavefront one 32 x 32 accumulator (64 MFMAs), so the
+// same update spreads over four times as many SIMDs; both whole 128-deep operands and the
+// feedback tile are requested at once and waited for once.  Sums are formed exactly as
+// above (ascending k from zero, then added to feedback).
+constexpr int kWholeChain = 128;
+constexpr int kSmallTile = 64;
+
+__global__ void __launch_bounds__(kUpdateThreads) block_update_small_tile_kernel(const UpdateArgs a) {
+    __shared__ __attribute__((aligned(16))) float deviation[kWholeChain][kSmallTile];     // [k][row]
+    __shared__ __attribute__((aligned(16))) float coefficient[kWholeChain][kSmallTile];   // [k][column]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int row0 = blockIdx.y * kSmallTile;
+    const int column0 = a.column_begin + blockIdx.x * kSmallTile;
+    const int wave_row = (wave >> 1) * 32, wave_column = (wave & 1) * 32;
+
+    // One instruction moves four k rows of a tile (4 x 64 floats; lane l's 16 bytes land at
+    // 16 l from the uniform LDS address); a wavefront moves k rows 32 wave ... 32 wave + 31.
+    const uint32_t left_lane = static_cast<uint32_t>(lane >> 4) * a.rows + (lane & 15) * 4;
+    const uint32_t right_lane = static_cast<uint32_t>(lane >> 4) * a.width + (lane & 15) * 4;
+    const size_t k_base = static_cast<size_t>(a.first_column + wave * 32);
+    const float *left = a.deviation_t + row0 + k_base * a.rows;
+    const float *right = a.coeff + column0 + k_base * a.width;
+#pragma unroll
+    for (int four = 0; four < 8; ++four) {
+        rows_to_lds(left + static_cast<size_t>(4 * four) * a.rows + left_lane, &deviation[wave * 32 + 4 * four][0]);
+        rows_to_lds(right + static_cast<size_t>(4 * four) * a.width + right_lane, &coefficient[wave * 32 + 4 * four][0]);
+    }
+
+    // This lane's cells of the 32 x 32 tile: rows (lane / 32) * 4 + ..., column lane % 32.
+    float *cells = a.feedback + static_cast<size_t>(row0 + wave_row + (lane >> 5) * 4) * a.width + column0 + wave_column + (lane & 31);
+    mk_f32x16 totals, sums;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        totals[r] = cells[static_cast<size_t>((r >> 2) * 8 + (r & 3)) * a.width];
+        sums[r] = 0.0f;
+    }
+    wait_for_loads();
+    __syncthreads();
+
+    const float *left_rows = &deviation[0][0] + (lane >> 5) * kSmallTile + wave_row + (lane & 31);
+    const float *right_rows = &coefficient[0][0] + (lane >> 5) * kSmallTile + wave_column + (lane & 31);
+#pragma unroll 16
+    for (int kk = 0; kk < kWholeChain; kk += 2)
+        sums = __builtin_amdgcn_mfma_f32_32x32x2f32(left_rows[kk * kSmallTile], right_rows[kk * kSmallTile], sums, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        cells[static_cast<size_t>((r >> 2) * 8 + (r & 3)) * a.width] = __fadd_rn(totals[r], sums[r]);
+}
+
 int launch_update(const UpdateArgs &a, hipStream_t stream) {
     MK_REQUIRE(mk_cdiv(a.rows, kTileRows) <= 65535, MK_ERR_UNSUPPORTED, "mk_feedback_block_update: too many rows");
     const dim3 grid(mk_cdiv(a.column_end - a.column_begin, kTileColumns), mk_cdiv(a.rows, kTileRows));
@@ -910,7 +963,10 @@ int launch_update(const UpdateArgs &a, hipStream_t stream) {
                         a.width % 4 == 0 && a.column_begin % 4 == 0 &&
                         (a.column_end - a.column_begin) % kTileColumns == 0 && a.chain_width % kDepthChunk == 0 &&
                         a.chain_width / kDepthChunk >= 4;   // the first chain spans the four steps that read feedback
-    if (staged)
+    // (launches that leave most of the GPU idle with 128 x 128 tiles)
+    if (staged && a.chains == 1 && a.chain_width == kWholeChain && grid.x * grid.y <= 128)
+        hipLaunchKernelGGL(block_update_small_tile_kernel, dim3(grid.x * 2, grid.y * 2), dim3(kUpdateThreads), 0, stream, a);
+    else if (staged)
         hipLaunchKernelGGL(block_update_from_deviations_kernel, grid, dim3(kUpdateThreads), 0, stream, a);
     else if (vec)
         hipLaunchKernelGGL((block_update_kernel<true>), grid, dim3(kUpdateThreads), 0, stream, a);
