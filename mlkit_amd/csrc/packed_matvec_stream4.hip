@@ -108,12 +108,10 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int waves = blockDim.x >> 6;
-    const int row_base = blockIdx.x * ROWS;
     const int part = lane / kRowLanes;                   // this lane's row within a step
     const int chunk_lane = wave * 64 + (lane & (kRowLanes - 1));
     const int sample_base = blockIdx.y * MT;
     const uint32_t row_bytes = static_cast<uint32_t>(a.width) >> 1;
-    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
     // Lanes past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
     // activations: they add nothing.
     const bool in_row = chunk_lane * kChunkCodes < a.width;
@@ -136,6 +134,18 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
     const uint32_t group_offset = static_cast<uint32_t>(part) * scale_row_bytes +
                                   ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
+    // Short rows (two per wavefront step): a workgroup takes every gridDim.x-th tile of ROWS
+    // rows and prepares its activations once, during the first tile's loads; tall matrices
+    // then pay for that preparation once per workgroup instead of once per tile.
+    constexpr bool kStrided = PARTS == 2;
+    XChunk<XT> x[MT];
+    float x_sum[MT], grid_term[MT];
+    const int tiles = a.rows / ROWS;
+    int tile = blockIdx.x;
+    bool first_tile = true;
+    do {
+    const int row_base = tile * ROWS;
+    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
     const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
     const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
                                         : nullptr;
@@ -155,9 +165,9 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
         __builtin_amdgcn_sched_barrier(0);  // in row order
     }
 
+    if (first_tile) {  // uniform
     // Each lane's chunk of every sample, through the wavefront's LDS buffer (LDS operations
     // of a wavefront complete in order, so no barrier is needed).
-    XChunk<XT> x[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
 #pragma unroll
@@ -166,7 +176,6 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     }
 
     // sum_k (min + step c_k) x_k = step * dot + min * sum(x) - step * (code-free part of dot).
-    float x_sum[MT], grid_term[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const uint32_t keep = in_row && sample_base + m < a.samples ? 0xffffffffu : 0u;
@@ -181,6 +190,8 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
         }
         grid_term[m] = a.grid_min * x_sum[m] - a.grid_step * code_free;
     }
+    }
+    first_tile = false;
 
     float sums[kSums];
 #pragma unroll
@@ -221,6 +232,10 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
             store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
         }
     }
+    if constexpr (!kStrided) break;
+    __syncthreads();  // `partials` is reused by the next tile
+    tile += gridDim.x;
+    } while (tile < tiles);
 }
 
 // ---- two to eight samples: the dot products on the matrix cores ---------------------------
@@ -242,6 +257,8 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
 
 template <int SETS, bool HAS_ZERO, int ROWS, int XT, int SLICES>
 __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a) {
+    // Short rows (one or two sub-slices per wavefront) leave registers for the tile loop below.
+    constexpr bool kStrided = SLICES <= 2;
     constexpr int kQuads = ROWS / 4;
     constexpr int kSlices = SLICES;                 // sub-slices of sixteen chunks per wavefront (rows of up to 512 / 1024 codes: 1 / 2)
     constexpr int kSteps = kQuads * kSlices;        // code loads per lane
@@ -259,13 +276,8 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     const int wave = tid >> 6;
     const int waves = blockDim.x >> 6;
     const int block = lane >> 2, t = lane & 3;
-    const int row_base = blockIdx.x * ROWS;
     const uint32_t row_bytes = static_cast<uint32_t>(a.width) >> 1;
-    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
-    const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
-    const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
-                                        : nullptr;
 
     // Chunks past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
     // activations: they add nothing.
@@ -304,26 +316,6 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
 #pragma unroll
         for (int s = 0; s < kSlices; ++s) chunk_from_swizzled_slice(x[set][s], x_slice + t * kSampleWords, s * 16 + block);
     }
-    // Scale (and offset) of row 4 q + t at every sub-slice, 2 bytes each.
-    uint16_t scale_raw[kSteps], zero_raw[HAS_ZERO ? kSteps : 1];
-#pragma unroll
-    for (int q = 0; q < kQuads; ++q)
-#pragma unroll
-        for (int s = 0; s < kSlices; ++s) {
-            const size_t quad_offset = static_cast<size_t>(4 * q) * scale_row_bytes;
-            scale_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(scale_base + quad_offset + group_offset[s]);
-            if constexpr (HAS_ZERO)
-                zero_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(zero_base + quad_offset + group_offset[s]);
-        }
-    __builtin_amdgcn_sched_barrier(0);
-
-    CodeChunk<4> codes[kSteps];
-#pragma unroll
-    for (int step = 0; step < kAhead; ++step) {
-        load_codes<4>(codes[step], codes_base + static_cast<size_t>(4 * (step / kSlices)) * row_bytes + code_offset[step % kSlices]);
-        __builtin_amdgcn_sched_barrier(0);  // in order
-    }
-
     float x_sum[SETS][kSlices], grid_term[SETS][kSlices];
 #pragma unroll
     for (int set = 0; set < SETS; ++set) {
@@ -345,6 +337,37 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
             }
             grid_term[set][s] = a.grid_min * x_sum[set][s] - a.grid_step * code_free;
         }
+    }
+
+    // A workgroup prepares its activations once and then (short rows) takes every
+    // gridDim.x-th tile of ROWS rows: tall matrices, with many more tiles than the GPU holds
+    // workgroups, pay for the preparation once per workgroup instead of once per tile.
+    const int tiles = a.rows / ROWS;
+    int tile = blockIdx.x;
+    do {
+    const int row_base = tile * ROWS;
+    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
+    const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
+    const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
+                                        : nullptr;
+    // Scale (and offset) of row 4 q + t at every sub-slice, 2 bytes each.
+    uint16_t scale_raw[kSteps], zero_raw[HAS_ZERO ? kSteps : 1];
+#pragma unroll
+    for (int q = 0; q < kQuads; ++q)
+#pragma unroll
+        for (int s = 0; s < kSlices; ++s) {
+            const size_t quad_offset = static_cast<size_t>(4 * q) * scale_row_bytes;
+            scale_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(scale_base + quad_offset + group_offset[s]);
+            if constexpr (HAS_ZERO)
+                zero_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(zero_base + quad_offset + group_offset[s]);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+
+    CodeChunk<4> codes[kSteps];
+#pragma unroll
+    for (int step = 0; step < kAhead; ++step) {
+        load_codes<4>(codes[step], codes_base + static_cast<size_t>(4 * (step / kSlices)) * row_bytes + code_offset[step % kSlices]);
+        __builtin_amdgcn_sched_barrier(0);  // in order
     }
 
     float sums[SETS][kSums];
@@ -436,14 +459,33 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
             store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
         }
     }
+    if constexpr (!kStrided) break;
+    __syncthreads();  // `partials` is reused by the next tile
+    tile += gridDim.x;
+    } while (tile < tiles);
+}
+
+// The number of workgroups of `kernel` the GPU holds at once, asked of the runtime the first
+// time and remembered per kernel (`known`).
+template <typename Kernel>
+int resident_workgroups(Kernel kernel, int threads, size_t dynamic_lds, int &known) {
+    if (known == 0) {
+        int per_cu = 0, device = 0, units = 256;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess || per_cu < 1)
+            per_cu = 4;
+        if (hipGetDevice(&device) == hipSuccess)
+            (void)hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device);
+        known = per_cu * units;
+    }
+    return known;
 }
 
 template <int SETS, int ROWS, int SLICES>
 void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
-    const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
     const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
     // at most 8 wavefronts x 4 samples x 4112 bytes = 129 KB of the CU's 160 KB
     const size_t slices = static_cast<size_t>(block.x / 64) * 4 * blocks_sample_words(SLICES) * sizeof(uint32_t);
+    dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
     // More than 64 KB of dynamic LDS has to be allowed per kernel (static LDS counts against
     // the CU's 160 KB too, so only what this launch needs is asked for).
     auto launch = [&](auto kernel) {
@@ -452,6 +494,13 @@ void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
             (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(slices));
             allowed = slices;
+        }
+        if constexpr (SLICES <= 2) {
+            // Short rows: as many workgroups as the GPU holds at once; each walks the tiles
+            // with that stride.  (Asked of the runtime once per kernel and workgroup size.)
+            static int resident[3] = {0, 0, 0};
+            const int known = resident_workgroups(kernel, static_cast<int>(block.x), slices, resident[block.x / 64]);
+            if (static_cast<int>(grid.x) > known) grid.x = known;
         }
         hipLaunchKernelGGL(kernel, grid, block, slices, stream, a);
     };
@@ -475,19 +524,23 @@ void launch_blocks(const Stream4Args &a, int tiles, hipStream_t stream) {
 
 template <int MT, int ROWS, int PARTS>
 void launch_tile_parts(const Stream4Args &a, int tiles, hipStream_t stream) {
-    const dim3 grid(tiles, mk_cdiv(a.samples, MT));
+    dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
+    auto launch = [&](auto kernel) {
+        if constexpr (PARTS == 2) {  // short rows: one wavefront per workgroup, which walks the tiles
+            static int known = 0;
+            const int resident = resident_workgroups(kernel, static_cast<int>(block.x), slices, known);
+            if (static_cast<int>(grid.x) > resident) grid.x = resident;
+        }
+        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a);
+    };
     if (a.x_dtype == MK_F16) {
-        if (a.zeros)
-            hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS, MK_F16, PARTS>), grid, block, slices, stream, a);
-        else
-            hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS, MK_F16, PARTS>), grid, block, slices, stream, a);
+        if (a.zeros) launch(stream4_kernel<MT, true, ROWS, MK_F16, PARTS>);
+        else launch(stream4_kernel<MT, false, ROWS, MK_F16, PARTS>);
     } else {
-        if (a.zeros)
-            hipLaunchKernelGGL((stream4_kernel<MT, true, ROWS, MK_BF16, PARTS>), grid, block, slices, stream, a);
-        else
-            hipLaunchKernelGGL((stream4_kernel<MT, false, ROWS, MK_BF16, PARTS>), grid, block, slices, stream, a);
+        if (a.zeros) launch(stream4_kernel<MT, true, ROWS, MK_BF16, PARTS>);
+        else launch(stream4_kernel<MT, false, ROWS, MK_BF16, PARTS>);
     }
 }
 
