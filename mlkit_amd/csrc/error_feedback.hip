@@ -352,7 +352,17 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
     // One step: round column 16 t + owner of every row, push its deviation into the later
     // columns.  `owner` is an int or a std::integral_constant.  `coefficients` is row
     // 16 t + owner of the tile as this lane reads it.
-    auto advance = [&](auto slot, auto owner, const float *coefficients, auto solving) __attribute__((always_inline)) {
+    // WHOLE: the coefficient row of a step is read from LDS during the step before it (the
+    // addresses are known in advance; read inside the step, every step waited for LDS at the
+    // head of its dependent chain).  Even steps use one set of registers, odd steps the other.
+    float row_even[kSlots], row_odd[kSlots];
+    auto load_row = [&](auto slot, auto owner, float (&row)[kSlots]) __attribute__((always_inline)) {
+        constexpr int t = decltype(slot)::value;
+        const float *coefficients = staged + (kRowLanes * t + decltype(owner)::value) * kNarrowTile + p;
+#pragma unroll
+        for (int later = t; later < kSlots; ++later) row[later] = coefficients[kRowLanes * later];
+    };
+    auto advance = [&](auto slot, auto owner, const float *coefficients, auto solving, const float (&row_ready)[kSlots]) __attribute__((always_inline)) {
         constexpr int t = decltype(slot)::value;
         constexpr bool kSolving = decltype(solving)::value;
         float pushed;
@@ -375,7 +385,7 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
             // owner's hold whatever the matrix has there; only the solve still reads its
             // running values of such columns afterwards, so it masks them.
 #pragma unroll
-            for (int later = t; later < kSlots; ++later) row_of[later] = coefficients[kRowLanes * later];
+            for (int later = t; later < kSlots; ++later) row_of[later] = row_ready[later];
             if constexpr (kSolving) row_of[t] = p > static_cast<int>(owner) ? row_of[t] : 0.0f;
         } else {
             float4 low = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -389,7 +399,19 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
             running[later] = __fadd_rn(running[later], __fmul_rn(pushed, row_of[later]));
     };
     auto step_of_whole = [&](auto slot, auto owner, auto solving) __attribute__((always_inline)) {
-        advance(slot, owner, staged + (kRowLanes * decltype(slot)::value + decltype(owner)::value) * kNarrowTile + p, solving);
+        constexpr int t = decltype(slot)::value, o = decltype(owner)::value;
+        constexpr bool kLast = t == kSlots - 1 && o == kRowLanes - 1;
+        using NextSlot = std::integral_constant<int, (o == kRowLanes - 1 && !kLast) ? t + 1 : t>;
+        using NextOwner = std::integral_constant<int, o == kRowLanes - 1 ? 0 : o + 1>;
+        if constexpr (o & 1) {
+            if constexpr (!kLast) load_row(NextSlot{}, NextOwner{}, row_even);
+            __builtin_amdgcn_sched_barrier(0);  // the reads stay ahead of this step's arithmetic
+            advance(slot, owner, nullptr, solving, row_odd);
+        } else {
+            load_row(NextSlot{}, NextOwner{}, row_odd);
+            __builtin_amdgcn_sched_barrier(0);
+            advance(slot, owner, nullptr, solving, row_even);
+        }
     };
     auto slot_of_steps = [&](auto slot, auto solving) __attribute__((always_inline)) {
         constexpr int t = decltype(slot)::value;
@@ -415,12 +437,13 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
             if (more) fetch_slot(a, t + 1, held);
             const float *mine_in_chunk = staged + (t & 1) * kRowLanes * kNarrowTile + p * kSlots;
             const int owners = min(kRowLanes, a.tile_width - kRowLanes * t);
-            for (int owner = 0; owner < owners; ++owner) advance(slot, owner, mine_in_chunk + owner * kNarrowTile, solving);
+            for (int owner = 0; owner < owners; ++owner) advance(slot, owner, mine_in_chunk + owner * kNarrowTile, solving, row_even);
             if (more) keep_slot(a, t + 1, staged + ((t + 1) & 1) * kRowLanes * kNarrowTile, held);
             __syncthreads();
         }
     };
     auto all_slots = [&](auto solving) __attribute__((always_inline)) {
+        if constexpr (WHOLE) load_row(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, row_even);
         slot_of_steps(std::integral_constant<int, 0>{}, solving);
         slot_of_steps(std::integral_constant<int, 1>{}, solving);
         slot_of_steps(std::integral_constant<int, 2>{}, solving);
