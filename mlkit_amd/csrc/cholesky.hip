@@ -46,23 +46,25 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
             return false;
         }
         const float reciprocal = 1.0f / sqrtf(pivot);
+        // Register rows below SIXTEEN hold only rows <= j (finished); register columns below
+        // SIXTEEN only columns < j, which for the rows still changing lie below the diagonal
+        // (never read): neither takes part, so a step costs (8 - SIXTEEN)^2 multiply-adds.
         float along_rows[kTile], along_columns[kTile];
 #pragma unroll
-        for (int u = 0; u < kTile; ++u) {
+        for (int u = SIXTEEN; u < kTile; ++u) {
             const int i = ty + 16 * u;
             along_rows[u] = i > j ? row[i] * reciprocal : 0.0f;      // U[j][i]; zero keeps rows <= j as they are
             along_columns[u] = row[tx + 16 * u] * reciprocal;        // U[j][k]
         }
-        // The pivot row's owners keep the scaled row (their entries of columns < j are zeros
-        // of the lower triangle and stay zero).
+        // The pivot row's owners keep the scaled row.
         if (ty == lane) {
 #pragma unroll
-            for (int v = 0; v < kTile; ++v) mine[SIXTEEN][v] = along_columns[v];
+            for (int v = SIXTEEN; v < kTile; ++v) mine[SIXTEEN][v] = along_columns[v];
         }
 #pragma unroll
-        for (int u = 0; u < kTile; ++u)
+        for (int u = SIXTEEN; u < kTile; ++u)
 #pragma unroll
-            for (int v = 0; v < kTile; ++v) mine[u][v] -= along_rows[u] * along_columns[v];
+            for (int v = SIXTEEN; v < kTile; ++v) mine[u][v] -= along_rows[u] * along_columns[v];
         // Row j + 1 is final now: its owners publish it for the next step.
         float *next = pivot_row[(j + 1) & 1];
         if (lane < 15) {
