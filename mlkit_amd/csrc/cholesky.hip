@@ -45,7 +45,8 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
             if (threadIdx.x == 0) *a.status = a.first_column + j + 1;
             return false;
         }
-        const float reciprocal = 1.0f / sqrtf(pivot);
+        // (one v_rsq_f32, accurate to an ulp; the IEEE square root and division were a fifth of a step's chain)
+        const float reciprocal = __builtin_amdgcn_rsqf(pivot);
         // Register rows below SIXTEEN hold only rows <= j (finished); register columns below
         // SIXTEEN only columns < j, which for the rows still changing lie below the diagonal
         // (never read): neither takes part, so a step costs (8 - SIXTEEN)^2 multiply-adds.
@@ -70,12 +71,12 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
         if (lane < 15) {
             if (ty == lane + 1) {
 #pragma unroll
-                for (int v = 0; v < kTile; ++v) next[tx + 16 * v] = mine[SIXTEEN][v];
+                for (int v = SIXTEEN; v < kTile; ++v) next[tx + 16 * v] = mine[SIXTEEN][v];   // columns < j are not read
             }
         } else if constexpr (SIXTEEN + 1 < kTile) {
             if (ty == 0) {
 #pragma unroll
-                for (int v = 0; v < kTile; ++v) next[tx + 16 * v] = mine[SIXTEEN + 1][v];
+                for (int v = SIXTEEN + 1; v < kTile; ++v) next[tx + 16 * v] = mine[SIXTEEN + 1][v];
             }
         }
         __syncthreads();
