@@ -5,7 +5,7 @@
 // unblocked panel kernel, so the blocked algorithm is driven from the host with library
 // triangular solves and matrix products for the block rows and the trailing updates, and
 // this file supplies the part that is neither: one workgroup factors a diagonal block of at
-// most 128 x 128 in LDS.
+// most 128 x 128 in registers.
 //
 // Replaces the `torch.linalg.cholesky_ex` call of `feedback_coefficients`
 // (quantization/algorithms/error_feedback.py:37-83 in /root/reference/src/mlkit) for large
@@ -30,53 +30,76 @@ struct BlockArgs {
 
 constexpr int kTile = kBlock / 16;
 
-// Steps 16 SIXTEEN ... 16 SIXTEEN + 15 of the factorisation below (the pivot rows of these
-// steps sit in register row SIXTEEN of their owners).  False after a pivot that is not
-// positive and finite, which every thread sees in the same step.
+// Columns 16 SIXTEEN ... 16 SIXTEEN + 15 of the factorisation below, two per step (their rows
+// sit in register row SIXTEEN of their owners).  False after a pivot that is not positive and
+// finite, which every thread sees in the same step.
+//
+// A step takes rows j and j + 1 as the updates of columns < j left them (`pivot_rows`), and
+// every thread derives what it needs of the two finished rows itself:
+//   U[j][k]     = A[j][k] / sqrt(A[j][j])
+//   U[j+1][k]   = (A[j+1][k] - U[j][j+1] U[j][k]) / sqrt(A[j+1][j+1] - U[j][j+1]^2)
+// and subtracts both outer products from its sub-block: one LDS round trip and one barrier
+// per two columns.
 template <int SIXTEEN>
-__device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[kTile][kTile], float (&pivot_row)[2][kBlock],
-                                              int tx, int ty) {
+__device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[kTile][kTile],
+                                              float (&pivot_rows)[2][2][kBlock], int tx, int ty) {
 #pragma unroll 1
-    for (int lane = 0; lane < 16; ++lane) {
+    for (int lane = 0; lane < 16; lane += 2) {
         const int j = 16 * SIXTEEN + lane;
-        const float *row = pivot_row[j & 1];
-        const float pivot = row[j];
+        const float *first = pivot_rows[(j >> 1) & 1][0], *second = pivot_rows[(j >> 1) & 1][1];
+        const float pivot = first[j];
         if (!(pivot > 0.0f) || !(pivot - pivot == 0.0f)) {
             if (threadIdx.x == 0) *a.status = a.first_column + j + 1;
             return false;
         }
         // (one v_rsq_f32, accurate to an ulp; the IEEE square root and division were a fifth of a step's chain)
         const float reciprocal = __builtin_amdgcn_rsqf(pivot);
+        const float link = first[j + 1] * reciprocal;                 // U[j][j+1]
+        const float next_pivot = second[j + 1] - link * link;
+        if (!(next_pivot > 0.0f) || !(next_pivot - next_pivot == 0.0f)) {
+            if (threadIdx.x == 0) *a.status = a.first_column + j + 2;
+            return false;
+        }
+        const float next_reciprocal = __builtin_amdgcn_rsqf(next_pivot);
         // Register rows below SIXTEEN hold only rows <= j (finished); register columns below
         // SIXTEEN only columns < j, which for the rows still changing lie below the diagonal
-        // (never read): neither takes part, so a step costs (8 - SIXTEEN)^2 multiply-adds.
-        float along_rows[kTile], along_columns[kTile];
+        // (never read): neither takes part, so a step costs 2 (8 - SIXTEEN)^2 multiply-adds.
+        float rows_first[kTile], rows_second[kTile], columns_first[kTile], columns_second[kTile];
 #pragma unroll
         for (int u = SIXTEEN; u < kTile; ++u) {
-            const int i = ty + 16 * u;
-            along_rows[u] = i > j ? row[i] * reciprocal : 0.0f;      // U[j][i]; zero keeps rows <= j as they are
-            along_columns[u] = row[tx + 16 * u] * reciprocal;        // U[j][k]
+            const int i = ty + 16 * u, k = tx + 16 * u;
+            const float upper = first[i] * reciprocal;                                   // U[j][i]
+            const float lower = (second[i] - link * upper) * next_reciprocal;            // U[j+1][i]
+            rows_first[u] = i > j + 1 ? upper : 0.0f;   // zero keeps rows <= j + 1 as they are
+            rows_second[u] = i > j + 1 ? lower : 0.0f;
+            columns_first[u] = first[k] * reciprocal;                                    // U[j][k]
+            columns_second[u] = (second[k] - link * columns_first[u]) * next_reciprocal; // U[j+1][k]
         }
-        // The pivot row's owners keep the scaled row.
+        // The two rows' owners keep the finished rows.
         if (ty == lane) {
 #pragma unroll
-            for (int v = SIXTEEN; v < kTile; ++v) mine[SIXTEEN][v] = along_columns[v];
+            for (int v = SIXTEEN; v < kTile; ++v) mine[SIXTEEN][v] = columns_first[v];
+        }
+        if (ty == lane + 1) {
+#pragma unroll
+            for (int v = SIXTEEN; v < kTile; ++v) mine[SIXTEEN][v] = columns_second[v];
         }
 #pragma unroll
         for (int u = SIXTEEN; u < kTile; ++u)
 #pragma unroll
-            for (int v = SIXTEEN; v < kTile; ++v) mine[u][v] -= along_rows[u] * along_columns[v];
-        // Row j + 1 is final now: its owners publish it for the next step.
-        float *next = pivot_row[(j + 1) & 1];
-        if (lane < 15) {
-            if (ty == lane + 1) {
+            for (int v = SIXTEEN; v < kTile; ++v)
+                mine[u][v] -= rows_first[u] * columns_first[v] + rows_second[u] * columns_second[v];
+        // Rows j + 2 and j + 3 have all their updates now: their owners publish them.
+        float (*next)[kBlock] = pivot_rows[((j >> 1) + 1) & 1];
+        if (lane < 14) {
+            if (ty == lane + 2 || ty == lane + 3) {
 #pragma unroll
-                for (int v = SIXTEEN; v < kTile; ++v) next[tx + 16 * v] = mine[SIXTEEN][v];   // columns < j are not read
+                for (int v = SIXTEEN; v < kTile; ++v) next[ty - lane - 2][tx + 16 * v] = mine[SIXTEEN][v];   // columns < j are not read
             }
         } else if constexpr (SIXTEEN + 1 < kTile) {
-            if (ty == 0) {
+            if (ty < 2) {
 #pragma unroll
-                for (int v = SIXTEEN + 1; v < kTile; ++v) next[tx + 16 * v] = mine[SIXTEEN + 1][v];
+                for (int v = SIXTEEN + 1; v < kTile; ++v) next[ty][tx + 16 * v] = mine[SIXTEEN + 1][v];
             }
         }
         __syncthreads();
@@ -88,15 +111,15 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
 // in the upper triangle, zeros below it.  A pivot that is not positive (or not finite)
 // records its column and leaves the block unspecified.
 //
-// Right-looking, one column per step.  The block lives in registers for the whole
+// Right-looking, two columns per step.  The block lives in registers for the whole
 // factorisation: thread (ty, tx) of a 16 x 16 grid owns entries (ty + 16 u, tx + 16 v),
-// an 8 x 8 sub-block.  Per step only the pivot row travels: the sixteen threads that own it
-// put it (unscaled) into one of two LDS row buffers, one barrier later every thread reads
-// the sixteen entries it needs, scales them by 1 / sqrt(pivot) and subtracts their outer
-// product from its sub-block.  Rows up to the pivot row are masked out of the update by a
-// zero factor, so finished rows keep their values.
+// an 8 x 8 sub-block.  Per step only the two pivot rows travel: the threads that own them
+// put them (as updated so far) into one of two LDS buffers, one barrier later every thread
+// reads the entries it needs, finishes the two rows for itself and subtracts their outer
+// products from its sub-block.  Rows up to the pivot rows are masked out of the update by
+// zero factors, so finished rows keep their values.
 __global__ void __launch_bounds__(kThreads) cholesky_block_kernel(const BlockArgs a) {
-    __shared__ float pivot_row[2][kBlock];
+    __shared__ float pivot_rows[2][2][kBlock];   // [buffer][row j, row j + 1][column]
     __shared__ int failed;
     const int n = a.size;
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
@@ -112,22 +135,22 @@ __global__ void __launch_bounds__(kThreads) cholesky_block_kernel(const BlockArg
             // Outside the block: an identity diagonal keeps every pivot of the padding at one.
             mine[u][v] = inside ? loaded : (row == column ? 1.0f : 0.0f);
         }
-    if (ty == 0) {
+    if (ty < 2) {
 #pragma unroll
-        for (int v = 0; v < kTile; ++v) pivot_row[0][tx + 16 * v] = mine[0][v];
+        for (int v = 0; v < kTile; ++v) pivot_rows[0][ty][tx + 16 * v] = mine[0][v];
     }
     __syncthreads();
     if (failed) return;
 
     // All 128 steps run (the padding is an identity): no data-dependent exit other than a bad pivot.
-    bool good = sixteen_steps<0>(a, mine, pivot_row, tx, ty);
-    good = good && sixteen_steps<1>(a, mine, pivot_row, tx, ty);
-    good = good && sixteen_steps<2>(a, mine, pivot_row, tx, ty);
-    good = good && sixteen_steps<3>(a, mine, pivot_row, tx, ty);
-    good = good && sixteen_steps<4>(a, mine, pivot_row, tx, ty);
-    good = good && sixteen_steps<5>(a, mine, pivot_row, tx, ty);
-    good = good && sixteen_steps<6>(a, mine, pivot_row, tx, ty);
-    good = good && sixteen_steps<7>(a, mine, pivot_row, tx, ty);
+    bool good = sixteen_steps<0>(a, mine, pivot_rows, tx, ty);
+    good = good && sixteen_steps<1>(a, mine, pivot_rows, tx, ty);
+    good = good && sixteen_steps<2>(a, mine, pivot_rows, tx, ty);
+    good = good && sixteen_steps<3>(a, mine, pivot_rows, tx, ty);
+    good = good && sixteen_steps<4>(a, mine, pivot_rows, tx, ty);
+    good = good && sixteen_steps<5>(a, mine, pivot_rows, tx, ty);
+    good = good && sixteen_steps<6>(a, mine, pivot_rows, tx, ty);
+    good = good && sixteen_steps<7>(a, mine, pivot_rows, tx, ty);
     if (!good) return;
 #pragma unroll
     for (int u = 0; u < kTile; ++u)
