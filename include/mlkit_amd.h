@@ -152,17 +152,22 @@ int mk_fwht(const void *source, int source_dtype, void *target, int target_dtype
 int mk_basis_mix(const float *source, float *target, const float *basis, long long rows, int order,
                  int power, int transpose, const float *signs_after, void *stream);
 
-/* Diagonal-block step of a blocked Cholesky factorisation, one workgroup: the upper triangle
- * of the symmetric positive definite size x size block at `matrix` (row-major, `leading`
- * floats per row, size <= 128) is replaced by U with block = U^T U, and the strict lower
- * triangle of the block by zeros.  *status (device memory, zero before the first block)
- * receives 1 + first_column + j if pivot j is not positive and finite, as
- * torch.linalg.cholesky_ex reports it; a block launched after a failure does nothing.  The
- * host drives the blocked algorithm with triangular solves and matrix products for the
- * panels and the trailing updates.
+/* Diagonal-block step of a blocked Cholesky factorisation: the upper triangle of the
+ * symmetric positive definite size x size block at `matrix` (row-major, `leading` floats per
+ * row, size <= 128) yields U with block = U^T U.  With row_columns == 0 (one workgroup) U
+ * replaces the block in place, zeros below the diagonal.  With row_columns > 0 the
+ * row_columns columns to the right of the block, in the same rows, take the same elimination
+ * and become U^-T times themselves (the block row of the factor), in place, one workgroup
+ * per 128 of them; the block itself is then left untouched and U goes to `factor_out`
+ * (size rows of 128 floats), because every workgroup reads the block.
+ * *status (device memory, zero before the first block) receives 1 + first_column + j if
+ * pivot j is not positive and finite, as torch.linalg.cholesky_ex reports it; a block
+ * launched after a failure does nothing.  The host drives the blocked algorithm with
+ * triangular solves and matrix products for the panels and the trailing updates.
  * Replaces: the factorisation inside feedback_coefficients,
  * quantization/algorithms/error_feedback.py:37-83 (torch.linalg.cholesky_ex). */
-int mk_cholesky_block(float *matrix, long long leading, int size, int first_column, int *status, void *stream);
+int mk_cholesky_block(float *matrix, long long leading, int size, int first_column, int row_columns,
+                      float *factor_out, int *status, void *stream);
 
 /* The blocked transform of a width order * power (power a power of two) in one launch:
  * every row [order, power] of `source` is multiplied by signs_before (NULL or

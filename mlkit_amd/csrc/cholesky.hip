@@ -26,9 +26,12 @@ struct BlockArgs {
     int size;            // rows = columns of the block, 1 ... 128
     int first_column;    // index of the block's first column in the whole matrix (for status)
     int *status;         // stays 0, or becomes 1 + the column whose pivot is not positive
+    int row_columns;     // columns to the right of the block, in the same rows, that take the same elimination
+    float *factor_out;   // where the factor goes when row_columns > 0 (128 floats per row); else in place
 };
 
 constexpr int kTile = kBlock / 16;
+constexpr int kRowFloats = 2 * kBlock;   // a published row: the block's columns, then the columns carried beside it
 
 // Columns 16 SIXTEEN ... 16 SIXTEEN + 15 of the factorisation below, two per step (their rows
 // sit in register row SIXTEEN of their owners).  False after a pivot that is not positive and
@@ -40,9 +43,12 @@ constexpr int kTile = kBlock / 16;
 //   U[j+1][k]   = (A[j+1][k] - U[j][j+1] U[j][k]) / sqrt(A[j+1][j+1] - U[j][j+1]^2)
 // and subtracts both outer products from its sub-block: one LDS round trip and one barrier
 // per two columns.
-template <int SIXTEEN>
-__device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[kTile][kTile],
-                                              float (&pivot_rows)[2][2][kBlock], int tx, int ty) {
+//
+// ROW: the workgroup also carries 128 columns to the right of the block (`beside`), which take
+// the same row operations and so become U_jj^-T A_jr, the block row of the factor.
+template <int SIXTEEN, bool ROW>
+__device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[kTile][kTile], float (&beside)[kTile][kTile],
+                                              float (&pivot_rows)[2][2][kRowFloats], int tx, int ty) {
 #pragma unroll 1
     for (int lane = 0; lane < 16; lane += 2) {
         const int j = 16 * SIXTEEN + lane;
@@ -75,31 +81,62 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
             columns_first[u] = first[k] * reciprocal;                                    // U[j][k]
             columns_second[u] = (second[k] - link * columns_first[u]) * next_reciprocal; // U[j+1][k]
         }
+        float beside_first[kTile], beside_second[kTile];
+        if constexpr (ROW) {
+#pragma unroll
+            for (int v = 0; v < kTile; ++v) {
+                const int c = kBlock + tx + 16 * v;
+                beside_first[v] = first[c] * reciprocal;
+                beside_second[v] = (second[c] - link * beside_first[v]) * next_reciprocal;
+            }
+        }
         // The two rows' owners keep the finished rows.
         if (ty == lane) {
 #pragma unroll
             for (int v = SIXTEEN; v < kTile; ++v) mine[SIXTEEN][v] = columns_first[v];
+            if constexpr (ROW) {
+#pragma unroll
+                for (int v = 0; v < kTile; ++v) beside[SIXTEEN][v] = beside_first[v];
+            }
         }
         if (ty == lane + 1) {
 #pragma unroll
             for (int v = SIXTEEN; v < kTile; ++v) mine[SIXTEEN][v] = columns_second[v];
+            if constexpr (ROW) {
+#pragma unroll
+                for (int v = 0; v < kTile; ++v) beside[SIXTEEN][v] = beside_second[v];
+            }
         }
 #pragma unroll
-        for (int u = SIXTEEN; u < kTile; ++u)
+        for (int u = SIXTEEN; u < kTile; ++u) {
 #pragma unroll
             for (int v = SIXTEEN; v < kTile; ++v)
                 mine[u][v] -= rows_first[u] * columns_first[v] + rows_second[u] * columns_second[v];
+            if constexpr (ROW) {
+#pragma unroll
+                for (int v = 0; v < kTile; ++v)
+                    beside[u][v] -= rows_first[u] * beside_first[v] + rows_second[u] * beside_second[v];
+            }
+        }
         // Rows j + 2 and j + 3 have all their updates now: their owners publish them.
-        float (*next)[kBlock] = pivot_rows[((j >> 1) + 1) & 1];
+        float (*next)[kRowFloats] = pivot_rows[((j >> 1) + 1) & 1];
         if (lane < 14) {
             if (ty == lane + 2 || ty == lane + 3) {
 #pragma unroll
                 for (int v = SIXTEEN; v < kTile; ++v) next[ty - lane - 2][tx + 16 * v] = mine[SIXTEEN][v];   // columns < j are not read
+                if constexpr (ROW) {
+#pragma unroll
+                    for (int v = 0; v < kTile; ++v) next[ty - lane - 2][kBlock + tx + 16 * v] = beside[SIXTEEN][v];
+                }
             }
         } else if constexpr (SIXTEEN + 1 < kTile) {
             if (ty < 2) {
 #pragma unroll
                 for (int v = SIXTEEN + 1; v < kTile; ++v) next[ty][tx + 16 * v] = mine[SIXTEEN + 1][v];
+                if constexpr (ROW) {
+#pragma unroll
+                    for (int v = 0; v < kTile; ++v) next[ty][kBlock + tx + 16 * v] = beside[SIXTEEN + 1][v];
+                }
             }
         }
         __syncthreads();
@@ -118,13 +155,18 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
 // reads the entries it needs, finishes the two rows for itself and subtracts their outer
 // products from its sub-block.  Rows up to the pivot rows are masked out of the update by
 // zero factors, so finished rows keep their values.
+template <bool ROW>
 __global__ void __launch_bounds__(kThreads) cholesky_block_kernel(const BlockArgs a) {
-    __shared__ float pivot_rows[2][2][kBlock];   // [buffer][row j, row j + 1][column]
+    __shared__ float pivot_rows[2][2][kRowFloats];   // [buffer][row j, row j + 1][column]
     __shared__ int failed;
     const int n = a.size;
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     if (threadIdx.x == 0) failed = *a.status != 0;   // an earlier block already failed: do nothing
-    float mine[kTile][kTile];
+    float mine[kTile][kTile], beside[kTile][kTile];
+    // ROW: workgroup b carries columns 128 b ... 128 b + 127 of the block row; every workgroup
+    // factors the block itself (from the matrix, which nobody overwrites: the factor goes to
+    // `factor_out`), and the first one stores it.
+    const int beside_first_column = n + kBlock * blockIdx.x;
 #pragma unroll
     for (int u = 0; u < kTile; ++u)
 #pragma unroll
@@ -134,43 +176,64 @@ __global__ void __launch_bounds__(kThreads) cholesky_block_kernel(const BlockArg
             const float loaded = a.matrix[(inside ? row : 0) * a.leading + (inside ? column : 0)];
             // Outside the block: an identity diagonal keeps every pivot of the padding at one.
             mine[u][v] = inside ? loaded : (row == column ? 1.0f : 0.0f);
+            beside[u][v] = 0.0f;
+            if constexpr (ROW) {
+                const bool present = row < n && kBlock * static_cast<int>(blockIdx.x) + column < a.row_columns;
+                const float carried = a.matrix[(present ? row : 0) * a.leading + (present ? beside_first_column + column : 0)];
+                beside[u][v] = present ? carried : 0.0f;
+            }
         }
     if (ty < 2) {
 #pragma unroll
-        for (int v = 0; v < kTile; ++v) pivot_rows[0][ty][tx + 16 * v] = mine[0][v];
+        for (int v = 0; v < kTile; ++v) {
+            pivot_rows[0][ty][tx + 16 * v] = mine[0][v];
+            if constexpr (ROW) pivot_rows[0][ty][kBlock + tx + 16 * v] = beside[0][v];
+        }
     }
     __syncthreads();
     if (failed) return;
 
-    // All 128 steps run (the padding is an identity): no data-dependent exit other than a bad pivot.
-    bool good = sixteen_steps<0>(a, mine, pivot_rows, tx, ty);
-    good = good && sixteen_steps<1>(a, mine, pivot_rows, tx, ty);
-    good = good && sixteen_steps<2>(a, mine, pivot_rows, tx, ty);
-    good = good && sixteen_steps<3>(a, mine, pivot_rows, tx, ty);
-    good = good && sixteen_steps<4>(a, mine, pivot_rows, tx, ty);
-    good = good && sixteen_steps<5>(a, mine, pivot_rows, tx, ty);
-    good = good && sixteen_steps<6>(a, mine, pivot_rows, tx, ty);
-    good = good && sixteen_steps<7>(a, mine, pivot_rows, tx, ty);
+    // All 128 columns run (the padding is an identity): no data-dependent exit other than a bad pivot.
+    bool good = sixteen_steps<0, ROW>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<1, ROW>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<2, ROW>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<3, ROW>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<4, ROW>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<5, ROW>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<6, ROW>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<7, ROW>(a, mine, beside, pivot_rows, tx, ty);
     if (!good) return;
+    float *factor = ROW ? a.factor_out : a.matrix;
+    const long long factor_leading = ROW ? kBlock : a.leading;
 #pragma unroll
     for (int u = 0; u < kTile; ++u)
 #pragma unroll
         for (int v = 0; v < kTile; ++v) {
             const int row = ty + 16 * u, column = tx + 16 * v;
-            if (row < n && column < n) a.matrix[row * a.leading + column] = column >= row ? mine[u][v] : 0.0f;
+            if (blockIdx.x == 0 && row < n && column < n) factor[row * factor_leading + column] = column >= row ? mine[u][v] : 0.0f;
+            if constexpr (ROW) {
+                if (row < n && kBlock * static_cast<int>(blockIdx.x) + column < a.row_columns)
+                    a.matrix[row * a.leading + beside_first_column + column] = beside[u][v];
+            }
         }
 }
 
 }  // namespace
 
-extern "C" int mk_cholesky_block(float *matrix, long long leading, int size, int first_column, int *status,
-                                 void *stream_) {
+extern "C" int mk_cholesky_block(float *matrix, long long leading, int size, int first_column, int row_columns,
+                                 float *factor_out, int *status, void *stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MK_REQUIRE(matrix && status, MK_ERR_INVALID, "mk_cholesky_block: null pointer");
     MK_REQUIRE(size >= 1 && size <= kBlock, MK_ERR_UNSUPPORTED, "mk_cholesky_block: blocks of 1 to %d rows (got %d)", kBlock, size);
-    MK_REQUIRE(leading >= size && first_column >= 0, MK_ERR_INVALID, "mk_cholesky_block: rows overlap");
-    BlockArgs a{matrix, leading, size, first_column, status};
-    hipLaunchKernelGGL(cholesky_block_kernel, dim3(1), dim3(kThreads), 0, stream, a);
+    MK_REQUIRE(row_columns >= 0 && leading >= static_cast<long long>(size) + row_columns && first_column >= 0, MK_ERR_INVALID,
+               "mk_cholesky_block: rows overlap");
+    MK_REQUIRE(row_columns == 0 || factor_out, MK_ERR_INVALID,
+               "mk_cholesky_block: a block row needs a separate place for the factor");
+    BlockArgs a{matrix, leading, size, first_column, status, row_columns, factor_out};
+    if (row_columns > 0)
+        hipLaunchKernelGGL(cholesky_block_kernel<true>, dim3(mk_cdiv(row_columns, kBlock)), dim3(kThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL(cholesky_block_kernel<false>, dim3(1), dim3(kThreads), 0, stream, a);
     MK_LAUNCH_CHECK("mk_cholesky_block");
     return MK_OK;
 }

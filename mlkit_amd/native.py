@@ -66,7 +66,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
         _c_void_p, _c_int, _c_void_p, _c_int, _c_longlong, _c_int, _c_void_p, _c_void_p, _c_int,
         _c_float, _c_void_p,
     ]),
-    "mk_cholesky_block": (_c_int, [_c_void_p, _c_longlong, _c_int, _c_int, _c_void_p, _c_void_p]),
+    "mk_cholesky_block": (_c_int, [_c_void_p, _c_longlong, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p]),
     "mk_rotate_blocks": (_c_int, [
         _c_void_p, _c_int, _c_void_p, _c_int, _c_longlong, _c_int, _c_int, _c_void_p, _c_int, _c_void_p,
         _c_void_p, _c_float, _c_void_p,

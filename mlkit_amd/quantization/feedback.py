@@ -43,8 +43,9 @@ def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
     HIP device, factored in place.  Two levels of right-looking blocking: panels of 512 columns
     update the rest of the matrix (a rank-512 product reads and writes the trailing matrix a
     quarter as often as rank-128 ones would); inside a panel's diagonal block the same scheme
-    runs with 128-column blocks, whose diagonal blocks ``mk_cholesky_block`` factors.
-    Block rows are triangular solves.
+    runs with 128-column blocks: ``mk_cholesky_block`` factors a diagonal block and carries its
+    block row inside the panel through the same elimination.  The panels' block rows are
+    triangular solves.
 
     Look-ahead: of a panel's trailing update only the band of rows the next panel consists of
     runs on the current stream; the rest runs on a second stream while the next panel's
@@ -59,6 +60,7 @@ def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
     device = matrix.device
     library = native.library()
     status = torch.zeros((), dtype=torch.int32, device=device)
+    factored = torch.empty((FACTORIZATION_BLOCK, FACTORIZATION_BLOCK), dtype=torch.float32, device=device)
     main = torch.cuda.current_stream(device)
     look_ahead = width >= LOOK_AHEAD_WIDTH   # narrower: the event traffic costs more than it hides
     side = torch.cuda.Stream(device) if look_ahead else None
@@ -85,10 +87,14 @@ def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
         raw_stream = native.current_stream(device)
         for start in range(panel_start, panel_stop, FACTORIZATION_BLOCK):
             stop = min(panel_stop, start + FACTORIZATION_BLOCK)
-            native.check(library.mk_cholesky_block(matrix[start, start:].data_ptr(), width, stop - start, start,
-                                                   status.data_ptr(), raw_stream))
-            if stop < panel_stop:
-                solve_block_row(start, stop, panel_stop)
+            # the block kernel also carries the rest of the panel's rows start:stop through the
+            # elimination (their block row of the factor); the factored block then comes back
+            # through `factored`, since every workgroup of that launch reads the block itself
+            beside = panel_stop - stop
+            native.check(library.mk_cholesky_block(matrix[start, start:].data_ptr(), width, stop - start, start, beside,
+                                                   factored.data_ptr() if beside else None, status.data_ptr(), raw_stream))
+            if beside:
+                matrix[start:stop, start:stop].copy_(factored[: stop - start, : stop - start])
                 subtract_outer_product(start, stop, stop, panel_stop, panel_stop)
         # the diagonal block's lower triangle holds leftovers of the products above
         matrix[panel_start:panel_stop, panel_start:panel_stop].triu_()
