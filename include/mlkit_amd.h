@@ -163,7 +163,7 @@ int mk_basis_mix(const float *source, float *target, const float *basis, long lo
  * *status (device memory, zero before the first block) receives 1 + first_column + j if
  * pivot j is not positive and finite, as torch.linalg.cholesky_ex reports it; a block
  * launched after a failure does nothing.  The host drives the blocked algorithm with
- * triangular solves and matrix products for the panels and the trailing updates.
+ * matrix products for the trailing updates.
  * Replaces: the factorisation inside feedback_coefficients,
  * quantization/algorithms/error_feedback.py:37-83 (torch.linalg.cholesky_ex). */
 int mk_cholesky_block(float *matrix, long long leading, int size, int first_column, int row_columns,

@@ -43,9 +43,9 @@ def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
     HIP device, factored in place.  Two levels of right-looking blocking: panels of 512 columns
     update the rest of the matrix (a rank-512 product reads and writes the trailing matrix a
     quarter as often as rank-128 ones would); inside a panel's diagonal block the same scheme
-    runs with 128-column blocks: ``mk_cholesky_block`` factors a diagonal block and carries its
-    block row inside the panel through the same elimination.  The panels' block rows are
-    triangular solves.
+    runs with 128-column blocks: ``mk_cholesky_block`` factors a diagonal block and carries the
+    rest of its rows, to the last column, through the same elimination, which makes them the
+    factor's block row; no triangular solve is left.
 
     Look-ahead: of a panel's trailing update only the band of rows the next panel consists of
     runs on the current stream; the rest runs on a second stream while the next panel's
@@ -65,13 +65,6 @@ def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
     look_ahead = width >= LOOK_AHEAD_WIDTH   # narrower: the event traffic costs more than it hides
     side = torch.cuda.Stream(device) if look_ahead else None
 
-    def solve_block_row(start: int, stop: int, limit: int) -> None:
-        # U_jr = U_jj^-T A_jr, solved in place as X U_jj = A_jr^T: the transposed view of the
-        # row-major block row is column-major, the layout the solver works in
-        row_block = matrix[start:stop, stop:limit]
-        torch.linalg.solve_triangular(matrix[start:stop, start:stop], row_block.T, upper=True, left=False,
-                                      out=row_block.T)
-
     def subtract_outer_product(start: int, stop: int, first_row: int, last_row: int, limit: int) -> None:
         """A[r, c] -= sum_k U[k, r] U[k, c] for k in start:stop, rows first_row:last_row, columns from
         the row band's first column to ``limit``: bands of rows, so that little below the diagonal
@@ -87,20 +80,22 @@ def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
         raw_stream = native.current_stream(device)
         for start in range(panel_start, panel_stop, FACTORIZATION_BLOCK):
             stop = min(panel_stop, start + FACTORIZATION_BLOCK)
-            # the block kernel also carries the rest of the panel's rows start:stop through the
-            # elimination (their block row of the factor); the factored block then comes back
+            # the block kernel also carries the rest of rows start:stop, to the matrix's last column,
+            # through the elimination (their block row of the factor); the factored block comes back
             # through `factored`, since every workgroup of that launch reads the block itself
-            beside = panel_stop - stop
+            beside = width - stop
             native.check(library.mk_cholesky_block(matrix[start, start:].data_ptr(), width, stop - start, start, beside,
                                                    factored.data_ptr() if beside else None, status.data_ptr(), raw_stream))
             if beside:
                 matrix[start:stop, start:stop].copy_(factored[: stop - start, : stop - start])
-                subtract_outer_product(start, stop, stop, panel_stop, panel_stop)
+            if stop < panel_stop:
+                # the rest of the panel's rows, over all columns to the right: what a triangular
+                # solve with the panel's whole diagonal block would otherwise do for them
+                subtract_outer_product(start, stop, stop, panel_stop, width)
         # the diagonal block's lower triangle holds leftovers of the products above
         matrix[panel_start:panel_stop, panel_start:panel_stop].triu_()
         if panel_stop == width:
             break
-        solve_block_row(panel_start, panel_stop, width)
         if not look_ahead:
             subtract_outer_product(panel_start, panel_stop, panel_stop, width, width)
             continue
