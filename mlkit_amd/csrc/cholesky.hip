@@ -3,9 +3,10 @@
 // The error-feedback coefficients are U blockdiag(U)^-1 for the damped Hessian H = U^T U
 // (K up to 16384).  The library factorisation spends most of its time in its small
 // unblocked panel kernel, so the blocked algorithm is driven from the host with library
-// triangular solves and matrix products for the block rows and the trailing updates, and
-// this file supplies the part that is neither: one workgroup factors a diagonal block of at
-// most 128 x 128 in registers.
+// matrix products for the trailing updates, and this file supplies the rest: a workgroup
+// factors a diagonal block of at most 128 x 128 in registers and, on request, carries 128
+// columns of the block's rows through the same elimination, which makes them the factor's
+// block row (one workgroup per 128 columns; no triangular solve is needed).
 //
 // Replaces the `torch.linalg.cholesky_ex` call of `feedback_coefficients`
 // (quantization/algorithms/error_feedback.py:37-83 in /root/reference/src/mlkit) for large

@@ -33,16 +33,16 @@ DEFERRED_TILES = 4  # tiles whose far-column updates are applied in one pass on 
 
 BLOCKED_FACTORIZATION_WIDTH = 1024  # narrower matrices go to the library factorisation
 FACTORIZATION_BLOCK = 128           # one workgroup factors a diagonal block of this size
-FACTORIZATION_PANEL = 512           # rank of the trailing updates of the whole matrix
-TRAILING_BAND = 2048                # rows per product of a trailing update (only the upper triangle is needed)
+FACTORIZATION_PANEL = 1024          # rank of the trailing updates of the whole matrix
+TRAILING_BAND = 1024                # rows per product of a trailing update (only the upper triangle is needed)
 LOOK_AHEAD_WIDTH = 8192             # from here on the far part of a trailing update runs on a second stream
 
 
 def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
     """``(U, status)`` with ``matrix = U^T U`` for a symmetric positive definite FP32 matrix on a
-    HIP device, factored in place.  Two levels of right-looking blocking: panels of 512 columns
-    update the rest of the matrix (a rank-512 product reads and writes the trailing matrix a
-    quarter as often as rank-128 ones would); inside a panel's diagonal block the same scheme
+    HIP device, factored in place.  Two levels of right-looking blocking: panels of 1024 columns
+    update the rest of the matrix (a rank-1024 product reads and writes the trailing matrix an
+    eighth as often as rank-128 ones would); inside a panel's diagonal block the same scheme
     runs with 128-column blocks: ``mk_cholesky_block`` factors a diagonal block and carries the
     rest of its rows, to the last column, through the same elimination, which makes them the
     factor's block row; no triangular solve is left.

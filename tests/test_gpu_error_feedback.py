@@ -172,6 +172,7 @@ def test_look_ahead_factorisation_equals_the_one_stream_order(width, monkeypatch
     inputs = rng.standard_normal((2 * width, width)).astype(np.float32)
     inputs[:, ::7] *= 4
     hessian = dev((inputs.T @ inputs / inputs.shape[0]).astype(np.float32))
+    monkeypatch.setattr(feedback, "FACTORIZATION_PANEL", 256)   # several panels at these widths
     monkeypatch.setattr(feedback, "LOOK_AHEAD_WIDTH", 1 << 30)
     expected, status = mk.feedback_coefficients(hessian.clone(), 1)
     assert status == 0
