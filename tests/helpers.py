@@ -1,5 +1,8 @@
 """Shared builders for the parity tests: seeded synthetic layers quantised by the oracle."""
 
+import concurrent.futures
+import os
+
 import numpy as np
 import torch
 
@@ -28,10 +31,27 @@ def activations(samples, width, seed, dtype=torch.float16):
     return torch.randn(samples, width, generator=generator).to(dtype)
 
 
+def _quantize_by_row_bands(weight, values, **options):
+    """scaling.quantize, with large matrices cut into row bands that run on a thread pool (the
+    codec is row-separable and numpy releases the interpreter lock inside its loops)."""
+    rows = weight.shape[0]
+    if weight.size < (1 << 22):
+        return scaling.quantize(weight, values, **options)
+    workers = min(16, os.cpu_count() or 1)
+    bands = np.array_split(np.arange(rows), min(rows, 4 * workers))
+    with concurrent.futures.ThreadPoolExecutor(workers) as pool:
+        parts = list(pool.map(lambda band: scaling.quantize(weight[band[0]:band[-1] + 1], values, **options), bands))
+    result = dict(parts[0])
+    for key in ("codes", "scales", "zero"):
+        result[key] = None if parts[0][key] is None else np.concatenate([part[key] for part in parts], 0)
+    result["side_bits"] = sum(part["side_bits"] for part in parts)
+    return result
+
+
 def quantised_layer(weight, values, *, bits, group, integer, asym=False, scale="absmax", fmt="fp16"):
     """Oracle quantisation + packing.  Returns a dict of numpy arrays."""
-    result = scaling.quantize(weight, values, group=group, integer=integer, asym=asym,
-                              scale=scale, fmt=fmt)
+    result = _quantize_by_row_bands(weight, values, group=group, integer=integer, asym=asym,
+                                    scale=scale, fmt=fmt)
     result["packed"] = bitstream.pack(result["codes"], bits)
     result["bits"] = bits
     result["shape"] = weight.shape

@@ -106,25 +106,81 @@ def test_gptq_on_device_matches_oracle_sweep(values, integer, asym, group, refit
     assert loss == pytest.approx(oracle_feedback.proxy_loss(weight, expected["w"], hessian), rel=1e-3)
 
 
-def test_gptq_full_width_layer_rows_match_oracle():
-    """N = 512 rows of the K = 11008 layer of the benchmark configuration (rows are
-    independent): the oracle sweeps the first 16 rows with the same coefficient matrix."""
-    rows, width, checked = 512, 11008, 16
+def test_config4_gptq_int4_g128_4096x11008_rows_match_oracle():
+    """The whole 4096 x 11008 layer of the benchmark configuration on the device (Hessian from
+    16384 tokens with 1 % of the channels x30, damp 0.01, block = refit = group = 128, natural
+    order).  Rows are independent, so the oracle sweeps 16 rows spread over the matrix with the
+    same coefficient matrix; codes, scales and reconstruction must equal it bit for bit, and
+    the decoded result must equal the sweep's output."""
+    rows, width = 4096, 11008
+    checked = np.linspace(0, rows - 1, 16).astype(np.int64)
     generator = torch.Generator(device="cuda").manual_seed(33)
     weight = (torch.randn((rows, width), device="cuda", generator=generator) * 0.02).half().float()
     inputs = torch.randn((16384, width), device="cuda", generator=generator).half()
     hot = torch.randperm(width, device="cuda", generator=generator)[: width // 100]
     inputs[:, hot] *= 30
-    hessian = (inputs.float().T @ inputs.float()) / inputs.shape[0]
+    hessian = torch.zeros((width, width), device="cuda")
+    for band in inputs.split(2048):                       # X^T X / n without a 721 MB fp32 copy of X
+        hessian.addmm_(band.float().T, band.float())
+    hessian /= inputs.shape[0]
     del inputs
     result = mk.gptq(mk.int(4, group=128))(weight, Ctx("down_proj", H=hessian))
     coeff = host(mk.feedback_coefficients(hessian.clone(), 1)[0])
-    expected = oracle_feedback.sweep(host(weight[:checked]), coeff, scaling.int_values(4), group=128, integer=True,
+    picked = torch.from_numpy(checked).cuda()
+    expected = oracle_feedback.sweep(host(weight[picked]), coeff, scaling.int_values(4), group=128, integer=True,
                                      refit=128, block=128)
-    np.testing.assert_array_equal(host(result.codes[:checked]), expected["codes"])
-    np.testing.assert_array_equal(host(result.params["scales"][:checked]), expected["scales"])
+    del coeff
+    np.testing.assert_array_equal(host(result.codes[picked]), expected["codes"])
+    np.testing.assert_array_equal(host(result.params["scales"][picked]), expected["scales"])
+    np.testing.assert_array_equal(host(result.w[picked]), expected["w"])
+    assert result.params["scales"].shape == (rows, width // 128) and result.codes.shape == (rows, width)
     rtn = mk.int(4, group=128)(weight).w
-    assert float(mk.proxy_loss(weight, result.w, hessian)) < 0.9 * float(mk.proxy_loss(weight, rtn, hessian))
+    loss = float(mk.proxy_loss(weight, result.w, hessian))
+    assert loss < 0.9 * float(mk.proxy_loss(weight, rtn, hessian))
+    sampled = oracle_feedback.proxy_loss(host(weight[picked]), expected["w"], host(hessian))
+    assert float(mk.proxy_loss(weight[picked], result.w[picked], hessian)) == pytest.approx(sampled, rel=1e-3)
+
+
+@pytest.mark.parametrize("values,integer,asym,group,refit", [
+    (scaling.int_values(4), True, False, 128, 128),
+    (scaling.int_values(4), True, True, 64, 128),
+    (scaling.NF4_VALUES, False, False, 64, 64),
+])
+def test_gptq_activation_order_on_device_matches_oracle(values, integer, asym, group, refit, rng):
+    """act_order=True: columns are swept by descending Hessian diagonal (dead channels count as
+    1).  The oracle sweeps the permuted weights with the device's coefficient matrix of the
+    permuted Hessian; codes and scales stay in sweep order, the reconstruction is returned in
+    the original column order (algorithms/error_feedback.py:276-283,196-197,228-232 in
+    /root/reference)."""
+    rows, width = 80, 512
+    weight = helpers.normal_weight(rows, width, seed=34)
+    inputs = rng.standard_normal((1536, width)).astype(F32)
+    inputs *= np.linspace(0.5, 3.0, width, dtype=F32)[rng.permutation(width)]
+    inputs[:, 77] = 0
+    hessian = (inputs.T @ inputs / 1536).astype(F32)
+    grid = mk.grid.int(4) if integer else mk.grid.values(values, bits=4)
+    quantizer = mk.gptq(mk.scaled(grid, group=group, asym=asym), refit=refit, act_order=True)
+    context = Ctx("layer", H=dev(hessian))
+    result = quantizer(dev(weight), context)
+    permutation = host(result.params["permutation"])
+    diagonal = np.diag(hessian).copy()
+    diagonal[diagonal == 0] = 1
+    assert sorted(permutation.tolist()) == list(range(width))
+    assert (np.diff(diagonal[permutation]) <= 0).all()                       # descending activation energy
+    coeff = host(mk.feedback_coefficients(dev(hessian).clone(), 1, permutation=dev(permutation))[0])
+    dead = (np.diag(hessian) == 0)
+    expected = oracle_feedback.sweep(weight[:, permutation], coeff, values, group=group, integer=integer,
+                                     refit=refit, block=128, asym=asym, dead=dead[permutation])
+    np.testing.assert_array_equal(host(result.codes), expected["codes"])
+    np.testing.assert_array_equal(host(result.params["scales"]), expected["scales"])
+    if asym:
+        np.testing.assert_array_equal(host(result.params["zero"]), expected["zero"])
+    np.testing.assert_array_equal(host(result.w), expected["w"][:, np.argsort(permutation)])
+    assert float(np.abs(host(result.w)[:, 77]).max()) == 0
+    plain = mk.gptq(mk.scaled(grid, group=group, asym=asym), refit=refit)(dev(weight), Ctx("layer", H=dev(hessian)))
+    assert result.bits == plain.bits and context.additional_bits == width * 9   # K * ceil(log2 K) bits of order
+    from mlkit_amd.inference.packed_linear import packed_compatible
+    assert not packed_compatible(result)
 
 
 @pytest.mark.parametrize("width", [28, 96, 896, 4864, 4096, 14336])

@@ -147,3 +147,61 @@ def test_fit_scales_c_equals_numpy():
         np.testing.assert_array_equal(scales, scaling.store_scale(expected, "fp16")[0])
         if asym:
             np.testing.assert_array_equal(zeros, scaling.stored_offset(zero, "fp16"))
+
+
+def classic_gptq_with_region_refits(weight, hessian_matrix, refit, group, asym, damp=0.01):
+    """The inverse-Cholesky loop in float64 where, at the first column of every region of
+    `refit` columns, the region's fp16 scales (and offsets) are fitted to the running weights
+    of that region -- the values its columns would take if nothing more were rounded
+    (algorithms/error_feedback.py:296-303,373-393 in /root/reference).  Scale fitting goes
+    through scaling.initial_scales / store_scale, not through the sweep's own C fit."""
+    h = hessian_matrix.astype(np.float64).copy()
+    h[np.diag_indices_from(h)] += damp * np.mean(np.diag(h))
+    upper = np.linalg.cholesky(np.linalg.inv(h)).T
+    w = weight.astype(np.float64).copy()
+    rows, width = w.shape
+    out = np.zeros_like(w)
+    all_scales, all_zeros = [], []
+    for j in range(width):
+        if j % refit == 0:
+            stop = min(width, j + refit)
+            fitted_group = min(group, stop - j)
+            scales, zero = scaling.initial_scales(w[:, j:stop].astype(F32), INT4, fitted_group, asym)
+            scales, _ = scaling.store_scale(scales, "fp16")
+            if zero is not None:
+                zero = scaling.stored_offset(zero, "fp16")
+                all_zeros.append(zero)
+            all_scales.append(scales)
+        slot = (j % refit) // fitted_group
+        scale = scales[:, slot].astype(np.float64)
+        offset = 0.0 if zero is None else zero[:, slot].astype(np.float64)
+        out[:, j] = np.clip(np.rint((w[:, j] - offset) / scale), -8, 7) * scale + offset
+        error = (w[:, j] - out[:, j]) / upper[j, j]
+        w[:, j + 1:] -= error[:, None] * upper[j, j + 1:][None, :]
+    return out, np.concatenate(all_scales, 1), np.concatenate(all_zeros, 1) if all_zeros else None
+
+
+@pytest.mark.parametrize("refit,group,block,asym", [
+    (32, 32, 32, False), (32, 32, 32, True), (64, 64, 64, False), (64, 64, 64, True),
+    (64, 16, 32, False), (64, 32, 64, True), (32, 8, 16, True), (64, 64, 16, False),
+    (48, 16, 48, False),                      # ragged: the last region holds 32 of 48 columns
+])
+def test_sweep_with_region_refits_follows_the_textbook_loop(refit, group, block, asym):
+    """Region refits (pending continuation -> targets -> scale fit -> tiles) against the float64
+    textbook loop: identical stored scales, reconstruction within 1e-6 + 1e-5 |w|."""
+    rows, width = 24, 128
+    weight = helpers.normal_weight(rows, width, seed=21 + refit + group)
+    h = hessian(width, seed=22 + block)
+    coeff, status = feedback.coefficients(h, 0.01)
+    assert status == 0
+    result = feedback.sweep(weight, coeff, INT4, group=group, integer=True, refit=refit, block=block, asym=asym)
+    expected, scales, zeros = classic_gptq_with_region_refits(weight, h, refit, group, asym)
+    np.testing.assert_array_equal(result["scales"], scales)
+    if asym:
+        np.testing.assert_array_equal(result["zero"], zeros)
+    assert (np.abs(result["w"] - expected) <= 1e-6 + 1e-5 * np.abs(expected)).all()
+    # Dropping the pending continuation (fitting to the original weights) must fail this pin.
+    naive = scaling.store_scale(scaling.initial_scales(weight[:, refit:2 * refit], INT4,
+                                                       min(group, refit), asym)[0], "fp16")[0]
+    per_region = -(-refit // min(group, refit))
+    assert not np.array_equal(naive, scales[:, per_region:2 * per_region])

@@ -138,6 +138,61 @@ def test_scale_search_against_float64_brute_force(values, integer):
     assert (chosen != scales).mean() > 0.3
 
 
+@pytest.mark.parametrize("values,integer,asym,fmt", [
+    (INT4, True, False, "fp16"), (INT4, True, True, "fp16"), (SEVEN, False, False, "fp16"),
+    (scaling.NF4_VALUES, False, False, "bf16"), (scaling.int_values(3), True, False, "fp16"),
+])
+def test_scale_search_selects_the_float64_winner_wherever_it_is_clear(values, integer, asym, fmt):
+    """Every group whose float64 least error beats every differently-stored candidate by more
+    than 1e-4 relative must get exactly that candidate: a wrong candidate order, a wrong
+    storage rounding of a candidate or a wrong comparison cannot hide inside a percentage."""
+    rows, width, group = 64, 640, 64
+    weight = helpers.normal_weight(rows, width, seed=31, student_t=True)
+    base, zero = scaling.initial_scales(weight, values, group, asym)
+    base, _ = scaling.store_scale(base, fmt)
+    fractions = np.linspace(0.5, 1.0, 20).astype(F32)
+    chosen = scaling.search_scales(weight, base, zero, values, fractions, group, fmt, integer)
+
+    blocks = weight.reshape(rows, -1, group)
+    centered = blocks if zero is None else (blocks - zero[..., None]).astype(F32)
+
+    def error64(candidate):
+        normalized = (centered / candidate[..., None]).astype(F32)
+        if integer:
+            rounded = np.clip(np.rint(normalized), values.min(), values.max())
+        else:
+            rounded = values[np.abs(normalized[..., None] - values).argmin(-1)]
+        return ((rounded.astype(np.float64) * candidate[..., None] - centered) ** 2).sum(-1)
+
+    candidates = [base] + [scaling.store_scale((base * f).astype(F32), fmt)[0] for f in fractions]
+    errors = np.stack([error64(c) for c in candidates])            # [21, rows, groups]
+    stack = np.stack(candidates)
+    winner = errors.argmin(0)                                       # first index of the least error
+    least = np.take_along_axis(errors, winner[None], 0)[0]
+    best_scale = np.take_along_axis(stack, winner[None], 0)[0]
+    rivals = np.where(stack != best_scale[None], errors, np.inf).min(0)
+    clear = rivals > least * (1 + 1e-4)
+    assert clear.mean() > 0.9, clear.mean()                         # the criterion must not be vacuous
+    np.testing.assert_array_equal(chosen[clear], best_scale[clear])
+    assert (chosen[clear] != base[clear]).mean() > 0.3              # and most winners are shrunken scales
+
+
+def test_scale_search_keeps_the_base_scale_on_an_exact_tie():
+    """A group of zeros has error exactly 0 under every candidate: the base scale stays
+    (grouped_scaling.py:343-350, `error < best_error`).  The fractions end below 1 so that
+    "the last candidate wins ties" would pick a different stored value; fp32 storage keeps the
+    candidates distinct."""
+    weight = helpers.normal_weight(4, 128, seed=32)
+    weight[1, 64:] = 0
+    weight[3, :64] = 0
+    fractions = np.array([0.5, 0.75], dtype=F32)
+    for values, integer in ((INT4, True), (SEVEN, False)):
+        base, _ = scaling.store_scale(scaling.initial_scales(weight, values, 64, False)[0], "fp32")
+        chosen = scaling.search_scales(weight, base, None, values, fractions, 64, "fp32", integer)
+        assert chosen[1, 1] == base[1, 1] and chosen[3, 0] == base[3, 0]
+        assert base[1, 1] != F32(base[1, 1] * F32(0.75))
+
+
 def test_ordered_group_error_is_a_sum_of_squares(rng):
     weight = helpers.normal_weight(8, 384, seed=8)
     scales = scaling.initial_scales(weight, INT4, 128, False)[0]
