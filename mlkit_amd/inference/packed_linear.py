@@ -130,16 +130,22 @@ class PackedLinear(nn.Module):
         return output.view(shape[:-1] + (self.out_features,))
 
     def _matvec(self, inputs: Tensor, output: Tensor, rows: int) -> None:
-        """One call into the C ABI with the layer's constant arguments bound once
-        (rebuilt after the buffers move or change dtype)."""
+        """One call into the C ABI.  The layer's constant arguments are bound once and kept
+        for as long as all five buffers stay where they were: the key is every buffer's
+        address, so a moved, cast, reassigned or reloaded ``scales`` / ``zeros`` / ``bias`` /
+        ``values`` / ``packed`` rebuilds them."""
+        buffers = self._buffers
+        packed, scales, values = buffers["packed"], buffers["scales"], buffers["values"]
+        zeros, bias = buffers["zeros"], buffers["bias"]
+        key = (packed.data_ptr(), scales.data_ptr(), values.data_ptr(),
+               0 if zeros is None else zeros.data_ptr(), 0 if bias is None else bias.data_ptr(),
+               scales.dtype, None if bias is None else bias.dtype)
         launch = self._launch
-        if launch is None or launch[0] != self.packed.data_ptr():  # a copy owns other buffers
-            scales, zeros, bias = self.scales, self.zeros, self.bias
+        if launch is None or launch[0] != key:
             launch = self._launch = (
-                self.packed.data_ptr(),
-                (self.packed.data_ptr(), scales.data_ptr(), native.dtype_code(scales), self.values.data_ptr(),
-                 self.values.numel(), native.pointer(zeros), native.pointer(bias),
-                 0 if bias is None else native.dtype_code(bias)),
+                key,
+                (key[0], key[1], native.dtype_code(scales), key[2], values.numel(), native.pointer(zeros),
+                 native.pointer(bias), 0 if bias is None else native.dtype_code(bias)),
                 (self.out_features, self.in_features, self.group, self.code_bits, int(self.uniform_grid),
                  self.grid_minimum, self.grid_step),
             )

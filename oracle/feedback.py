@@ -150,7 +150,7 @@ def sweep(weight, coeff, values, *, group, integer, refit=128, block=128, asym=F
     ``weight`` [N, K], ``coeff`` = unit upper ``A`` [K, K] fp32.  Returns codes (uint8),
     scales/zero concatenated over regions, and the fp32 reconstruction.
     """
-    original = np.array(weight, dtype=F32)
+    original = np.array(weight, dtype=F32, order="C")   # the C routines index rows of `width` floats
     rows, width = original.shape
     if dead is not None:
         original[:, dead] = 0

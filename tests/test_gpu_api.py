@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 import torch
 from torch import nn
+import torch.nn.functional as functional
 
 import mlkit_amd as mk
 from mlkit_amd.quantization.core import Ctx
@@ -289,6 +290,30 @@ def test_packed_linear_can_be_copied_and_cast_after_launching():
         result = single(inputs.float().cuda())
         torch.testing.assert_close(result, expected.float(), rtol=2e-3, atol=2e-3)
         assert result.dtype == torch.float32
+
+
+def test_packed_linear_follows_replaced_side_buffers():
+    """After a launch, new `scales`, `zeros` and `bias` tensors (assignment, a partial
+    load_state_dict(assign=True), re-registration) must be the ones the next launch reads."""
+    packed, _ = packed_and_reference(mk.int(4, group=64, asym=True), dtype=torch.float16)
+    layer = packed.module[0]
+    inputs = torch.randn(2, 256, dtype=torch.float16, device="cuda")
+
+    def dense_product():
+        return functional.linear(inputs.float(), layer.weight.float(),
+                                 None if layer.bias is None else layer.bias.float())
+
+    with torch.inference_mode():
+        torch.testing.assert_close(layer(inputs).float(), dense_product(), rtol=2e-3, atol=2e-3)
+        before = layer(inputs).clone()
+        layer.scales = (layer.scales.float() * 1.5).half()                      # plain assignment
+        torch.testing.assert_close(layer(inputs).float(), dense_product(), rtol=2e-3, atol=2e-3)
+        assert not torch.allclose(layer(inputs), before, rtol=1e-2, atol=1e-3)
+        state = {"zeros": (layer.zeros.float() + 0.01).half(), "bias": torch.full_like(layer.bias, 0.25)}
+        layer.load_state_dict(state, strict=False, assign=True)                 # partial reload
+        torch.testing.assert_close(layer(inputs).float(), dense_product(), rtol=2e-3, atol=2e-3)
+        layer.register_buffer("scales", (layer.scales.float() * 0.5).half())   # re-registration
+        torch.testing.assert_close(layer(inputs).float(), dense_product(), rtol=2e-3, atol=2e-3)
 
 
 WIDTH_FORMATS = {

@@ -205,3 +205,18 @@ def test_sweep_with_region_refits_follows_the_textbook_loop(refit, group, block,
                                                        min(group, refit), asym)[0], "fp16")[0]
     per_region = -(-refit // min(group, refit))
     assert not np.array_equal(naive, scales[:, per_region:2 * per_region])
+
+
+def test_sweep_accepts_column_permuted_views():
+    """Fancy-indexed columns come back from numpy in column-major order; the sweep must read
+    them as rows all the same (activation order hands it `weight[:, permutation]`)."""
+    rows, width = 16, 96
+    weight = helpers.normal_weight(rows, width, seed=40)
+    coeff, _ = feedback.coefficients(hessian(width, seed=41), 0.01)
+    permutation = np.random.default_rng(3).permutation(width)
+    view = weight[:, permutation]
+    direct = feedback.sweep(view, coeff, INT4, group=32, integer=True, refit=32, block=32)
+    copied = feedback.sweep(np.ascontiguousarray(view), coeff, INT4, group=32, integer=True, refit=32, block=32)
+    np.testing.assert_array_equal(direct["codes"], copied["codes"])
+    first = np.clip(np.rint(view[:, 0] / direct["scales"][:, 0]), -8, 7) + 8
+    np.testing.assert_array_equal(direct["codes"][:, 0], first.astype(np.uint8))
