@@ -60,6 +60,26 @@ int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packed, const vo
                      int input_width, int group, int bits, int uniform, float grid_min,
                      float grid_step, void *stream);
 
+/* mk_packed_matvec for `count` (1..8) weight matrices that read the same activations:
+ * y[i] = x @ dequant(packed[i])^T (+ bias[i]) for every i, each with output_widths[i] rows.
+ * The matrices share x, samples, input_width, group, bits, the grid (uniform, grid_min,
+ * grid_step, values) and the dtypes; either every matrix has offsets or none has.  packed,
+ * scales, zeros (NULL = none), bias (NULL = none; single entries may be NULL) and y are HOST
+ * arrays of `count` device pointers, output_widths a host array of `count` ints; the arrays
+ * are read before the call returns.  Layouts the INT4 streaming kernels take (4-bit uniform
+ * grid, 16-bit activations and scales, input_width a multiple of 32 up to 16384) run as ONE
+ * launch whose workgroups are spread over all the matrices; every other layout runs as
+ * `count` launches of mk_packed_matvec.  Results equal those of `count` separate calls bit
+ * for bit.
+ * Replaces: the consecutive launches of kernels/packed_linear.py:181-226 that sibling layers
+ * fed by one tensor make (attention q/k/v, MLP gate/up: the model calls
+ * PackedLinear.forward, inference/packed_linear.py:148-245, once per layer). */
+int mk_packed_matvec_group(const void *x, int x_dtype, int count, const uint8_t *const *packed,
+                           const void *const *scales, int scale_dtype, const float *values, int n_values,
+                           const void *const *zeros, const void *const *bias, int bias_dtype,
+                           void *const *y, const int *output_widths, int samples, int input_width,
+                           int group, int bits, int uniform, float grid_min, float grid_step, void *stream);
+
 /* out[n, k] = dequant(code[n, k]) in out_dtype, same dequantisation as mk_packed_matvec
  * with multiply and add kept separate (no fused multiply-add).
  * Replaces: kernels/packed_linear.py:279-313 (decode / decode_rows). */

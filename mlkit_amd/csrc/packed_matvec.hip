@@ -106,9 +106,20 @@ size_t lds_bytes_for(const Plan &p, int groups, bool uniform, bool has_zero) {
     return floats * sizeof(float);
 }
 
-int tuning(const char *name, int fallback) {
-    const char *text = std::getenv(name);
-    return text && *text ? std::atoi(text) : fallback;
+// Development switches, read from the environment once per process (not per launch).
+struct Tuning {
+    int no_stream4, no_pairs, workgroups, rows_parallel;  // rows_parallel 0: planned
+};
+const Tuning &tuning() {
+    static const Tuning values = [] {
+        auto read = [](const char *name, int fallback) {
+            const char *text = std::getenv(name);
+            return text && *text ? std::atoi(text) : fallback;
+        };
+        return Tuning{read("MK_MATVEC_NO_STREAM4", 0), read("MK_MATVEC_NO_PAIRS", 0), read("MK_MATVEC_WORKGROUPS", 512),
+                      read("MK_MATVEC_ROWS_PARALLEL", 0)};
+    }();
+    return values;
 }
 
 // Chooses the lane/row decomposition of the chunked kernel; returns false when the
@@ -134,11 +145,11 @@ bool plan_chunked(int samples, int rows, int width, int group, int groups, int b
     const int seg = lanes <= 64 ? next_pow2(lanes) : 64 * mk_cdiv(lanes, 64);
     const int rows_per_thread = mk_matvec::kThreadRows;
     int rows_parallel = seg < 64 ? 64 / seg : 1;
-    const int wanted_workgroups = tuning("MK_MATVEC_WORKGROUPS", 512);
+    const int wanted_workgroups = tuning().workgroups;
     while (seg * rows_parallel * 2 <= 256 &&
            rows / (rows_parallel * 2 * rows_per_thread) >= wanted_workgroups)
         rows_parallel *= 2;
-    rows_parallel = tuning("MK_MATVEC_ROWS_PARALLEL", rows_parallel);
+    if (tuning().rows_parallel > 0) rows_parallel = tuning().rows_parallel;
     const int threads = seg * rows_parallel;
     if (threads % 64 != 0 || threads > 512) return false;
     p.sample_tile = mt;
@@ -151,6 +162,26 @@ bool plan_chunked(int samples, int rows, int width, int group, int groups, int b
     if (p.lds_bytes > 60 * 1024) return false;
     p.grid_x = 0;
     return true;
+}
+
+// Rows [first_row, output_width) through the word-at-a-time kernel.
+int launch_words(const void *x, int x_dtype, const uint8_t *packed, const void *scales, int scale_dtype,
+                 const float *values, const void *zeros, const void *bias, int bias_dtype, void *y, int samples,
+                 int output_width, int input_width, int group, int bits, int uniform, float grid_min,
+                 float grid_step, int first_row, hipStream_t stream) {
+    const int divisor = mk_gcd(bits, 8);
+    WordArgs w;
+    w.x = x; w.packed = packed; w.scales = scales; w.zeros = zeros; w.values = values; w.bias = bias;
+    w.y = y; w.samples = samples; w.rows = output_width; w.width = input_width; w.group = group;
+    w.groups = mk_cdiv(input_width, group); w.first_row = first_row;
+    w.x_dtype = x_dtype; w.scale_dtype = scale_dtype; w.bias_dtype = bias_dtype;
+    w.bits = bits;
+    w.bytes_per_word = bits / divisor; w.codes_per_word = 8 / divisor; w.uniform = uniform;
+    w.grid_min = grid_min; w.grid_step = grid_step;
+    dim3 grid(mk_cdiv(output_width - first_row, 4), mk_cdiv(samples, 8));
+    hipLaunchKernelGGL(packed_matvec_words_kernel, grid, dim3(256), 0, stream, w);
+    MK_LAUNCH_CHECK("mk_packed_matvec");
+    return MK_OK;
 }
 
 }  // namespace
@@ -191,10 +222,9 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
                          (reinterpret_cast<uintptr_t>(bias) & 3u) == 0 &&
                          (reinterpret_cast<uintptr_t>(x) & 15u) == 0 &&
                          (static_cast<size_t>(input_width) * mk_dtype_bytes(x_dtype)) % 16 == 0;
-    const int divisor = mk_gcd(bits, 8);
     int done_rows = 0;  // rows [0, done_rows) are covered by a chunked kernel
     Plan plan;
-    if (aligned && !tuning("MK_MATVEC_NO_STREAM4", 0) &&
+    if (aligned && !tuning().no_stream4 &&
         mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
         (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
         mk_matvec::Stream4Args s4;
@@ -204,8 +234,9 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
         s4.values = values; s4.n_values = n_values; s4.uniform = uniform; s4.bits = bits;
         s4.x_dtype = x_dtype; s4.scale_dtype = scale_dtype;
         done_rows = mk_matvec::stream4_launch(s4, stream);
+        MK_REQUIRE(done_rows >= 0, MK_ERR_HIP, "mk_packed_matvec: the runtime refused the kernel's LDS size");
         if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
-    } else if (aligned && !tuning("MK_MATVEC_NO_PAIRS", 0) &&
+    } else if (aligned && !tuning().no_pairs &&
                mk_matvec::pairs_accepts(input_width, group, bits, x_dtype, scale_dtype) &&
                (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
         mk_matvec::Stream4Args s4;
@@ -247,18 +278,75 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
             }
         }
     }
-    if (done_rows < output_width) {
-        WordArgs w;
-        w.x = x; w.packed = packed; w.scales = scales; w.zeros = zeros; w.values = values; w.bias = bias;
-        w.y = y; w.samples = samples; w.rows = output_width; w.width = input_width; w.group = group;
-        w.groups = groups; w.first_row = done_rows;
-        w.x_dtype = x_dtype; w.scale_dtype = scale_dtype; w.bias_dtype = bias_dtype;
-        w.bits = bits;
-        w.bytes_per_word = bits / divisor; w.codes_per_word = 8 / divisor; w.uniform = uniform;
-        w.grid_min = grid_min; w.grid_step = grid_step;
-        dim3 grid(mk_cdiv(output_width - done_rows, 4), mk_cdiv(samples, 8));
-        hipLaunchKernelGGL(packed_matvec_words_kernel, grid, dim3(256), 0, stream, w);
-        MK_LAUNCH_CHECK("mk_packed_matvec");
+    if (done_rows < output_width)
+        return launch_words(x, x_dtype, packed, scales, scale_dtype, values, zeros, bias, bias_dtype, y, samples,
+                            output_width, input_width, group, bits, uniform, grid_min, grid_step, done_rows, stream);
+    return MK_OK;
+}
+
+extern "C" int mk_packed_matvec_group(const void *x, int x_dtype, int count, const uint8_t *const *packed,
+                                      const void *const *scales, int scale_dtype, const float *values, int n_values,
+                                      const void *const *zeros, const void *const *bias, int bias_dtype,
+                                      void *const *y, const int *output_widths, int samples, int input_width,
+                                      int group, int bits, int uniform, float grid_min, float grid_step,
+                                      void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(count >= 1 && count <= mk_matvec::kMaxGroupMembers, MK_ERR_INVALID,
+               "mk_packed_matvec_group: 1 to %d matrices per call", mk_matvec::kMaxGroupMembers);
+    MK_REQUIRE(x && packed && scales && y && output_widths, MK_ERR_INVALID, "mk_packed_matvec_group: null argument");
+    MK_REQUIRE(samples >= 1 && input_width >= 1 && group >= 1, MK_ERR_INVALID,
+               "mk_packed_matvec_group: sizes must be positive");
+    bool with_zeros = zeros && zeros[0];
+    bool one_launch = mk_dtype_valid(x_dtype) && mk_dtype_valid(scale_dtype) && (!bias || mk_dtype_valid(bias_dtype)) &&
+                      bits == 4 && !tuning().no_stream4 &&
+                      mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
+                      (reinterpret_cast<uintptr_t>(x) & 15u) == 0 &&
+                      (static_cast<size_t>(input_width) * mk_dtype_bytes(x_dtype)) % 16 == 0;
+    for (int i = 0; i < count; ++i) {
+        MK_REQUIRE(packed[i] && scales[i] && y[i] && output_widths[i] >= 1, MK_ERR_INVALID,
+                   "mk_packed_matvec_group: matrix %d has a null pointer or no rows", i);
+        MK_REQUIRE(((zeros && zeros[i]) != 0) == with_zeros, MK_ERR_INVALID,
+                   "mk_packed_matvec_group: either every matrix has offsets or none has");
+        const void *bias_i = bias ? bias[i] : nullptr;
+        one_launch = one_launch && (reinterpret_cast<uintptr_t>(packed[i]) & 3u) == 0 &&
+                     (reinterpret_cast<uintptr_t>(scales[i]) & 3u) == 0 &&
+                     (reinterpret_cast<uintptr_t>(with_zeros ? zeros[i] : nullptr) & 3u) == 0 &&
+                     (reinterpret_cast<uintptr_t>(bias_i) & 3u) == 0;
+    }
+    if (!one_launch) {  // the same results, one launch per matrix
+        for (int i = 0; i < count; ++i)
+            if (int status = mk_packed_matvec(x, x_dtype, packed[i], scales[i], scale_dtype, values, n_values,
+                                              with_zeros ? zeros[i] : nullptr, bias ? bias[i] : nullptr, bias_dtype,
+                                              y[i], samples, output_widths[i], input_width, group, bits, uniform,
+                                              grid_min, grid_step, stream_))
+                return status;
+        return MK_OK;
+    }
+    mk_matvec::Stream4Args shared{};
+    shared.x = x; shared.samples = samples; shared.width = input_width; shared.group = group;
+    shared.groups = mk_cdiv(input_width, group); shared.bias_dtype = bias_dtype; shared.grid_min = grid_min;
+    shared.grid_step = grid_step; shared.values = values; shared.n_values = n_values; shared.uniform = uniform;
+    shared.bits = bits; shared.x_dtype = x_dtype; shared.scale_dtype = scale_dtype;
+    mk_matvec::Stream4Group members{};
+    members.count = count;
+    for (int i = 0; i < count; ++i) {
+        members.member[i].packed = packed[i];
+        members.member[i].scales = scales[i];
+        members.member[i].zeros = with_zeros ? zeros[i] : nullptr;
+        members.member[i].bias = bias ? bias[i] : nullptr;
+        members.member[i].y = y[i];
+    }
+    int rows_per_tile = 0;
+    MK_REQUIRE(mk_matvec::stream4_launch_group(shared, members, output_widths, &rows_per_tile, stream) == 0, MK_ERR_HIP,
+               "mk_packed_matvec_group: the runtime refused the kernel's LDS size");
+    MK_LAUNCH_CHECK("mk_packed_matvec_group");
+    for (int i = 0; i < count; ++i) {  // rows past a member's last whole tile
+        const int covered = output_widths[i] / rows_per_tile * rows_per_tile;
+        if (covered < output_widths[i])
+            if (int status = launch_words(x, x_dtype, packed[i], scales[i], scale_dtype, values, members.member[i].zeros,
+                                          members.member[i].bias, bias_dtype, y[i], samples, output_widths[i],
+                                          input_width, group, bits, uniform, grid_min, grid_step, covered, stream))
+                return status;
     }
     return MK_OK;
 }

@@ -67,11 +67,64 @@ struct Stream4Args {
     int n_values, uniform, bits;
     int x_dtype, scale_dtype;  // pair-table kernel: MK_F16 or MK_BF16 each
 };
+// Several weight matrices that share the activations, the row width and the codec, multiplied
+// by one launch: workgroup `v` of the grid belongs to the member with the largest
+// first_tile <= v and multiplies that member's tile v - first_tile.  count == 0: the single
+// matrix described by Stream4Args.
+constexpr int kMaxGroupMembers = 8;
+struct Stream4Member {
+    const uint8_t *packed;
+    const void *scales, *zeros, *bias;
+    void *y;
+    int rows;        // output width of this member (row stride of y)
+    int first_tile;  // tiles of all earlier members
+};
+struct Stream4Group {
+    int count, total_tiles;
+    Stream4Member member[kMaxGroupMembers];
+};
+
+// What one tile of rows reads and writes.
+struct TileSource {
+    const uint8_t *packed;
+    const uint8_t *scales, *zeros;
+    const void *bias;
+    void *y;
+    int rows, tile;
+};
+
+// Wavefront-uniform (v comes from blockIdx and the grid size): the member table is read with
+// scalar loads.
+__device__ __forceinline__ TileSource tile_source(const Stream4Args &a, const Stream4Group &g, int v) {
+    TileSource s{a.packed, static_cast<const uint8_t *>(a.scales), static_cast<const uint8_t *>(a.zeros), a.bias, a.y,
+                 a.rows, v};
+    if (g.count > 0) {
+        int m = 0;
+#pragma unroll
+        for (int i = 1; i < kMaxGroupMembers; ++i)
+            if (i < g.count && v >= g.member[i].first_tile) m = i;
+        const Stream4Member &chosen = g.member[m];
+        s.packed = chosen.packed;
+        s.scales = static_cast<const uint8_t *>(chosen.scales);
+        s.zeros = static_cast<const uint8_t *>(chosen.zeros);
+        s.bias = chosen.bias;
+        s.y = chosen.y;
+        s.rows = chosen.rows;
+        s.tile = v - chosen.first_tile;
+    }
+    return s;
+}
+
 // Pair-table kernel (packed_matvec_pairs.hip): 2-, 3- and 4-bit codes of any scalar grid.
 bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype);
 int pairs_launch(const Stream4Args &a, hipStream_t stream);
 bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
+// The same for a group (Stream4Args carries what the members share; its packed / scales /
+// zeros / bias / y / rows are ignored).  `rows_per_tile` receives the tile height chosen for
+// all members: rows beyond the last whole tile of a member are left to the caller.
+int stream4_launch_group(const Stream4Args &shared, Stream4Group &group, const int *member_rows, int *rows_per_tile,
+                         hipStream_t stream);
 
 // ---------------------------------------------------------------------------------
 // Activation registers.  XT: MK_F32 keeps 32 floats per chunk; MK_F16 / MK_BF16 keep

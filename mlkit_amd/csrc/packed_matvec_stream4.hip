@@ -20,6 +20,7 @@
 
 #include "packed_matvec_impl.h"
 
+#include <atomic>
 #include <type_traits>
 
 namespace mk_matvec {
@@ -92,7 +93,7 @@ __device__ __forceinline__ void chunk_dot_bf16(const CodeChunk<4> &codes, const 
 // row and lanes 32 - 63 the next, so that a step covers two rows instead of leaving half the
 // wavefront without codes.
 template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS>
-__global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
+__global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const Stream4Group members) {
     static_assert(ROWS * MT <= 64 && ROWS % PARTS == 0, "one transposed reduction per workgroup");
     __shared__ float partials[64 * 8];  // [row sum][wavefront]
     // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
@@ -140,15 +141,15 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
     constexpr bool kStrided = PARTS == 2;
     XChunk<XT> x[MT];
     float x_sum[MT], grid_term[MT];
-    const int tiles = a.rows / ROWS;
+    const int tiles = members.count > 0 ? members.total_tiles : a.rows / ROWS;
     int tile = blockIdx.x;
     bool first_tile = true;
     do {
-    const int row_base = tile * ROWS;
-    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
-    const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
-    const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
-                                        : nullptr;
+    const TileSource source = tile_source(a, members, tile);  // uniform
+    const int row_base = source.tile * ROWS;
+    const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
+    const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
+    const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
     uint16_t scale_raw[kStreamRows], zero_raw[HAS_ZERO ? kStreamRows : 1];
 #pragma unroll
     for (int r = 0; r < kStreamRows; ++r) {
@@ -228,8 +229,8 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
         const int row = row_base + PARTS * j + (tid - value * PARTS);
         const int sample = sample_base + m;
         if (sample < a.samples) {
-            if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
-            store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
+            if (source.bias) total += mk_load_as_float(source.bias, row, a.bias_dtype);
+            store_output<XT>(source.y, static_cast<size_t>(sample) * source.rows + row, total);
         }
     }
     if constexpr (!kStrided) break;
@@ -256,7 +257,7 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a) {
 // and reach the multiply as DPP quad broadcasts.
 
 template <int SETS, bool HAS_ZERO, int ROWS, int XT, int SLICES>
-__global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a) {
+__global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a, const Stream4Group members) {
     // Short rows (one or two sub-slices per wavefront) leave registers for the tile loop below.
     constexpr bool kStrided = SLICES <= 2;
     constexpr int kQuads = ROWS / 4;
@@ -342,14 +343,14 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     // A workgroup prepares its activations once and then (short rows) takes every
     // gridDim.x-th tile of ROWS rows: tall matrices, with many more tiles than the GPU holds
     // workgroups, pay for the preparation once per workgroup instead of once per tile.
-    const int tiles = a.rows / ROWS;
+    const int tiles = members.count > 0 ? members.total_tiles : a.rows / ROWS;
     int tile = blockIdx.x;
     do {
-    const int row_base = tile * ROWS;
-    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
-    const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
-    const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
-                                        : nullptr;
+    const TileSource source = tile_source(a, members, tile);  // uniform
+    const int row_base = source.tile * ROWS;
+    const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
+    const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
+    const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
     // Scale (and offset) of row 4 q + t at every sub-slice, 2 bytes each.
     uint16_t scale_raw[kSteps], zero_raw[HAS_ZERO ? kSteps : 1];
 #pragma unroll
@@ -455,8 +456,8 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
         const int set = index / (ROWS * 4), row = row_base + (index / 4) % ROWS;
         const int sample = blockIdx.y * 4 * SETS + 4 * set + (index & 3);
         if (sample < a.samples) {
-            if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
-            store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
+            if (source.bias) total += mk_load_as_float(source.bias, row, a.bias_dtype);
+            store_output<XT>(source.y, static_cast<size_t>(sample) * source.rows + row, total);
         }
     }
     if constexpr (!kStrided) break;
@@ -468,104 +469,107 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
 // The number of workgroups of `kernel` the GPU holds at once, asked of the runtime the first
 // time and remembered per kernel (`known`).
 template <typename Kernel>
-int resident_workgroups(Kernel kernel, int threads, size_t dynamic_lds, int &known) {
-    if (known == 0) {
+int resident_workgroups(Kernel kernel, int threads, size_t dynamic_lds, std::atomic<int> &known) {
+    int value = known.load(std::memory_order_relaxed);
+    if (value == 0) {  // two threads asking at once both get the same answer
         int per_cu = 0, device = 0, units = 256;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess || per_cu < 1)
             per_cu = 4;
         if (hipGetDevice(&device) == hipSuccess)
             (void)hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device);
-        known = per_cu * units;
+        value = per_cu * units;
+        known.store(value, std::memory_order_relaxed);
     }
-    return known;
+    return value;
 }
 
 template <int SETS, int ROWS, int SLICES>
-void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
+int launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
     // at most 8 wavefronts x 4 samples x 4112 bytes = 129 KB of the CU's 160 KB
     const size_t slices = static_cast<size_t>(block.x / 64) * 4 * blocks_sample_words(SLICES) * sizeof(uint32_t);
     dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
     // More than 64 KB of dynamic LDS has to be allowed per kernel (static LDS counts against
     // the CU's 160 KB too, so only what this launch needs is asked for).
-    auto launch = [&](auto kernel) {
-        static size_t allowed = 64 * 1024;
-        if (slices > allowed) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      static_cast<int>(slices));
-            allowed = slices;
+    auto launch = [&](auto kernel) -> int {
+        static std::atomic<size_t> allowed{64 * 1024};
+        if (slices > allowed.load(std::memory_order_relaxed)) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    static_cast<int>(slices)) != hipSuccess)
+                return -1;
+            allowed.store(slices, std::memory_order_relaxed);
         }
         if constexpr (SLICES <= 2) {
             // Short rows: as many workgroups as the GPU holds at once; each walks the tiles
             // with that stride.  (Asked of the runtime once per kernel and workgroup size.)
-            static int resident[3] = {0, 0, 0};
+            static std::atomic<int> resident[3];
             const int known = resident_workgroups(kernel, static_cast<int>(block.x), slices, resident[block.x / 64]);
             if (static_cast<int>(grid.x) > known) grid.x = known;
         }
-        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a);
+        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
+        return 0;
     };
     if (a.x_dtype == MK_F16) {
-        if (a.zeros) launch(stream4_blocks_kernel<SETS, true, ROWS, MK_F16, SLICES>);
-        else launch(stream4_blocks_kernel<SETS, false, ROWS, MK_F16, SLICES>);
-    } else {
-        if (a.zeros) launch(stream4_blocks_kernel<SETS, true, ROWS, MK_BF16, SLICES>);
-        else launch(stream4_blocks_kernel<SETS, false, ROWS, MK_BF16, SLICES>);
+        if (a.zeros) return launch(stream4_blocks_kernel<SETS, true, ROWS, MK_F16, SLICES>);
+        return launch(stream4_blocks_kernel<SETS, false, ROWS, MK_F16, SLICES>);
     }
+    if (a.zeros) return launch(stream4_blocks_kernel<SETS, true, ROWS, MK_BF16, SLICES>);
+    return launch(stream4_blocks_kernel<SETS, false, ROWS, MK_BF16, SLICES>);
 }
 
 // A wavefront covers 512 codes per sub-slice: short rows get fewer sub-slices, so that no
 // sub-slice lies wholly past the end of the row.
 template <int SETS, int ROWS>
-void launch_blocks(const Stream4Args &a, int tiles, hipStream_t stream) {
-    if (a.width <= 512) launch_blocks_sliced<SETS, ROWS, 1>(a, tiles, stream);
-    else if (a.width <= 1024) launch_blocks_sliced<SETS, ROWS, 2>(a, tiles, stream);
-    else launch_blocks_sliced<SETS, ROWS, 4>(a, tiles, stream);
+int launch_blocks(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
+    if (a.width <= 512) return launch_blocks_sliced<SETS, ROWS, 1>(a, members, tiles, stream);
+    if (a.width <= 1024) return launch_blocks_sliced<SETS, ROWS, 2>(a, members, tiles, stream);
+    return launch_blocks_sliced<SETS, ROWS, 4>(a, members, tiles, stream);
 }
 
 template <int MT, int ROWS, int PARTS>
-void launch_tile_parts(const Stream4Args &a, int tiles, hipStream_t stream) {
+int launch_tile_parts(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     dim3 grid(tiles, mk_cdiv(a.samples, MT));
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
-    auto launch = [&](auto kernel) {
+    auto launch = [&](auto kernel) -> int {
         if constexpr (PARTS == 2) {  // short rows: one wavefront per workgroup, which walks the tiles
-            static int known = 0;
+            static std::atomic<int> known{0};
             const int resident = resident_workgroups(kernel, static_cast<int>(block.x), slices, known);
             if (static_cast<int>(grid.x) > resident) grid.x = resident;
         }
-        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a);
+        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
+        return 0;
     };
     if (a.x_dtype == MK_F16) {
-        if (a.zeros) launch(stream4_kernel<MT, true, ROWS, MK_F16, PARTS>);
-        else launch(stream4_kernel<MT, false, ROWS, MK_F16, PARTS>);
-    } else {
-        if (a.zeros) launch(stream4_kernel<MT, true, ROWS, MK_BF16, PARTS>);
-        else launch(stream4_kernel<MT, false, ROWS, MK_BF16, PARTS>);
+        if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_F16, PARTS>);
+        return launch(stream4_kernel<MT, false, ROWS, MK_F16, PARTS>);
     }
+    if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_BF16, PARTS>);
+    return launch(stream4_kernel<MT, false, ROWS, MK_BF16, PARTS>);
 }
 
 template <int MT, int ROWS>
-void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
-    if (a.width <= 1024) launch_tile_parts<MT, ROWS, 2>(a, tiles, stream);
-    else launch_tile_parts<MT, ROWS, 1>(a, tiles, stream);
+int launch_tile(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
+    if (a.width <= 1024) return launch_tile_parts<MT, ROWS, 2>(a, members, tiles, stream);
+    return launch_tile_parts<MT, ROWS, 1>(a, members, tiles, stream);
 }
 
+// Launches `tiles` tiles of ROWS rows (of the single matrix, or of all members of a group);
+// returns 0, or -1 when the runtime refused a launch attribute.
 template <int ROWS>
-int launch_rows(const Stream4Args &a, hipStream_t stream) {
-    const int tiles = a.rows / ROWS;
+int launch_rows(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     if (tiles == 0) return 0;
     // One or two samples: v_dot2 kernel.  Three and more: matrix-core blocks (measured at
     // 4096 x 14336: 9.5 against 10.8 us for four samples, 13.3 against 17.6 us for eight).
     if (a.samples >= 3) {
-        if (a.samples <= 4) launch_blocks<1, ROWS>(a, tiles, stream);
-        else launch_blocks<2, ROWS>(a, tiles, stream);
-    } else if (a.samples == 2) {
-        launch_tile<2, ROWS>(a, tiles, stream);
-    } else {
-        launch_tile<1, ROWS>(a, tiles, stream);
+        if (a.samples <= 4) return launch_blocks<1, ROWS>(a, members, tiles, stream);
+        return launch_blocks<2, ROWS>(a, members, tiles, stream);
     }
-    return tiles * ROWS;
+    if (a.samples == 2) return launch_tile<2, ROWS>(a, members, tiles, stream);
+    return launch_tile<1, ROWS>(a, members, tiles, stream);
 }
+
+constexpr int kComputeUnits = 256;
 
 }  // namespace
 
@@ -577,11 +581,37 @@ bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, i
            (group % kChunkCodes == 0 || group >= width);
 }
 
-// Multiplies the leading whole tiles of rows; returns the number of rows covered.
+// Multiplies the leading whole tiles of rows; returns the number of rows covered, or -1 when
+// the runtime refused a launch attribute.
 int stream4_launch(const Stream4Args &a, hipStream_t stream) {
-    constexpr int kComputeUnits = 256;
-    if (a.rows / kWideRows >= kComputeUnits) return launch_rows<kWideRows>(a, stream);
-    return launch_rows<kNarrowRows>(a, stream);
+    Stream4Group none;
+    none.count = 0;
+    none.total_tiles = 0;
+    if (a.rows / kWideRows >= kComputeUnits) {
+        const int tiles = a.rows / kWideRows;
+        return launch_rows<kWideRows>(a, none, tiles, stream) ? -1 : tiles * kWideRows;
+    }
+    const int tiles = a.rows / kNarrowRows;
+    return launch_rows<kNarrowRows>(a, none, tiles, stream) ? -1 : tiles * kNarrowRows;
+}
+
+int stream4_launch_group(const Stream4Args &shared, Stream4Group &group, const int *member_rows, int *rows_per_tile,
+                         hipStream_t stream) {
+    long long wide_tiles = 0;
+    for (int i = 0; i < group.count; ++i) wide_tiles += member_rows[i] / kWideRows;
+    const int rows = wide_tiles >= kComputeUnits ? kWideRows : kNarrowRows;
+    int first = 0;
+    for (int i = 0; i < group.count; ++i) {
+        group.member[i].rows = member_rows[i];
+        group.member[i].first_tile = first;
+        first += member_rows[i] / rows;
+    }
+    group.total_tiles = first;
+    *rows_per_tile = rows;
+    Stream4Args a = shared;
+    a.zeros = group.member[0].zeros;  // selects the kernel variant; the members agree on it
+    if (rows == kWideRows) return launch_rows<kWideRows>(a, group, first, stream);
+    return launch_rows<kNarrowRows>(a, group, first, stream);
 }
 
 }  // namespace mk_matvec

@@ -6,6 +6,7 @@ packed_linear.py:43-79,181-226,279-313); the launches go to ``mk_packed_matvec``
 ``mk_packed_decode`` of ``libmlkit_amd.so`` on the current HIP stream.
 """
 
+import ctypes
 import math
 from dataclasses import dataclass
 
@@ -104,6 +105,62 @@ def matrix_vector(
         grid_minimum, grid_step, native.current_stream(device),
     )
     native.check(status)
+
+
+class GroupLaunch:
+    """Bound arguments of ``mk_packed_matvec_group`` for sibling layers that read the same
+    activations: the host arrays of device pointers are built once and reused by every call."""
+
+    def __init__(self, packed: list[Tensor], scales: list[Tensor], values: Tensor, zeros: list[Tensor | None],
+                 bias: list[Tensor | None], output_widths: list[int], input_width: int, group: int, layout: PackedLayout,
+                 *, uniform_grid: bool, grid_minimum: float, grid_step: float) -> None:
+        count = len(packed)
+        if not 1 <= count <= 8 or not (len(scales) == len(zeros) == len(bias) == len(output_widths) == count):
+            raise ValueError("a launch group holds one to eight matrices with one entry per matrix in every list")
+        self.device = native.require_device(values, *packed, *scales, *zeros, *bias)
+        with_zeros = zeros[0] is not None
+        for index in range(count):
+            if packed[index].dtype != torch.uint8 or packed[index].numel() != output_widths[index] * layout.row_bytes(input_width):
+                raise ValueError("packed byte count does not match the layer shape and precision")
+            if scales[index].dtype != scales[0].dtype or (zeros[index] is not None) != with_zeros:
+                raise ValueError("the matrices of a launch group share the scale dtype and the use of offsets")
+            if zeros[index] is not None and zeros[index].dtype != scales[0].dtype:
+                raise ValueError("zeros must have the dtype of scales")
+        bias_dtypes = {entry.dtype for entry in bias if entry is not None}
+        if len(bias_dtypes) > 1:
+            raise ValueError("the biases of a launch group share one dtype")
+        pointers = ctypes.c_void_p * count
+        self.keep = (packed, scales, values, zeros, bias)
+        self.count = count
+        self.output_widths = list(output_widths)
+        self.input_width = input_width
+        self._y = pointers()
+        self._constant = (
+            pointers(*[entry.data_ptr() for entry in packed]), pointers(*[entry.data_ptr() for entry in scales]),
+            native.dtype_code(scales[0]), values.data_ptr(), values.numel(),
+            pointers(*[native.pointer(entry) for entry in zeros]) if with_zeros else None,
+            pointers(*[native.pointer(entry) for entry in bias]) if bias_dtypes else None,
+            native.DTYPE_CODES[next(iter(bias_dtypes))] if bias_dtypes else 0,
+        )
+        self._widths = (ctypes.c_int * count)(*output_widths)
+        self._tail = (input_width, group, layout.bits, int(uniform_grid), grid_minimum, grid_step)
+
+    def __call__(self, inputs: Tensor, outputs: list[Tensor], stream: int | None = None) -> None:
+        """``outputs[i][m, n] = sum_k dequant(code_i[n, k]) * inputs[m, k] (+ bias_i[n])`` on the current stream."""
+        samples = inputs.shape[0]
+        if not inputs.is_cuda or inputs.device != self.device or not inputs.is_contiguous() or inputs.shape[1] != self.input_width:
+            raise ValueError("grouped packed matvec needs contiguous inputs of the layers' width on their device")
+        for index, output in enumerate(outputs):
+            if (output.dtype != inputs.dtype or tuple(output.shape) != (samples, self.output_widths[index])
+                    or not output.is_contiguous() or output.device != self.device):
+                raise ValueError("outputs must be contiguous [samples, output_width] tensors of the inputs' dtype")
+            self._y[index] = output.data_ptr()
+        if len(outputs) != self.count:
+            raise ValueError("one output per matrix of the group")
+        status = native.library().mk_packed_matvec_group(
+            inputs.data_ptr(), native.dtype_code(inputs), self.count, *self._constant, self._y, self._widths, samples,
+            *self._tail, native.current_stream(self.device) if stream is None else stream)
+        native.check(status)
 
 
 def decode(

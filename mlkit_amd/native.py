@@ -37,6 +37,10 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
         _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
         _c_float, _c_float, _c_void_p,
     ]),
+    "mk_packed_matvec_group": (_c_int, [
+        _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
+        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
+    ]),
     "mk_packed_decode": (_c_int, [
         _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,

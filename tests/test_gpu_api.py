@@ -177,7 +177,8 @@ def test_gptq_activation_order_on_device_matches_oracle(values, integer, asym, g
     if asym:
         np.testing.assert_array_equal(host(result.params["zero"]), expected["zero"])
     np.testing.assert_array_equal(host(result.w), expected["w"][:, np.argsort(permutation)])
-    assert float(np.abs(host(result.w)[:, 77]).max()) == 0
+    if not asym:   # an asymmetric grid need not contain zero
+        assert float(np.abs(host(result.w)[:, 77]).max()) == 0
     plain = mk.gptq(mk.scaled(grid, group=group, asym=asym), refit=refit)(dev(weight), Ctx("layer", H=dev(hessian)))
     assert result.bits == plain.bits and context.additional_bits == width * 9   # K * ceil(log2 K) bits of order
     from mlkit_amd.inference.packed_linear import packed_compatible

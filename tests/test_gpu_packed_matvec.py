@@ -3,6 +3,7 @@ reconstruct-then-matmul.  Tolerances: fp16/bf16 activations, max |y - y_ref| <= 
 (fp32 accumulate) against a float64 yardstick, plus the reference's own allclose bounds
 (tests/inference/test_packed_linear.py:13-24,91-98,162-186)."""
 
+import ctypes
 import functools
 
 import numpy as np
@@ -342,3 +343,79 @@ def test_widest_rows_fill_the_lds_of_the_block_kernels(name, values, bits, integ
     for samples in (1, 4, 8):
         x = helpers.activations(samples, width, seed=32 + samples)
         check(run_matvec(layer, x), layer, x)
+
+
+def run_group(layers, x, biases=None, scale_dtype=torch.float16):
+    from mlkit_amd.kernels import packed_linear
+
+    first = layers[0]
+    width = first["shape"][1]
+    layout = packed_linear.layout_for(first["bits"], width, first["group"])
+    uniform, minimum, step = helpers.uniform_grid(first["values"])
+    tensors = [helpers.to_device(layer, scale_dtype) for layer in layers]
+    biases = [None] * len(layers) if biases is None else [None if b is None else b.cuda() for b in biases]
+    launch = packed_linear.GroupLaunch(
+        [t["packed"] for t in tensors], [t["scales"] for t in tensors], tensors[0]["values"],
+        [t["zeros"] for t in tensors], biases, [layer["shape"][0] for layer in layers], width, first["group"], layout,
+        uniform_grid=uniform, grid_minimum=minimum, grid_step=step)
+    inputs = x.cuda().contiguous()
+    outputs = [torch.full((inputs.shape[0], layer["shape"][0]), float("nan"), dtype=inputs.dtype, device="cuda")
+               for layer in layers]
+    launch(inputs, outputs)
+    torch.cuda.synchronize()
+    return outputs
+
+
+@pytest.mark.parametrize("width,rows,asym", [
+    (4096, (4096, 1024, 1024), False),      # q / k / v of an 8B-class decoder
+    (4096, (14336, 14336), False),          # gate / up
+    (896, (896, 128, 128), True),           # q / k / v of the 0.5B-class decoder, short rows, offsets
+    (896, (4864, 4864), False),
+    (2080, (50, 37, 16), False),            # ragged: rows past the last whole tile, partly filled wavefront
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_grouped_launch_equals_separate_launches(width, rows, asym, dtype):
+    """One launch over sibling matrices sharing the activations returns, bit for bit, what one
+    launch per matrix returns (which the tests above hold against the oracle), for every row
+    count, with and without bias; and the first member is checked against the oracle directly."""
+    layers = [helpers.quantised_layer(helpers.normal_weight(n, width, seed=70 + i, outlier_fraction=0.001), INT4,
+                                      bits=4, group=32 if width % 128 else 128, integer=True, asym=asym)
+              for i, n in enumerate(rows)]
+    for samples in (1, 2, 3, 4, 8):
+        x = helpers.activations(samples, width, seed=80 + samples, dtype=dtype)
+        biases = [helpers.activations(1, n, seed=90 + i, dtype=dtype)[0] if i != 1 else None for i, n in enumerate(rows)]
+        for with_bias in (False, True):
+            chosen = biases if with_bias else None
+            grouped = run_group(layers, x, chosen)
+            for index, layer in enumerate(layers):
+                bias = None if chosen is None else chosen[index]
+                separate = run_matvec(layer, x, bias=bias)
+                assert np.array_equal(grouped[index].float().cpu().numpy(), separate), (index, samples, with_bias)
+            check(grouped[0].float().cpu().numpy(), layers[0], x, None if chosen is None else chosen[0],
+                  relative=1e-3 if dtype == torch.float16 else 8e-3)
+
+
+def test_grouped_launch_of_other_codecs_runs_one_launch_per_matrix():
+    """Layouts the INT4 streaming kernels do not take go through the same entry point as
+    separate launches: same results as mk_packed_matvec."""
+    layers = [helpers.quantised_layer(helpers.normal_weight(n, 2048, seed=75 + i, student_t=True), scaling.NF4_VALUES,
+                                      bits=4, group=64, integer=False) for i, n in enumerate((64, 40))]
+    x = helpers.activations(2, 2048, seed=76)
+    grouped = run_group(layers, x)
+    for index, layer in enumerate(layers):
+        assert np.array_equal(grouped[index].float().cpu().numpy(), run_matvec(layer, x))
+        check(grouped[index].float().cpu().numpy(), layer, x)
+
+
+def test_grouped_launch_validation():
+    from mlkit_amd import native
+
+    lib = native.library()
+    x = torch.zeros(1, 256, device="cuda", dtype=torch.float16)
+    pointers = (ctypes.c_void_p * 9)(*([x.data_ptr()] * 9))
+    widths = (ctypes.c_int * 9)(*([16] * 9))
+    arguments = lambda count: (x.data_ptr(), 1, count, pointers, pointers, 1, None, 0, None, None, 0, pointers, widths,  # noqa: E731
+                               1, 256, 128, 4, 1, -8.0, 1.0, None)
+    assert lib.mk_packed_matvec_group(*arguments(9)) == native.MK_ERR_INVALID
+    assert "1 to 8 matrices" in native.last_error()
+    assert lib.mk_packed_matvec_group(*arguments(0)) == native.MK_ERR_INVALID
