@@ -80,6 +80,23 @@ int mk_packed_matvec_group(const void *x, int x_dtype, int count, const uint8_t 
                            void *const *y, const int *output_widths, int samples, int input_width,
                            int group, int bits, int uniform, float grid_min, float grid_step, void *stream);
 
+/* The online input rotation of a rotated layer and its packed matvec from one call:
+ * rotated = T(x * signs), T = (basis (x) H_power) * scale along the input width
+ * (input_width = order * power, power a power of two; order == 1: a plain Walsh-Hadamard
+ * transform, basis unused), written to `rotated` ([samples, input_width] of x_dtype, a
+ * buffer of the caller's that must not alias x), then mk_packed_matvec on `rotated` with the
+ * remaining arguments.  signs: NULL or [input_width] fp32 of +-1.  Results equal mk_fwht /
+ * mk_rotate_blocks followed by mk_packed_matvec bit for bit; MK_ERR_UNSUPPORTED when
+ * mk_rotate_blocks does not take (order, power).
+ * Replaces: the rotate_inputs forward pre-hook (conversion/model_transforms.py:116-128) in
+ * front of PackedLinear.forward (inference/packed_linear.py:148-245). */
+int mk_rotated_packed_matvec(const void *x, int x_dtype, void *rotated, int order, int power,
+                             const float *basis, const float *signs, float scale, const uint8_t *packed,
+                             const void *scales, int scale_dtype, const float *values, int n_values,
+                             const void *zeros, const void *bias, int bias_dtype, void *y, int samples,
+                             int output_width, int input_width, int group, int bits, int uniform,
+                             float grid_min, float grid_step, void *stream);
+
 /* out[n, k] = dequant(code[n, k]) in out_dtype, same dequantisation as mk_packed_matvec
  * with multiply and add kept separate (no fused multiply-add).
  * Replaces: kernels/packed_linear.py:279-313 (decode / decode_rows). */
@@ -87,6 +104,29 @@ int mk_packed_decode(const uint8_t *packed, const void *scales, int scale_dtype,
                      const float *values, int n_values, const void *zeros, void *out,
                      int out_dtype, int output_width, int input_width, int group, int bits,
                      int uniform, float grid_min, float grid_step, void *stream);
+
+/* Rows rows[0 .. n_rows) of the [output_width, input_width] packed matrix, decoded as by
+ * mk_packed_decode into out [n_rows, input_width]: the embedding lookup of a tied output
+ * projection.  rows: device int64; an index outside [0, output_width) decodes row 0.
+ * Replaces: the gather + unpack + decode_scaled of PackedEmbedding.forward
+ * (inference/packed_linear.py:273-287). */
+int mk_packed_decode_rows(const uint8_t *packed, const void *scales, int scale_dtype, const float *values,
+                          int n_values, const void *zeros, const long long *rows, int n_rows, void *out,
+                          int out_dtype, int output_width, int input_width, int group, int bits, int uniform,
+                          float grid_min, float grid_step, void *stream);
+
+/* packed = the little-endian bit stream of `count` codes of `bits` (1..16) bits: code i
+ * occupies stream bits [i * bits, (i + 1) * bits), byte j holds stream bits [8 j, 8 j + 8);
+ * ceil(count * bits / 8) bytes are written, the last one zero padded.  codes: uint8
+ * (code_bytes 1) or signed int16 / int32 / int64 (code_bytes 2 / 4 / 8).  *overflow (device
+ * int, NULL to skip; the caller zeroes it) becomes 1 when a code lies outside [0, 2^bits).
+ * Replaces: quantization/operations/bit_packing.py:13-77 (pack). */
+int mk_pack(const void *codes, int code_bytes, long long count, int bits, uint8_t *packed, int *overflow,
+            void *stream);
+
+/* codes[i] = code i of the stream written by mk_pack: uint8 for bits <= 8, int32 above.
+ * Replaces: quantization/operations/bit_packing.py:80-135 (unpack). */
+int mk_unpack(const uint8_t *packed, long long count, int bits, void *codes, void *stream);
 
 /* Scale storage formats of the scalar codec (formats/scale_storage.py:11-26). */
 #define MK_SCALE_FP32 0

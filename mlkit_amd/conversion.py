@@ -29,17 +29,30 @@ def record_transform(model: nn.Module, descriptor: dict[str, Any]) -> None:
     model.__dict__["_mlkit_transforms"] = descriptors
 
 
+class RotateInputs:
+    """The forward pre-hook of a rotated layer: its first positional input goes through the
+    layer's online rotation (fp16 / bf16 inputs are transformed in fp32 inside the kernel and
+    rounded once).  A class rather than a closure so that a packed layer can recognise the
+    hook and run the rotation in the same library call as its matvec."""
+
+    def __init__(self, rotation: OnlineRotation) -> None:
+        self.rotation = rotation
+
+    def __call__(self, layer: nn.Module, arguments: tuple) -> tuple:
+        return (self.rotation(arguments[0]), *arguments[1:])
+
+
 def install_transform(model: nn.Module, descriptor: dict[str, Any]) -> None:
     """Attach the online half of a recorded transform to the layer it names."""
     if descriptor["kind"] != "rotation":
         raise ValueError(f"unknown model transform {descriptor['kind']!r}")
-    rotation = OnlineRotation(descriptor["seed"])
-
-    def rotate_inputs(layer: nn.Module, arguments: tuple) -> tuple:
-        # fp16 / bf16 inputs are transformed in fp32 inside the kernel and rounded once
-        return (rotation(arguments[0]), *arguments[1:])
-
-    model.get_submodule(descriptor["name"]).register_forward_pre_hook(rotate_inputs)
+    layer = model.get_submodule(descriptor["name"])
+    hook = RotateInputs(OnlineRotation(descriptor["seed"]))
+    absorb = getattr(layer, "absorb_input_rotation", None)
+    if absorb is not None and not layer._forward_pre_hooks:
+        absorb(hook.rotation)  # a packed layer runs the rotation inside its own launch sequence
+    else:
+        layer.register_forward_pre_hook(hook)
 
 
 @dataclass

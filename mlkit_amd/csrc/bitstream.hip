@@ -1,0 +1,211 @@
+// Integer codes <-> little-endian bit stream on gfx950.
+//
+// Code i of width b occupies stream bits [i b, (i + 1) b); byte j holds stream bits
+// [8 j, 8 j + 8), least significant first; the stream is ceil(count b / 8) bytes.  A thread
+// owns 32 consecutive codes, which are exactly b dwords of the stream whatever b is, so no
+// two threads share a byte: the codes pass through a 64-bit shift register and leave (or
+// enter) as whole dwords.  The codes past the last whole run of 32 go byte by byte.
+//
+// Replaces the tensor operations of the reference's `pack` / `unpack`
+// (quantization/operations/bit_packing.py:13-135 in /root/reference/src/mlkit).
+
+#include <type_traits>
+
+#include "mk_common.h"
+
+namespace {
+
+constexpr int kRun = 32;  // codes per thread
+
+struct StreamArgs {
+    const void *codes_in;   // pack: source codes
+    void *codes_out;        // unpack: uint8 (bits <= 8) or int32 codes
+    uint8_t *packed;        // pack: target stream
+    const uint8_t *stream;  // unpack: source stream
+    long long count;
+    int bits;
+    int *overflow;
+};
+
+// Code `index` as an unsigned value; `bad` collects what does not fit `bits` bits.
+template <int CODE_BYTES>
+__device__ __forceinline__ uint32_t code_at(const void *codes, long long index, int bits, uint32_t &bad) {
+    if constexpr (CODE_BYTES == 1) {
+        const uint32_t value = static_cast<const uint8_t *>(codes)[index];
+        bad |= value >> bits;
+        return value;
+    } else if constexpr (CODE_BYTES == 2) {
+        const int value = static_cast<const int16_t *>(codes)[index];
+        bad |= static_cast<uint32_t>(value) >> bits;  // a negative value has high bits set
+        return static_cast<uint32_t>(value);
+    } else if constexpr (CODE_BYTES == 4) {
+        const int value = static_cast<const int32_t *>(codes)[index];
+        bad |= static_cast<uint32_t>(value) >> bits;
+        return static_cast<uint32_t>(value);
+    } else {
+        const long long value = static_cast<const long long *>(codes)[index];
+        bad |= (static_cast<unsigned long long>(value) >> bits) != 0 ? 1u : 0u;
+        return static_cast<uint32_t>(value);
+    }
+}
+
+// ALIGNED: the stream starts on a 4-byte boundary and whole runs are stored as dwords.
+template <int CODE_BYTES, bool ALIGNED>
+__global__ void __launch_bounds__(256) pack_kernel(const StreamArgs a) {
+    const long long whole_runs = a.count / kRun;
+    const long long runs = whole_runs + (a.count % kRun ? 1 : 0);
+    const uint32_t mask = (1u << a.bits) - 1u;
+    uint32_t bad = 0;
+    for (long long run = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; run < runs;
+         run += static_cast<long long>(gridDim.x) * blockDim.x) {
+        const long long first = run * kRun;
+        uint8_t *target = a.packed + run * (4 * a.bits);
+        if (run < whole_runs) {
+            uint64_t window = 0;
+            int filled = 0, word = 0;
+#pragma unroll
+            for (int i = 0; i < kRun; ++i) {
+                window |= static_cast<uint64_t>(code_at<CODE_BYTES>(a.codes_in, first + i, a.bits, bad) & mask) << filled;
+                filled += a.bits;
+                if (filled >= 32) {
+                    const uint32_t out = static_cast<uint32_t>(window);
+                    if constexpr (ALIGNED) {
+                        reinterpret_cast<uint32_t *>(target)[word] = out;
+                    } else {
+                        for (int b = 0; b < 4; ++b) target[4 * word + b] = static_cast<uint8_t>(out >> (8 * b));
+                    }
+                    ++word;
+                    window >>= 32;
+                    filled -= 32;
+                }
+            }
+        } else {  // the last, partial run: whole bytes, the final one zero padded
+            const int left = static_cast<int>(a.count - first);
+            uint64_t window = 0;
+            int filled = 0, byte = 0;
+            for (int i = 0; i < left; ++i) {
+                window |= static_cast<uint64_t>(code_at<CODE_BYTES>(a.codes_in, first + i, a.bits, bad) & mask) << filled;
+                filled += a.bits;
+                while (filled >= 8) {
+                    target[byte++] = static_cast<uint8_t>(window);
+                    window >>= 8;
+                    filled -= 8;
+                }
+            }
+            if (filled > 0) target[byte] = static_cast<uint8_t>(window);
+        }
+    }
+    if (bad && a.overflow) atomicOr(a.overflow, 1);
+}
+
+template <bool WIDE_CODES, bool ALIGNED>
+__global__ void __launch_bounds__(256) unpack_kernel(const StreamArgs a) {
+    const long long whole_runs = a.count / kRun;
+    const long long runs = whole_runs + (a.count % kRun ? 1 : 0);
+    const long long stream_bytes = (a.count * a.bits + 7) / 8;
+    const uint32_t mask = (1u << a.bits) - 1u;
+    for (long long run = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; run < runs;
+         run += static_cast<long long>(gridDim.x) * blockDim.x) {
+        const long long first = run * kRun;
+        const long long source_byte = run * (4 * a.bits);
+        const uint8_t *source = a.stream + source_byte;
+        const int left = run < whole_runs ? kRun : static_cast<int>(a.count - first);
+        uint64_t window = 0;
+        int filled = 0, word = 0;
+        uint32_t out[kRun];
+#pragma unroll
+        for (int i = 0; i < kRun; ++i) {
+            if (filled < a.bits && i < left) {
+                uint32_t next = 0;
+                if (ALIGNED && run < whole_runs) {
+                    next = reinterpret_cast<const uint32_t *>(source)[word];
+                } else {
+                    for (int b = 0; b < 4; ++b)
+                        if (source_byte + 4 * word + b < stream_bytes) next |= static_cast<uint32_t>(source[4 * word + b]) << (8 * b);
+                }
+                ++word;
+                window |= static_cast<uint64_t>(next) << filled;
+                filled += 32;
+            }
+            out[i] = static_cast<uint32_t>(window) & mask;
+            window >>= a.bits;
+            filled -= a.bits;
+        }
+        if constexpr (WIDE_CODES) {
+            int32_t *target = static_cast<int32_t *>(a.codes_out) + first;
+#pragma unroll
+            for (int i = 0; i < kRun; ++i)  // constant indices keep `out` in registers
+                if (i < left) target[i] = static_cast<int32_t>(out[i]);
+        } else {
+            uint8_t *target = static_cast<uint8_t *>(a.codes_out) + first;
+            if (left == kRun && (reinterpret_cast<uintptr_t>(target) & 3u) == 0) {
+#pragma unroll
+                for (int q = 0; q < kRun / 4; ++q)
+                    reinterpret_cast<uint32_t *>(target)[q] =
+                        out[4 * q] | (out[4 * q + 1] << 8) | (out[4 * q + 2] << 16) | (out[4 * q + 3] << 24);
+            } else {
+#pragma unroll
+                for (int i = 0; i < kRun; ++i)
+                    if (i < left) target[i] = static_cast<uint8_t>(out[i]);
+            }
+        }
+    }
+}
+
+unsigned grid_for(long long count) {
+    const long long runs = (count + kRun - 1) / kRun;
+    long long blocks = (runs + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    return static_cast<unsigned>(blocks < 1 ? 1 : blocks);
+}
+
+}  // namespace
+
+extern "C" int mk_pack(const void *codes, int code_bytes, long long count, int bits, uint8_t *packed, int *overflow,
+                       void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(bits >= 1 && bits <= 16, MK_ERR_INVALID, "mk_pack: packing supports one through sixteen bits");
+    MK_REQUIRE(count >= 0, MK_ERR_INVALID, "mk_pack: negative count");
+    MK_REQUIRE(code_bytes == 1 || code_bytes == 2 || code_bytes == 4 || code_bytes == 8, MK_ERR_INVALID,
+               "mk_pack: codes are uint8, int16, int32 or int64");
+    if (count == 0) return MK_OK;
+    MK_REQUIRE(codes && packed, MK_ERR_INVALID, "mk_pack: null tensor pointer");
+    StreamArgs a{};
+    a.codes_in = codes; a.packed = packed; a.count = count; a.bits = bits; a.overflow = overflow;
+    const bool aligned = (reinterpret_cast<uintptr_t>(packed) & 3u) == 0;
+    const dim3 grid(grid_for(count)), block(256);
+    auto launch = [&](auto aligned_tag) {
+        constexpr bool A = decltype(aligned_tag)::value;
+        switch (code_bytes) {
+            case 1: hipLaunchKernelGGL((pack_kernel<1, A>), grid, block, 0, stream, a); break;
+            case 2: hipLaunchKernelGGL((pack_kernel<2, A>), grid, block, 0, stream, a); break;
+            case 4: hipLaunchKernelGGL((pack_kernel<4, A>), grid, block, 0, stream, a); break;
+            default: hipLaunchKernelGGL((pack_kernel<8, A>), grid, block, 0, stream, a); break;
+        }
+    };
+    if (aligned) launch(std::true_type{});
+    else launch(std::false_type{});
+    MK_LAUNCH_CHECK("mk_pack");
+    return MK_OK;
+}
+
+extern "C" int mk_unpack(const uint8_t *packed, long long count, int bits, void *codes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(bits >= 1 && bits <= 16, MK_ERR_INVALID, "mk_unpack: one through sixteen bits");
+    MK_REQUIRE(count >= 0, MK_ERR_INVALID, "mk_unpack: negative count");
+    if (count == 0) return MK_OK;
+    MK_REQUIRE(packed && codes, MK_ERR_INVALID, "mk_unpack: null tensor pointer");
+    StreamArgs a{};
+    a.stream = packed; a.codes_out = codes; a.count = count; a.bits = bits;
+    const bool aligned = (reinterpret_cast<uintptr_t>(packed) & 3u) == 0;
+    const dim3 grid(grid_for(count)), block(256);
+    if (bits > 8) {
+        if (aligned) hipLaunchKernelGGL((unpack_kernel<true, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((unpack_kernel<true, false>), grid, block, 0, stream, a);
+    } else {
+        if (aligned) hipLaunchKernelGGL((unpack_kernel<false, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((unpack_kernel<false, false>), grid, block, 0, stream, a);
+    }
+    MK_LAUNCH_CHECK("mk_unpack");
+    return MK_OK;
+}

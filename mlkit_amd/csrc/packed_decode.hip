@@ -25,7 +25,16 @@ struct DecodeArgs {
     int bits, bytes_per_word, codes_per_word, uniform, n_values;
     float grid_min, grid_step;
     int chunks_per_group_shift;   // log2(group / 32) when that is a power of two (31: one group per row), else -1
+    const long long *row_index;   // null, or the source row of every output row (a gather of rows)
+    int source_rows;              // rows of the packed matrix; an index outside [0, source_rows) reads row 0
 };
+
+// The row of the packed matrix that output row `row` decodes.
+__device__ __forceinline__ size_t source_row_of(const DecodeArgs &a, size_t row) {
+    if (!a.row_index) return row;
+    const long long wanted = a.row_index[row];
+    return wanted >= 0 && wanted < a.source_rows ? static_cast<size_t>(wanted) : 0;
+}
 
 __global__ void packed_decode_kernel(const DecodeArgs a) {
     const int row_words = a.width / a.codes_per_word;
@@ -35,13 +44,14 @@ __global__ void packed_decode_kernel(const DecodeArgs a) {
          word += static_cast<size_t>(gridDim.x) * blockDim.x) {
         const size_t row = word / row_words;
         const int word_in_row = static_cast<int>(word - row * row_words);
-        const uint8_t *source = a.packed + word * a.bytes_per_word;
+        const size_t from = source_row_of(a, row);
+        const uint8_t *source = a.packed + (from * row_words + word_in_row) * a.bytes_per_word;
         uint64_t bits = 0;
         for (int b = 0; b < a.bytes_per_word; ++b) bits |= static_cast<uint64_t>(source[b]) << (8 * b);
         for (int i = 0; i < a.codes_per_word; ++i) {
             const int k = word_in_row * a.codes_per_word + i;
             const uint32_t code = static_cast<uint32_t>((bits >> (i * a.bits)) & mask);
-            const size_t slot = row * a.groups + k / a.group;
+            const size_t slot = from * a.groups + k / a.group;
             float weight;
             if (a.uniform) {
                 const float stepped = __fmul_rn(static_cast<float>(code), a.grid_step);
@@ -100,17 +110,18 @@ __global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeA
         const uint32_t chunk_in_row = chunk - row * row_chunks;
         const int first = static_cast<int>(chunk_in_row) * mk_matvec::kChunkCodes;
         mk_matvec::CodeChunk<BITS> codes;
-        mk_matvec::load_codes<BITS>(codes, a.packed + static_cast<size_t>(chunk) * (4 * BITS));
+        const size_t from = source_row_of(a, row);
+        mk_matvec::load_codes<BITS>(codes, a.packed + (from * row_chunks + chunk_in_row) * (4 * BITS));
         const uint32_t group_in_row = a.chunks_per_group_shift >= 0 ? chunk_in_row >> a.chunks_per_group_shift
                                                                     : static_cast<uint32_t>(first) / static_cast<uint32_t>(a.group);
-        size_t slot = static_cast<size_t>(row) * a.groups + group_in_row;
+        size_t slot = from * a.groups + group_in_row;
         float scale = mk_load_as_float(a.scales, slot, a.scale_dtype);
         float zero = has_zero ? mk_load_as_float(a.zeros, slot, a.scale_dtype) : 0.0f;
         float out[32];
 #pragma unroll
         for (int k = 0; k < 32; ++k) {
             if (!one_slot) {
-                slot = static_cast<size_t>(row) * a.groups + (first + k) / a.group;
+                slot = from * a.groups + (first + k) / a.group;
                 scale = mk_load_as_float(a.scales, slot, a.scale_dtype);
                 if (has_zero) zero = mk_load_as_float(a.zeros, slot, a.scale_dtype);
             }
@@ -141,7 +152,12 @@ __global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeA
             }
             mine[lane * (PIECES + 1) + q] = piece;
         }
-        // LDS operations of a wavefront complete in order: no barrier between the two loops.
+        // The pieces cross lanes through LDS: the wavefront's writes are ordered before its reads
+        // (the hardware completes a wavefront's LDS operations in order; the fence keeps the
+        // compiler from moving a read above a write it cannot prove distinct).
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         mk_u32x4 *target = static_cast<mk_u32x4 *>(a.out) + static_cast<size_t>(first_chunk) * PIECES;
         const size_t pieces_left = static_cast<size_t>(total - first_chunk) * PIECES;
 #pragma unroll
@@ -150,6 +166,9 @@ __global__ void __launch_bounds__(256) packed_decode_chunks_kernel(const DecodeA
             const mk_u32x4 piece = mine[(index / PIECES) * (PIECES + 1) + index % PIECES];
             if (static_cast<size_t>(index) < pieces_left) target[index] = piece;
         }
+        // ... and this trip's reads before the next trip's writes.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
@@ -176,26 +195,26 @@ void launch_chunks(const DecodeArgs &a, hipStream_t stream) {
 
 }  // namespace
 
-extern "C" int mk_packed_decode(const uint8_t *packed, const void *scales, int scale_dtype,
-                                const float *values, int n_values, const void *zeros, void *out,
-                                int out_dtype, int output_width, int input_width, int group, int bits,
-                                int uniform, float grid_min, float grid_step, void *stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
-    MK_REQUIRE(packed && scales && out, MK_ERR_INVALID, "mk_packed_decode: null tensor pointer");
-    MK_REQUIRE(mk_dtype_valid(scale_dtype) && mk_dtype_valid(out_dtype), MK_ERR_INVALID,
-               "mk_packed_decode: unknown dtype code");
-    MK_REQUIRE(output_width >= 1 && input_width >= 1 && group >= 1, MK_ERR_INVALID,
-               "mk_packed_decode: sizes must be positive");
-    MK_REQUIRE(bits >= 1 && bits <= 8, MK_ERR_INVALID, "mk_packed_decode: code width must be 1..8 bits");
+namespace {
+
+int decode_rows(const uint8_t *packed, const void *scales, int scale_dtype, const float *values, int n_values,
+                const void *zeros, void *out, int out_dtype, int output_rows, int input_width, int group, int bits,
+                int uniform, float grid_min, float grid_step, const long long *row_index, int source_rows,
+                const char *name, hipStream_t stream) {
+    MK_REQUIRE(packed && scales && out, MK_ERR_INVALID, "%s: null tensor pointer", name);
+    MK_REQUIRE(mk_dtype_valid(scale_dtype) && mk_dtype_valid(out_dtype), MK_ERR_INVALID, "%s: unknown dtype code", name);
+    MK_REQUIRE(output_rows >= 1 && input_width >= 1 && group >= 1, MK_ERR_INVALID, "%s: sizes must be positive", name);
+    MK_REQUIRE(bits >= 1 && bits <= 8, MK_ERR_INVALID, "%s: code width must be 1..8 bits", name);
     MK_REQUIRE(uniform || (values && n_values >= 1 && n_values <= (1 << bits)), MK_ERR_INVALID,
-               "mk_packed_decode: a value table of at most 2^bits entries is required");
+               "%s: a value table of at most 2^bits entries is required", name);
     MK_REQUIRE(mk_packed_layout_supported(bits, input_width, group), MK_ERR_UNSUPPORTED,
-               "mk_packed_decode: rows or scale groups split a packing word (bits=%d width=%d group=%d)",
-               bits, input_width, group);
+               "%s: rows or scale groups split a packing word (bits=%d width=%d group=%d)", name, bits, input_width,
+               group);
     DecodeArgs a;
     a.packed = packed; a.scales = scales; a.zeros = zeros; a.values = values; a.out = out;
-    a.rows = output_width; a.width = input_width; a.group = group; a.groups = mk_cdiv(input_width, group);
+    a.rows = output_rows; a.width = input_width; a.group = group; a.groups = mk_cdiv(input_width, group);
     a.scale_dtype = scale_dtype; a.out_dtype = out_dtype; a.bits = bits;
+    a.row_index = row_index; a.source_rows = source_rows;
     const int divisor = mk_gcd(bits, 8);
     a.bytes_per_word = bits / divisor; a.codes_per_word = 8 / divisor; a.uniform = uniform;
     a.grid_min = grid_min; a.grid_step = grid_step;
@@ -212,7 +231,7 @@ extern "C" int mk_packed_decode(const uint8_t *packed, const void *scales, int s
     }
     const bool wide = input_width % mk_matvec::kChunkCodes == 0 && (reinterpret_cast<uintptr_t>(packed) & 3u) == 0 &&
                       (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && bits >= 2 &&
-                      static_cast<long long>(output_width) * (input_width / mk_matvec::kChunkCodes) < (1ll << 31) - (1 << 24);
+                      static_cast<long long>(output_rows) * (input_width / mk_matvec::kChunkCodes) < (1ll << 31) - (1 << 24);
     if (wide) {
         switch (bits) {
             case 2: launch_chunks<2>(a, stream); break;
@@ -223,13 +242,37 @@ extern "C" int mk_packed_decode(const uint8_t *packed, const void *scales, int s
             case 7: launch_chunks<7>(a, stream); break;
             default: launch_chunks<8>(a, stream); break;
         }
-        MK_LAUNCH_CHECK("mk_packed_decode");
+        MK_LAUNCH_CHECK(name);
         return MK_OK;
     }
-    const size_t words = static_cast<size_t>(output_width) * (input_width / a.codes_per_word);
+    const size_t words = static_cast<size_t>(output_rows) * (input_width / a.codes_per_word);
     size_t blocks = (words + 255) / 256;
     if (blocks > 256u * 32u) blocks = 256u * 32u;
     hipLaunchKernelGGL(packed_decode_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
-    MK_LAUNCH_CHECK("mk_packed_decode");
+    MK_LAUNCH_CHECK(name);
     return MK_OK;
+}
+
+}  // namespace
+
+extern "C" int mk_packed_decode(const uint8_t *packed, const void *scales, int scale_dtype,
+                                const float *values, int n_values, const void *zeros, void *out,
+                                int out_dtype, int output_width, int input_width, int group, int bits,
+                                int uniform, float grid_min, float grid_step, void *stream) {
+    return decode_rows(packed, scales, scale_dtype, values, n_values, zeros, out, out_dtype, output_width, input_width,
+                       group, bits, uniform, grid_min, grid_step, nullptr, output_width, "mk_packed_decode",
+                       static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mk_packed_decode_rows(const uint8_t *packed, const void *scales, int scale_dtype,
+                                     const float *values, int n_values, const void *zeros, const long long *rows,
+                                     int n_rows, void *out, int out_dtype, int output_width, int input_width,
+                                     int group, int bits, int uniform, float grid_min, float grid_step,
+                                     void *stream) {
+    MK_REQUIRE(n_rows >= 0 && output_width >= 1, MK_ERR_INVALID, "mk_packed_decode_rows: sizes must be positive");
+    if (n_rows == 0) return MK_OK;
+    MK_REQUIRE(rows, MK_ERR_INVALID, "mk_packed_decode_rows: null row list");
+    return decode_rows(packed, scales, scale_dtype, values, n_values, zeros, out, out_dtype, n_rows, input_width, group,
+                       bits, uniform, grid_min, grid_step, rows, output_width, "mk_packed_decode_rows",
+                       static_cast<hipStream_t>(stream));
 }

@@ -19,6 +19,8 @@
 // (kernels/packed_linear.py:107-173 in /root/reference/src/mlkit).
 
 #pragma once
+#include <cstddef>
+
 #include "mk_common.h"
 
 namespace mk_matvec {
@@ -68,49 +70,56 @@ struct Stream4Args {
     int x_dtype, scale_dtype;  // pair-table kernel: MK_F16 or MK_BF16 each
 };
 // Several weight matrices that share the activations, the row width and the codec, multiplied
-// by one launch: workgroup `v` of the grid belongs to the member with the largest
-// first_tile <= v and multiplies that member's tile v - first_tile.  count == 0: the single
-// matrix described by Stream4Args.
+// by one launch: the grid's z index selects the member, x walks that member's tiles of rows
+// (workgroups past a shorter member's last tile leave at once).  count == 0: the single
+// matrix described by Stream4Args.  The member is known from the workgroup's index alone, so
+// its table entry is fetched together with the other arguments, not behind them.
 constexpr int kMaxGroupMembers = 8;
 struct Stream4Member {
     const uint8_t *packed;
     const void *scales, *zeros, *bias;
     void *y;
-    int rows;        // output width of this member (row stride of y)
-    int first_tile;  // tiles of all earlier members
+    int rows;   // output width of this member (row stride of y)
+    int tiles;  // whole tiles of rows this launch multiplies
 };
 struct Stream4Group {
-    int count, total_tiles;
+    int count, widest_tiles;
     Stream4Member member[kMaxGroupMembers];
 };
 
-// What one tile of rows reads and writes.
+// What a workgroup's matrix is: pointers, row count and number of tiles (wavefront-uniform).
 struct TileSource {
     const uint8_t *packed;
     const uint8_t *scales, *zeros;
     const void *bias;
     void *y;
-    int rows, tile;
+    int rows, tiles;
 };
 
-// Wavefront-uniform (v comes from blockIdx and the grid size): the member table is read with
-// scalar loads.
-__device__ __forceinline__ TileSource tile_source(const Stream4Args &a, const Stream4Group &g, int v) {
+// The kernels take (Stream4Args, Stream4Group) by value, i.e. in the kernel-argument segment,
+// which is constant memory: member `member` of the table is read from there with one scalar
+// load at a computed offset.  (Indexing the by-value parameter itself with a run-time index
+// makes the compiler copy the whole table to scratch memory first.)
+constexpr size_t kGroupTableOffset = (sizeof(Stream4Args) + alignof(Stream4Group) - 1) / alignof(Stream4Group) *
+                                     alignof(Stream4Group);
+
+template <int ROWS>
+__device__ __forceinline__ TileSource tile_source(const Stream4Args &a, const Stream4Group &g, int member) {
     TileSource s{a.packed, static_cast<const uint8_t *>(a.scales), static_cast<const uint8_t *>(a.zeros), a.bias, a.y,
-                 a.rows, v};
+                 a.rows, a.rows / ROWS};
     if (g.count > 0) {
-        int m = 0;
-#pragma unroll
-        for (int i = 1; i < kMaxGroupMembers; ++i)
-            if (i < g.count && v >= g.member[i].first_tile) m = i;
-        const Stream4Member &chosen = g.member[m];
-        s.packed = chosen.packed;
-        s.scales = static_cast<const uint8_t *>(chosen.scales);
-        s.zeros = static_cast<const uint8_t *>(chosen.zeros);
-        s.bias = chosen.bias;
-        s.y = chosen.y;
-        s.rows = chosen.rows;
-        s.tile = v - chosen.first_tile;
+        typedef const Stream4Member __attribute__((address_space(4))) *ConstantMember;
+        typedef const char __attribute__((address_space(4))) *ConstantBytes;
+        const ConstantBytes segment = (ConstantBytes)__builtin_amdgcn_kernarg_segment_ptr();
+        const ConstantMember chosen =
+            reinterpret_cast<ConstantMember>(segment + kGroupTableOffset + offsetof(Stream4Group, member)) + member;
+        s.packed = chosen->packed;
+        s.scales = static_cast<const uint8_t *>(chosen->scales);
+        s.zeros = static_cast<const uint8_t *>(chosen->zeros);
+        s.bias = chosen->bias;
+        s.y = chosen->y;
+        s.rows = chosen->rows;
+        s.tiles = chosen->tiles;
     }
     return s;
 }

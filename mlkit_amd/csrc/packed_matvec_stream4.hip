@@ -32,9 +32,12 @@ namespace {
 // per wavefront (both values swept on the GPU together with 8 / 32 rows and 4 - 16 ahead).
 constexpr int kWideRows = 16, kNarrowRows = 4;
 
+#ifndef MK_S4_AHEAD
+#define MK_S4_AHEAD 8
+#endif
 template <int ROWS>
 constexpr int rows_ahead_of() {
-    return ROWS < 8 ? ROWS : 8;
+    return ROWS < MK_S4_AHEAD ? ROWS : MK_S4_AHEAD;
 }
 
 // ---- bf16 activations ----------------------------------------------------------------------
@@ -93,7 +96,7 @@ __device__ __forceinline__ void chunk_dot_bf16(const CodeChunk<4> &codes, const 
 // row and lanes 32 - 63 the next, so that a step covers two rows instead of leaving half the
 // wavefront without codes.
 template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS>
-__global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const Stream4Group members) {
+__device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4Group &members) {
     static_assert(ROWS * MT <= 64 && ROWS % PARTS == 0, "one transposed reduction per workgroup");
     __shared__ float partials[64 * 8];  // [row sum][wavefront]
     // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
@@ -105,6 +108,8 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const
     constexpr int kSums = kStreamRows * MT;
     constexpr int kRowLanes = 64 / PARTS;
 
+    const TileSource source = tile_source<ROWS>(a, members, blockIdx.z);
+    if (static_cast<int>(blockIdx.x) >= source.tiles) return;  // a shorter member of a group: the whole workgroup leaves
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -121,16 +126,23 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const
 
     // The workgroup is aligned first: a compute unit serves loads first come, first served,
     // and a wavefront that starts late would queue its small loads behind the others' codes.
+#ifndef MK_S4_NO_LEAD_BARRIER
     __syncthreads();
+#endif
 
     // Activations: 32 per sample, as 16 fp16 pairs (L2 hits), requested first.
     mk_u32x4 pieces[MT][4];
+    auto request_activations = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        const int sample = sample_base + m < a.samples ? sample_base + m : a.samples - 1;
+        for (int m = 0; m < MT; ++m) {
+            const int sample = sample_base + m < a.samples ? sample_base + m : a.samples - 1;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) pieces[m][i] = request_piece(a, sample, wave * 2048, i, lane);
-    }
+            for (int i = 0; i < 4; ++i) pieces[m][i] = request_piece(a, sample, wave * 2048, i, lane);
+        }
+    };
+#ifndef MK_S4_CODES_FIRST
+    request_activations();
+#endif
     // The scale (and offset) of this lane's chunk in every row, 2 bytes each.
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
     const uint32_t group_offset = static_cast<uint32_t>(part) * scale_row_bytes +
@@ -141,30 +153,40 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const
     constexpr bool kStrided = PARTS == 2;
     XChunk<XT> x[MT];
     float x_sum[MT], grid_term[MT];
-    const int tiles = members.count > 0 ? members.total_tiles : a.rows / ROWS;
     int tile = blockIdx.x;
     bool first_tile = true;
     do {
-    const TileSource source = tile_source(a, members, tile);  // uniform
-    const int row_base = source.tile * ROWS;
+    const int row_base = tile * ROWS;
     const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
     const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
     const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
     uint16_t scale_raw[kStreamRows], zero_raw[HAS_ZERO ? kStreamRows : 1];
-#pragma unroll
-    for (int r = 0; r < kStreamRows; ++r) {
-        scale_raw[r] = *reinterpret_cast<const uint16_t *>(scale_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
-        if constexpr (HAS_ZERO)
-            zero_raw[r] = *reinterpret_cast<const uint16_t *>(zero_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
     CodeChunk<4> codes[kStreamRows];
+    auto request_sides = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int r = 0; r < kStreamAhead; ++r) {
-        load_codes<4>(codes[r], codes_base + static_cast<size_t>(PARTS * r) * row_bytes + code_offset);
-        __builtin_amdgcn_sched_barrier(0);  // in row order
-    }
+        for (int r = 0; r < kStreamRows; ++r) {
+            scale_raw[r] = *reinterpret_cast<const uint16_t *>(scale_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
+            if constexpr (HAS_ZERO)
+                zero_raw[r] = *reinterpret_cast<const uint16_t *>(zero_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto request_codes = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < kStreamAhead; ++r) {
+            load_codes<4>(codes[r], codes_base + static_cast<size_t>(PARTS * r) * row_bytes + code_offset);
+            __builtin_amdgcn_sched_barrier(0);  // in row order
+        }
+    };
+#ifdef MK_S4_CODES_FIRST
+    request_codes();
+    if (first_tile) request_activations();
+    __builtin_amdgcn_sched_barrier(0);
+    request_sides();
+#else
+    request_sides();
+    request_codes();
+#endif
 
     if (first_tile) {  // uniform
     // Each lane's chunk of every sample, through the wavefront's LDS buffer (LDS operations
@@ -236,8 +258,31 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const
     if constexpr (!kStrided) break;
     __syncthreads();  // `partials` is reused by the next tile
     tile += gridDim.x;
-    } while (tile < tiles);
+    } while (tile < source.tiles);
 }
+
+template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS>
+__global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const Stream4Group members) {
+    stream4_body<MT, HAS_ZERO, ROWS, XT, PARTS>(a, members);
+}
+
+#ifdef MK_S4_FLAT
+// Experiment: one sample, fp16, no offsets, with the arguments as scalars so that the first
+// of them can be preloaded into scalar registers at dispatch.
+__global__ void __launch_bounds__(512) stream4_flat_kernel(const void *x, const uint8_t *packed, const void *scales,
+                                                           int width, int samples, int group, int groups, int rows,
+                                                           void *y, const void *bias, int bias_dtype, float grid_min,
+                                                           float grid_step, int scale_dtype) {
+    Stream4Args a;
+    a.x = x; a.packed = packed; a.scales = scales; a.zeros = nullptr; a.bias = bias; a.y = y;
+    a.samples = samples; a.rows = rows; a.width = width; a.group = group; a.groups = groups;
+    a.bias_dtype = bias_dtype; a.grid_min = grid_min; a.grid_step = grid_step; a.values = nullptr;
+    a.n_values = 0; a.uniform = 1; a.bits = 4; a.x_dtype = MK_F16; a.scale_dtype = scale_dtype;
+    Stream4Group none;
+    none.count = 0;
+    stream4_body<1, false, 16, MK_F16, 1>(a, none);
+}
+#endif
 
 // ---- two to eight samples: the dot products on the matrix cores ---------------------------
 //
@@ -272,6 +317,8 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     constexpr int kSampleWords = blocks_sample_words(SLICES);
     uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * (4 * kSampleWords);
 
+    const TileSource source = tile_source<ROWS>(a, members, blockIdx.z);
+    if (static_cast<int>(blockIdx.x) >= source.tiles) return;  // a shorter member of a group: the whole workgroup leaves
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -343,11 +390,9 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     // A workgroup prepares its activations once and then (short rows) takes every
     // gridDim.x-th tile of ROWS rows: tall matrices, with many more tiles than the GPU holds
     // workgroups, pay for the preparation once per workgroup instead of once per tile.
-    const int tiles = members.count > 0 ? members.total_tiles : a.rows / ROWS;
     int tile = blockIdx.x;
     do {
-    const TileSource source = tile_source(a, members, tile);  // uniform
-    const int row_base = source.tile * ROWS;
+    const int row_base = tile * ROWS;
     const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
     const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
     const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
@@ -463,7 +508,7 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     if constexpr (!kStrided) break;
     __syncthreads();  // `partials` is reused by the next tile
     tile += gridDim.x;
-    } while (tile < tiles);
+    } while (tile < source.tiles);
 }
 
 // The number of workgroups of `kernel` the GPU holds at once, asked of the runtime the first
@@ -488,7 +533,7 @@ int launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int 
     const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
     // at most 8 wavefronts x 4 samples x 4112 bytes = 129 KB of the CU's 160 KB
     const size_t slices = static_cast<size_t>(block.x / 64) * 4 * blocks_sample_words(SLICES) * sizeof(uint32_t);
-    dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
+    dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS), members.count > 0 ? members.count : 1);
     // More than 64 KB of dynamic LDS has to be allowed per kernel (static LDS counts against
     // the CU's 160 KB too, so only what this launch needs is asked for).
     auto launch = [&](auto kernel) -> int {
@@ -504,7 +549,7 @@ int launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int 
             // with that stride.  (Asked of the runtime once per kernel and workgroup size.)
             static std::atomic<int> resident[3];
             const int known = resident_workgroups(kernel, static_cast<int>(block.x), slices, resident[block.x / 64]);
-            if (static_cast<int>(grid.x) > known) grid.x = known;
+            if (grid.x * grid.z > static_cast<unsigned>(known)) grid.x = mk_cdiv(known, static_cast<int>(grid.z));
         }
         hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
         return 0;
@@ -528,18 +573,25 @@ int launch_blocks(const Stream4Args &a, const Stream4Group &members, int tiles, 
 
 template <int MT, int ROWS, int PARTS>
 int launch_tile_parts(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
-    dim3 grid(tiles, mk_cdiv(a.samples, MT));
+    dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1);
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
     auto launch = [&](auto kernel) -> int {
         if constexpr (PARTS == 2) {  // short rows: one wavefront per workgroup, which walks the tiles
             static std::atomic<int> known{0};
             const int resident = resident_workgroups(kernel, static_cast<int>(block.x), slices, known);
-            if (static_cast<int>(grid.x) > resident) grid.x = resident;
+            if (grid.x * grid.z > static_cast<unsigned>(resident)) grid.x = mk_cdiv(resident, static_cast<int>(grid.z));
         }
         hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
         return 0;
     };
+#ifdef MK_S4_FLAT
+    if (MT == 1 && ROWS == 16 && PARTS == 1 && a.x_dtype == MK_F16 && !a.zeros && members.count == 0) {
+        hipLaunchKernelGGL(stream4_flat_kernel, grid, block, slices, stream, a.x, a.packed, a.scales, a.width, a.samples,
+                           a.group, a.groups, a.rows, a.y, a.bias, a.bias_dtype, a.grid_min, a.grid_step, a.scale_dtype);
+        return 0;
+    }
+#endif
     if (a.x_dtype == MK_F16) {
         if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_F16, PARTS>);
         return launch(stream4_kernel<MT, false, ROWS, MK_F16, PARTS>);
@@ -586,7 +638,7 @@ bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, i
 int stream4_launch(const Stream4Args &a, hipStream_t stream) {
     Stream4Group none;
     none.count = 0;
-    none.total_tiles = 0;
+    none.widest_tiles = 0;
     if (a.rows / kWideRows >= kComputeUnits) {
         const int tiles = a.rows / kWideRows;
         return launch_rows<kWideRows>(a, none, tiles, stream) ? -1 : tiles * kWideRows;
@@ -600,18 +652,18 @@ int stream4_launch_group(const Stream4Args &shared, Stream4Group &group, const i
     long long wide_tiles = 0;
     for (int i = 0; i < group.count; ++i) wide_tiles += member_rows[i] / kWideRows;
     const int rows = wide_tiles >= kComputeUnits ? kWideRows : kNarrowRows;
-    int first = 0;
+    int widest = 0;
     for (int i = 0; i < group.count; ++i) {
         group.member[i].rows = member_rows[i];
-        group.member[i].first_tile = first;
-        first += member_rows[i] / rows;
+        group.member[i].tiles = member_rows[i] / rows;
+        if (group.member[i].tiles > widest) widest = group.member[i].tiles;
     }
-    group.total_tiles = first;
+    group.widest_tiles = widest;
     *rows_per_tile = rows;
     Stream4Args a = shared;
     a.zeros = group.member[0].zeros;  // selects the kernel variant; the members agree on it
-    if (rows == kWideRows) return launch_rows<kWideRows>(a, group, first, stream);
-    return launch_rows<kNarrowRows>(a, group, first, stream);
+    if (rows == kWideRows) return launch_rows<kWideRows>(a, group, widest, stream);
+    return launch_rows<kNarrowRows>(a, group, widest, stream);
 }
 
 }  // namespace mk_matvec

@@ -1,0 +1,50 @@
+// Online input rotation followed by the packed matvec, enqueued from one call.
+//
+// A rotated layer (the reference's `rotate_inputs` forward pre-hook,
+// conversion/model_transforms.py:116-128 in /root/reference/src/mlkit, in front of
+// PackedLinear.forward, inference/packed_linear.py:148-245) multiplies its packed weight with
+// T(x * signs), T = (basis (x) H_power) / sqrt(power) along the input width.  The rotated
+// activations are at most 8 x 16384 values: they are written to a small buffer by the
+// Walsh-Hadamard / blocked-rotation kernel and read back, from L2, by the matvec kernel
+// enqueued right behind it on the same stream.  One library call replaces a Python hook, an
+// allocation and two calls.
+
+#include "mk_common.h"
+
+namespace {
+
+int rotate_then_multiply(const void *x, int x_dtype, void *rotated, int order, int power, const float *basis,
+                         const float *signs, float scale, const uint8_t *packed, const void *scales, int scale_dtype,
+                         const float *values, int n_values, const void *zeros, const void *bias, int bias_dtype, void *y,
+                         int samples, int output_width, int input_width, int group, int bits, int uniform,
+                         float grid_min, float grid_step, void *stream) {
+    MK_REQUIRE(x && rotated && x != rotated, MK_ERR_INVALID,
+               "mk_rotated_packed_matvec: activations and their rotated copy must be two buffers");
+    MK_REQUIRE(order >= 1 && power >= 1 && static_cast<long long>(order) * power == input_width, MK_ERR_INVALID,
+               "mk_rotated_packed_matvec: order * power must equal the input width (%d * %d != %d)", order, power,
+               input_width);
+    MK_REQUIRE(order == 1 || basis, MK_ERR_INVALID, "mk_rotated_packed_matvec: a blocked rotation needs its basis");
+    int status;
+    if (order == 1)
+        status = mk_fwht(x, x_dtype, rotated, x_dtype, samples, input_width, signs, nullptr, signs ? input_width : 0, scale,
+                         stream);
+    else
+        status = mk_rotate_blocks(x, x_dtype, rotated, x_dtype, samples, order, power, basis, 0, signs, nullptr, scale,
+                                  stream);
+    if (status) return status;
+    return mk_packed_matvec(rotated, x_dtype, packed, scales, scale_dtype, values, n_values, zeros, bias, bias_dtype, y,
+                            samples, output_width, input_width, group, bits, uniform, grid_min, grid_step, stream);
+}
+
+}  // namespace
+
+extern "C" int mk_rotated_packed_matvec(const void *x, int x_dtype, void *rotated, int order, int power,
+                                        const float *basis, const float *signs, float scale, const uint8_t *packed,
+                                        const void *scales, int scale_dtype, const float *values, int n_values,
+                                        const void *zeros, const void *bias, int bias_dtype, void *y, int samples,
+                                        int output_width, int input_width, int group, int bits, int uniform,
+                                        float grid_min, float grid_step, void *stream) {
+    return rotate_then_multiply(x, x_dtype, rotated, order, power, basis, signs, scale, packed, scales, scale_dtype, values,
+                                n_values, zeros, bias, bias_dtype, y, samples, output_width, input_width, group, bits,
+                                uniform, grid_min, grid_step, stream);
+}

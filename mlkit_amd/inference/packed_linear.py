@@ -1,21 +1,30 @@
 """A linear layer (and a tied embedding) that execute packed scalar-grid codes.
 
-Mirrors /root/reference/src/mlkit/inference/packed_linear.py: ``PackedLinear`` (:41-245),
-``PackedEmbedding`` (:248-287), ``packed_compatible`` (:290-304) -- same buffers
+Drop-in for /root/reference/src/mlkit/inference/packed_linear.py: ``PackedLinear`` (:41-245),
+``PackedEmbedding`` (:248-287), ``packed_compatible`` (:290-304) -- the same buffers
 (``packed``, ``scales``, ``values``, ``zeros``, ``bias``; ``_dense_weight`` non-persistent),
-attributes and error messages.  Up to ``maximum_fused_rows`` input rows go to
-``mk_packed_matvec``; larger inputs decode the weight once (``mk_packed_decode``) and use an
-ordinary matrix product.
+attributes and error messages.
+
+How a call is served here:
+
+* up to ``maximum_fused_rows`` input rows: one ``mk_packed_matvec`` launch, or, when the layer
+  has absorbed its online input rotation, one ``mk_rotated_packed_matvec`` call (rotation
+  kernel and matvec enqueued back to back, the rotated activations staying in a small buffer
+  of the layer);
+* more rows, or a layout without a fused kernel: the weight is decoded once
+  (``mk_packed_decode``) and an ordinary matrix product follows;
+* a tied embedding decodes only the requested rows (``mk_packed_decode_rows``).
 """
 
 from collections.abc import Callable
+from dataclasses import dataclass
 
 import torch
 import torch.nn.functional as functional
 from torch import Tensor, nn
 
 from mlkit_amd import native
-from mlkit_amd.kernels.packed_linear import MAXIMUM_CODE_BITS, decode, layout_for, packed_matvec_op
+from mlkit_amd.kernels.packed_linear import MAXIMUM_CODE_BITS, PackedLayout, decode, layout_for, packed_matvec_op
 from mlkit_amd.quantization.bitstream import pack, unpack
 from mlkit_amd.quantization.codecs import decode_scaled
 from mlkit_amd.quantization.core import Q
@@ -32,6 +41,41 @@ def preserve_input_processing(original: nn.Module, replacement: nn.Module) -> No
     for name, value in original.named_buffers(recurse=False):
         if name.startswith("_mlkit_"):
             replacement.register_buffer(name, value.detach().clone())
+
+
+def packed_compatible(quantized: Q) -> bool:
+    """Whether ``quantized`` can be held as a packed stream: a complete ``scaled`` / ``feedback``
+    codec of one to eight bits whose table fits the code width, in natural column order, with
+    no code offset and refit regions made of whole scale groups."""
+    if quantized.codec not in ("scaled", "feedback") or quantized.codes is None:
+        return False
+    parameters = quantized.params
+    width = quantized.metadata.get("code_bits")
+    if not isinstance(width, int) or not 1 <= width <= MAXIMUM_CODE_BITS:
+        return False
+    if parameters["values"].numel() > (1 << width):
+        return False
+    if parameters.get("permutation") is not None or parameters.get("offset", 0) != 0:
+        return False
+    group = parameters["group"]
+    return parameters.get("refit", group) % group == 0
+
+
+@dataclass(frozen=True)
+class _Grid:
+    """The value table as the kernels see it: affine grids need no table lookup."""
+
+    uniform: bool
+    minimum: float
+    step: float
+
+    @staticmethod
+    def of(values: Tensor) -> "_Grid":
+        table = values.detach().float().cpu()
+        if table.numel() < 2:
+            return _Grid(False, float(table[0]) if table.numel() else 0.0, 1.0)
+        gaps = table[1:] - table[:-1]
+        return _Grid(bool(torch.allclose(gaps, gaps[0].expand_as(gaps))), float(table[0]), float(gaps[0]))
 
 
 class PackedLinear(nn.Module):
@@ -54,86 +98,120 @@ class PackedLinear(nn.Module):
             raise ValueError(
                 "PackedLinear requires a complete scalar-grid codec of at most eight bits in "
                 "its original column order with refit boundaries aligned to scale groups")
-        assert quantized.codes is not None
         device = original.weight.device
         if device.type != "cuda":
             raise ValueError("PackedLinear requires CUDA weights")
-        native.library()  # fail here, not at the first forward, when the kernels are not built
+        native.library()  # a missing kernel library is reported here, not at the first forward
+        parameters, metadata = quantized.params, quantized.metadata
         self.in_features, self.out_features = original.in_features, original.out_features
-        self.group = quantized.params["group"]
-        self.code_bits = int(quantized.metadata["code_bits"])
+        self.group: int = parameters["group"]
+        self.code_bits = int(metadata["code_bits"])
         self.storage_dtype = original.weight.dtype
         self.cache_dense = cache_dense
-        scales = quantized.params["scales"]
-        side_dtype = SCALE_STORAGE_DTYPES.get(str(quantized.metadata.get("scale_fmt")), scales.dtype)
-        zero = quantized.params.get("zero")
-        self.register_buffer("packed", pack(quantized.codes, self.code_bits).to(device))
-        self.register_buffer("scales", scales.to(device=device, dtype=side_dtype).contiguous())
-        self.register_buffer("values", quantized.params["values"].to(device=device, dtype=torch.float32).contiguous())
-        self.register_buffer("zeros", None if zero is None else zero.to(device=device, dtype=side_dtype).contiguous())
+        # Side information is kept in the 16-bit format it was rounded to, when there is one.
+        side_dtype = SCALE_STORAGE_DTYPES.get(str(metadata.get("scale_fmt")), parameters["scales"].dtype)
+
+        def resident(tensor: Tensor | None, dtype: torch.dtype) -> Tensor | None:
+            return None if tensor is None else tensor.detach().to(device=device, dtype=dtype).contiguous()
+
+        self.register_buffer("packed", pack(quantized.codes.to(device), self.code_bits))
+        self.register_buffer("scales", resident(parameters["scales"], side_dtype))
+        self.register_buffer("values", resident(parameters["values"], torch.float32))
+        self.register_buffer("zeros", resident(parameters.get("zero"), side_dtype))
         self.register_buffer("bias", None if original.bias is None else original.bias.detach().clone())
         self.register_buffer("_dense_weight", None, persistent=False)
-        table = quantized.params["values"].detach().cpu().float()
-        steps = table.diff()
-        self.uniform_grid = bool(len(steps) and torch.allclose(steps, steps[0].expand_as(steps)))
-        self.grid_minimum = float(table[0])
-        self.grid_step = float(steps[0]) if len(steps) else 1.0
-        self.layout = layout_for(self.code_bits, self.in_features, self.group)
-        self.maximum_fused_rows = 0 if self.layout is None else MAXIMUM_FUSED_ROWS
+        grid = _Grid.of(parameters["values"])
+        self.uniform_grid, self.grid_minimum, self.grid_step = grid.uniform, grid.minimum, grid.step
+        self.layout: PackedLayout | None = layout_for(self.code_bits, self.in_features, self.group)
+        self.maximum_fused_rows = MAXIMUM_FUSED_ROWS if self.layout is not None else 0
         self._launch: tuple | None = None
+        self._rotation = None          # an absorbed OnlineRotation
+        self._rotation_launch: tuple | None = None
         preserve_input_processing(original, self)
+        self._absorb_rotation_hook()
+
+    # -- online input rotation ---------------------------------------------------------------
+
+    def absorb_input_rotation(self, rotation) -> None:
+        """Run ``rotation`` (an ``OnlineRotation``) on the inputs inside ``forward`` instead of
+        in a forward pre-hook: short inputs then take one library call for rotation + matvec."""
+        self._rotation = rotation
+        self._rotation_launch = None
+
+    def _absorb_rotation_hook(self) -> None:
+        """A carried-over ``RotateInputs`` pre-hook is taken in when it is the only pre-hook
+        (so the order in which input transforms apply cannot change)."""
+        from mlkit_amd.conversion import RotateInputs
+
+        hooks = self._forward_pre_hooks
+        if len(hooks) == 1 and not self._forward_pre_hooks_with_kwargs:
+            (key, hook), = hooks.items()
+            if isinstance(hook, RotateInputs):
+                del hooks[key]
+                self.absorb_input_rotation(hook.rotation)
+
+    # -- module plumbing ---------------------------------------------------------------------
 
     def _apply(self, fn: Callable[[Tensor], Tensor], recurse: bool = True) -> "PackedLinear":
-        self._launch = None
+        self._launch = self._rotation_launch = None
         self._dense_weight = None
         return super()._apply(fn, recurse)
 
     @property
     def weight(self) -> Tensor:
-        if self._dense_weight is not None:
-            return self._dense_weight
-        if self.layout is None:
-            codes = unpack(self.packed, self.code_bits, (self.out_features, self.in_features))
-            dense = decode_scaled(codes, scales=self.scales.float(), values=self.values, group=self.group,
-                                  zero=None if self.zeros is None else self.zeros.float()).to(self.storage_dtype)
-        else:
-            dense = torch.empty((self.out_features, self.in_features), device=self.packed.device,
-                                dtype=self.storage_dtype)
+        """The dense ``[out_features, in_features]`` weight in the storage dtype."""
+        cached = self._dense_weight
+        if cached is not None:
+            return cached
+        shape = (self.out_features, self.in_features)
+        if self.layout is not None:
+            dense = torch.empty(shape, device=self.packed.device, dtype=self.storage_dtype)
             decode(self.packed, self.scales, self.values, self.zeros, dense, self.group, self.layout,
                    self.uniform_grid, self.grid_minimum, self.grid_step)
+        else:  # rows or groups split a packing word: unpack the stream, then the scalar decoder
+            offsets = self.zeros.float() if self.zeros is not None else None
+            dense = decode_scaled(unpack(self.packed, self.code_bits, shape), scales=self.scales.float(),
+                                  values=self.values, group=self.group, zero=offsets).to(self.storage_dtype)
         if self.cache_dense:
             self._dense_weight = dense
         return dense
 
+    # -- forward -----------------------------------------------------------------------------
+
     def forward(self, inputs: Tensor) -> Tensor:
-        width = self.in_features
-        shape = inputs.shape
-        if shape[-1] != width:
+        if inputs.shape[-1] != self.in_features:
             raise ValueError("input width does not match the packed linear")
         if not inputs.is_cuda:
             raise ValueError("packed inference requires CUDA inputs")
-        rows = inputs.numel() // width
-        if rows > self.maximum_fused_rows or rows == 0 or inputs.dtype not in native.DTYPE_CODES:
+        rows = inputs.numel() // self.in_features
+        fused = 0 < rows <= self.maximum_fused_rows and inputs.dtype in native.DTYPE_CODES
+        compiling = torch.compiler.is_compiling()
+        rotate_here = False
+        if self._rotation is not None:
+            if fused and not compiling and self._rotation_arguments(inputs) is not None:
+                rotate_here = True
+            else:
+                inputs = self._rotation(inputs)   # the general path: rotate, then as an unrotated layer
+        if not fused:
             return functional.linear(inputs, self.weight.to(inputs.dtype), self.bias)
         if inputs.requires_grad and torch.is_grad_enabled():
             raise RuntimeError("packed CUDA inference does not support autograd")
-        flat = inputs.reshape(rows, width)
+        flat = inputs.reshape(rows, self.in_features)
         if not flat.is_contiguous():
             flat = flat.contiguous()
-        if torch.compiler.is_compiling():
+        if compiling:
             output = packed_matvec_op(flat, self.packed, self.scales, self.values, self.zeros, self.bias,
                                       self.out_features, self.group, self.code_bits, self.uniform_grid,
                                       self.grid_minimum, self.grid_step)
         else:
             output = inputs.new_empty((rows, self.out_features))
-            self._matvec(flat, output, rows)
-        return output.view(shape[:-1] + (self.out_features,))
+            self._matvec(flat, output, rows, rotate_here)
+        return output.view(inputs.shape[:-1] + (self.out_features,))
 
-    def _matvec(self, inputs: Tensor, output: Tensor, rows: int) -> None:
-        """One call into the C ABI.  The layer's constant arguments are bound once and kept
-        for as long as all five buffers stay where they were: the key is every buffer's
-        address, so a moved, cast, reassigned or reloaded ``scales`` / ``zeros`` / ``bias`` /
-        ``values`` / ``packed`` rebuilds them."""
+    def _bound_arguments(self) -> tuple:
+        """The layer's constant launch arguments, bound once and kept for as long as all five
+        buffers stay where they were: the key is every buffer's address and dtype, so a moved,
+        cast, reassigned or reloaded buffer rebuilds them."""
         buffers = self._buffers
         packed, scales, values = buffers["packed"], buffers["scales"], buffers["values"]
         zeros, bias = buffers["zeros"], buffers["bias"]
@@ -149,10 +227,36 @@ class PackedLinear(nn.Module):
                 (self.out_features, self.in_features, self.group, self.code_bits, int(self.uniform_grid),
                  self.grid_minimum, self.grid_step),
             )
-        _, tensors, constants = launch
-        status = native.library().mk_packed_matvec(
-            inputs.data_ptr(), native.DTYPE_CODES[inputs.dtype], *tensors, output.data_ptr(), rows, *constants,
-            native.current_stream(inputs.device))
+        return launch
+
+    def _rotation_arguments(self, inputs: Tensor) -> tuple | None:
+        """``(key, rotated buffer, leading arguments of mk_rotated_packed_matvec, keep)`` for
+        this device and input dtype, or None when the rotation kernels do not take the width."""
+        key = (inputs.device, inputs.dtype)
+        bound = self._rotation_launch
+        if bound is None or bound[0] != key:
+            arguments = self._rotation.launch_arguments(self.in_features, inputs.device)
+            if arguments is None:
+                bound = self._rotation_launch = (key, None, None, None)
+            else:
+                order, power, basis, signs, scale, keep = arguments
+                rotated = torch.empty((MAXIMUM_FUSED_ROWS, self.in_features), dtype=inputs.dtype, device=inputs.device)
+                bound = self._rotation_launch = (key, rotated, (order, power, basis, signs, scale), keep)
+        return None if bound[1] is None else bound
+
+    def _matvec(self, inputs: Tensor, output: Tensor, rows: int, rotate: bool = False) -> None:
+        """One call into the C ABI on the current stream."""
+        _, tensors, constants = self._bound_arguments()
+        stream = native.current_stream(inputs.device)
+        code = native.DTYPE_CODES[inputs.dtype]
+        if rotate:
+            _, rotated, rotation, _ = self._rotation_arguments(inputs)
+            status = native.library().mk_rotated_packed_matvec(
+                inputs.data_ptr(), code, rotated.data_ptr(), *rotation, *tensors, output.data_ptr(), rows, *constants,
+                stream)
+        else:
+            status = native.library().mk_packed_matvec(inputs.data_ptr(), code, *tensors, output.data_ptr(), rows,
+                                                       *constants, stream)
         if status:
             native.check(status)
 
@@ -184,24 +288,13 @@ class PackedEmbedding(nn.Module):
 
     def forward(self, indices: Tensor) -> Tensor:
         head = self.projection
-        rows = indices.reshape(-1)
-        taken = head.packed.view(self.num_embeddings, -1)[rows]
-        codes = unpack(taken.reshape(-1), head.code_bits, (rows.numel(), self.embedding_dim))
-        embedded = decode_scaled(codes, scales=head.scales[rows].float(), values=head.values, group=head.group,
-                                 zero=None if head.zeros is None else head.zeros[rows].float())
-        return embedded.to(head.storage_dtype).view(*indices.shape, self.embedding_dim)
-
-
-def packed_compatible(quantized: Q) -> bool:
-    """A complete scalar codec of at most eight bits, unpermuted, with refit regions that are
-    whole scale groups."""
-    if quantized.codec not in {"scaled", "feedback"}:
-        return False
-    group = quantized.params["group"]
-    code_bits = quantized.metadata.get("code_bits")
-    return (isinstance(code_bits, int) and 1 <= code_bits <= MAXIMUM_CODE_BITS
-            and quantized.codes is not None
-            and quantized.params["values"].numel() <= 2**code_bits
-            and quantized.params.get("offset", 0) == 0
-            and quantized.params.get("permutation") is None
-            and quantized.params.get("refit", group) % group == 0)
+        device = head.packed.device
+        tokens = indices.reshape(-1).to(device=device, dtype=torch.int64).contiguous()
+        embedded = torch.empty((tokens.numel(), self.embedding_dim), dtype=head.storage_dtype, device=device)
+        if tokens.numel():
+            native.check(native.library().mk_packed_decode_rows(
+                head.packed.data_ptr(), head.scales.data_ptr(), native.dtype_code(head.scales), head.values.data_ptr(),
+                head.values.numel(), native.pointer(head.zeros), tokens.data_ptr(), tokens.numel(), embedded.data_ptr(),
+                native.dtype_code(embedded), self.num_embeddings, self.embedding_dim, head.group, head.code_bits,
+                int(head.uniform_grid), head.grid_minimum, head.grid_step, native.current_stream(device)))
+        return embedded.view(*indices.shape, self.embedding_dim)

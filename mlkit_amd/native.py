@@ -41,10 +41,21 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
         _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
     ]),
+    "mk_rotated_packed_matvec": (_c_int, [
+        _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_float,
+        _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
+    ]),
     "mk_packed_decode": (_c_int, [
         _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
     ]),
+    "mk_packed_decode_rows": (_c_int, [
+        _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
+    ]),
+    "mk_pack": (_c_int, [_c_void_p, _c_int, _c_longlong, _c_int, _c_void_p, _c_void_p, _c_void_p]),
+    "mk_unpack": (_c_int, [_c_void_p, _c_longlong, _c_int, _c_void_p, _c_void_p]),
     "mk_scalar_encode": (_c_int, [
         _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int,
         _c_int, _c_int, _c_float, _c_float, _c_void_p,

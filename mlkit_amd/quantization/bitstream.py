@@ -1,10 +1,14 @@
-"""Packing of integer codes into a little-endian bit stream, and back.
+"""Integer codes as a little-endian bit stream, and back.
 
 Code ``i`` of width ``b`` occupies stream bits ``[i*b, (i+1)*b)``; byte ``j`` holds stream
-bits ``[8j, 8j+8)``, least significant first.  Same layout, return types and errors as the
-reference's ``pack`` / ``unpack`` (/root/reference/src/mlkit/quantization/operations/
+bits ``[8j, 8j+8)``, least significant first.  Layout, return types and errors are those of
+the reference's ``pack`` / ``unpack`` (/root/reference/src/mlkit/quantization/operations/
 bit_packing.py:13-135); the stream is what ``PackedLinear.packed`` and checkpoints hold.
-These are tensor operations on whatever device the codes live on.
+
+Tensors on a HIP device go through ``mk_pack`` / ``mk_unpack`` (one thread per 32 codes, no
+temporaries).  Host tensors are packed as bit planes: the stream *is* the codes' bits laid
+end to end, so the codes are spread into one uint8 per bit, regrouped eight at a time and
+weighted by powers of two.
 """
 
 import math
@@ -12,11 +16,13 @@ import math
 import torch
 from torch import Tensor
 
+_KERNEL_CODE_BYTES = {torch.uint8: 1, torch.int16: 2, torch.int32: 4, torch.int64: 8}
 
-def _period(bits: int) -> tuple[int, int]:
-    """(codes, bytes) of the shortest run of whole codes that fills whole bytes."""
-    common = math.gcd(bits, 8)
-    return 8 // common, bits // common
+
+def _bit_planes(values: Tensor, bits: int) -> Tensor:
+    """``[n, bits]`` uint8: bit ``t`` of every value, least significant first."""
+    shifts = torch.arange(bits, device=values.device, dtype=torch.int32)
+    return ((values.to(torch.int32).unsqueeze(1) >> shifts) & 1).to(torch.uint8)
 
 
 def pack(codes: Tensor, bits: int) -> Tensor:
@@ -25,26 +31,30 @@ def pack(codes: Tensor, bits: int) -> Tensor:
         raise ValueError("packing supports one through sixteen bits")
     if codes.is_floating_point() or codes.is_complex():
         raise TypeError("codes must have an integer dtype")
-    flat = codes.detach().reshape(-1).to(torch.int64)
-    if flat.numel() and (int(flat.min()) < 0 or int(flat.max()) >= 1 << bits):
-        raise ValueError(f"codes exceed the unsigned capacity of {bits} bits")
+    flat = codes.detach().reshape(-1)
     count = flat.numel()
-    per_period, period_bytes = _period(bits)
-    padded = -(-count // per_period) * per_period
-    if padded != count:
-        flat = torch.cat([flat, flat.new_zeros(padded - count)])
-    # A period of codes is at most 16 * 8 = 128 bits: assemble it in two 64-bit halves
-    # only when needed; with bits <= 8 a period is at most 64 bits.
-    grouped = flat.view(-1, per_period)
-    out = torch.zeros((grouped.shape[0], period_bytes), dtype=torch.int64, device=codes.device)
-    for index in range(per_period):
-        start = index * bits
-        value = grouped[:, index]
-        first_byte, shift = divmod(start, 8)
-        spread = value << shift  # at most 16 + 7 bits
-        for byte in range((shift + bits + 7) // 8):
-            out[:, first_byte + byte] |= (spread >> (8 * byte)) & 0xFF
-    return out.to(torch.uint8).reshape(-1)[: (count * bits + 7) // 8]
+    size = (count * bits + 7) // 8
+    if flat.is_cuda:
+        from mlkit_amd import native
+
+        if flat.dtype not in _KERNEL_CODE_BYTES:
+            flat = flat.to(torch.int32)
+        flat = flat.contiguous()
+        packed = torch.empty(size, dtype=torch.uint8, device=flat.device)
+        overflow = torch.zeros(1, dtype=torch.int32, device=flat.device)
+        native.check(native.library().mk_pack(flat.data_ptr(), _KERNEL_CODE_BYTES[flat.dtype], count, bits,
+                                              packed.data_ptr(), overflow.data_ptr(),
+                                              native.current_stream(flat.device)))
+        if int(overflow.item()):
+            raise ValueError(f"codes exceed the unsigned capacity of {bits} bits")
+        return packed
+    if count and (int(flat.min()) < 0 or int(flat.max()) >= 1 << bits):
+        raise ValueError(f"codes exceed the unsigned capacity of {bits} bits")
+    stream = _bit_planes(flat, bits).reshape(-1)
+    if stream.numel() % 8:
+        stream = torch.cat([stream, stream.new_zeros(8 - stream.numel() % 8)])
+    weights = (1 << torch.arange(8, dtype=torch.int32)).to(torch.uint8)
+    return (stream.view(-1, 8) * weights).sum(dim=1, dtype=torch.int32).to(torch.uint8)[:size]
 
 
 def unpack(packed: Tensor, bits: int, shape: tuple[int, ...]) -> Tensor:
@@ -55,21 +65,17 @@ def unpack(packed: Tensor, bits: int, shape: tuple[int, ...]) -> Tensor:
     if any(dimension < 0 for dimension in shape):
         raise ValueError("shape dimensions must be nonnegative")
     count = math.prod(shape)
-    needed = (count * bits + 7) // 8
-    if packed.numel() != needed:
+    if packed.numel() != (count * bits + 7) // 8:
         raise ValueError(f"packed byte count {packed.numel()} does not match shape {shape} at {bits} bits")
-    per_period, period_bytes = _period(bits)
-    periods = -(-count // per_period)
-    stream = packed.reshape(-1).to(torch.int64)
-    if stream.numel() != periods * period_bytes:
-        stream = torch.cat([stream, stream.new_zeros(periods * period_bytes - stream.numel())])
-    grouped = stream.view(periods, period_bytes)
-    out = torch.empty((periods, per_period), dtype=torch.int64, device=packed.device)
-    mask = (1 << bits) - 1
-    for index in range(per_period):
-        first_byte, shift = divmod(index * bits, 8)
-        value = torch.zeros(periods, dtype=torch.int64, device=packed.device)
-        for byte in range((shift + bits + 7) // 8):
-            value |= grouped[:, first_byte + byte] << (8 * byte)
-        out[:, index] = (value >> shift) & mask
-    return out.reshape(-1)[:count].to(torch.uint8 if bits <= 8 else torch.int32).reshape(shape)
+    code_dtype = torch.uint8 if bits <= 8 else torch.int32
+    if packed.is_cuda:
+        from mlkit_amd import native
+
+        stream = packed.reshape(-1).contiguous()
+        codes = torch.empty(count, dtype=code_dtype, device=packed.device)
+        native.check(native.library().mk_unpack(stream.data_ptr(), count, bits, codes.data_ptr(),
+                                                native.current_stream(packed.device)))
+        return codes.reshape(shape)
+    planes = _bit_planes(packed.reshape(-1), 8).reshape(-1)[: count * bits].view(count, bits)
+    weights = 1 << torch.arange(bits, dtype=torch.int32)
+    return (planes.to(torch.int32) * weights).sum(dim=1, dtype=torch.int32).to(code_dtype).reshape(shape)

@@ -195,6 +195,23 @@ class OnlineRotation:
             plan = self._plans[key] = self._prepare(value)
         return plan(value)
 
+    def launch_arguments(self, width: int, device: torch.device) -> tuple | None:
+        """``(order, power, basis pointer or None, signs pointer, scale, keep)`` for
+        ``mk_rotated_packed_matvec``, or None when the rotation kernels do not take this width
+        (``keep`` holds the tensors the pointers belong to)."""
+        order, power, basis = transform_factor(width)
+        if power > MAXIMUM_KERNEL_WIDTH or order > MAXIMUM_KERNEL_ORDER:
+            return None
+        from mlkit_amd.kernels import hadamard as kernel
+
+        signs = _cached_signs(width, self.seed, device)
+        if basis is None:
+            return 1, width, None, signs.data_ptr(), kernel.normaliser(width), (signs,)
+        if not kernel.fits_one_launch(order, power):
+            return None
+        basis_on_device = _basis_on(width, device)
+        return order, power, basis_on_device.data_ptr(), signs.data_ptr(), kernel.normaliser(power), (signs, basis_on_device)
+
     def _prepare(self, value: Tensor):
         seed = self.seed
         width = value.shape[-1]

@@ -499,7 +499,7 @@ class Block(nn.Module):
 
 def test_online_rotation_survives_quantization_packing_and_checkpoints(tmp_path):
     """Rotated down projection (4864 = 76 x 64, Paley order 76): same function before
-    quantization; after quantization the packed model keeps the input hook, and a checkpoint
+    quantization; after quantization the packed model keeps the input rotation, and a checkpoint
     restores both the codes and the rotation."""
     torch.manual_seed(45)
     module = Block().cuda()
@@ -513,7 +513,8 @@ def test_online_rotation_survives_quantization_packing_and_checkpoints(tmp_path)
     assert converted.transforms == module._mlkit_transforms
     quantized_output = converted(inputs)
     packed = mk.optimize(converted, backend="packed")
-    assert isinstance(packed.module.down_proj, mk.PackedLinear) and len(packed.module.down_proj._forward_pre_hooks) == 1
+    down = packed.module.down_proj   # the packed layer runs the rotation itself (one library call per forward)
+    assert isinstance(down, mk.PackedLinear) and not down._forward_pre_hooks and down._rotation is not None
     with torch.inference_mode():
         torch.testing.assert_close(packed(inputs), quantized_output, rtol=1e-4, atol=1e-4)
     mk.save(converted, tmp_path / "rotated")
@@ -557,6 +558,42 @@ def test_config5_rotated_int4_layer_end_to_end(rows, width):
         exact = host(x.float() @ plain.T)
         relative = np.linalg.norm(host(y.float()) - exact) / np.linalg.norm(exact)
         assert relative < 0.15, relative   # 4-bit rounding noise of a Gaussian layer
+
+
+@pytest.mark.parametrize("rows,width", [(256, 4096), (512, 14336), (64, 896)])
+def test_packed_layer_absorbs_its_online_rotation(rows, width):
+    """mk.optimize turns the rotate_inputs pre-hook of a rotated layer into a rotation inside
+    PackedLinear.forward: one library call (rotation kernel + matvec) for up to eight rows.
+    The result equals hook-then-matvec bit for bit (the same two kernels), for fp16 and bf16,
+    for more than eight rows (dense path) and after deepcopy / state reload."""
+    from mlkit_amd.conversion import RotateInputs
+    from mlkit_amd.quantization.transforms import OnlineRotation
+
+    torch.manual_seed(48)
+    layer = nn.Linear(width, rows, bias=True, dtype=torch.float16)
+    module = nn.ModuleDict({"down_proj": layer}).cuda()
+    mk.rotate(seed=4)(module)
+    assert any(isinstance(hook, RotateInputs) for hook in module["down_proj"]._forward_pre_hooks.values())
+    converted = mk.quantize(module, mk.int(4, group=128), calib=None)
+    packed = mk.optimize(converted, backend="packed")
+    fused = packed.module["down_proj"]
+    assert isinstance(fused, mk.PackedLinear) and not fused._forward_pre_hooks and fused._rotation is not None
+    seed = mk.layer_seed("down_proj", 4)
+    hook = OnlineRotation(seed)
+    plain = copy.deepcopy(fused)
+    plain._rotation = None                       # the unrotated layer, fed rotated inputs by hand
+    for dtype in (torch.float16, torch.bfloat16):
+        for samples in (1, 3, 8, 20):
+            if samples > 8 and dtype != layer.weight.dtype:
+                continue   # the dense path multiplies in the layer's own dtype (bias included)
+            x = torch.randn(samples, width, device="cuda").to(dtype)
+            with torch.inference_mode():
+                assert torch.equal(fused(x), plain(hook(x))), (dtype, samples)
+                assert torch.equal(fused(x.view(1, samples, width)), plain(hook(x)).view(1, samples, rows))
+    duplicate = copy.deepcopy(packed).module["down_proj"]
+    x = torch.randn(2, width, device="cuda").half()
+    with torch.inference_mode():
+        assert torch.equal(duplicate(x), fused(x))
 
 
 def test_checkpoint_mirrors_of_the_reference_tests(tmp_path):
