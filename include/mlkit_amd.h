@@ -97,6 +97,22 @@ int mk_rotated_packed_matvec(const void *x, int x_dtype, void *rotated, int orde
                              int output_width, int input_width, int group, int bits, int uniform,
                              float grid_min, float grid_step, void *stream);
 
+/* mk_rotated_packed_matvec without the `rotated` argument: the rotated activations go to a
+ * fixed 512 KiB array inside the library's own device memory (one per GPU, held until the
+ * process ends), so the call allocates nothing and asks the caller for no workspace.
+ * samples * input_width * (bytes of x_dtype) must not exceed 524288 (8 rows of 16384 fp32
+ * values); larger requests return MK_ERR_INVALID and name mk_rotated_packed_matvec.  All
+ * calls on one GPU share the array: calls that overlap on one GPU (different streams) race,
+ * calls on one stream do not.  Results equal mk_rotated_packed_matvec bit for bit.
+ * No counterpart in the reference: it exists for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). */
+int mk_rotated_packed_matvec_static(const void *x, int x_dtype, int order, int power, const float *basis,
+                                    const float *signs, float scale, const uint8_t *packed,
+                                    const void *scales, int scale_dtype, const float *values, int n_values,
+                                    const void *zeros, const void *bias, int bias_dtype, void *y, int samples,
+                                    int output_width, int input_width, int group, int bits, int uniform,
+                                    float grid_min, float grid_step, void *stream);
+
 /* out[n, k] = dequant(code[n, k]) in out_dtype, same dequantisation as mk_packed_matvec
  * with multiply and add kept separate (no fused multiply-add).
  * Replaces: kernels/packed_linear.py:279-313 (decode / decode_rows). */

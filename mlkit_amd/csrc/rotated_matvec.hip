@@ -9,6 +9,8 @@
 // enqueued right behind it on the same stream.  One library call replaces a Python hook, an
 // allocation and two calls.
 
+#include <mutex>
+
 #include "mk_common.h"
 
 namespace {
@@ -44,6 +46,64 @@ extern "C" int mk_rotated_packed_matvec(const void *x, int x_dtype, void *rotate
                                         const void *zeros, const void *bias, int bias_dtype, void *y, int samples,
                                         int output_width, int input_width, int group, int bits, int uniform,
                                         float grid_min, float grid_step, void *stream) {
+    return rotate_then_multiply(x, x_dtype, rotated, order, power, basis, signs, scale, packed, scales, scale_dtype, values,
+                                n_values, zeros, bias, bias_dtype, y, samples, output_width, input_width, group, bits,
+                                uniform, grid_min, grid_step, stream);
+}
+
+// ---- the same without a buffer from the caller ---------------------------------------------
+//
+// For callers that cannot allocate (code under HIP graph capture, serving loops that own no
+// allocator): the rotated activations go to a fixed array in the library's own device
+// memory.  Every GPU the library runs on holds one copy of the array until the process ends;
+// all calls on a GPU share it, so calls that overlap on one GPU (two streams) race.
+
+namespace {
+
+constexpr size_t kStaticRotatedBytes = 512 * 1024;  // 8 rows x 16384 values x 4 bytes
+constexpr int kMaxDevices = 64;
+
+static __device__ __align__(256) unsigned char scratch[kStaticRotatedBytes];
+
+// The device address of `scratch` on the current device, looked up once per device.  (In host
+// code the array's name is only a handle for this lookup, not an address a kernel can use.)
+int static_rotated_buffer(void **buffer) {
+    static std::mutex guard;
+    static void *address[kMaxDevices];
+    int device = 0;
+    hipError_t status = hipGetDevice(&device);
+    if (status != hipSuccess || device < 0 || device >= kMaxDevices)
+        return mk_fail(MK_ERR_HIP, "mk_rotated_packed_matvec_static: no current device (%s)", hipGetErrorString(status));
+    std::lock_guard<std::mutex> lock(guard);
+    if (!address[device]) {
+        void *found = nullptr;
+        status = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+        if (status != hipSuccess || !found)
+            return mk_fail(MK_ERR_HIP, "mk_rotated_packed_matvec_static: the library's buffer has no address on device %d (%s)",
+                           device, hipGetErrorString(status));
+        address[device] = found;
+    }
+    *buffer = address[device];
+    return MK_OK;
+}
+
+}  // namespace
+
+extern "C" int mk_rotated_packed_matvec_static(const void *x, int x_dtype, int order, int power, const float *basis,
+                                               const float *signs, float scale, const uint8_t *packed,
+                                               const void *scales, int scale_dtype, const float *values,
+                                               int n_values, const void *zeros, const void *bias, int bias_dtype,
+                                               void *y, int samples, int output_width, int input_width, int group,
+                                               int bits, int uniform, float grid_min, float grid_step, void *stream) {
+    MK_REQUIRE(mk_dtype_valid(x_dtype) && samples >= 1 && input_width >= 1, MK_ERR_INVALID,
+               "mk_rotated_packed_matvec_static: unknown dtype code or empty input");
+    const unsigned long long needed = static_cast<unsigned long long>(samples) * input_width * mk_dtype_bytes(x_dtype);
+    MK_REQUIRE(needed <= kStaticRotatedBytes, MK_ERR_INVALID,
+               "mk_rotated_packed_matvec_static: %d x %d activations of %d bytes need %llu bytes, the library's buffer "
+               "holds %llu; use mk_rotated_packed_matvec with a buffer of the caller's",
+               samples, input_width, mk_dtype_bytes(x_dtype), needed, static_cast<unsigned long long>(kStaticRotatedBytes));
+    void *rotated = nullptr;
+    if (int status = static_rotated_buffer(&rotated)) return status;
     return rotate_then_multiply(x, x_dtype, rotated, order, power, basis, signs, scale, packed, scales, scale_dtype, values,
                                 n_values, zeros, bias, bias_dtype, y, samples, output_width, input_width, group, bits,
                                 uniform, grid_min, grid_step, stream);

@@ -46,6 +46,11 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
         _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
     ]),
+    "mk_rotated_packed_matvec_static": (_c_int, [
+        _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float,
+        _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
+    ]),
     "mk_packed_decode": (_c_int, [
         _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p,
