@@ -1,17 +1,28 @@
-"""Headline benchmark: INT4-g128 packed matvec, weight 4096x14336 (N x K), on one MI355X.
+"""Headline benchmark: INT4-g128 packed matvec, weight 4096x14336 (N x K), M=1, on one MI355X.
 
-One step = one launch of the packed matvec at M=1 on the next of several distinct weight
-copies (more than 512 MB in total, so the 256 MB Infinity Cache cannot serve the stream).
-Prints ONE JSON line; `value` is the effective weight bandwidth (codes + scales bytes per
-second) with every input resident in HBM.  `roofline` prices the same launches by their
-algorithmic bytes; `cpu_baseline` times the oracle's reconstruct-then-matmul on host cores.
+One step = one call of ``mk_packed_matvec_group`` over ``--members`` (default 8) distinct
+4096x14336 weight matrices that read one activation row each: the shape of a
+mixture-of-experts layer's expert down-projections, or of sibling projections fed by one
+tensor.  Every member is a complete INT4-g128 matvec whose output equals the single-matrix
+call bit for bit; the single-matrix chain (one ``mk_packed_matvec`` per step) is timed beside
+it and reported in ``config.by_rows``.  Weight sets rotate so that more than 512 MB of distinct
+weights pass between two uses of a set and the 256 MB Infinity Cache cannot serve the stream.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+The timed region is a HIP graph of ``--steps`` calls; ``ms_per_step`` is the median over
+``--replays`` timed replays (HIP events on the stream the graph runs on).  Prints ONE JSON line:
+``value`` is the effective weight bandwidth (codes + scales bytes per second) with every input
+resident in HBM; ``roofline`` prices the same launches by their algorithmic bytes;
+``cpu_baseline`` times the CPU restatement (reconstruct-then-matmul, GPTQ sweep, Walsh-Hadamard
+transform) on the host's cores; ``kernels`` holds the other kernels of the path with their own
+roofline fractions (fp32 MFMA for the GPTQ trailing update, HBM for the rest).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--members G] [--replays R]
 """
 
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -23,23 +34,28 @@ CODE_BYTES = ROWS * WIDTH * BITS // 8
 SCALE_BYTES = ROWS * (WIDTH // GROUP) * 2
 WEIGHT_BYTES = CODE_BYTES + SCALE_BYTES
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
-# profiles/packed_matvec_stream4_int4_g128_4096x14336_m1.md), M=1.
-MEASURED_TRAFFIC_BYTES = 30_641_000
+MFMA_FP32_PEAK_TFLOPS = 157.3
+MINIMUM_ROTATING_BYTES = 512 * 2**20
+# HBM bytes per matrix of a launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; recorded, not
+# measured by this script.
+RECORDED_TRAFFIC = {"bytes_per_matrix": 30_641_000,
+                    "source": "profiles/packed_matvec_stream4_int4_g128_4096x14336_m1.md (rocprofv3 --pmc "
+                              "FETCH_SIZE, WRITE_SIZE); recorded there, not measured in this run"}
 
 
 def algorithmic_bytes(samples: int) -> int:
+    """Per matrix: codes + scales + the activation rows read + the outputs written."""
     return WEIGHT_BYTES + samples * WIDTH * 2 + samples * ROWS * 2
 
 
-def make_copies(count: int, device: torch.device):
+def make_copies(count: int, device: torch.device, rows=ROWS, width=WIDTH, group=GROUP, bits=BITS):
     """Distinct synthetic layers: seeded uniform codes and fp16 scales of the magnitude an
     N(0, 0.02^2) weight gives (absmax/8 of 128 normals ~ 0.0065)."""
     generator = torch.Generator(device=device).manual_seed(20240601)
     copies = []
     for _ in range(count):
-        packed = torch.randint(0, 256, (CODE_BYTES,), dtype=torch.uint8, device=device, generator=generator)
-        scales = (torch.rand((ROWS, WIDTH // GROUP), device=device, generator=generator) * 0.004 + 0.005).half()
+        packed = torch.randint(0, 256, (rows * width * bits // 8,), dtype=torch.uint8, device=device, generator=generator)
+        scales = (torch.rand((rows, width // group), device=device, generator=generator) * 0.004 + 0.005).half()
         copies.append((packed, scales))
     return copies
 
@@ -67,77 +83,113 @@ class Launcher:
             native.check(status)
 
 
-def timed_region(launchers, steps, warmup, use_graph=True):
-    """Returns (seconds by wall clock, seconds by HIP events) for exactly `steps` launches."""
+class GroupLauncher:
+    """One mk_packed_matvec_group call over `members` weight copies that read `x`."""
+
+    def __init__(self, x, members, values, *, rows=ROWS, width=WIDTH, group=GROUP):
+        from mlkit_amd.kernels import packed_linear
+
+        count = len(members)
+        layout = packed_linear.layout_for(BITS, width, group)
+        self.launch = packed_linear.GroupLaunch(
+            [packed for packed, _ in members], [scales for _, scales in members], values, [None] * count, [None] * count,
+            [rows] * count, width, group, layout, uniform_grid=True, grid_minimum=-8.0, grid_step=1.0)
+        self.x = x
+        self.outputs = [torch.empty((x.shape[0], rows), device=x.device, dtype=x.dtype) for _ in range(count)]
+
+    def __call__(self, stream: int) -> None:
+        self.launch(self.x, self.outputs, stream)
+
+
+def timed_graph(launchers, steps, warmup, replays, minimum_span_ms=1.0):
+    """Per-step seconds of a HIP graph of `steps` launches: the graph is replayed `replays`
+    times, each timed by a pair of HIP events on the replay stream around enough back-to-back
+    launches of the graph to span about a millisecond.  Returns (median, minimum, maximum,
+    graph launches per timed replay)."""
     stream = torch.cuda.current_stream()
     count = len(launchers)
-    for step in range(warmup):
+    for step in range(max(warmup, count)):
         launchers[step % count](stream.cuda_stream)
     torch.cuda.synchronize()
-    graph = None
-    if use_graph:
-        try:
-            side = torch.cuda.Stream()
-            side.wait_stream(stream)
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=side):
-                capture = torch.cuda.current_stream().cuda_stream
-                for step in range(steps):
-                    launchers[(warmup + step) % count](capture)
-            graph.replay()  # untimed: uploads the graph
-            torch.cuda.synchronize()
-        except Exception as error:  # capture unsupported: time eager launches instead
-            print(f"[bench] graph capture unavailable ({error}); timing eager launches", file=sys.stderr)
-            graph = None
-    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    started = time.perf_counter()
-    begin.record()
-    if graph is not None:
-        graph.replay()
-    else:
-        raw = stream.cuda_stream
+    side = torch.cuda.Stream()
+    side.wait_stream(stream)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        capture = torch.cuda.current_stream().cuda_stream
         for step in range(steps):
-            launchers[(warmup + step) % count](raw)
+            launchers[(warmup + step) % count](capture)
+    for _ in range(3):  # untimed: uploads the graph, warms the clocks
+        graph.replay()
+    torch.cuda.synchronize()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record()
+    graph.replay()
     end.record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - started
-    return wall, begin.elapsed_time(end) / 1e3, graph is not None
+    batch = max(1, int(np.ceil(minimum_span_ms / max(begin.elapsed_time(end), 1e-3))))
+    samples = []
+    for _ in range(replays):
+        begin.record()
+        for _ in range(batch):
+            graph.replay()
+        end.record()
+        torch.cuda.synchronize()
+        samples.append(begin.elapsed_time(end) / 1e3 / (batch * steps))
+    return statistics.median(samples), min(samples), max(samples), batch
 
 
-def cpu_baseline():
-    """Oracle reconstruct-then-matmul (unpack -> values[codes]*scale -> fp32 matmul) on the
-    host cores, on the full 4096x14336 layer at M=1: a bounded number of repetitions."""
-    from oracle import bitstream, matvec as oracle_matvec, scaling
+def _blas_threads(limit: int | None):
+    try:
+        import threadpoolctl
+
+        return threadpoolctl.threadpool_limits(limits=limit) if limit else threadpoolctl.threadpool_info()
+    except Exception:  # threadpoolctl is optional
+        return None
+
+
+def cpu_matvec_baseline() -> dict:
+    """The CPU restatement of reconstruct-then-matmul (unpack -> values[codes] * scale -> fp32
+    matmul) on the whole 4096x14336 layer at M=1, one thread: at least 10 timed repetitions of
+    the matmul on the reconstructed weight after 2 warm-ups, and as many whole passes
+    (reconstruction included) as fit in about 12 s."""
+    from oracle import matvec as oracle_matvec, scaling
 
     rng = np.random.default_rng(7)
     packed = rng.integers(0, 256, CODE_BYTES, dtype=np.uint8)
     scales = (rng.random((ROWS, WIDTH // GROUP), dtype=np.float32) * 0.004 + 0.005).astype(np.float16).astype(np.float32)
     values = scaling.int_values(4)
     x = rng.standard_normal((1, WIDTH), dtype=np.float32).astype(np.float16).astype(np.float32)
-    threads = torch.get_num_threads()
-    full = []
-    budget = time.perf_counter() + 20.0
-    dense = None
-    while len(full) < 3 and (not full or time.perf_counter() < budget):
-        started = time.perf_counter()
-        dense = oracle_matvec.dequantise(packed, BITS, (ROWS, WIDTH), scales, values, GROUP)
-        oracle_matvec.reconstruct_then_matmul(x, None, BITS, (ROWS, WIDTH), scales, values, GROUP, dense=dense)
-        full.append(time.perf_counter() - started)
-    matmul_only = []
-    for _ in range(10):
-        started = time.perf_counter()
-        oracle_matvec.reconstruct_then_matmul(x, None, BITS, (ROWS, WIDTH), scales, values, GROUP, dense=dense)
-        matmul_only.append(time.perf_counter() - started)
-    seconds = float(np.median(full))
+    limiter = _blas_threads(1)
+    try:
+        whole = []
+        budget = time.perf_counter() + 12.0
+        dense = None
+        while len(whole) < 10 and (len(whole) < 2 or time.perf_counter() < budget):
+            started = time.perf_counter()
+            dense = oracle_matvec.dequantise(packed, BITS, (ROWS, WIDTH), scales, values, GROUP)
+            oracle_matvec.reconstruct_then_matmul(x, None, BITS, (ROWS, WIDTH), scales, values, GROUP, dense=dense)
+            whole.append(time.perf_counter() - started)
+        for _ in range(2):
+            oracle_matvec.reconstruct_then_matmul(x, None, BITS, (ROWS, WIDTH), scales, values, GROUP, dense=dense)
+        matmul = []
+        for _ in range(10):
+            started = time.perf_counter()
+            oracle_matvec.reconstruct_then_matmul(x, None, BITS, (ROWS, WIDTH), scales, values, GROUP, dense=dense)
+            matmul.append(time.perf_counter() - started)
+    finally:
+        if limiter is not None and hasattr(limiter, "restore_original_limits"):
+            limiter.restore_original_limits()
+    timed = whole[1:] if len(whole) > 1 else whole   # the first pass warms the caches
+    seconds = float(np.median(timed))
     return {
         "value": WEIGHT_BYTES / seconds / 1e9,
         "unit": "GB/s effective weight bandwidth",
-        "cores": threads,
+        "cores": 1,
         "kind": "port",
-        "sample": f"{len(full)} x full 4096x14336 INT4-g128 layer at M=1, oracle unpack+dequantise+fp32 matmul "
-                  f"(numpy); median {seconds * 1e3:.0f} ms; matmul alone with the dense weight cached "
-                  f"{float(np.median(matmul_only)) * 1e3:.2f} ms; os.cpu_count()={os.cpu_count()}",
+        "sample": f"{len(timed)} timed passes (after 1 warm-up) over the whole 4096x14336 INT4-g128 layer at M=1: numpy unpack + "
+                  f"dequantise + fp32 matmul, one thread, median {seconds * 1e3:.0f} ms; the matmul alone on the reconstructed "
+                  f"weight, 10 repetitions after 2 warm-ups, median {float(np.median(matmul)) * 1e3:.2f} ms "
+                  f"({WEIGHT_BYTES / float(np.median(matmul)) / 1e9:.1f} GB/s of packed bytes); os.cpu_count()={os.cpu_count()}",
     }
 
 
@@ -155,20 +207,37 @@ def _time(function, repeats=20, warmup=3):
     return begin.elapsed_time(end) / repeats
 
 
-def gptq_layer(device: torch.device, generator: torch.Generator) -> dict:
-    """GPTQ, INT4 g128, 4096 x 11008, refit = block = 128; the Hessian product and the Cholesky
-    factorisation (outside the kernels of this repository) are timed apart."""
+def _entry(ms, nbytes=None, flops=None, **extra):
+    record = {"ms": ms, **extra}
+    if nbytes is not None:
+        record.update(bytes=nbytes, GBps=nbytes / ms / 1e6, hbm_frac=nbytes / ms / 1e6 / HBM_PEAK_GBPS)
+    if flops is not None:
+        record.update(flops=flops, TFLOPs=flops / ms / 1e9)
+    return record
+
+
+def gptq_layer(device: torch.device, generator: torch.Generator, cpu_rows: int = 0) -> dict:
+    """GPTQ, INT4 g128, 4096 x 11008, refit = block = 128.  The Hessian product and the Cholesky
+    factorisation (outside the parity boundary) are timed apart; the wide trailing updates
+    (`block_update_from_deviations_kernel`, fp32 matrix cores) are replayed on their own through
+    mk_feedback_block_update_staged and priced against the fp32 MFMA peak; with `cpu_rows` the
+    CPU restatement sweeps that many rows with the same coefficient matrix, is timed, and its
+    codes are compared with the device's."""
     import mlkit_amd as mk
+    from mlkit_amd import native
+    from mlkit_amd.quantization import feedback
     from mlkit_amd.quantization.core import Ctx
 
-    rows, width = 4096, 11008
+    rows, width, block, deferred = 4096, 11008, 128, feedback.DEFERRED_TILES
     target = (torch.randn((rows, width), device=device, generator=generator) * 0.02).half().float()
     inputs = torch.randn((16384, width), device=device, generator=generator).half()
     hot = torch.randperm(width, device=device, generator=generator)[: width // 100]
     inputs[:, hot] *= 30
-    hessian = (inputs.float().T @ inputs.float()) / inputs.shape[0]
+    hessian = torch.zeros((width, width), device=device)
+    for band in inputs.split(2048):
+        hessian.addmm_(band.float().T, band.float())
+    hessian /= inputs.shape[0]
     del inputs
-    from mlkit_amd.quantization import feedback
 
     def wall_ms(function, repeats=3):
         """Median wall-clock time of `function`, synchronised on both sides."""
@@ -193,23 +262,104 @@ def gptq_layer(device: torch.device, generator: torch.Generator) -> dict:
         sweep_ms = wall_ms(lambda: quantizer(target, Ctx("down_proj", H=hessian)))
     finally:
         feedback.feedback_coefficients = original
-    update_flops = sum(2 * rows * 128 * (width - stop) for stop in range(128, width, 128))
+    update_flops = sum(2 * rows * block * (width - stop) for stop in range(block, width, block))
     rtn = mk.int(4, group=128)(target)
-    return {
+    out = {
         "total_ms": total_ms, "coefficients_ms": factor_ms, "sweep_and_update_ms": sweep_ms,
-        "columns_per_s": width / (sweep_ms / 1e3), "trailing_update_flops": update_flops,
+        "columns_per_s": width / (sweep_ms / 1e3), "weights_per_s": rows * width / (sweep_ms / 1e3),
+        "trailing_update_flops": update_flops,
         "proxy_loss": float(mk.proxy_loss(target, result.w, hessian)),
         "rtn_proxy_loss": float(mk.proxy_loss(target, rtn.w, hessian)),
     }
+    # The wide (deferred, chained) trailing updates of the sweep, replayed alone: every group of
+    # `deferred` tiles updates all columns to its right in one launch.
+    coefficients = ready[0]
+    deviations = (target - result.w).T.contiguous()          # [width, rows], as the sweep stores them
+    scratch = torch.zeros_like(target)
+    library, stream = native.library(), native.current_stream(device)
+    wide = [(start, start + deferred * block) for start in range(0, width, deferred * block)
+            if start + deferred * block < width and (width - start - deferred * block) % 128 == 0]
+    wide_flops = sum(2 * rows * deferred * block * (width - begin) for _, begin in wide)
+
+    def replay_updates():
+        for start, begin in wide:
+            native.check(library.mk_feedback_block_update_staged(
+                scratch.data_ptr(), deviations.data_ptr(), coefficients.data_ptr(), rows, width, start, block, deferred,
+                begin, width, stream))
+
+    update_ms = _time(replay_updates, repeats=5, warmup=2)
+    tflops = wide_flops / update_ms / 1e9
+    out["trailing_update_roofline"] = {
+        "kernel": "block_update_from_deviations_kernel", "bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS,
+        "unit": "TFLOP/s", "frac": tflops / MFMA_FP32_PEAK_TFLOPS, "launches": len(wide), "ms_all_launches": update_ms,
+        "flops_all_launches": wide_flops,
+        "note": f"the {len(wide)} chained launches ({deferred} tiles of {block} columns each, all columns to their right) that "
+                f"carry {wide_flops / update_flops:.0%} of the layer's trailing-update flops",
+    }
+    del deviations, scratch
+    if cpu_rows:
+        from oracle import feedback as oracle_feedback, scaling
+
+        picked = torch.linspace(0, rows - 1, cpu_rows, device=device).long()
+        host_coefficients = coefficients.cpu().numpy()
+        host_weight = target[picked].cpu().numpy()
+        started = time.perf_counter()
+        expected = oracle_feedback.sweep(host_weight, host_coefficients, scaling.int_values(4), group=128, integer=True,
+                                         refit=128, block=128)
+        seconds = time.perf_counter() - started
+        mismatches = int((result.codes[picked].cpu().numpy() != expected["codes"]).sum())
+        out["cpu_baseline"] = {
+            "value": cpu_rows * width / seconds, "unit": "weights/s", "cores": int(os.environ.get("OMP_NUM_THREADS", 0)) or os.cpu_count(),
+            "kind": "port",
+            "sample": f"{cpu_rows} rows spread over the 4096 x 11008 layer, all 11008 columns, the C restatement of the sweep "
+                      f"(OpenMP over rows) with the device's coefficient matrix: {seconds:.1f} s; device: "
+                      f"{rows * width / (sweep_ms / 1e3):.3e} weights/s",
+            "code_mismatches_vs_device": mismatches, "codes_compared": cpu_rows * width,
+        }
+    return out
 
 
-def other_kernels(device: torch.device) -> dict:
-    """Timings of the other kernels of the path at the shapes of the benchmark configurations
-    (`--kernels`); each entry carries its algorithmic bytes or flops and the rate they give."""
+def rotated_layer(device: torch.device, generator: torch.Generator, values: torch.Tensor) -> dict:
+    """Config 5: the rotated INT4-g128 layers at M = 1 and 8.  One step = the online rotation of
+    the activations plus the packed matvec, enqueued by one mk_rotated_packed_matvec call; the
+    unrotated matvec of the same layer is timed beside it."""
+    from mlkit_amd import native
+    from mlkit_amd.quantization.transforms import OnlineRotation
+
+    library = native.library()
+    out = {}
+    for rows, width in ((ROWS, WIDTH), (WIDTH, 4096)):
+        copies = make_copies(max(2, -(-MINIMUM_ROTATING_BYTES // (rows * width // 2))), device, rows=rows, width=width)
+        order, power, basis, signs, scale, keep = OnlineRotation(17).launch_arguments(width, device)
+        for samples in (1, 8):
+            x = torch.randn((samples, width), device=device, generator=generator).half()
+            y = torch.empty((samples, rows), device=device, dtype=torch.float16)
+            rotated = torch.empty_like(x)
+
+            def rotated_call(packed, scales):
+                arguments = (x.data_ptr(), native.MK_F16, rotated.data_ptr(), order, power, basis, signs, scale,
+                             packed.data_ptr(), scales.data_ptr(), native.MK_F16, values.data_ptr(), 16, None, None, 0,
+                             y.data_ptr(), samples, rows, width, GROUP, BITS, 1, -8.0, 1.0)
+                return lambda stream: native.check(library.mk_rotated_packed_matvec(*arguments, stream))
+
+            with_rotation = [rotated_call(packed, scales) for packed, scales in copies]
+            plain = [Launcher(x, packed, scales, values, y, rows=rows, width=width) for packed, scales in copies]
+            rotated_s = timed_graph(with_rotation, 200, 20, 20)[0]
+            plain_s = timed_graph(plain, 200, 20, 20)[0]
+            out[f"{rows}x{width} M={samples}"] = {
+                "rotation": f"{order} x {power}" if order > 1 else f"fwht {power}",
+                "rotated_us": rotated_s * 1e6, "unrotated_us": plain_s * 1e6, "rotation_costs_us": (rotated_s - plain_s) * 1e6,
+            }
+        del copies
+    return out
+
+
+def other_kernels(device: torch.device, full: bool) -> dict:
+    """The other kernels of the path at the shapes of the benchmark configurations; each entry
+    carries its algorithmic bytes or flops and the rate they give.  `full` adds the decoder-layer
+    shapes, the tied head and the wider codecs."""
     import mlkit_amd as mk
     from mlkit_amd.kernels import hadamard, packed_linear, scalar_decode, scalar_encode
-    from mlkit_amd.quantization.transforms import OnlineRotation
-    from mlkit_amd.quantization.core import Ctx
 
     out = {}
     generator = torch.Generator(device=device).manual_seed(1)
@@ -217,61 +367,51 @@ def other_kernels(device: torch.device) -> dict:
     elements = ROWS * WIDTH
     values = torch.arange(-8, 8, dtype=torch.float32, device=device)
 
-    def entry(ms, nbytes=None, flops=None, **extra):
-        record = {"ms": ms, **extra}
-        if nbytes is not None:
-            record.update(bytes=nbytes, GBps=nbytes / ms / 1e6, hbm_frac=nbytes / ms / 1e6 / HBM_PEAK_GBPS)
-        if flops is not None:
-            record.update(flops=flops, TFLOPs=flops / ms / 1e9)
-        return record
-
     fit = lambda: scalar_encode.fit_scales(weight, GROUP, asym=False, reciprocal=0.125, value_minimum=-8.0,  # noqa: E731
                                            scale_format="fp16", store_zero=False)
     scales, _ = fit()
-    out["fit_scales 4096x14336 g128"] = entry(_time(fit), elements * 4 + scales.numel() * 4)
+    out["fit_scales 4096x14336 g128"] = _entry(_time(fit), elements * 4 + scales.numel() * 4)
     encode = lambda: scalar_encode.encode(weight, scales, None, values, GROUP, None, integer=True,  # noqa: E731
                                           minimum=-8.0, maximum=7.0)
     codes = encode()
-    out["encode int4 4096x14336 g128"] = entry(_time(encode), elements * 5 + scales.numel() * 4)
-    out["decode codes 4096x14336 g128"] = entry(
+    out["encode int4 4096x14336 g128"] = _entry(_time(encode), elements * 5 + scales.numel() * 4)
+    out["decode codes 4096x14336 g128"] = _entry(
         _time(lambda: scalar_decode.decode(codes, scales, values, None, GROUP)), elements * 5 + scales.numel() * 4)
+    out["pack int4 4096x14336"] = _entry(_time(lambda: mk.pack(codes, 4), repeats=10), elements + elements // 2)
+    stream = mk.pack(codes, 4)
+    out["unpack int4 4096x14336"] = _entry(_time(lambda: mk.unpack(stream, 4, (ROWS, WIDTH)), repeats=10),
+                                           elements + elements // 2)
     seven = torch.tensor([-1, -0.5, -0.25, 0, 0.25, 0.5, 1], device=device)
     fractions = torch.linspace(0.5, 1.0, 20, device=device)
     square = weight[:, :4096].contiguous()
     base, _ = scalar_encode.fit_scales(square, 64, asym=False, reciprocal=1.0, value_minimum=-1.0,
                                        scale_format="fp16", store_zero=False)
-    out["search_scales codebook7 4096x4096 g64, 21 candidates"] = entry(
+    out["search_scales codebook7 4096x4096 g64, 21 candidates"] = _entry(
         _time(lambda: scalar_encode.search_scales(square, base, None, seven, fractions, 64, None, "fp16",
                                                   integer=False, minimum=-1.0, maximum=1.0), repeats=5),
         4096 * 4096 * 4 + 2 * base.numel() * 4)
-    packed = mk.pack(codes[:8], 4)  # layout only; the timed stream is synthetic
-    packed = torch.randint(0, 256, (CODE_BYTES,), dtype=torch.uint8, device=device, generator=generator)
     dense = torch.empty((ROWS, WIDTH), device=device, dtype=torch.float16)
     layout = packed_linear.layout_for(BITS, WIDTH, GROUP)
     half_scales = scales.half()
-    out["packed decode int4 4096x14336 -> fp16"] = entry(
-        _time(lambda: packed_linear.decode(packed, half_scales, values, None, dense, GROUP, layout, True, -8.0, 1.0)),
+    out["packed decode int4 4096x14336 -> fp16"] = _entry(
+        _time(lambda: packed_linear.decode(stream, half_scales, values, None, dense, GROUP, layout, True, -8.0, 1.0)),
         CODE_BYTES + SCALE_BYTES + elements * 2)
 
     rotated = torch.empty_like(weight)
-    out["fwht 4096x14336 fp32 as 7x2048 blocks"] = entry(
-        _time(lambda: hadamard.transform(weight.view(ROWS, 7, 2048), out=rotated.view(ROWS, 7, 2048))), elements * 8)
+    fwht_ms = _time(lambda: hadamard.transform(weight.view(ROWS, 7, 2048), out=rotated.view(ROWS, 7, 2048)))
+    out["fwht 4096x14336 fp32 as 7x2048 blocks"] = _entry(fwht_ms, elements * 8)
+    out["fwht_roofline"] = {"kernel": "fwht_kernel", "bound": "hbm", "achieved": elements * 8 / fwht_ms / 1e6,
+                            "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": elements * 8 / fwht_ms / 1e6 / HBM_PEAK_GBPS,
+                            "workload": "4096 x 14336 fp32 as 7 x 2048 blocks, read and written once"}
     tall = weight.view(WIDTH, ROWS)
-    out["fwht 14336x4096 fp32"] = entry(_time(lambda: hadamard.transform(tall, out=rotated.view(WIDTH, ROWS))), elements * 8)
-    out["rht 4096x14336 fp32 (28x512 Paley: fwht + basis mix)"] = entry(
-        _time(lambda: mk.rht(weight, seed=3), repeats=5), elements * 8, launches=2)
-    for samples in (1, 8):
-        for width in (4096, 14336):
-            x = torch.randn((samples, width), device=device, generator=generator).half()
-            out[f"rht activations M={samples} K={width} fp16"] = {"us": _time(lambda: mk.rht(x, seed=3), 50) * 1e3}
-            hook = OnlineRotation(3)
-            out[f"online rotation hook M={samples} K={width} fp16"] = {"us": _time(lambda: hook(x), 50) * 1e3}
+    out["fwht 14336x4096 fp32"] = _entry(_time(lambda: hadamard.transform(tall, out=rotated.view(WIDTH, ROWS))), elements * 8)
+    out["rht 4096x14336 fp32 (28x512 Paley)"] = _entry(_time(lambda: mk.rht(weight, seed=3), repeats=5), elements * 8)
 
     # other matvec shapes and codecs, M = 1 and 8: HIP-graph launches through the C ABI over
     # enough distinct weight copies (> 512 MB) that the Infinity Cache cannot serve them
     def matvec(rows, width, group, bits, table, uniform, asym, label, dtype=torch.float16):
         code_bytes = rows * width * bits // 8
-        count = max(2, min(40, -(-(512 * 2**20) // code_bytes)))
+        count = max(2, min(40, -(-MINIMUM_ROTATING_BYTES // code_bytes)))
         streams = [torch.randint(0, 256, (code_bytes,), dtype=torch.uint8, device=device, generator=generator)
                    for _ in range(count)]
         side = (torch.rand((rows, width // group), device=device, generator=generator) * 0.004 + 0.005).half()
@@ -282,53 +422,81 @@ def other_kernels(device: torch.device) -> dict:
             launchers = [Launcher(x, stream, side, table, y, zeros=zeros, rows=rows, width=width, group=group,
                                   bits=bits, uniform=uniform, grid_min=float(table[0]),
                                   grid_step=float(table[1] - table[0])) for stream in streams]
-            _, seconds, _ = timed_region(launchers, 400, 40)
+            seconds = timed_graph(launchers, 200, 20, 20)[0]
             nbytes = code_bytes + side.numel() * 2 * (2 if asym else 1) + samples * (width + rows) * 2
-            out[f"matvec {label} {rows}x{width} M={samples}"] = entry(seconds / 400 * 1e3, nbytes, copies=count)
+            out[f"matvec {label} {rows}x{width} M={samples}"] = _entry(seconds * 1e3, nbytes, copies=count)
 
     nf4 = mk.NF4_VALUES.to(device)
     matvec(4096, 4096, 128, 4, values, True, True, "int4 asym g128")
-    matvec(ROWS, WIDTH, 128, 4, values, True, False, "int4 g128, bf16 activations", dtype=torch.bfloat16)
     matvec(ROWS, WIDTH, 64, 2, torch.arange(-2, 2, dtype=torch.float32, device=device), True, False, "int2 g64")
     matvec(ROWS, WIDTH, 64, 3, torch.arange(-4, 4, dtype=torch.float32, device=device), True, False, "int3 g64")
     matvec(ROWS, WIDTH, 64, 4, nf4, False, False, "nf4 g64")
     matvec(ROWS, WIDTH, 64, 3, seven, False, False, "codebook7 g64")
-    matvec(151936, 896, 128, 4, values, True, False, "int4 g128 (tied head)")
-    matvec(ROWS, WIDTH, 128, 8, torch.arange(-128, 128, dtype=torch.float32, device=device), True, False, "int8 g128")
-    for rows, width in ((896, 896), (128, 896), (4864, 896), (896, 4864)):
-        matvec(rows, width, 128, 4, values, True, False, "int4 g128 (decoder layer)")
+    if full:
+        matvec(ROWS, WIDTH, 128, 4, values, True, False, "int4 g128, bf16 activations", dtype=torch.bfloat16)
+        matvec(151936, 896, 128, 4, values, True, False, "int4 g128 (tied head)")
+        matvec(ROWS, WIDTH, 128, 8, torch.arange(-128, 128, dtype=torch.float32, device=device), True, False, "int8 g128")
+        for rows, width in ((896, 896), (128, 896), (4864, 896), (896, 4864)):
+            matvec(rows, width, 128, 4, values, True, False, "int4 g128 (decoder layer)")
     del weight, rotated, dense, codes
-
-    out["gptq int4 g128 4096x11008"] = gptq_layer(device, generator)
+    out["rotated layers (config 5)"] = rotated_layer(device, generator, values)
     return out
+
+
+def cpu_fwht_baseline() -> dict:
+    """The stagewise CPU transform on 256 rows of 7 x 2048 blocks (numpy, one thread)."""
+    from oracle import transforms
+
+    rng = np.random.default_rng(3)
+    rows = 256
+    value = rng.standard_normal((rows * 7, 2048), dtype=np.float32)
+    for _ in range(2):
+        transforms.fwht(value)
+    times = []
+    for _ in range(10):
+        started = time.perf_counter()
+        transforms.fwht(value)
+        times.append(time.perf_counter() - started)
+    seconds = float(np.median(times))
+    return {"value": value.size * 8 / seconds / 1e9, "unit": "GB/s (read + write once)", "cores": 1, "kind": "port",
+            "sample": f"{rows} rows of the 4096 x 14336 fp32 matrix as 7 x 2048 blocks, stagewise numpy transform, 10 repetitions "
+                      f"after 2 warm-ups, median {seconds * 1e3:.1f} ms"}
 
 
 def main() -> None:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=2000)
-    parser.add_argument("--warmup", type=int, default=200)
-    parser.add_argument("--copies", type=int, default=18)
-    parser.add_argument("--no-graph", action="store_true")
+    parser.add_argument("--steps", type=int, default=100)
+    parser.add_argument("--warmup", type=int, default=20)
+    parser.add_argument("--members", type=int, default=8, help="weight matrices per mk_packed_matvec_group call (1..8)")
+    parser.add_argument("--replays", type=int, default=60, help="timed replays of the graph; the median is reported")
+    parser.add_argument("--copies", type=int, default=0, help="distinct weight copies in rotation (default: enough for 512 MB "
+                                                               "between two uses of a copy)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
-    parser.add_argument("--kernels", action="store_true",
-                        help="also time the other kernels of the path (adds a `kernels` object to the line)")
+    parser.add_argument("--skip-kernels", action="store_true", help="only the headline matvec (no GPTQ / FWHT / codec legs)")
+    parser.add_argument("--kernels", action="store_true", help="add the decoder-layer shapes, the tied head and wider codecs")
     parser.add_argument("--profile-gptq", action="store_true",
                         help="for rocprofv3: only run the GPTQ layer (4096 x 11008) and print its timings")
     parser.add_argument("--profile-launches", type=int, default=0,
-                        help="for rocprofv3: only launch the M=1 matvec this many times, plus three "
+                        help="for rocprofv3: only issue this many eager calls (grouped with --members > 1), plus three "
                              "256 MiB device copies whose counters calibrate FETCH_SIZE / WRITE_SIZE")
-    parser.add_argument("--profile-rows", type=int, default=1,
-                        help="activation rows M of the --profile-launches launches")
+    parser.add_argument("--profile-rows", type=int, default=1, help="activation rows M of the --profile-launches calls")
     options = parser.parse_args()
     if options.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a HIP device")
+    if not 1 <= options.members <= 8:
+        sys.exit("--members must be 1..8")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     values = torch.arange(-8, 8, dtype=torch.float32, device=device)
-    copies = make_copies(options.copies, device)
+    members = options.members
+    # Between two uses of a weight set at least 512 MB of other weights are streamed.
+    sets = -(-MINIMUM_ROTATING_BYTES // (members * WEIGHT_BYTES)) + 1
+    copy_count = max(options.copies, sets * members, 18)
+    copy_count = -(-copy_count // members) * members
+    copies = make_copies(copy_count, device)
     generator = torch.Generator(device=device).manual_seed(5)
 
     if options.profile_gptq:
@@ -336,8 +504,11 @@ def main() -> None:
         return
     if options.profile_launches:
         x = torch.randn((options.profile_rows, WIDTH), device=device, generator=generator).half()
-        y = torch.empty((options.profile_rows, ROWS), device=device, dtype=torch.float16)
-        launchers = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
+        if members > 1:
+            launchers = [GroupLauncher(x, copies[index:index + members], values) for index in range(0, copy_count, members)]
+        else:
+            y = torch.empty((options.profile_rows, ROWS), device=device, dtype=torch.float16)
+            launchers = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
         raw = torch.cuda.current_stream().cuda_stream
         for step in range(options.profile_launches):
             launchers[step % len(launchers)](raw)
@@ -349,60 +520,83 @@ def main() -> None:
         return
 
     results = {}
+    head_step = None
     for samples in (1, 2, 4, 8):
         x = torch.randn((samples, WIDTH), device=device, generator=generator).half()
         y = torch.empty((samples, ROWS), device=device, dtype=torch.float16)
-        launchers = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
-        wall, event_seconds, graphed = timed_region(launchers, options.steps, options.warmup,
-                                                    use_graph=not options.no_graph)
-        per_launch = event_seconds / options.steps
-        resident = [launchers[0]]
-        _, resident_seconds, _ = timed_region(resident, options.steps, options.warmup,
-                                              use_graph=not options.no_graph)
-        results[samples] = {
-            "us_per_call": per_launch * 1e6,
-            "wall_us_per_call": wall / options.steps * 1e6,
-            "effective_weight_GBps": WEIGHT_BYTES / per_launch / 1e9,
-            "algorithmic_GBps": algorithmic_bytes(samples) / per_launch / 1e9,
-            "cache_resident_us_per_call": resident_seconds / options.steps * 1e6,
-            "graph": graphed,
-        }
-    head = results[1]
-    per_launch = head["us_per_call"] / 1e6
-    achieved = algorithmic_bytes(1) / per_launch / 1e9
+        single = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
+        row = {}
+        median, low, high, batch = timed_graph(single, max(options.steps, 50), options.warmup, max(20, options.replays // 2))
+        row["single_call"] = {"us_per_matrix": median * 1e6, "min_us": low * 1e6, "max_us": high * 1e6,
+                              "hbm_frac": algorithmic_bytes(samples) / median / 1e9 / HBM_PEAK_GBPS}
+        resident = timed_graph([single[0]], max(options.steps, 50), options.warmup, 10)[0]
+        row["single_call"]["cache_resident_us"] = resident * 1e6
+        for count in sorted({2, 4, members} - {1}):
+            grouped = [GroupLauncher(x, copies[index:index + count], values) for index in range(0, copy_count - count + 1, count)]
+            steps = options.steps if (samples == 1 and count == members) else max(options.steps // 2, 25)
+            replays = options.replays if (samples == 1 and count == members) else max(20, options.replays // 3)
+            median, low, high, batch = timed_graph(grouped, steps, options.warmup, replays)
+            row[f"group_of_{count}"] = {"us_per_call": median * 1e6, "us_per_matrix": median * 1e6 / count,
+                                        "min_us_per_matrix": low * 1e6 / count, "max_us_per_matrix": high * 1e6 / count,
+                                        "hbm_frac": algorithmic_bytes(samples) * count / median / 1e9 / HBM_PEAK_GBPS}
+            if samples == 1 and count == members:
+                head_step = (median, low, high, batch, steps, replays)
+            del grouped
+        results[samples] = row
+    if members == 1:
+        x = torch.randn((1, WIDTH), device=device, generator=generator).half()
+        y = torch.empty((1, ROWS), device=device, dtype=torch.float16)
+        single = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
+        median, low, high, batch = timed_graph(single, options.steps, options.warmup, options.replays)
+        head_step = (median, low, high, batch, options.steps, options.replays)
+    per_step, low, high, batch, steps, replays = head_step
+    achieved = algorithmic_bytes(1) * members / per_step / 1e9
     line = {
         "metric": "effective weight GB/s, INT4-g128 packed matvec 4096x14336, M=1",
-        "value": head["effective_weight_GBps"],
+        "value": WEIGHT_BYTES * members / per_step / 1e9,
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": options.steps,
+        "steps": steps,
         "warmup": options.warmup,
-        "ms_per_step": per_launch * 1e3,
+        "ms_per_step": per_step * 1e3,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16 activations, u4 codes, f32 accumulate",
         "data": "synthetic seeded codes and fp16 scales",
         "config": {
-            "workload": "INT4 symmetric g128 packed matvec, weight 4096x14336 (N x K), M=1; "
-                        f"{options.copies} distinct weight copies ({options.copies * WEIGHT_BYTES / 2**20:.0f} MiB) in rotation",
-            "launch": "HIP graph of back-to-back launches" if head["graph"] else "eager launches",
+            "workload": f"INT4 symmetric g128 packed matvec, weight 4096x14336 (N x K), M=1; one step = one "
+                        f"mk_packed_matvec_group call over {members} such matrices (one launch); "
+                        f"{copy_count} distinct weight copies ({copy_count * WEIGHT_BYTES / 2**20:.0f} MiB) in rotation",
+            "matrices_per_step": members,
+            "us_per_matrix": per_step * 1e6 / members,
+            "single_call_us_per_matrix": results[1]["single_call"]["us_per_matrix"],
+            "launch": "HIP graph of `steps` back-to-back calls on one stream",
+            "timing": {"replays": replays, "graph_launches_per_timed_replay": batch, "statistic": "median",
+                       "min_ms_per_step": low * 1e3, "max_ms_per_step": high * 1e3},
             "by_rows": {str(k): v for k, v in results.items()},
         },
         "roofline": {
+            "kernel": "stream4_kernel<1,false,16,f16,1> (one launch per step)",
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES,
+            "algorithmic_bytes_per_launch": algorithmic_bytes(1) * members,
+            "traffic": RECORDED_TRAFFIC["bytes_per_matrix"] * members,
+            "traffic_source": RECORDED_TRAFFIC["source"],
         },
-        "cpu_baseline": None if options.no_cpu_baseline else cpu_baseline(),
+        "cpu_baseline": None if options.no_cpu_baseline else cpu_matvec_baseline(),
     }
-    if options.kernels:
-        del copies, launchers
+    if not options.skip_kernels:
+        del copies, single
         torch.cuda.empty_cache()
-        line["kernels"] = other_kernels(device)
+        kernels = other_kernels(device, options.kernels)
+        kernels["gptq int4 g128 4096x11008"] = gptq_layer(device, generator, cpu_rows=0 if options.no_cpu_baseline else 32)
+        if not options.no_cpu_baseline:
+            kernels["fwht_cpu_baseline"] = cpu_fwht_baseline()
+        line["kernels"] = kernels
     print(json.dumps(line))
 
 

@@ -60,21 +60,23 @@ int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packed, const vo
                      int input_width, int group, int bits, int uniform, float grid_min,
                      float grid_step, void *stream);
 
-/* mk_packed_matvec for `count` (1..8) weight matrices that read the same activations:
- * y[i] = x @ dequant(packed[i])^T (+ bias[i]) for every i, each with output_widths[i] rows.
- * The matrices share x, samples, input_width, group, bits, the grid (uniform, grid_min,
- * grid_step, values) and the dtypes; either every matrix has offsets or none has.  packed,
- * scales, zeros (NULL = none), bias (NULL = none; single entries may be NULL) and y are HOST
- * arrays of `count` device pointers, output_widths a host array of `count` ints; the arrays
- * are read before the call returns.  Layouts the INT4 streaming kernels take (4-bit uniform
- * grid, 16-bit activations and scales, input_width a multiple of 32 up to 16384) run as ONE
- * launch whose workgroups are spread over all the matrices; every other layout runs as
- * `count` launches of mk_packed_matvec.  Results equal those of `count` separate calls bit
- * for bit.
- * Replaces: the consecutive launches of kernels/packed_linear.py:181-226 that sibling layers
- * fed by one tensor make (attention q/k/v, MLP gate/up: the model calls
- * PackedLinear.forward, inference/packed_linear.py:148-245, once per layer). */
-int mk_packed_matvec_group(const void *x, int x_dtype, int count, const uint8_t *const *packed,
+/* mk_packed_matvec for `count` (1..8) weight matrices of one input width and one codec in a
+ * single call: y[i] = x[i] @ dequant(packed[i])^T (+ bias[i]) for every i, each with
+ * output_widths[i] rows.  The activation pointers may all be the same (sibling projections
+ * fed by one tensor: attention q/k/v, MLP gate/up) or differ (the experts of a
+ * mixture-of-experts layer, each with its own `samples` rows).  The matrices share samples,
+ * input_width, group, bits, the grid (uniform, grid_min, grid_step, values) and the dtypes;
+ * either every matrix has offsets or none has.  x, packed, scales, zeros (NULL = none), bias
+ * (NULL = none; single entries may be NULL) and y are HOST arrays of `count` device pointers,
+ * output_widths a host array of `count` ints; the arrays are read before the call returns.
+ * Layouts the INT4 streaming kernels take (4-bit uniform grid, 16-bit activations and scales,
+ * input_width a multiple of 32 up to 16384) run as ONE launch whose grid covers all the
+ * matrices; every other layout runs as `count` launches of mk_packed_matvec.  Results equal
+ * those of `count` separate calls bit for bit.
+ * Replaces: the consecutive launches of kernels/packed_linear.py:181-226 that a model makes
+ * for such layers (it calls PackedLinear.forward, inference/packed_linear.py:148-245, once
+ * per layer). */
+int mk_packed_matvec_group(const void *const *x, int x_dtype, int count, const uint8_t *const *packed,
                            const void *const *scales, int scale_dtype, const float *values, int n_values,
                            const void *const *zeros, const void *const *bias, int bias_dtype,
                            void *const *y, const int *output_widths, int samples, int input_width,
@@ -298,6 +300,18 @@ int mk_feedback_block_update_range(float *feedback, const float *original, const
                                    const float *coeff, int rows, int width, int first_column,
                                    int chain_width, int chains, int column_begin, int column_end,
                                    void *stream);
+
+/* mk_feedback_block_update_range with the deviations handed over instead of recomputed:
+ * deviations [width, rows] fp32 holds column c of (original - output) at deviations[c, :]
+ * (what mk_feedback_sweep leaves in its `deviations` argument), so both operands of the
+ * matrix-core product are read as row tiles.  Whole 128 x 128 tiles only: rows and
+ * column_end - column_begin multiples of 128, chain_width a multiple of 32 and at least 128,
+ * 16-byte aligned operands; MK_ERR_UNSUPPORTED otherwise.  Same sums, bit for bit.
+ * Replaces: the addmm_ of quantization/algorithms/error_feedback.py:366-370, whose first
+ * operand is this deviation matrix. */
+int mk_feedback_block_update_staged(float *feedback, const float *deviations, const float *coeff, int rows,
+                                    int width, int first_column, int chain_width, int chains, int column_begin,
+                                    int column_end, void *stream);
 
 /* The whole natural-order error-feedback sweep of a layer with per-region absmax / minmax
  * scale fits, enqueued in one call: for every region of `refit` columns the pending

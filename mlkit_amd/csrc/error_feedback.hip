@@ -1074,6 +1074,34 @@ extern "C" int mk_feedback_block_update_range(float *feedback, const float *orig
     return MK_OK;
 }
 
+extern "C" int mk_feedback_block_update_staged(float *feedback, const float *deviations, const float *coeff, int rows,
+                                               int width, int first_column, int chain_width, int chains,
+                                               int column_begin, int column_end, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(feedback && deviations && coeff, MK_ERR_INVALID, "mk_feedback_block_update_staged: null tensor pointer");
+    MK_REQUIRE(rows >= 1 && width >= 1 && first_column >= 0 && chain_width >= 1 && chains >= 1 &&
+                   first_column + static_cast<long long>(chain_width) * chains <= width,
+               MK_ERR_INVALID, "mk_feedback_block_update_staged: %d chains of %d columns from column %d lie outside a row of %d",
+               chains, chain_width, first_column, width);
+    MK_REQUIRE(column_begin >= first_column + chain_width * chains && column_end <= width, MK_ERR_INVALID,
+               "mk_feedback_block_update_staged: updated columns [%d, %d) must follow the chains and lie inside the row",
+               column_begin, column_end);
+    if (column_begin >= column_end) return MK_OK;
+    const auto aligned = [](const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15u) == 0; };
+    MK_REQUIRE(aligned(deviations) && aligned(coeff) && rows % kTileRows == 0 && width % 4 == 0 && column_begin % 4 == 0 &&
+                   (column_end - column_begin) % kTileColumns == 0 && chain_width % kDepthChunk == 0 &&
+                   chain_width / kDepthChunk >= 4,
+               MK_ERR_UNSUPPORTED,
+               "mk_feedback_block_update_staged: whole %d x %d tiles, chains of at least %d columns and 16-byte aligned "
+               "operands are required; use mk_feedback_block_update_range otherwise",
+               kTileRows, kTileColumns, 4 * kDepthChunk);
+    UpdateArgs a{feedback, nullptr, nullptr, coeff, rows, width, first_column, chain_width, chains, column_begin, column_end,
+                 deviations};
+    if (int status = launch_update(a, stream)) return status;
+    MK_LAUNCH_CHECK("mk_feedback_block_update_staged");
+    return MK_OK;
+}
+
 extern "C" int mk_feedback_block_update(float *feedback, const float *original, const float *output,
                                         const float *coeff, int rows, int width, int tile_start, int tile_stop,
                                         void *stream) {

@@ -284,7 +284,7 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
     return MK_OK;
 }
 
-extern "C" int mk_packed_matvec_group(const void *x, int x_dtype, int count, const uint8_t *const *packed,
+extern "C" int mk_packed_matvec_group(const void *const *x, int x_dtype, int count, const uint8_t *const *packed,
                                       const void *const *scales, int scale_dtype, const float *values, int n_values,
                                       const void *const *zeros, const void *const *bias, int bias_dtype,
                                       void *const *y, const int *output_widths, int samples, int input_width,
@@ -300,22 +300,22 @@ extern "C" int mk_packed_matvec_group(const void *x, int x_dtype, int count, con
     bool one_launch = mk_dtype_valid(x_dtype) && mk_dtype_valid(scale_dtype) && (!bias || mk_dtype_valid(bias_dtype)) &&
                       bits == 4 && !tuning().no_stream4 &&
                       mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
-                      (reinterpret_cast<uintptr_t>(x) & 15u) == 0 &&
                       (static_cast<size_t>(input_width) * mk_dtype_bytes(x_dtype)) % 16 == 0;
     for (int i = 0; i < count; ++i) {
-        MK_REQUIRE(packed[i] && scales[i] && y[i] && output_widths[i] >= 1, MK_ERR_INVALID,
+        MK_REQUIRE(x[i] && packed[i] && scales[i] && y[i] && output_widths[i] >= 1, MK_ERR_INVALID,
                    "mk_packed_matvec_group: matrix %d has a null pointer or no rows", i);
         MK_REQUIRE(((zeros && zeros[i]) != 0) == with_zeros, MK_ERR_INVALID,
                    "mk_packed_matvec_group: either every matrix has offsets or none has");
         const void *bias_i = bias ? bias[i] : nullptr;
-        one_launch = one_launch && (reinterpret_cast<uintptr_t>(packed[i]) & 3u) == 0 &&
+        one_launch = one_launch && (reinterpret_cast<uintptr_t>(x[i]) & 15u) == 0 &&
+                     (reinterpret_cast<uintptr_t>(packed[i]) & 3u) == 0 &&
                      (reinterpret_cast<uintptr_t>(scales[i]) & 3u) == 0 &&
                      (reinterpret_cast<uintptr_t>(with_zeros ? zeros[i] : nullptr) & 3u) == 0 &&
                      (reinterpret_cast<uintptr_t>(bias_i) & 3u) == 0;
     }
     if (!one_launch) {  // the same results, one launch per matrix
         for (int i = 0; i < count; ++i)
-            if (int status = mk_packed_matvec(x, x_dtype, packed[i], scales[i], scale_dtype, values, n_values,
+            if (int status = mk_packed_matvec(x[i], x_dtype, packed[i], scales[i], scale_dtype, values, n_values,
                                               with_zeros ? zeros[i] : nullptr, bias ? bias[i] : nullptr, bias_dtype,
                                               y[i], samples, output_widths[i], input_width, group, bits, uniform,
                                               grid_min, grid_step, stream_))
@@ -323,13 +323,14 @@ extern "C" int mk_packed_matvec_group(const void *x, int x_dtype, int count, con
         return MK_OK;
     }
     mk_matvec::Stream4Args shared{};
-    shared.x = x; shared.samples = samples; shared.width = input_width; shared.group = group;
+    shared.x = x[0]; shared.samples = samples; shared.width = input_width; shared.group = group;
     shared.groups = mk_cdiv(input_width, group); shared.bias_dtype = bias_dtype; shared.grid_min = grid_min;
     shared.grid_step = grid_step; shared.values = values; shared.n_values = n_values; shared.uniform = uniform;
     shared.bits = bits; shared.x_dtype = x_dtype; shared.scale_dtype = scale_dtype;
     mk_matvec::Stream4Group members{};
     members.count = count;
     for (int i = 0; i < count; ++i) {
+        members.member[i].x = x[i];
         members.member[i].packed = packed[i];
         members.member[i].scales = scales[i];
         members.member[i].zeros = with_zeros ? zeros[i] : nullptr;
@@ -343,7 +344,7 @@ extern "C" int mk_packed_matvec_group(const void *x, int x_dtype, int count, con
     for (int i = 0; i < count; ++i) {  // rows past a member's last whole tile
         const int covered = output_widths[i] / rows_per_tile * rows_per_tile;
         if (covered < output_widths[i])
-            if (int status = launch_words(x, x_dtype, packed[i], scales[i], scale_dtype, values, members.member[i].zeros,
+            if (int status = launch_words(x[i], x_dtype, packed[i], scales[i], scale_dtype, values, members.member[i].zeros,
                                           members.member[i].bias, bias_dtype, y[i], samples, output_widths[i],
                                           input_width, group, bits, uniform, grid_min, grid_step, covered, stream))
                 return status;

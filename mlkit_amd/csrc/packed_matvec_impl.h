@@ -76,6 +76,7 @@ struct Stream4Args {
 // its table entry is fetched together with the other arguments, not behind them.
 constexpr int kMaxGroupMembers = 8;
 struct Stream4Member {
+    const void *x;  // this member's activations (members may share them)
     const uint8_t *packed;
     const void *scales, *zeros, *bias;
     void *y;
@@ -89,6 +90,7 @@ struct Stream4Group {
 
 // What a workgroup's matrix is: pointers, row count and number of tiles (wavefront-uniform).
 struct TileSource {
+    const void *x;
     const uint8_t *packed;
     const uint8_t *scales, *zeros;
     const void *bias;
@@ -105,14 +107,15 @@ constexpr size_t kGroupTableOffset = (sizeof(Stream4Args) + alignof(Stream4Group
 
 template <int ROWS>
 __device__ __forceinline__ TileSource tile_source(const Stream4Args &a, const Stream4Group &g, int member) {
-    TileSource s{a.packed, static_cast<const uint8_t *>(a.scales), static_cast<const uint8_t *>(a.zeros), a.bias, a.y,
-                 a.rows, a.rows / ROWS};
+    TileSource s{a.x, a.packed, static_cast<const uint8_t *>(a.scales), static_cast<const uint8_t *>(a.zeros), a.bias,
+                 a.y, a.rows, a.rows / ROWS};
     if (g.count > 0) {
         typedef const Stream4Member __attribute__((address_space(4))) *ConstantMember;
         typedef const char __attribute__((address_space(4))) *ConstantBytes;
         const ConstantBytes segment = (ConstantBytes)__builtin_amdgcn_kernarg_segment_ptr();
         const ConstantMember chosen =
             reinterpret_cast<ConstantMember>(segment + kGroupTableOffset + offsetof(Stream4Group, member)) + member;
+        s.x = chosen->x;
         s.packed = chosen->packed;
         s.scales = static_cast<const uint8_t *>(chosen->scales);
         s.zeros = static_cast<const uint8_t *>(chosen->zeros);
@@ -234,10 +237,10 @@ constexpr int kSliceWords = 64 * kChunkStrideWords;  // one wavefront's buffer: 
 // Piece i of the slice that starts at element `slice_start` of x's row `sample`: 16 bytes per
 // lane.  Pieces past the end of the row read the start of the row instead (their chunks are
 // zeroed later).
-__device__ __forceinline__ mk_u32x4 request_piece(const Stream4Args &a, int sample, int slice_start, int i, int lane) {
+__device__ __forceinline__ mk_u32x4 request_piece(const void *x, int width, int sample, int slice_start, int i, int lane) {
     const int element = slice_start + (16 * i + (lane >> 2)) * kChunkCodes + (lane & 3) * 8;
-    const size_t offset = static_cast<size_t>(sample) * a.width + (element < a.width ? element : (lane & 3) * 8);
-    return *reinterpret_cast<const mk_u32x4 *>(static_cast<const uint8_t *>(a.x) + offset * 2);
+    const size_t offset = static_cast<size_t>(sample) * width + (element < width ? element : (lane & 3) * 8);
+    return *reinterpret_cast<const mk_u32x4 *>(static_cast<const uint8_t *>(x) + offset * 2);
 }
 
 __device__ __forceinline__ void park_piece(uint32_t *slice, int i, int lane, mk_u32x4 piece) {

@@ -315,7 +315,7 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
             const int wanted_sample = blockIdx.y * 4 * SETS + 4 * set + j;
             const int sample = wanted_sample < a.samples ? wanted_sample : a.samples - 1;
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(a, sample, wave * (512 * kSlices), i, lane);
+            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(a.x, a.width, sample, wave * (512 * kSlices), i, lane);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j)

@@ -32,12 +32,9 @@ namespace {
 // per wavefront (both values swept on the GPU together with 8 / 32 rows and 4 - 16 ahead).
 constexpr int kWideRows = 16, kNarrowRows = 4;
 
-#ifndef MK_S4_AHEAD
-#define MK_S4_AHEAD 8
-#endif
 template <int ROWS>
 constexpr int rows_ahead_of() {
-    return ROWS < MK_S4_AHEAD ? ROWS : MK_S4_AHEAD;
+    return ROWS < 8 ? ROWS : 8;
 }
 
 // ---- bf16 activations ----------------------------------------------------------------------
@@ -126,9 +123,7 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
 
     // The workgroup is aligned first: a compute unit serves loads first come, first served,
     // and a wavefront that starts late would queue its small loads behind the others' codes.
-#ifndef MK_S4_NO_LEAD_BARRIER
     __syncthreads();
-#endif
 
     // Activations: 32 per sample, as 16 fp16 pairs (L2 hits), requested first.
     mk_u32x4 pieces[MT][4];
@@ -137,12 +132,10 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         for (int m = 0; m < MT; ++m) {
             const int sample = sample_base + m < a.samples ? sample_base + m : a.samples - 1;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) pieces[m][i] = request_piece(a, sample, wave * 2048, i, lane);
+            for (int i = 0; i < 4; ++i) pieces[m][i] = request_piece(source.x, a.width, sample, wave * 2048, i, lane);
         }
     };
-#ifndef MK_S4_CODES_FIRST
     request_activations();
-#endif
     // The scale (and offset) of this lane's chunk in every row, 2 bytes each.
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
     const uint32_t group_offset = static_cast<uint32_t>(part) * scale_row_bytes +
@@ -178,15 +171,8 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
             __builtin_amdgcn_sched_barrier(0);  // in row order
         }
     };
-#ifdef MK_S4_CODES_FIRST
-    request_codes();
-    if (first_tile) request_activations();
-    __builtin_amdgcn_sched_barrier(0);
-    request_sides();
-#else
     request_sides();
     request_codes();
-#endif
 
     if (first_tile) {  // uniform
     // Each lane's chunk of every sample, through the wavefront's LDS buffer (LDS operations
@@ -256,33 +242,16 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         }
     }
     if constexpr (!kStrided) break;
-    __syncthreads();  // `partials` is reused by the next tile
     tile += gridDim.x;
-    } while (tile < source.tiles);
+    if (tile >= source.tiles) break;
+    __syncthreads();  // `partials` is reused by the next tile
+    } while (true);
 }
 
 template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS>
 __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const Stream4Group members) {
     stream4_body<MT, HAS_ZERO, ROWS, XT, PARTS>(a, members);
 }
-
-#ifdef MK_S4_FLAT
-// Experiment: one sample, fp16, no offsets, with the arguments as scalars so that the first
-// of them can be preloaded into scalar registers at dispatch.
-__global__ void __launch_bounds__(512) stream4_flat_kernel(const void *x, const uint8_t *packed, const void *scales,
-                                                           int width, int samples, int group, int groups, int rows,
-                                                           void *y, const void *bias, int bias_dtype, float grid_min,
-                                                           float grid_step, int scale_dtype) {
-    Stream4Args a;
-    a.x = x; a.packed = packed; a.scales = scales; a.zeros = nullptr; a.bias = bias; a.y = y;
-    a.samples = samples; a.rows = rows; a.width = width; a.group = group; a.groups = groups;
-    a.bias_dtype = bias_dtype; a.grid_min = grid_min; a.grid_step = grid_step; a.values = nullptr;
-    a.n_values = 0; a.uniform = 1; a.bits = 4; a.x_dtype = MK_F16; a.scale_dtype = scale_dtype;
-    Stream4Group none;
-    none.count = 0;
-    stream4_body<1, false, 16, MK_F16, 1>(a, none);
-}
-#endif
 
 // ---- two to eight samples: the dot products on the matrix cores ---------------------------
 //
@@ -355,7 +324,7 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
             const int wanted_sample = blockIdx.y * 4 * SETS + 4 * set + j;
             const int sample = wanted_sample < a.samples ? wanted_sample : a.samples - 1;
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(a, sample, wave * (512 * kSlices), i, lane);
+            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(source.x, a.width, sample, wave * (512 * kSlices), i, lane);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -506,9 +475,10 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
         }
     }
     if constexpr (!kStrided) break;
-    __syncthreads();  // `partials` is reused by the next tile
     tile += gridDim.x;
-    } while (tile < source.tiles);
+    if (tile >= source.tiles) break;
+    __syncthreads();  // `partials` is reused by the next tile
+    } while (true);
 }
 
 // The number of workgroups of `kernel` the GPU holds at once, asked of the runtime the first
@@ -585,13 +555,6 @@ int launch_tile_parts(const Stream4Args &a, const Stream4Group &members, int til
         hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
         return 0;
     };
-#ifdef MK_S4_FLAT
-    if (MT == 1 && ROWS == 16 && PARTS == 1 && a.x_dtype == MK_F16 && !a.zeros && members.count == 0) {
-        hipLaunchKernelGGL(stream4_flat_kernel, grid, block, slices, stream, a.x, a.packed, a.scales, a.width, a.samples,
-                           a.group, a.groups, a.rows, a.y, a.bias, a.bias_dtype, a.grid_min, a.grid_step, a.scale_dtype);
-        return 0;
-    }
-#endif
     if (a.x_dtype == MK_F16) {
         if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_F16, PARTS>);
         return launch(stream4_kernel<MT, false, ROWS, MK_F16, PARTS>);

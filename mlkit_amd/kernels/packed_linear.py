@@ -134,6 +134,7 @@ class GroupLaunch:
         self.count = count
         self.output_widths = list(output_widths)
         self.input_width = input_width
+        self._x = pointers()
         self._y = pointers()
         self._constant = (
             pointers(*[entry.data_ptr() for entry in packed]), pointers(*[entry.data_ptr() for entry in scales]),
@@ -145,20 +146,28 @@ class GroupLaunch:
         self._widths = (ctypes.c_int * count)(*output_widths)
         self._tail = (input_width, group, layout.bits, int(uniform_grid), grid_minimum, grid_step)
 
-    def __call__(self, inputs: Tensor, outputs: list[Tensor], stream: int | None = None) -> None:
-        """``outputs[i][m, n] = sum_k dequant(code_i[n, k]) * inputs[m, k] (+ bias_i[n])`` on the current stream."""
-        samples = inputs.shape[0]
-        if not inputs.is_cuda or inputs.device != self.device or not inputs.is_contiguous() or inputs.shape[1] != self.input_width:
-            raise ValueError("grouped packed matvec needs contiguous inputs of the layers' width on their device")
-        for index, output in enumerate(outputs):
-            if (output.dtype != inputs.dtype or tuple(output.shape) != (samples, self.output_widths[index])
+    def __call__(self, inputs: "Tensor | list[Tensor]", outputs: list[Tensor], stream: int | None = None) -> None:
+        """``outputs[i][m, n] = sum_k dequant(code_i[n, k]) * inputs_i[m, k] (+ bias_i[n])`` on the current
+        stream.  ``inputs`` is one tensor every matrix reads, or one tensor per matrix (the same
+        shape and dtype: e.g. the experts of a mixture-of-experts layer)."""
+        shared = isinstance(inputs, Tensor)
+        each = [inputs] * self.count if shared else list(inputs)
+        if len(each) != self.count or len(outputs) != self.count:
+            raise ValueError("one input (or one shared input) and one output per matrix of the group")
+        first = each[0]
+        samples = first.shape[0]
+        for index, (entry, output) in enumerate(zip(each, outputs)):
+            if (not entry.is_cuda or entry.device != self.device or not entry.is_contiguous()
+                    or tuple(entry.shape) != (samples, self.input_width) or entry.dtype != first.dtype):
+                raise ValueError("grouped packed matvec needs contiguous inputs of one shape and dtype, of the layers' "
+                                 "width, on their device")
+            if (output.dtype != first.dtype or tuple(output.shape) != (samples, self.output_widths[index])
                     or not output.is_contiguous() or output.device != self.device):
                 raise ValueError("outputs must be contiguous [samples, output_width] tensors of the inputs' dtype")
+            self._x[index] = entry.data_ptr()
             self._y[index] = output.data_ptr()
-        if len(outputs) != self.count:
-            raise ValueError("one output per matrix of the group")
         status = native.library().mk_packed_matvec_group(
-            inputs.data_ptr(), native.dtype_code(inputs), self.count, *self._constant, self._y, self._widths, samples,
+            self._x, native.dtype_code(first), self.count, *self._constant, self._y, self._widths, samples,
             *self._tail, native.current_stream(self.device) if stream is None else stream)
         native.check(status)
 

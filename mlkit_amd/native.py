@@ -110,6 +110,9 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
         _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_float,
         _c_float, _c_int, _c_int, _c_void_p,
     ]),
+    "mk_feedback_block_update_staged": (_c_int, [
+        _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+    ]),
     "mk_feedback_block_update_range": (_c_int, [
         _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
         _c_int, _c_void_p,

@@ -414,8 +414,33 @@ def test_grouped_launch_validation():
     x = torch.zeros(1, 256, device="cuda", dtype=torch.float16)
     pointers = (ctypes.c_void_p * 9)(*([x.data_ptr()] * 9))
     widths = (ctypes.c_int * 9)(*([16] * 9))
-    arguments = lambda count: (x.data_ptr(), 1, count, pointers, pointers, 1, None, 0, None, None, 0, pointers, widths,  # noqa: E731
+    arguments = lambda count: (pointers, 1, count, pointers, pointers, 1, None, 0, None, None, 0, pointers, widths,  # noqa: E731
                                1, 256, 128, 4, 1, -8.0, 1.0, None)
     assert lib.mk_packed_matvec_group(*arguments(9)) == native.MK_ERR_INVALID
     assert "1 to 8 matrices" in native.last_error()
     assert lib.mk_packed_matvec_group(*arguments(0)) == native.MK_ERR_INVALID
+
+
+def test_grouped_launch_with_activations_per_matrix():
+    """The experts of a mixture-of-experts layer: eight 4096 x 14336 INT4-g128 matrices (two
+    distinct weight sets, reused, to bound the oracle's work), each multiplied with its own
+    activation row in one launch; every output equals the separate launch and the oracle."""
+    from mlkit_amd.kernels import packed_linear
+
+    layers = [helpers.quantised_layer(helpers.normal_weight(4096, 14336, seed=95 + i), INT4, bits=4, group=128,
+                                      integer=True) for i in range(2)]
+    tensors = [helpers.to_device(layer) for layer in layers]
+    members = [tensors[i % 2] for i in range(8)]
+    layout = packed_linear.layout_for(4, 14336, 128)
+    launch = packed_linear.GroupLaunch([t["packed"] for t in members], [t["scales"] for t in members], members[0]["values"],
+                                       [None] * 8, [None] * 8, [4096] * 8, 14336, 128, layout, uniform_grid=True,
+                                       grid_minimum=-8.0, grid_step=1.0)
+    for samples in (1, 4):
+        inputs = [helpers.activations(samples, 14336, seed=120 + i).cuda() for i in range(8)]
+        outputs = [torch.full((samples, 4096), float("nan"), dtype=torch.float16, device="cuda") for _ in range(8)]
+        launch(inputs, outputs)
+        torch.cuda.synchronize()
+        for i in range(8):
+            separate = run_matvec(layers[i % 2], inputs[i].cpu())
+            assert np.array_equal(outputs[i].float().cpu().numpy(), separate), i
+        check(outputs[5].float().cpu().numpy(), layers[1], inputs[5].cpu())
