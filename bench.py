@@ -38,9 +38,10 @@ MFMA_FP32_PEAK_TFLOPS = 157.3
 MINIMUM_ROTATING_BYTES = 512 * 2**20
 # HBM bytes per matrix of a launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; recorded, not
 # measured by this script.
-RECORDED_TRAFFIC = {"bytes_per_matrix": 30_641_000,
-                    "source": "profiles/packed_matvec_stream4_int4_g128_4096x14336_m1.md (rocprofv3 --pmc "
-                              "FETCH_SIZE, WRITE_SIZE); recorded there, not measured in this run"}
+RECORDED_TRAFFIC = {"bytes_per_matrix": 30_331_800,
+                    "source": "profiles/packed_matvec_stream4_int4_g128_4096x14336_m1_group8.md (rocprofv3 --pmc "
+                              "FETCH_SIZE, WRITE_SIZE of the 8-matrix launch, per matrix); recorded there, not measured in "
+                              "this run"}
 
 
 def algorithmic_bytes(samples: int) -> int:

@@ -87,9 +87,9 @@ int mk_packed_matvec_group(const void *const *x, int x_dtype, int count, const u
  * (input_width = order * power, power a power of two; order == 1: a plain Walsh-Hadamard
  * transform, basis unused), written to `rotated` ([samples, input_width] of x_dtype, a
  * buffer of the caller's that must not alias x), then mk_packed_matvec on `rotated` with the
- * remaining arguments.  signs: NULL or [input_width] fp32 of +-1.  Results equal mk_fwht /
- * mk_rotate_blocks followed by mk_packed_matvec bit for bit; MK_ERR_UNSUPPORTED when
- * mk_rotate_blocks does not take (order, power).
+ * remaining arguments.  signs: NULL or [input_width] fp32 of +-1.  Results equal
+ * mk_rotate_rows followed by mk_packed_matvec bit for bit; MK_ERR_UNSUPPORTED when
+ * mk_rotate_rows does not take (order, power).
  * Replaces: the rotate_inputs forward pre-hook (conversion/model_transforms.py:116-128) in
  * front of PackedLinear.forward (inference/packed_linear.py:148-245). */
 int mk_rotated_packed_matvec(const void *x, int x_dtype, void *rotated, int order, int power,
@@ -260,6 +260,18 @@ int mk_cholesky_block(float *matrix, long long leading, int size, int first_colu
 int mk_rotate_blocks(const void *source, int source_dtype, void *target, int target_dtype, long long rows,
                      int order, int power, const float *basis, int transpose, const float *signs_before,
                      const float *signs_after, float scale, void *stream);
+
+/* The rotation of mk_rotate_blocks for a few activation rows, on order * rows workgroups:
+ * target[r, f', :] = scale * H_power( sum_f basis[f', f] * (source[r, f, :] * signs[f, :]) ),
+ * the same transform with the mix applied before the Walsh-Hadamard stages (they commute),
+ * so every output block is independent work.  basis == NULL: the +-1 Hadamard matrix of
+ * size `order` (a power of two), which makes the whole a Walsh-Hadamard transform of
+ * order * power points.  32 <= power <= 1024; rows, order <= 65535.  Results agree with
+ * mk_rotate_blocks / mk_fwht to fp32 rounding (another summation order), not bit for bit.
+ * Replaces: the rotate_inputs hook of conversion/model_transforms.py:116-128
+ * (quantization/operations/orthogonal_transforms.py:101-122) for activations. */
+int mk_rotate_rows(const void *source, int source_dtype, void *target, int target_dtype, int rows, int order,
+                   int power, const float *basis, const float *signs, float scale, void *stream);
 
 /* Error-feedback sweep over columns [tile_start, tile_start + tile_width) of every row:
  * target = original + correction; the nearest grid value (as in mk_scalar_encode, with the

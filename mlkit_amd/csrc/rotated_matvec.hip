@@ -5,8 +5,8 @@
 // PackedLinear.forward, inference/packed_linear.py:148-245) multiplies its packed weight with
 // T(x * signs), T = (basis (x) H_power) / sqrt(power) along the input width.  The rotated
 // activations are at most 8 x 16384 values: they are written to a small buffer by the
-// Walsh-Hadamard / blocked-rotation kernel and read back, from L2, by the matvec kernel
-// enqueued right behind it on the same stream.  One library call replaces a Python hook, an
+// row-rotation kernel (mk_rotate_rows: order * samples short workgroups) and read back, from
+// L2, by the matvec kernel enqueued right behind it on the same stream.  One library call replaces a Python hook, an
 // allocation and two calls.
 
 #include <mutex>
@@ -26,13 +26,20 @@ int rotate_then_multiply(const void *x, int x_dtype, void *rotated, int order, i
                "mk_rotated_packed_matvec: order * power must equal the input width (%d * %d != %d)", order, power,
                input_width);
     MK_REQUIRE(order == 1 || basis, MK_ERR_INVALID, "mk_rotated_packed_matvec: a blocked rotation needs its basis");
+    // The rotation runs on order * samples short workgroups (mk_rotate_rows); a plain
+    // power-of-two width is split as H_width = H_blocks (x) H_points with about sqrt(width)
+    // points per block.
     int status;
-    if (order == 1)
-        status = mk_fwht(x, x_dtype, rotated, x_dtype, samples, input_width, signs, nullptr, signs ? input_width : 0, scale,
-                         stream);
-    else
-        status = mk_rotate_blocks(x, x_dtype, rotated, x_dtype, samples, order, power, basis, 0, signs, nullptr, scale,
-                                  stream);
+    if (order == 1) {
+        MK_REQUIRE((input_width & (input_width - 1)) == 0 && input_width >= 32, MK_ERR_UNSUPPORTED,
+                   "mk_rotated_packed_matvec: a Walsh-Hadamard rotation needs a power-of-two width of at least 32");
+        int points = 32;
+        while (points * points < input_width && points < 1024) points *= 2;
+        status = mk_rotate_rows(x, x_dtype, rotated, x_dtype, samples, input_width / points, points, nullptr, signs, scale,
+                                stream);
+    } else {
+        status = mk_rotate_rows(x, x_dtype, rotated, x_dtype, samples, order, power, basis, signs, scale, stream);
+    }
     if (status) return status;
     return mk_packed_matvec(rotated, x_dtype, packed, scales, scale_dtype, values, n_values, zeros, bias, bias_dtype, y,
                             samples, output_width, input_width, group, bits, uniform, grid_min, grid_step, stream);

@@ -91,6 +91,9 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
         _c_void_p, _c_int, _c_void_p, _c_int, _c_longlong, _c_int, _c_int, _c_void_p, _c_int, _c_void_p,
         _c_void_p, _c_float, _c_void_p,
     ]),
+    "mk_rotate_rows": (_c_int, [
+        _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p,
+    ]),
     "mk_basis_mix": (_c_int, [
         _c_void_p, _c_void_p, _c_void_p, _c_longlong, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
     ]),

@@ -113,6 +113,7 @@ def _basis_on(width: int, device: torch.device) -> Tensor:
 
 
 ONE_LAUNCH_ROWS = 256
+ROW_KERNEL_ROWS = 64   # activation rows the per-block rotation kernel takes (mk_rotate_rows)
 
 
 def rotate(value: Tensor, *, inverse: bool = False, signs: Tensor | None = None) -> Tensor:
@@ -197,73 +198,60 @@ class OnlineRotation:
 
     def launch_arguments(self, width: int, device: torch.device) -> tuple | None:
         """``(order, power, basis pointer or None, signs pointer, scale, keep)`` for
-        ``mk_rotated_packed_matvec``, or None when the rotation kernels do not take this width
-        (``keep`` holds the tensors the pointers belong to)."""
+        ``mk_rotate_rows`` / ``mk_rotated_packed_matvec``, or None when the row-rotation kernel
+        does not take this width (``keep`` holds the tensors the pointers belong to).  A plain
+        power-of-two width is ``(1, width, None, ...)``."""
         order, power, basis = transform_factor(width)
-        if power > MAXIMUM_KERNEL_WIDTH or order > MAXIMUM_KERNEL_ORDER:
-            return None
         from mlkit_amd.kernels import hadamard as kernel
 
         signs = _cached_signs(width, self.seed, device)
         if basis is None:
+            if width < 32 or width > MAXIMUM_KERNEL_WIDTH:
+                return None
             return 1, width, None, signs.data_ptr(), kernel.normaliser(width), (signs,)
-        if not kernel.fits_one_launch(order, power):
+        if not 32 <= power <= 1024 or order > 65535:
             return None
         basis_on_device = _basis_on(width, device)
         return order, power, basis_on_device.data_ptr(), signs.data_ptr(), kernel.normaliser(power), (signs, basis_on_device)
 
     def _prepare(self, value: Tensor):
+        """The callable for tensors of this width, device and dtype.  Up to ROW_KERNEL_ROWS rows
+        (decode-time activations) go to ``mk_rotate_rows``: one short workgroup per output block
+        and row.  Taller inputs take the transform-then-mix kernels of ``rotate``."""
         seed = self.seed
         width = value.shape[-1]
-        order, power, basis = transform_factor(width)
 
         def general(tensor: Tensor) -> Tensor:
             return randomized_transform(tensor, seed=seed)
 
-        if not (_on_kernel(value) and power <= MAXIMUM_KERNEL_WIDTH and order <= MAXIMUM_KERNEL_ORDER):
+        arguments = self.launch_arguments(width, value.device) if _on_kernel(value) else None
+        if arguments is None:
             return general
         from mlkit_amd import native
-        from mlkit_amd.kernels import hadamard as kernel
 
+        order, power, basis, signs, scale, keep = arguments
+        if order == 1:  # H_width = H_blocks (x) H_points, about sqrt(width) points per block
+            points = 32
+            while points * points < width and points < 1024:
+                points *= 2
+            order, power = width // points, points
         device = value.device
-        signs = _cached_signs(width, seed, device)
-        library = native.library()
         code = native.dtype_code(value)
-        sign_pointer = signs.data_ptr()
-        if basis is None:
-            scale = kernel.normaliser(width)
-            launch = library.mk_fwht
+        launch = native.library().mk_rotate_rows
 
-            def whole(tensor: Tensor) -> Tensor:
-                if not tensor.is_contiguous():
-                    tensor = tensor.contiguous()
-                output = torch.empty_like(tensor)
-                native.check(launch(tensor.data_ptr(), code, output.data_ptr(), code, tensor.numel() // width, width,
-                                    sign_pointer, None, width, scale, native.current_stream(device)))
-                return output
-
-            whole.keeps = (signs,)
-            return whole
-        if not kernel.fits_one_launch(order, power):
-            return general
-        basis_on_device = _basis_on(width, device)
-        basis_pointer = basis_on_device.data_ptr()
-        scale = kernel.normaliser(power)
-        launch = library.mk_rotate_blocks
-
-        def blocked(tensor: Tensor) -> Tensor:
+        def by_rows(tensor: Tensor) -> Tensor:
             rows = tensor.numel() // width
-            if rows > ONE_LAUNCH_ROWS:
+            if rows > ROW_KERNEL_ROWS or rows == 0:
                 return general(tensor)
             if not tensor.is_contiguous():
                 tensor = tensor.contiguous()
             output = torch.empty_like(tensor)
-            native.check(launch(tensor.data_ptr(), code, output.data_ptr(), code, rows, order, power, basis_pointer, 0,
-                                sign_pointer, None, scale, native.current_stream(device)))
+            native.check(launch(tensor.data_ptr(), code, output.data_ptr(), code, rows, order, power, basis, signs, scale,
+                                native.current_stream(device)))
             return output
 
-        blocked.keeps = (signs, basis_on_device)
-        return blocked
+        by_rows.keeps = keep
+        return by_rows
 
 
 def rht(value: Tensor, *, seed: int = 0, inverse: bool = False) -> Tensor:

@@ -701,19 +701,33 @@ def test_incoherent_quantization_on_device_and_checkpoint(tmp_path):
 @pytest.mark.parametrize("width", [4096, 14336, 896, 12])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_online_rotation_hook_equals_rht(width, dtype):
-    """The prepared launch of the forward pre-hook against ``mk.rht`` on the same input:
-    equal bit for bit, for one row, a batch, more rows than the one-launch kernel takes,
-    and a non-contiguous view."""
+    """The prepared launch of the forward pre-hook against ``mk.rht`` on the same input.  Up to
+    64 rows take the per-block kernel (mix, then transform: the same linear map summed in
+    another order), so results agree to fp32 rounding: fp32 outputs to 1e-5, 16-bit outputs
+    identical except where the rounding of the output sits on a near-tie.  Taller inputs take
+    ``rht``'s own kernels and are equal bit for bit; so is a width without a kernel."""
     from mlkit_amd.quantization.transforms import OnlineRotation
 
     rotation = OnlineRotation(seed=11)
     generator = torch.Generator(device="cuda").manual_seed(width)
+
+    def close(ours, theirs):
+        if width < 32:
+            return torch.equal(ours, theirs)
+        if dtype == torch.float32:
+            return torch.allclose(ours, theirs, rtol=1e-5, atol=2e-5)
+        step = 2.0 ** (-10 if dtype == torch.float16 else -7) * float(theirs.float().abs().max())
+        return float((ours.float() - theirs.float()).abs().max()) <= step and float((ours == theirs).float().mean()) > 0.99
+
     for rows in (1, 8, 300):
         value = torch.randn((rows, width), device="cuda", generator=generator).to(dtype)
-        assert torch.equal(rotation(value), mk.rht(value, seed=11))
+        if rows > 64:
+            assert torch.equal(rotation(value), mk.rht(value, seed=11))
+        else:
+            assert close(rotation(value), mk.rht(value, seed=11))
     wide = torch.randn((4, 2 * width), device="cuda", generator=generator).to(dtype)
     view = wide[:, :width]
-    assert torch.equal(rotation(view), mk.rht(view, seed=11))
+    assert close(rotation(view), mk.rht(view, seed=11))
     batched = torch.randn((2, 3, width), device="cuda", generator=generator).to(dtype)
-    assert torch.equal(rotation(batched), mk.rht(batched, seed=11))
+    assert close(rotation(batched), mk.rht(batched, seed=11))
     assert rotation(batched).shape == batched.shape

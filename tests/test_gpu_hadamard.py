@@ -150,3 +150,32 @@ def test_weight_sized_rotation_keeps_norms():
     torch.testing.assert_close(hadamard.transform(blocks).view_as(weight), weight, rtol=1e-5, atol=1e-6)
     sample = weight[:3].cpu().numpy().reshape(3, 7, 2048)
     np.testing.assert_array_equal(host(blocks[:3]), transforms.fwht(sample))
+
+
+@pytest.mark.parametrize("width", [32, 64, 512, 896, 4096, 4864, 11008, 14336, 32768])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_row_rotation_kernel_matches_oracle(width, dtype):
+    """mk_rotate_rows (mix, then one Walsh-Hadamard transform per output block; the online
+    rotation of activations) against the oracle's transform-then-mix: the same linear map in
+    another summation order, so fp32 results agree to rounding (the reference's own bound for
+    the basis product, rtol 1e-5 of the row norm scale), and rows are independent."""
+    from mlkit_amd.quantization.transforms import OnlineRotation, random_signs
+
+    rotation = OnlineRotation(seed=width + 1)
+    signs = host(random_signs(width, width + 1, "cuda"))
+    for rows in (1, 8, 33):
+        generator = torch.Generator().manual_seed(width + rows)
+        value = torch.randn((rows, width), generator=generator).to(dtype)
+        rotated = rotation(value.cuda())
+        assert rotated.dtype == dtype and rotated.shape == value.shape
+        expected = transforms.randomized(value.float().numpy(), signs)
+        if dtype == torch.float32:
+            np.testing.assert_allclose(host(rotated), expected, rtol=1e-5, atol=2e-5)
+            np.testing.assert_allclose(np.linalg.norm(host(rotated), axis=1), np.linalg.norm(value.numpy(), axis=1), rtol=1e-5)
+        else:
+            rounded = torch.from_numpy(expected).to(dtype).float().numpy()
+            step = 2.0 ** (-10 if dtype == torch.float16 else -7)
+            assert np.abs(host(rotated.float()) - rounded).max() <= step * np.abs(expected).max()
+            assert (host(rotated.float()) == rounded).mean() > 0.99          # one rounding: only near-ties move
+    first = rotation(value[:1].cuda())
+    assert torch.equal(first, rotated[:1])
