@@ -410,7 +410,7 @@ def other_kernels(device: torch.device, full: bool) -> dict:
 
     # other matvec shapes and codecs, M = 1 and 8: HIP-graph launches through the C ABI over
     # enough distinct weight copies (> 512 MB) that the Infinity Cache cannot serve them
-    def matvec(rows, width, group, bits, table, uniform, asym, label, dtype=torch.float16):
+    def matvec(rows, width, group, bits, table, uniform, asym, label, dtype=torch.float16, grouped=False):
         code_bytes = rows * width * bits // 8
         count = max(2, min(40, -(-MINIMUM_ROTATING_BYTES // code_bytes)))
         streams = [torch.randint(0, 256, (code_bytes,), dtype=torch.uint8, device=device, generator=generator)
@@ -426,13 +426,25 @@ def other_kernels(device: torch.device, full: bool) -> dict:
             seconds = timed_graph(launchers, 200, 20, 20)[0]
             nbytes = code_bytes + side.numel() * 2 * (2 if asym else 1) + samples * (width + rows) * 2
             out[f"matvec {label} {rows}x{width} M={samples}"] = _entry(seconds * 1e3, nbytes, copies=count)
+            if grouped and count >= 16:   # eight matrices per launch (mk_packed_matvec_group)
+                layout = packed_linear.layout_for(bits, width, group)
+                calls = []
+                for first in range(0, count - 7, 8):
+                    launch = packed_linear.GroupLaunch(streams[first:first + 8], [side] * 8, table, [zeros] * 8, [None] * 8,
+                                                       [rows] * 8, width, group, layout, uniform_grid=uniform,
+                                                       grid_minimum=float(table[0]), grid_step=float(table[1] - table[0]))
+                    outputs = [torch.empty((samples, rows), device=device, dtype=dtype) for _ in range(8)]
+                    calls.append(lambda stream, launch=launch, outputs=outputs: launch(x, outputs, stream))
+                seconds = timed_graph(calls, 50, 8, 20)[0]
+                out[f"matvec {label} {rows}x{width} M={samples}, 8 matrices per launch"] = _entry(
+                    seconds * 1e3, 8 * nbytes, us_per_matrix=seconds * 1e6 / 8, copies=count)
 
     nf4 = mk.NF4_VALUES.to(device)
     matvec(4096, 4096, 128, 4, values, True, True, "int4 asym g128")
-    matvec(ROWS, WIDTH, 64, 2, torch.arange(-2, 2, dtype=torch.float32, device=device), True, False, "int2 g64")
-    matvec(ROWS, WIDTH, 64, 3, torch.arange(-4, 4, dtype=torch.float32, device=device), True, False, "int3 g64")
-    matvec(ROWS, WIDTH, 64, 4, nf4, False, False, "nf4 g64")
-    matvec(ROWS, WIDTH, 64, 3, seven, False, False, "codebook7 g64")
+    matvec(ROWS, WIDTH, 64, 2, torch.arange(-2, 2, dtype=torch.float32, device=device), True, False, "int2 g64", grouped=True)
+    matvec(ROWS, WIDTH, 64, 3, torch.arange(-4, 4, dtype=torch.float32, device=device), True, False, "int3 g64", grouped=True)
+    matvec(ROWS, WIDTH, 64, 4, nf4, False, False, "nf4 g64", grouped=True)
+    matvec(ROWS, WIDTH, 64, 3, seven, False, False, "codebook7 g64", grouped=True)
     if full:
         matvec(ROWS, WIDTH, 128, 4, values, True, False, "int4 g128, bf16 activations", dtype=torch.bfloat16)
         matvec(151936, 896, 128, 4, values, True, False, "int4 g128 (tied head)")

@@ -297,10 +297,15 @@ extern "C" int mk_packed_matvec_group(const void *const *x, int x_dtype, int cou
     MK_REQUIRE(samples >= 1 && input_width >= 1 && group >= 1, MK_ERR_INVALID,
                "mk_packed_matvec_group: sizes must be positive");
     bool with_zeros = zeros && zeros[0];
-    bool one_launch = mk_dtype_valid(x_dtype) && mk_dtype_valid(scale_dtype) && (!bias || mk_dtype_valid(bias_dtype)) &&
-                      bits == 4 && !tuning().no_stream4 &&
-                      mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
-                      (static_cast<size_t>(input_width) * mk_dtype_bytes(x_dtype)) % 16 == 0;
+    const bool dtypes_valid = mk_dtype_valid(x_dtype) && mk_dtype_valid(scale_dtype) && (!bias || mk_dtype_valid(bias_dtype)) &&
+                              bits >= 1 && bits <= 8;
+    // The kernels that take a group: the INT4 streaming kernels, else the table kernels.
+    const bool streaming = dtypes_valid && !tuning().no_stream4 &&
+                           mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0);
+    const bool tables = dtypes_valid && !streaming && !tuning().no_pairs && (uniform || (values && n_values >= 1 && n_values <= (1 << bits))) &&
+                        mk_packed_layout_supported(bits, input_width, group) &&
+                        mk_matvec::pairs_accepts(input_width, group, bits, x_dtype, scale_dtype);
+    bool one_launch = (streaming || tables) && (static_cast<size_t>(input_width) * mk_dtype_bytes(x_dtype)) % 16 == 0;
     for (int i = 0; i < count; ++i) {
         MK_REQUIRE(x[i] && packed[i] && scales[i] && y[i] && output_widths[i] >= 1, MK_ERR_INVALID,
                    "mk_packed_matvec_group: matrix %d has a null pointer or no rows", i);
@@ -338,8 +343,11 @@ extern "C" int mk_packed_matvec_group(const void *const *x, int x_dtype, int cou
         members.member[i].y = y[i];
     }
     int rows_per_tile = 0;
-    MK_REQUIRE(mk_matvec::stream4_launch_group(shared, members, output_widths, &rows_per_tile, stream) == 0, MK_ERR_HIP,
-               "mk_packed_matvec_group: the runtime refused the kernel's LDS size");
+    if (streaming)
+        MK_REQUIRE(mk_matvec::stream4_launch_group(shared, members, output_widths, &rows_per_tile, stream) == 0, MK_ERR_HIP,
+                   "mk_packed_matvec_group: the runtime refused the kernel's LDS size");
+    else
+        mk_matvec::pairs_launch_group(shared, members, output_widths, &rows_per_tile, stream);
     MK_LAUNCH_CHECK("mk_packed_matvec_group");
     for (int i = 0; i < count; ++i) {  // rows past a member's last whole tile
         const int covered = output_widths[i] / rows_per_tile * rows_per_tile;

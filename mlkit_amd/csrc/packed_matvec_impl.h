@@ -130,6 +130,8 @@ __device__ __forceinline__ TileSource tile_source(const Stream4Args &a, const St
 // Pair-table kernel (packed_matvec_pairs.hip): 2-, 3- and 4-bit codes of any scalar grid.
 bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype);
 int pairs_launch(const Stream4Args &a, hipStream_t stream);
+int pairs_launch_group(const Stream4Args &shared, Stream4Group &group, const int *member_rows, int *rows_per_tile,
+                       hipStream_t stream);
 bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
 // The same for a group (Stream4Args carries what the members share; its packed / scales /

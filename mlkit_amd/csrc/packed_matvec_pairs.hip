@@ -112,7 +112,7 @@ __device__ __forceinline__ void fill_table(uint32_t *table, const Stream4Args &a
 }
 
 template <int BITS, int MT, bool HAS_ZERO, int XT, int LOOKUP, int ROWS>
-__global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
+__global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const Stream4Group members) {
     constexpr int kLookup = LOOKUP;
     constexpr int kPairRows = ROWS;
     constexpr int kPairAhead = rows_in_flight<BITS>();
@@ -124,6 +124,9 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
     constexpr int kReduceRows = pair_reduce_rows<MT, ROWS>();
     constexpr int kSums = kReduceRows * MT;
 
+    // The matrix of this workgroup: the launch's only one, or member blockIdx.z of a group.
+    const TileSource source = tile_source<ROWS>(a, members, blockIdx.z);
+    if (static_cast<int>(blockIdx.x) >= source.tiles) return;  // a shorter member: the whole workgroup leaves
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -131,7 +134,7 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
     const int row_base = blockIdx.x * kPairRows;
     const int sample_base = blockIdx.y * MT;
     const uint32_t row_bytes = (static_cast<uint32_t>(a.width) * BITS) >> 3;
-    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
+    const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
     // Lanes past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
     // activations: they add nothing.
     const bool in_row = tid * kChunkCodes < a.width;
@@ -146,13 +149,12 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int sample = sample_base + m < a.samples ? sample_base + m : a.samples - 1;
-        load_x_chunk<XT>(x[m], a.x, static_cast<size_t>(sample) * a.width + static_cast<size_t>(chunk) * kChunkCodes);
+        load_x_chunk<XT>(x[m], source.x, static_cast<size_t>(sample) * a.width + static_cast<size_t>(chunk) * kChunkCodes);
     }
     const uint32_t group_offset = ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
-    const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
-    const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
-                                        : nullptr;
+    const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
+    const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
     uint16_t scale_raw[kPairRows], zero_raw[HAS_ZERO ? kPairRows : 1];
 #pragma unroll
     for (int r = 0; r < kPairRows; ++r) {
@@ -240,12 +242,8 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
             const int row = row_base + pass * kReduceRows + j;
             const int sample = sample_base + m;
             if (sample < a.samples) {
-                if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
-                const size_t index = static_cast<size_t>(sample) * a.rows + row;
-                if constexpr (XT == MK_F16)
-                    static_cast<_Float16 *>(a.y)[index] = static_cast<_Float16>(total);
-                else
-                    static_cast<uint16_t *>(a.y)[index] = mk_float_to_bf16(total);
+                if (source.bias) total += mk_load_as_float(source.bias, row, a.bias_dtype);
+                store_output<XT>(source.y, static_cast<size_t>(sample) * source.rows + row, total);
             }
         }
     }
@@ -261,7 +259,7 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a) {
 // four sub-slices of sixteen chunks; the four row sums of a result lane take their scales
 // from the four lanes of its quad.
 template <int BITS, int SETS, bool HAS_ZERO, int XT, int LOOKUP, int SLICES>
-__global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) {
+__global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, const Stream4Group members) {
     constexpr int kQuads = kPairRows / 4;
     constexpr int kSlices = SLICES;  // sub-slices of sixteen chunks per wavefront (rows of up to 512 / 1024 codes: 1 / 2)
     constexpr int kSteps = kQuads * kSlices;
@@ -273,6 +271,9 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
     constexpr int kSampleWords = blocks_sample_words(SLICES);
 
+    // The matrix of this workgroup: the launch's only one, or member blockIdx.z of a group.
+    const TileSource source = tile_source<kPairRows>(a, members, blockIdx.z);
+    if (static_cast<int>(blockIdx.x) >= source.tiles) return;  // a shorter member: the whole workgroup leaves
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -281,11 +282,10 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
     uint32_t *const x_slice = x_slices_storage + wave * (4 * kSampleWords);   // one buffer per sample of a set
     const int row_base = blockIdx.x * kPairRows;
     const uint32_t row_bytes = (static_cast<uint32_t>(a.width) * BITS) >> 3;
-    const uint8_t *codes_base = a.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
+    const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
-    const uint8_t *scale_base = static_cast<const uint8_t *>(a.scales) + static_cast<size_t>(row_base) * scale_row_bytes;
-    const uint8_t *zero_base = HAS_ZERO ? static_cast<const uint8_t *>(a.zeros) + static_cast<size_t>(row_base) * scale_row_bytes
-                                        : nullptr;
+    const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
+    const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
 
     fill_table<BITS, LOOKUP, XT>(table, a);
 
@@ -315,7 +315,7 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
             const int wanted_sample = blockIdx.y * 4 * SETS + 4 * set + j;
             const int sample = wanted_sample < a.samples ? wanted_sample : a.samples - 1;
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(a.x, a.width, sample, wave * (512 * kSlices), i, lane);
+            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(source.x, a.width, sample, wave * (512 * kSlices), i, lane);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -437,15 +437,15 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a) 
         const int set = index / (kPairRows * 4), row = row_base + (index / 4) % kPairRows;
         const int sample = blockIdx.y * 4 * SETS + 4 * set + (index & 3);
         if (sample < a.samples) {
-            if (a.bias) total += mk_load_as_float(a.bias, row, a.bias_dtype);
-            store_output<XT>(a.y, static_cast<size_t>(sample) * a.rows + row, total);
+            if (source.bias) total += mk_load_as_float(source.bias, row, a.bias_dtype);
+            store_output<XT>(source.y, static_cast<size_t>(sample) * source.rows + row, total);
         }
     }
 }
 
 template <int BITS, int SETS, int XT, int LOOKUP, int SLICES>
-void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
-    const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS));
+void launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
+    const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS), members.count > 0 ? members.count : 1);
     const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * 4 * blocks_sample_words(SLICES) * sizeof(uint32_t);
     // More than 64 KB of dynamic LDS has to be allowed per kernel (static LDS counts against
@@ -457,7 +457,7 @@ void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
                                       static_cast<int>(slices));
             allowed = slices;
         }
-        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a);
+        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
     };
     if (a.zeros) launch(pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP, SLICES>);
     else launch(pairs_blocks_kernel<BITS, SETS, false, XT, LOOKUP, SLICES>);
@@ -465,93 +465,93 @@ void launch_blocks_sliced(const Stream4Args &a, int tiles, hipStream_t stream) {
 
 // Short rows get fewer sub-slices per wavefront, so that none lies wholly past the row's end.
 template <int BITS, int SETS, int XT, int LOOKUP>
-void launch_blocks_with(const Stream4Args &a, int tiles, hipStream_t stream) {
-    if (a.width <= 1024) launch_blocks_sliced<BITS, SETS, XT, LOOKUP, 2>(a, tiles, stream);
-    else launch_blocks_sliced<BITS, SETS, XT, LOOKUP, 4>(a, tiles, stream);
+void launch_blocks_with(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
+    if (a.width <= 1024) launch_blocks_sliced<BITS, SETS, XT, LOOKUP, 2>(a, members, tiles, stream);
+    else launch_blocks_sliced<BITS, SETS, XT, LOOKUP, 4>(a, members, tiles, stream);
 }
 
 template <int BITS, int MT, int XT, int LOOKUP>
-void launch_tile_with(const Stream4Args &a, int tiles, hipStream_t stream) {
-    const dim3 grid(tiles, mk_cdiv(a.samples, MT));
+void launch_tile_with(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
+    const dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1);
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     if constexpr (MT == 1) {
         if (tile_rows(a) == kShortTileRows) {
             if (a.zeros)
-                hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP, kShortTileRows>), grid, block, 0, stream, a);
+                hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP, kShortTileRows>), grid, block, 0, stream, a, members);
             else
-                hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, LOOKUP, kShortTileRows>), grid, block, 0, stream, a);
+                hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, LOOKUP, kShortTileRows>), grid, block, 0, stream, a, members);
             return;
         }
     }
     if (a.zeros)
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP, kPairRows>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP, kPairRows>), grid, block, 0, stream, a, members);
     else
-        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, LOOKUP, kPairRows>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, LOOKUP, kPairRows>), grid, block, 0, stream, a, members);
 }
 
 // Field width per code width: the widest whose table a workgroup fills quickly.
 template <int BITS, int MT, int XT>
-void launch_tile_as(const Stream4Args &a, int tiles, hipStream_t stream) {
+void launch_tile_as(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     if constexpr (BITS == 2) {
-        launch_tile_with<BITS, MT, XT, 4>(a, tiles, stream);                                   // 256 entries
+        launch_tile_with<BITS, MT, XT, 4>(a, members, tiles, stream);                                   // 256 entries
     } else if constexpr (BITS == 3) {
-        if (a.width >= 8192) launch_tile_with<BITS, MT, XT, 4>(a, tiles, stream);              // 4096 entries
-        else launch_tile_with<BITS, MT, XT, 2>(a, tiles, stream);                              // 64
+        if (a.width >= 8192) launch_tile_with<BITS, MT, XT, 4>(a, members, tiles, stream);              // 4096 entries
+        else launch_tile_with<BITS, MT, XT, 2>(a, members, tiles, stream);                              // 64
     } else if constexpr (BITS <= 5) {
-        launch_tile_with<BITS, MT, XT, 2>(a, tiles, stream);                                   // 256 / 1024
+        launch_tile_with<BITS, MT, XT, 2>(a, members, tiles, stream);                                   // 256 / 1024
     } else if constexpr (BITS == 6) {
-        if (a.width >= 4096) launch_tile_with<BITS, MT, XT, 2>(a, tiles, stream);              // 4096
-        else launch_tile_with<BITS, MT, XT, 1>(a, tiles, stream);                              // 64
+        if (a.width >= 4096) launch_tile_with<BITS, MT, XT, 2>(a, members, tiles, stream);              // 4096
+        else launch_tile_with<BITS, MT, XT, 1>(a, members, tiles, stream);                              // 64
     } else {
-        launch_tile_with<BITS, MT, XT, 1>(a, tiles, stream);                                   // 128 / 256
+        launch_tile_with<BITS, MT, XT, 1>(a, members, tiles, stream);                                   // 128 / 256
     }
 }
 
 template <int BITS, int MT>
-void launch_tile(const Stream4Args &a, int tiles, hipStream_t stream) {
-    if (a.x_dtype == MK_F16) launch_tile_as<BITS, MT, MK_F16>(a, tiles, stream);
-    else launch_tile_as<BITS, MT, MK_BF16>(a, tiles, stream);
+void launch_tile(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
+    if (a.x_dtype == MK_F16) launch_tile_as<BITS, MT, MK_F16>(a, members, tiles, stream);
+    else launch_tile_as<BITS, MT, MK_BF16>(a, members, tiles, stream);
 }
 
 // The same field widths for the matrix-core kernel.
 template <int BITS, int SETS, int XT>
-void launch_blocks_as(const Stream4Args &a, int tiles, hipStream_t stream) {
+void launch_blocks_as(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     if constexpr (BITS == 2) {
-        launch_blocks_with<BITS, SETS, XT, 4>(a, tiles, stream);
+        launch_blocks_with<BITS, SETS, XT, 4>(a, members, tiles, stream);
     } else if constexpr (BITS == 3) {
         // (eight wavefronts' activation buffers leave no room for the 32 KB table)
-        if (a.width >= 8192 && a.width <= 14336) launch_blocks_with<BITS, SETS, XT, 4>(a, tiles, stream);
-        else launch_blocks_with<BITS, SETS, XT, 2>(a, tiles, stream);
+        if (a.width >= 8192 && a.width <= 14336) launch_blocks_with<BITS, SETS, XT, 4>(a, members, tiles, stream);
+        else launch_blocks_with<BITS, SETS, XT, 2>(a, members, tiles, stream);
     } else if constexpr (BITS <= 5) {
-        launch_blocks_with<BITS, SETS, XT, 2>(a, tiles, stream);
+        launch_blocks_with<BITS, SETS, XT, 2>(a, members, tiles, stream);
     } else if constexpr (BITS == 6) {
-        if (a.width >= 4096) launch_blocks_with<BITS, SETS, XT, 2>(a, tiles, stream);
-        else launch_blocks_with<BITS, SETS, XT, 1>(a, tiles, stream);
+        if (a.width >= 4096) launch_blocks_with<BITS, SETS, XT, 2>(a, members, tiles, stream);
+        else launch_blocks_with<BITS, SETS, XT, 1>(a, members, tiles, stream);
     } else {
-        launch_blocks_with<BITS, SETS, XT, 1>(a, tiles, stream);
+        launch_blocks_with<BITS, SETS, XT, 1>(a, members, tiles, stream);
     }
 }
 
 template <int BITS, int SETS>
-void launch_blocks(const Stream4Args &a, int tiles, hipStream_t stream) {
-    if (a.x_dtype == MK_F16) launch_blocks_as<BITS, SETS, MK_F16>(a, tiles, stream);
-    else launch_blocks_as<BITS, SETS, MK_BF16>(a, tiles, stream);
+void launch_blocks(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
+    if (a.x_dtype == MK_F16) launch_blocks_as<BITS, SETS, MK_F16>(a, members, tiles, stream);
+    else launch_blocks_as<BITS, SETS, MK_BF16>(a, members, tiles, stream);
 }
 
 template <int BITS>
-void launch_bits(const Stream4Args &a, int tiles, hipStream_t stream) {
+void launch_bits(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     if (a.samples >= 3) {  // measured against the v_dot2 kernel at 4096 x 14336
-        if (a.samples <= 4) launch_blocks<BITS, 1>(a, tiles, stream);
-        else launch_blocks<BITS, 2>(a, tiles, stream);
+        if (a.samples <= 4) launch_blocks<BITS, 1>(a, members, tiles, stream);
+        else launch_blocks<BITS, 2>(a, members, tiles, stream);
         return;
     }
     int tile = 1;
     while (tile < a.samples && tile < 8) tile <<= 1;
     switch (tile) {
-        case 1: launch_tile<BITS, 1>(a, tiles, stream); break;
-        case 2: launch_tile<BITS, 2>(a, tiles, stream); break;
-        case 4: launch_tile<BITS, 4>(a, tiles, stream); break;
-        default: launch_tile<BITS, 8>(a, tiles, stream); break;
+        case 1: launch_tile<BITS, 1>(a, members, tiles, stream); break;
+        case 2: launch_tile<BITS, 2>(a, members, tiles, stream); break;
+        case 4: launch_tile<BITS, 4>(a, members, tiles, stream); break;
+        default: launch_tile<BITS, 8>(a, members, tiles, stream); break;
     }
 }
 
@@ -562,21 +562,50 @@ bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype)
            width <= 16384 && (group % kChunkCodes == 0 || group >= width);
 }
 
-// Multiplies rows [0, 16 * tiles); returns the number of rows covered.
+namespace {
+
+void launch_for_bits(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
+    switch (a.bits) {
+        case 2: launch_bits<2>(a, members, tiles, stream); break;
+        case 3: launch_bits<3>(a, members, tiles, stream); break;
+        case 4: launch_bits<4>(a, members, tiles, stream); break;
+        case 5: launch_bits<5>(a, members, tiles, stream); break;
+        case 6: launch_bits<6>(a, members, tiles, stream); break;
+        case 7: launch_bits<7>(a, members, tiles, stream); break;
+        default: launch_bits<8>(a, members, tiles, stream); break;
+    }
+}
+
+}  // namespace
+
+// Multiplies the leading whole tiles of rows; returns the number of rows covered.
 int pairs_launch(const Stream4Args &a, hipStream_t stream) {
     const int tile = tile_rows(a);
     const int tiles = a.rows / tile;
     if (tiles == 0) return 0;
-    switch (a.bits) {
-        case 2: launch_bits<2>(a, tiles, stream); break;
-        case 3: launch_bits<3>(a, tiles, stream); break;
-        case 4: launch_bits<4>(a, tiles, stream); break;
-        case 5: launch_bits<5>(a, tiles, stream); break;
-        case 6: launch_bits<6>(a, tiles, stream); break;
-        case 7: launch_bits<7>(a, tiles, stream); break;
-        default: launch_bits<8>(a, tiles, stream); break;
-    }
+    Stream4Group none;
+    none.count = 0;
+    none.widest_tiles = 0;
+    launch_for_bits(a, none, tiles, stream);
     return tiles * tile;
+}
+
+int pairs_launch_group(const Stream4Args &shared, Stream4Group &group, const int *member_rows, int *rows_per_tile,
+                       hipStream_t stream) {
+    const int tile = tile_rows(shared);
+    int widest = 0;
+    for (int i = 0; i < group.count; ++i) {
+        group.member[i].rows = member_rows[i];
+        group.member[i].tiles = member_rows[i] / tile;
+        if (group.member[i].tiles > widest) widest = group.member[i].tiles;
+    }
+    group.widest_tiles = widest;
+    *rows_per_tile = tile;
+    if (widest == 0) return 0;
+    Stream4Args a = shared;
+    a.zeros = group.member[0].zeros;  // selects the kernel variant; the members agree on it
+    launch_for_bits(a, group, widest, stream);
+    return 0;
 }
 
 }  // namespace mk_matvec

@@ -395,16 +395,41 @@ def test_grouped_launch_equals_separate_launches(width, rows, asym, dtype):
                   relative=1e-3 if dtype == torch.float16 else 8e-3)
 
 
-def test_grouped_launch_of_other_codecs_runs_one_launch_per_matrix():
-    """Layouts the INT4 streaming kernels do not take go through the same entry point as
-    separate launches: same results as mk_packed_matvec."""
-    layers = [helpers.quantised_layer(helpers.normal_weight(n, 2048, seed=75 + i, student_t=True), scaling.NF4_VALUES,
-                                      bits=4, group=64, integer=False) for i, n in enumerate((64, 40))]
-    x = helpers.activations(2, 2048, seed=76)
-    grouped = run_group(layers, x)
+GROUP_CODECS = {
+    "int2": (scaling.int_values(2), 2, True), "int3": (scaling.int_values(3), 3, True),
+    "nf4": (scaling.NF4_VALUES, 4, False), "codebook7": (np.array([-1, -.5, -.25, 0, .25, .5, 1], dtype=np.float32), 3, False),
+    "int8": (scaling.int_values(8), 8, True),
+}
+
+
+@pytest.mark.parametrize("name", GROUP_CODECS)
+@pytest.mark.parametrize("width,rows", [(2048, (64, 40, 16)), (896, (128, 128)), (8192, (48, 32))])
+def test_grouped_launch_of_table_codecs(name, width, rows):
+    """Sub-byte, codebook and 8-bit codecs through the grouped entry point (one launch of the
+    table kernels, members of different heights, rows past a member's last whole tile): equal
+    to separate launches bit for bit for every row count, with and without offsets; the first
+    member is also held against the oracle."""
+    values, bits, integer = GROUP_CODECS[name]
+    for asym in (False, True):
+        layers = [helpers.quantised_layer(helpers.normal_weight(n, width, seed=75 + i, student_t=True), values, bits=bits,
+                                          group=64, integer=integer, asym=asym) for i, n in enumerate(rows)]
+        for samples in (1, 2, 3, 8):
+            x = helpers.activations(samples, width, seed=76 + samples)
+            grouped = run_group(layers, x)
+            for index, layer in enumerate(layers):
+                assert np.array_equal(grouped[index].float().cpu().numpy(), run_matvec(layer, x)), (index, samples, asym)
+            check(grouped[0].float().cpu().numpy(), layers[0], x)
+
+
+def test_grouped_launch_of_layouts_without_a_group_kernel():
+    """fp32 activations (the generic kernel) go through the same entry point as one launch per
+    matrix: same results as mk_packed_matvec."""
+    layers = [helpers.quantised_layer(helpers.normal_weight(n, 256, seed=77 + i), INT4, bits=4, group=64, integer=True,
+                                      fmt="fp32") for i, n in enumerate((37, 21))]
+    x = helpers.activations(2, 256, seed=78, dtype=torch.float32)
+    grouped = run_group(layers, x, scale_dtype=torch.float32)
     for index, layer in enumerate(layers):
-        assert np.array_equal(grouped[index].float().cpu().numpy(), run_matvec(layer, x))
-        check(grouped[index].float().cpu().numpy(), layer, x)
+        assert np.array_equal(grouped[index].cpu().numpy(), run_matvec(layer, x, scale_dtype=torch.float32))
 
 
 def test_grouped_launch_validation():
