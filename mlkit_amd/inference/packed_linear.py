@@ -16,6 +16,7 @@ How a call is served here:
 * a tied embedding decodes only the requested rows (``mk_packed_decode_rows``).
 """
 
+import copy
 from collections.abc import Callable
 from dataclasses import dataclass
 
@@ -24,13 +25,15 @@ import torch.nn.functional as functional
 from torch import Tensor, nn
 
 from mlkit_amd import native
-from mlkit_amd.kernels.packed_linear import MAXIMUM_CODE_BITS, PackedLayout, decode, layout_for, packed_matvec_op
+from mlkit_amd.kernels.packed_linear import (MAXIMUM_CODE_BITS, GroupLaunch, PackedLayout, decode, layout_for,
+                                             packed_matvec_op)
 from mlkit_amd.quantization.bitstream import pack, unpack
 from mlkit_amd.quantization.codecs import decode_scaled
 from mlkit_amd.quantization.core import Q
 
 SCALE_STORAGE_DTYPES = {"fp16": torch.float16, "bf16": torch.bfloat16}
 MAXIMUM_FUSED_ROWS = 8
+_LAUNCH_BUFFERS = frozenset({"packed", "scales", "values", "zeros", "bias"})
 
 
 def preserve_input_processing(original: nn.Module, replacement: nn.Module) -> None:
@@ -127,6 +130,7 @@ class PackedLinear(nn.Module):
         self._launch: tuple | None = None
         self._rotation = None          # an absorbed OnlineRotation
         self._rotation_launch: tuple | None = None
+        self._siblings: SiblingLaunch | None = None
         preserve_input_processing(original, self)
         self._absorb_rotation_hook()
 
@@ -152,9 +156,26 @@ class PackedLinear(nn.Module):
 
     # -- module plumbing ---------------------------------------------------------------------
 
+    def __setattr__(self, name: str, value) -> None:
+        if name in _LAUNCH_BUFFERS:   # a replaced buffer: bound launch arguments are stale
+            self.__dict__["_launch"] = None
+            siblings = self.__dict__.get("_siblings")
+            if siblings is not None:
+                siblings.reset()
+        super().__setattr__(name, value)
+
+    def register_buffer(self, name: str, tensor, persistent: bool = True) -> None:
+        if name in _LAUNCH_BUFFERS and "_siblings" in self.__dict__:
+            self.__dict__["_launch"] = None
+            if self.__dict__["_siblings"] is not None:
+                self.__dict__["_siblings"].reset()
+        super().register_buffer(name, tensor, persistent)
+
     def _apply(self, fn: Callable[[Tensor], Tensor], recurse: bool = True) -> "PackedLinear":
         self._launch = self._rotation_launch = None
         self._dense_weight = None
+        if self._siblings is not None:
+            self._siblings.reset()
         return super()._apply(fn, recurse)
 
     @property
@@ -203,10 +224,28 @@ class PackedLinear(nn.Module):
             output = packed_matvec_op(flat, self.packed, self.scales, self.values, self.zeros, self.bias,
                                       self.out_features, self.group, self.code_bits, self.uniform_grid,
                                       self.grid_minimum, self.grid_step)
+        elif self._siblings is not None and not rotate_here:
+            output = self._siblings.output_for(self, inputs, flat)
         else:
             output = inputs.new_empty((rows, self.out_features))
             self._matvec(flat, output, rows, rotate_here)
         return output.view(inputs.shape[:-1] + (self.out_features,))
+
+    # -- grouped launches with sibling layers ------------------------------------------------
+
+    @property
+    def groupable(self) -> bool:
+        """Whether this layer may share a launch with siblings: a fused layout, no input
+        transform of its own."""
+        return (self.layout is not None and self._rotation is None and not self._forward_pre_hooks
+                and not self._forward_pre_hooks_with_kwargs)
+
+    @property
+    def group_key(self) -> tuple:
+        """What sibling layers must have in common to share a launch."""
+        return (self.in_features, self.group, self.code_bits, self.uniform_grid, self.grid_minimum, self.grid_step,
+                tuple(self.values.tolist()), self.scales.dtype, self.zeros is None,
+                None if self.bias is None else self.bias.dtype, self.packed.device)
 
     def _bound_arguments(self) -> tuple:
         """The layer's constant launch arguments, bound once and kept for as long as all five
@@ -259,6 +298,80 @@ class PackedLinear(nn.Module):
                                                        *constants, stream)
         if status:
             native.check(status)
+
+
+class SiblingLaunch:
+    """Packed layers that read the same activations, multiplied by one launch.
+
+    The first member whose ``forward`` sees an input runs ``mk_packed_matvec_group`` for all
+    members and keeps the others' outputs; each other member, called with the *same tensor*
+    (same object, or same memory, shape and version), takes its output from there, once.  The
+    kept input is referenced for as long as outputs are pending, so its memory cannot be
+    handed to another tensor meanwhile; an in-place change is noticed through the tensor's
+    version counter where one exists (not under ``torch.inference_mode``: there the model must
+    not modify the shared input between the sibling calls).  Anything else -- another input, a
+    member called twice -- simply starts a new grouped launch, so results never depend on the
+    cache being hit."""
+
+    MAXIMUM = 8
+
+    def __init__(self, layers: list[PackedLinear]) -> None:
+        self.layers = tuple(layers)
+        for layer in self.layers:
+            layer._siblings = self
+        self._launch: GroupLaunch | None = None
+        self._pending: tuple | None = None
+
+    def reset(self) -> None:
+        self._launch = None
+        self._pending = None
+
+    def __deepcopy__(self, memo: dict) -> "SiblingLaunch":
+        """A copy links the copied layers and binds its own launch arguments on first use."""
+        clone = SiblingLaunch.__new__(SiblingLaunch)
+        memo[id(self)] = clone
+        clone.layers = tuple(copy.deepcopy(layer, memo) for layer in self.layers)
+        clone._launch = None
+        clone._pending = None
+        return clone
+
+    @staticmethod
+    def _version(tensor: Tensor) -> int | None:
+        try:
+            return tensor._version
+        except RuntimeError:  # inference tensors keep no version counter
+            return None
+
+    def _bound(self) -> GroupLaunch:
+        if self._launch is None:
+            first = self.layers[0]
+            self._launch = GroupLaunch(
+                [layer.packed for layer in self.layers], [layer.scales for layer in self.layers], first.values,
+                [layer.zeros for layer in self.layers], [layer.bias for layer in self.layers],
+                [layer.out_features for layer in self.layers], first.in_features, first.group, first.layout,
+                uniform_grid=first.uniform_grid, grid_minimum=first.grid_minimum, grid_step=first.grid_step)
+        return self._launch
+
+    def output_for(self, layer: PackedLinear, original: Tensor, flat: Tensor) -> Tensor:
+        pending = self._pending
+        if pending is not None:
+            kept, version, outputs = pending
+            # without a version counter only the very same tensor object counts as the same input
+            same = kept is original or (version is not None and kept.data_ptr() == original.data_ptr()
+                                        and kept.shape == original.shape and kept.dtype == original.dtype
+                                        and kept.stride() == original.stride())
+            if same and version == self._version(original) and id(layer) in outputs:
+                output = outputs.pop(id(layer))
+                if not outputs:
+                    self._pending = None
+                return output
+        rows = flat.shape[0]
+        results = [flat.new_empty((rows, member.out_features)) for member in self.layers]
+        self._bound()(flat, results)
+        outputs = {id(member): result for member, result in zip(self.layers, results)}
+        mine = outputs.pop(id(layer))
+        self._pending = (original, self._version(original), outputs) if outputs else None
+        return mine
 
 
 class PackedEmbedding(nn.Module):

@@ -317,6 +317,60 @@ def test_packed_linear_follows_replaced_side_buffers():
         torch.testing.assert_close(layer(inputs).float(), dense_product(), rtol=2e-3, atol=2e-3)
 
 
+class Attention(nn.Module):
+    """q / k / v read the same hidden state; o reads something else."""
+
+    def __init__(self, width=896, heads_kv=128):
+        super().__init__()
+        self.q_proj = nn.Linear(width, width, bias=True)
+        self.k_proj = nn.Linear(width, heads_kv, bias=True)
+        self.v_proj = nn.Linear(width, heads_kv, bias=True)
+        self.o_proj = nn.Linear(width, width, bias=False)
+
+    def forward(self, x):
+        q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+        mixed = q * (k.sum(-1, keepdim=True) + v.mean(-1, keepdim=True))
+        return self.o_proj(mixed)
+
+
+def test_sibling_layers_share_one_launch():
+    """optimize(group_siblings=True): q / k / v (same parent, same input width and codec) are
+    linked; the model's output equals the ungrouped packed model bit for bit, for fp16 rows 1..8,
+    under inference_mode and plain no_grad, when an input is modified in place between calls,
+    when a member is called alone, after deepcopy, and after a buffer is replaced."""
+    torch.manual_seed(49)
+    module = Attention().half().cuda()
+    converted = mk.quantize(module, mk.int(4, group=128), calib=None)
+    plain = mk.optimize(converted, backend="packed")
+    grouped = mk.optimize(converted, backend="packed", group_siblings=True)
+    attention = grouped.module
+    assert attention.q_proj._siblings is attention.k_proj._siblings is attention.v_proj._siblings is not None
+    assert attention.o_proj._siblings is None and len(attention.q_proj._siblings.layers) == 3
+    for context in (torch.inference_mode, torch.no_grad):
+        for rows in (1, 2, 5, 8, 12):
+            x = torch.randn(rows, 896, device="cuda").half()
+            with context():
+                assert torch.equal(grouped(x), plain(x)), (context, rows)
+    with torch.no_grad():
+        x = torch.randn(2, 896, device="cuda").half()
+        q = attention.q_proj(x)                      # leaves k and v pending for this x
+        x.mul_(2)                                    # the version changes: pending outputs must not be used
+        assert torch.equal(attention.k_proj(x), plain.module.k_proj(x))
+        assert torch.equal(q * 0 + attention.q_proj(x), plain.module.q_proj(x))
+        other = torch.randn(2, 896, device="cuda").half()
+        assert torch.equal(attention.v_proj(other), plain.module.v_proj(other))   # another tensor: a new launch
+        assert torch.equal(attention.v_proj(other), plain.module.v_proj(other))   # a member called twice
+    duplicate = copy.deepcopy(grouped)
+    assert duplicate.module.q_proj._siblings is not attention.q_proj._siblings
+    assert duplicate.module.q_proj._siblings.layers[1] is duplicate.module.k_proj
+    with torch.inference_mode():
+        x = torch.randn(1, 896, device="cuda").half()
+        assert torch.equal(duplicate(x), plain(x))
+        attention.k_proj.scales = (attention.k_proj.scales.float() * 2).half()     # a replaced buffer is picked up
+        plain.module.k_proj.scales = (plain.module.k_proj.scales.float() * 2).half()
+        assert torch.equal(grouped(x), plain(x))
+
+
 WIDTH_FORMATS = {
     "int2": lambda: mk.int(2, group=64),
     "int3": lambda: mk.int(3, group=64),
