@@ -10,7 +10,6 @@ without the buffers of packed layers, which are rebuilt from the codes.
 
 import hashlib
 import json
-import os
 import shutil
 import tempfile
 from collections.abc import Callable
@@ -113,55 +112,87 @@ def restore_layer(tensors: dict[str, Tensor], name: str, entry: dict[str, Any]) 
              metadata={**entry.get("metadata", {}), "code_bits": entry["code_bits"]})
 
 
+class _StateCollector:
+    """The part of a module's state a checkpoint stores as ``state.<name>``: everything except
+    the rounded weights (they come back from the codes), parameters tied to them, and the
+    derived buffers of packed layers.  Tensors that are views of the same memory are stored
+    once; the other names are recorded as aliases of the first."""
+
+    DERIVED_BUFFERS = frozenset({"packed", "scales", "values", "zeros"})
+
+    def __init__(self, model: QModel) -> None:
+        self.rounded = set(model.quantized)
+        self.skipped = {_weight_name(name) for name in model.quantized} | set(model.tied_weights)
+        self.tensors: dict[str, Tensor] = {}
+        self.aliases: dict[str, str] = {}
+        self._owner_of_memory: dict[tuple, str] = {}
+
+    def wanted(self, name: str) -> bool:
+        if name in self.skipped:
+            return False
+        module_name, _, leaf = name.rpartition(".")
+        return not (module_name in self.rounded and leaf in self.DERIVED_BUFFERS)
+
+    def add(self, name: str, value: Tensor) -> None:
+        memory = (value.device, value.data_ptr(), value.dtype, tuple(value.shape), tuple(value.stride()))
+        owner = self._owner_of_memory.get(memory)
+        if owner is None:
+            self._owner_of_memory[memory] = name
+            self.tensors[f"state.{name}"] = value.detach().cpu().contiguous().clone()
+        else:
+            self.aliases[name] = owner
+
+
+def _manifest(model: QModel, layers: dict[str, Any], aliases: dict[str, str], tensors: dict[str, Tensor]) -> dict[str, Any]:
+    reference_parameter = next(model.module.parameters(), None)
+    dtype = torch.float32 if reference_parameter is None else reference_parameter.dtype
+    return {
+        "format_version": FORMAT_VERSION, "name": model.name, "architecture": "external",
+        "dtype": str(dtype).removeprefix("torch."), "layers": layers, "reports": [], "pass_reports": [],
+        "stability_reports": {}, "logical_bpw": model.bpw, "model_bpw": model.model_bpw,
+        "parameter_accounting": None, "transforms": list(model.transforms), "activations": {}, "kv": None,
+        "state_aliases": aliases, "tied_weights": model.tied_weights,
+        "tensor_bytes": sum(tensor.numel() * tensor.element_size() for tensor in tensors.values()),
+    }
+
+
+def _publish(staged: Path, destination: Path) -> None:
+    """Move a fully written checkpoint directory into place.  An existing checkpoint is set
+    aside under a fresh name first and removed only after the new one is in place; if the new
+    one cannot be moved in, the old one returns."""
+    if not destination.exists():
+        staged.rename(destination)
+        return
+    aside = Path(tempfile.mkdtemp(prefix=f".{destination.name}.replaced_", dir=destination.parent))
+    aside.rmdir()                      # only the unique name is wanted
+    destination.rename(aside)
+    try:
+        staged.rename(destination)
+    except BaseException:
+        aside.rename(destination)
+        raise
+    shutil.rmtree(aside, ignore_errors=True)
+
+
 def save(model: QModel, path: "str | Path", *, overwrite: bool = False) -> None:
+    """Write ``mlkit.json`` + ``weights.safetensors`` under ``path``; the directory appears (or is
+    replaced, with ``overwrite``) only once both files are complete."""
     destination = Path(path).resolve()
     if destination.exists() and not overwrite:
         raise FileExistsError(f"checkpoint destination already exists: {destination}")
     destination.parent.mkdir(parents=True, exist_ok=True)
-    staging = Path(tempfile.mkdtemp(prefix="mlkit_checkpoint_", dir=destination.parent))
-    try:
-        tensors, layers = describe_layers(model.quantized)
-        omitted = {_weight_name(name) for name in model.quantized} | set(model.tied_weights)
-        first_of_storage: dict[tuple, str] = {}
-        aliases: dict[str, str] = {}
-        for name, value in model.module.state_dict().items():
-            owner, _, field = name.rpartition(".")
-            if name in omitted or (owner in model.quantized and field in {"packed", "scales", "values", "zeros"}):
-                continue
-            identity = (value.device, value.data_ptr(), value.dtype, tuple(value.shape), tuple(value.stride()))
-            first = first_of_storage.setdefault(identity, name)
-            if first == name:
-                tensors[f"state.{name}"] = value.detach().cpu().contiguous().clone()
-            else:
-                aliases[name] = first
-        save_file(tensors, str(staging / WEIGHTS_FILE))
-        parameter = next(model.module.parameters(), None)
-        dtype = torch.float32 if parameter is None else parameter.dtype
-        manifest = {
-            "format_version": FORMAT_VERSION, "name": model.name, "architecture": "external",
-            "dtype": str(dtype).removeprefix("torch."), "layers": layers, "reports": [], "pass_reports": [],
-            "stability_reports": {}, "logical_bpw": model.bpw, "model_bpw": model.model_bpw,
-            "parameter_accounting": None, "transforms": list(model.transforms), "activations": {}, "kv": None,
-            "state_aliases": aliases, "tied_weights": model.tied_weights,
-            "tensor_bytes": sum(t.numel() * t.element_size() for t in tensors.values()),
-        }
-        (staging / MANIFEST_FILE).write_text(json.dumps(manifest, indent=2) + "\n")
-        if destination.exists():
-            previous = destination.with_name(f"{destination.name}.previous")
-            if previous.exists():
-                raise FileExistsError(f"checkpoint backup already exists: {previous}")
-            os.replace(destination, previous)
-            try:
-                os.replace(staging, destination)
-            except BaseException:
-                os.replace(previous, destination)
-                raise
-            shutil.rmtree(previous)
-        else:
-            os.replace(staging, destination)
-    finally:
-        if staging.exists():
-            shutil.rmtree(staging)
+    tensors, layers = describe_layers(model.quantized)
+    state = _StateCollector(model)
+    for name, value in model.module.state_dict().items():
+        if state.wanted(name):
+            state.add(name, value)
+    tensors.update(state.tensors)
+    with tempfile.TemporaryDirectory(prefix="mlkit_checkpoint_", dir=destination.parent) as scratch:
+        staged = Path(scratch) / "checkpoint"
+        staged.mkdir()
+        save_file(tensors, str(staged / WEIGHTS_FILE))
+        (staged / MANIFEST_FILE).write_text(json.dumps(_manifest(model, layers, state.aliases, tensors), indent=2) + "\n")
+        _publish(staged, destination)
 
 
 def load_checkpoint(path: "str | Path", *, model: "nn.Module | Callable[[], nn.Module]", device: str = "cuda") -> QModel:

@@ -1,9 +1,11 @@
 """What a quantizer qualifies for: fused kernels, checkpoint form, packed execution.
 
-Mirrors /root/reference/src/mlkit/evaluation/capability_report.py:24-133 (``Capabilities``,
+Same fields and report strings as the reference's capability report
+(/root/reference/src/mlkit/evaluation/capability_report.py:24-133: ``Capabilities``,
 ``capabilities``, ``error_feedback_path``, ``packed_inference_path``,
-``online_activation_path``) with the same field names and the same report strings for the
-scalar formats this package implements.
+``online_activation_path``), for the scalar formats this package implements.  Each of the
+three "path" questions is answered by walking a short list of (condition, answer) rules, the
+first that applies wins; ``capabilities`` rounds a seeded random matrix once and asks them.
 """
 
 from dataclasses import dataclass, fields
@@ -19,11 +21,7 @@ from mlkit_amd.quantization.core import Ctx, FittedRounder, FunctionQuantizer, Q
 from mlkit_amd.quantization.feedback import FUSED_CODEBOOK_LIMIT
 from mlkit_amd.quantization.scaled import SCALE_FORMAT_BITS, Scaled
 
-
-def _shown(value: Any) -> str:
-    if value is None:
-        return "unknown"
-    return f"{value:.4f}" if isinstance(value, float) else str(value)
+FUSED = "fused kernel"
 
 
 @dataclass
@@ -41,40 +39,51 @@ class Capabilities:
     online_activations: str
 
     def __str__(self) -> str:
-        labels = [field.name.replace("_", " ") for field in fields(self)]
-        pad = max(map(len, labels))
-        return "\n".join(f"{label.ljust(pad)}  {_shown(getattr(self, field.name))}"
-                         for label, field in zip(labels, fields(self), strict=True))
+        rows = []
+        for field in fields(self):
+            value = getattr(self, field.name)
+            text = "unknown" if value is None else (f"{value:.4f}" if isinstance(value, float) else str(value))
+            rows.append((field.name.replace("_", " "), text))
+        width = max(len(label) for label, _ in rows)
+        return "\n".join(f"{label:<{width}}  {text}" for label, text in rows)
+
+
+def _fitted_scalar(quantization: Quantizer, weight: Tensor):
+    """The scalar rounding state the quantizer fits on ``weight`` (None when it fits none)."""
+    with torch.no_grad():
+        fitted = quantization.fit(weight, Ctx("capabilities", X=weight.new_zeros((1, weight.shape[1]))))
+    return fitted.scalar if isinstance(fitted, FittedRounder) else None
 
 
 def error_feedback_path(quantization: Any, weight: Tensor) -> str:
-    if isinstance(quantization, FunctionQuantizer) or not isinstance(quantization, Quantizer):
+    plain_function = isinstance(quantization, FunctionQuantizer) or not isinstance(quantization, Quantizer)
+    if plain_function:
         return "reference rounding; the function is called on every column block"
     if type(quantization).fit is Quantizer.fit:
         return "not an inner format; it does not implement Quantizer.fit"
-    context = Ctx("capabilities", X=weight.new_zeros((1, weight.shape[1])))
-    with torch.no_grad():
-        rounder = quantization.fit(weight, context)
-    scalar = rounder.scalar if isinstance(rounder, FittedRounder) else None
-    if scalar is not None and scalar.grid.bits <= 8 and scalar.values.numel() <= FUSED_CODEBOOK_LIMIT:
-        return "fused scalar kernel at step=1"
-    return "reference rounding with the fitted rounder"
+    scalar = _fitted_scalar(quantization, weight)
+    kernel_ready = scalar is not None and scalar.grid.bits <= 8 and scalar.values.numel() <= FUSED_CODEBOOK_LIMIT
+    return "fused scalar kernel at step=1" if kernel_ready else "reference rounding with the fitted rounder"
 
 
 def packed_inference_path(result: Q, input_width: int) -> str:
-    if not registered(result.codec) or result.codec not in {"scaled", "feedback"} or not packed_compatible(result):
+    scalar_codes = registered(result.codec) and result.codec in ("scaled", "feedback") and packed_compatible(result)
+    if not scalar_codes:
         return "no; dense weights"
-    if layout_for(result.metadata["code_bits"], input_width, result.params["group"]) is None:
-        return "packed storage with dense execution; rows or groups split a packing word"
-    return "fused kernel"
+    whole_words = layout_for(result.metadata["code_bits"], input_width, result.params["group"]) is not None
+    return FUSED if whole_words else "packed storage with dense execution; rows or groups split a packing word"
 
 
 def online_activation_path(quantization: Any) -> str:
     if not isinstance(quantization, Scaled):
         return "reference rounding; not restorable from a checkpoint"
-    fused = (quantization.grid.dim == 1 and quantization.grid.values is not None and quantization.scale == "absmax"
-             and isinstance(quantization.scale_fmt, str) and quantization.scale_fmt in SCALE_FORMAT_BITS)
-    return "fused kernel" if fused else "reference rounding"
+    requirements = (
+        quantization.grid.dim == 1,
+        quantization.grid.values is not None,
+        quantization.scale == "absmax",
+        isinstance(quantization.scale_fmt, str) and quantization.scale_fmt in SCALE_FORMAT_BITS,
+    )
+    return FUSED if all(requirements) else "reference rounding"
 
 
 def capabilities(quantization: Any, shape: tuple[int, int] = (64, 256), *, device: str = "cuda") -> Capabilities:
@@ -82,23 +91,23 @@ def capabilities(quantization: Any, shape: tuple[int, int] = (64, 256), *, devic
 
     The bit cost includes side information and therefore depends on ``shape``.
     """
+    rows, width = shape
     generator = torch.Generator(device=device).manual_seed(0)
-    weight = torch.randn(shape, device=device, generator=generator)
-    inputs = torch.randn((4 * shape[1], shape[1]), device=device, generator=generator)
-    context = Ctx("capabilities", X=inputs)
+    weight = torch.randn((rows, width), device=device, generator=generator)
+    context = Ctx("capabilities", X=torch.randn((4 * width, width), device=device, generator=generator))
     with torch.no_grad():
         result = as_q(quantization(weight, context))
-        restored = result.w
-    if restored.shape != weight.shape or not bool(torch.isfinite(restored).all()):
+        reconstruction = result.w
+    if reconstruction.shape != weight.shape or not bool(torch.isfinite(reconstruction).all()):
         raise ValueError("the quantizer returned an invalid reconstruction")
-    bits = None if result.bits is None else result.bits + context.additional_bits
-    portable = result.codes is not None and registered(result.codec)
+    total_bits = None if result.bits is None else result.bits + context.additional_bits
+    stored_as_codes = result.codes is not None and registered(result.codec)
     return Capabilities(
         quantizer=repr(quantization),
-        bits_per_weight=None if bits is None else bits / weight.numel(),
+        bits_per_weight=None if total_bits is None else total_bits / weight.numel(),
         codec=result.codec,
-        checkpoint="codes with a registered codec" if portable else "dense reconstruction",
+        checkpoint="codes with a registered codec" if stored_as_codes else "dense reconstruction",
         error_feedback=error_feedback_path(quantization, weight),
-        packed_inference=packed_inference_path(result, shape[1]),
+        packed_inference=packed_inference_path(result, width),
         online_activations=online_activation_path(quantization),
     )

@@ -1,11 +1,16 @@
 """Incoherence processing: an inner quantizer applied in a randomly rotated basis.
 
-Mirrors /root/reference/src/mlkit/quantization/algorithms/incoherence.py:15-98 (``Incoherent``,
-``incoherent``): rows and columns are multiplied by hash-derived signs and rotated with the
-structured transform before the inner quantizer sees them; calibration statistics are
-rotated the same way; a portable inner representation is wrapped in the ``"basis"`` codec,
-which rotates the reconstruction back on decode.  On a HIP device every rotation is one or
-two kernel launches with the sign flips fused.
+Same call surface and results as the reference's ``Incoherent`` / ``incoherent``
+(/root/reference/src/mlkit/quantization/algorithms/incoherence.py:15-98): the weight is seen by
+the inner quantizer as ``U W V^T`` with ``U``, ``V`` sign-randomised structured transforms of
+the output and input side (signs from ``deterministic_signs`` of the layer seed and seed + 1),
+calibration statistics move to the same basis, and a portable inner representation comes back
+wrapped in the ``"basis"`` codec, which undoes the rotation on decode.
+
+Here the two sides are objects (``_Side``) that know how to move a matrix into their basis and
+back along either axis, so the quantizer itself reads as: rotate, describe the statistics in
+the new basis, round, wrap or rotate back.  On a HIP device each move is one or two kernel
+launches with the sign flips fused.
 """
 
 from collections.abc import Callable
@@ -17,16 +22,55 @@ from mlkit_amd.quantization.codecs import compose, deterministic_signs, register
 from mlkit_amd.quantization.core import Ctx, Q, Quantizer, as_q, layer_seed
 from mlkit_amd.quantization.transforms import rotate
 
+SIDE_KINDS = (None, "rht")
 
-def _rows(value: Tensor, signs: Tensor, inverse: bool = False) -> Tensor:
-    """The transform along the first dimension."""
-    return rotate(value.T.contiguous(), inverse=inverse, signs=signs).T
+
+class _Side:
+    """One sign-randomised structured transform ``T diag(signs)`` of a given width."""
+
+    def __init__(self, width: int, seed: int, device) -> None:
+        self.seed = seed
+        self.signs = deterministic_signs(width, seed, device)
+
+    def along_columns(self, matrix: Tensor, back: bool = False) -> Tensor:
+        """``matrix @ (T diag(signs))^T`` (every row transformed), or its inverse."""
+        return rotate(matrix.contiguous(), inverse=back, signs=self.signs)
+
+    def along_rows(self, matrix: Tensor, back: bool = False) -> Tensor:
+        """``(T diag(signs)) @ matrix`` (every column transformed), or its inverse."""
+        return self.along_columns(matrix.T, back).T
+
+    def conjugate(self, symmetric: Tensor) -> Tensor:
+        """``(T S) M (T S)^T`` for a square matrix over this side's width."""
+        return self.along_rows(self.along_columns(symmetric))
+
+
+def _statistics_in(side: _Side, ctx: Ctx, device) -> Callable[[str, Callable | None, str], Tensor]:
+    """Calibration statistics as the inner quantizer must see them once the inputs are rotated
+    by ``side``: everything is recomputed from the rotated inputs (or conjugated, for H)."""
+    upstream = ctx._provider
+
+    def provide(name: str, function: Callable | None, reduce: str) -> Tensor:
+        if name == "H":
+            return side.conjugate(ctx.H.to(device))
+        rotated_inputs = side.along_columns(ctx.X.to(device))
+        known = {"X": lambda: rotated_inputs, "act_absmean": lambda: rotated_inputs.abs().mean(0),
+                 "act_absmax": lambda: rotated_inputs.abs().amax(0)}
+        if name in known:
+            return known[name]()
+        if function is not None:
+            return function(rotated_inputs)
+        if upstream is None:
+            raise KeyError(name)
+        return upstream(name, function, reduce)
+
+    return provide
 
 
 class Incoherent(Quantizer):
     def __init__(self, inner: Callable[..., "Q | Tensor"], *, left: str | None = "rht", right: str | None = "rht",
                  train_signs: bool = False) -> None:
-        if left not in {None, "rht"} or right not in {None, "rht"}:
+        if left not in SIDE_KINDS or right not in SIDE_KINDS:
             raise ValueError("incoherence transforms must be rht or None")
         self.inner, self.left, self.right, self.train_signs = inner, left, right, train_signs
 
@@ -35,61 +79,45 @@ class Incoherent(Quantizer):
 
     def __call__(self, w: Tensor, ctx: Ctx | None = None) -> Q:
         ctx = ctx or Ctx(device=w.device)
-        seed = layer_seed(ctx.name, ctx._seed) % 2**32
-        left_signs = deterministic_signs(w.shape[0], seed, w.device) if self.left else None
-        right_signs = deterministic_signs(w.shape[1], seed + 1, w.device) if self.right else None
-        rotated = w.float()
-        if left_signs is not None:
-            rotated = _rows(rotated, left_signs)
-        if right_signs is not None:
-            rotated = rotate(rotated.contiguous(), signs=right_signs)
-        inner_ctx = ctx.replace()
-        if right_signs is not None:
-            fallback = ctx._provider
+        base_seed = layer_seed(ctx.name, ctx._seed) % 2**32
+        rows, columns = w.shape
+        output_side = _Side(rows, base_seed, w.device) if self.left else None
+        input_side = _Side(columns, base_seed + 1, w.device) if self.right else None
 
-            def rotated_statistic(name: str, fn: Callable | None, reduce: str) -> Tensor:
-                if name == "H":
-                    hessian = ctx.H.to(w.device) * right_signs[:, None] * right_signs[None, :]
-                    return rotate(rotate(hessian.contiguous()).T.contiguous()).T
-                inputs = rotate(ctx.X.to(w.device).contiguous(), signs=right_signs)
-                if name == "X":
-                    return inputs
-                if name == "act_absmean":
-                    return inputs.abs().mean(0)
-                if name == "act_absmax":
-                    return inputs.abs().amax(0)
-                if fn is not None:
-                    return fn(inputs)
-                if fallback is not None:
-                    return fallback(name, fn, reduce)
-                raise KeyError(name)
-
-            inner_ctx = ctx.derive(rotated_statistic)
-        quantized = as_q(self.inner(rotated, inner_ctx))
+        in_basis = w.float()
+        if output_side is not None:
+            in_basis = output_side.along_rows(in_basis)
+        if input_side is not None:
+            in_basis = input_side.along_columns(in_basis)
+        inner_ctx = ctx.replace() if input_side is None else ctx.derive(_statistics_in(input_side, ctx, w.device))
+        rounded = as_q(self.inner(in_basis, inner_ctx))
         ctx.add_bits(inner_ctx.additional_bits)
-        if quantized.codes is not None and registered(quantized.codec):
-            result = compose(quantized, "basis", {
-                "shape": tuple(w.shape),
-                "left_seed": seed if self.left else None,
-                "right_seed": (seed + 1) % 2**32 if self.right else None,
-                "left_signs": left_signs if self.train_signs else None,
-                "right_signs": right_signs if self.train_signs else None,
-            })
+
+        portable = rounded.codes is not None and registered(rounded.codec)
+        if not portable:
             if self.train_signs:
-                for key, signs in (("left_signs", left_signs), ("right_signs", right_signs)):
-                    if signs is not None:
-                        result.metadata["trainable"].append(key)
-                        result.metadata["parameter_formats"][key] = "fp16"
-                        ctx.add_bits(16 * signs.numel())
-            return result
-        if self.train_signs:
-            raise ValueError("trainable signs require an inner quantizer with a registered codec")
-        restored = quantized.w
-        if right_signs is not None:
-            restored = rotate(restored.contiguous(), inverse=True, signs=right_signs)
-        if left_signs is not None:
-            restored = _rows(restored, left_signs, inverse=True)
-        return Q(restored, bits=quantized.bits)
+                raise ValueError("trainable signs require an inner quantizer with a registered codec")
+            restored = rounded.w
+            if input_side is not None:
+                restored = input_side.along_columns(restored, back=True)
+            if output_side is not None:
+                restored = output_side.along_rows(restored, back=True)
+            return Q(restored, bits=rounded.bits)
+
+        kept_signs = {"left_signs": output_side.signs if output_side is not None and self.train_signs else None,
+                      "right_signs": input_side.signs if input_side is not None and self.train_signs else None}
+        wrapped = compose(rounded, "basis", {
+            "shape": (rows, columns),
+            "left_seed": None if output_side is None else output_side.seed,
+            "right_seed": None if input_side is None else input_side.seed % 2**32,
+            **kept_signs,
+        })
+        for key, signs in kept_signs.items():  # trainable sign vectors are stored, as fp16
+            if signs is not None:
+                wrapped.metadata["trainable"].append(key)
+                wrapped.metadata["parameter_formats"][key] = "fp16"
+                ctx.add_bits(16 * signs.numel())
+        return wrapped
 
 
 def incoherent(inner: Callable[..., "Q | Tensor"], **options: Any) -> Incoherent:
