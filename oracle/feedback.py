@@ -15,7 +15,11 @@ Two places have no order fixed by the reference (its torch calls leave it to the
 the trailing block update (``addmm_``) and the triangular solve of the pending
 continuation.  This oracle fixes them -- fmaf over ascending k from zero, then one add;
 right-looking forward substitution -- and the HIP kernels follow the same orders.
-Against the reference's own torch backend these two orders are *parity unpinned*.
+Against the reference's own torch backend these two bit-level orders are *parity
+unpinned* (the reference asserts its own backends against each other at rtol 1e-5).
+Everything else of ``sweep`` -- including the region refits (pending continuation,
+targets, scale fit) -- is pinned by the float64 textbook loops of
+tests/test_oracle_feedback.py.
 
 The sequential pieces run in C (``csrc/gptq_ref.c``); ``round_tile_numpy`` is the same
 tile arithmetic in numpy and pins the C against a second implementation.

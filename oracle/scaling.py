@@ -16,9 +16,12 @@ Follows, in the reference:
   codecs/scaled.py:19-101                   decode_grouped / decode_scaled / decode_feedback
 
 ``search_scales`` fixes one summation order for the per-group squared error (stated in
-its docstring); the reference leaves that order to ``Tensor.sum`` / ``tl.sum``, so the
-exact candidate chosen on a near tie is *parity unpinned* against the reference and is
-only checked at the reference's own tolerance.
+its docstring); the reference leaves that order to ``Tensor.sum`` / ``tl.sum``.  The tests
+pin the candidate order, the storage rounding of candidates, the strict comparison and the
+"base scale wins ties" rule against a float64 brute force wherever the winner is clear (a
+gap above 1e-4 relative) and on an exact tie; only the candidate chosen when the two best
+errors lie within 1e-4 relative of each other is *parity unpinned* against the reference
+(its own two code paths may disagree there too).
 """
 
 import numpy as np
