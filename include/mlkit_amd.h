@@ -346,6 +346,35 @@ int mk_feedback_sweep(const float *original, float *feedback, float *output, uin
                       float reciprocal, float value_minimum, int scale_format, int deferred_tiles,
                       void *stream);
 
+/* Index of the nearest codeword for `count` vectors of `dimension` (2, 4, 8 or 16) fp32
+ * coordinates: the smallest sum over ascending coordinates of squared differences, the
+ * lowest index on ties.  codebook: [codebook_size, dimension] fp32.  With lattice != 0 the
+ * codebook is the E8P table (65,536 points of 8 coordinates followed by the 256 magnitude
+ * patterns that generate them) and the search is the structured one: per coset, every
+ * magnitude pattern scored against |v - shift|, a pattern whose sign parity disagrees with the
+ * input's paying for the flip of its cheapest coordinate; code = pattern * 128 + sign bits
+ * (+ 32768 for the -1/4 coset).  codes: [count] int32.
+ * Replaces: kernels/lattice_search.py:10-70 (nearest_lattice_code, nearest_lattice, search)
+ * and the device side of quantization/operations/search.py:34-79 (nearest). */
+int mk_vector_nearest(const float *vectors, long long count, int dimension, const float *codebook,
+                      int codebook_size, int lattice, int32_t *codes, void *stream);
+
+/* Columns [tile_start, tile_start + tile_width) of every row, rounded in blocks of
+ * `dimension` columns with LDL error feedback: target = weight + correction, code = the
+ * codeword nearest to target / scale (search as in mk_vector_nearest), reconstruction =
+ * codeword * scale, and the block's deviations times their coefficient rows (products
+ * rounded one by one, summed over ascending coordinate) added to the corrections of the
+ * tile's later columns.  original, feedback, output: [rows, width] fp32; coeff: [width,
+ * width]; scales: [rows, groups_per_row] fp32, group `(column - region_start) / group`;
+ * encoded: [rows, width / dimension] int32.  At most 256 columns per call; width, tile bounds
+ * and group multiples of `dimension`.
+ * Replaces: kernels/error_feedback.py:146-274 (round_vector_feedback_tile, round_vector_tile). */
+int mk_feedback_round_vector_tile(const float *original, const float *feedback, const float *coeff,
+                                  const float *scales, const float *codebook, float *output,
+                                  int32_t *encoded, int rows, int width, int region_start,
+                                  int tile_start, int tile_width, int group, int groups_per_row,
+                                  int dimension, int codebook_size, int lattice, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

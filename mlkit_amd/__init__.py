@@ -2,7 +2,7 @@
 
 The public names are the reference's (``import mlkit_amd as mk``): ``mk.scaled`` /
 ``mk.int`` / ``mk.nf4`` / ``mk.mxfp4``, ``mk.grid``, ``mk.codec``, ``mk.gptq`` / ``mk.ldlq``,
-``mk.pack`` / ``mk.unpack``, ``mk.hadamard`` / ``mk.rht``, ``mk.snap``, ``mk.proxy_loss``,
+``mk.pack`` / ``mk.unpack``, ``mk.hadamard`` / ``mk.rht``, ``mk.snap`` / ``mk.nearest``, ``mk.proxy_loss``,
 ``mk.PackedLinear``, ``mk.optimize``, ``mk.capabilities``, ``mk.Q`` / ``mk.Ctx`` /
 ``mk.Quantizer`` / ``mk.quantizer``, ``mk.save`` / ``mk.load_checkpoint``.  Every fused path
 runs a hand-written HIP kernel from ``libmlkit_amd.so`` (``python -m mlkit_amd.build``) and
@@ -22,7 +22,7 @@ from mlkit_amd.quantization.feedback import feedback_coefficients, gptq, ldlq, p
 from mlkit_amd.quantization.grids import NF4_VALUES, Grid, grid
 from mlkit_amd.quantization.incoherence import Incoherent, incoherent
 from mlkit_amd.quantization.scaled import Scaled, int, mxfp4, nf4, scaled, store_scale  # noqa: A004
-from mlkit_amd.quantization.search import snap
+from mlkit_amd.quantization.search import nearest, snap
 from mlkit_amd.quantization.transforms import hadamard, paley_matrix, rht, structured_transform, transform_factor
 
 __version__ = "0.1.0"
@@ -38,6 +38,6 @@ __all__ = [
     "Capabilities", "Ctx", "Grid", "Model", "NF4_VALUES", "PackedEmbedding", "PackedLinear", "Q", "QModel",
     "Quantizer", "Rotate", "Scaled", "capabilities", "codec", "concatenate_rows", "deterministic_signs",
     "feedback_coefficients", "gptq", "grid", "hadamard", "incoherent", "install_transform", "int", "layer_seed", "ldlq", "load_checkpoint", "mxfp4",
-    "nf4", "optimize", "pack", "packed_compatible", "paley_matrix", "proxy_loss", "quantize", "quantizer", "rht",
+    "nearest", "nf4", "optimize", "pack", "packed_compatible", "paley_matrix", "proxy_loss", "quantize", "quantizer", "rht",
     "rotate", "rtn", "save", "scaled", "snap", "store_scale", "structured_transform", "transform_factor", "unpack",
 ]

@@ -39,7 +39,7 @@ def translation_units() -> list[tuple[str, pathlib.Path, list[str]]]:
     for width in MATVEC_WIDTHS:
         units.append((f"packed_matvec_b{width}", CSRC / "packed_matvec_bits.hip",
                       [f"-DMK_MATVEC_BITS={width}"]))
-    exact = {"packed_decode", "scalar_codec", "error_feedback", "hadamard"}
+    exact = {"packed_decode", "scalar_codec", "error_feedback", "hadamard", "vector_feedback"}
     for source in sorted(CSRC.glob("*.hip")):
         if source.name == "packed_matvec_bits.hip":
             continue

@@ -181,3 +181,44 @@ def sweep(
         native.current_stream(device),
     ))
     return scales, zeros
+
+
+MAXIMUM_VECTOR_TILE_WIDTH = 256
+
+
+def round_vector_tile(
+    original: Tensor,
+    feedback: Tensor,
+    coefficients: Tensor,
+    scales: Tensor,
+    codebook: Tensor,
+    output: Tensor,
+    encoded: Tensor,
+    *,
+    region_start: int,
+    tile_start: int,
+    tile_width: int,
+    group: int,
+    dimension: int,
+    codebook_size: int,
+    lattice: bool,
+) -> None:
+    """Round columns ``tile_start`` to ``tile_start + tile_width`` of every row in blocks of
+    ``dimension`` columns (/root/reference/src/mlkit/kernels/error_feedback.py:241-274).
+    ``codebook`` holds the reconstruction of every code; for the lattice its 256 magnitude
+    patterns follow the ``codebook_size`` points."""
+    device = native.require_device(original, feedback, coefficients, scales, codebook, output, encoded)
+    rows, width = original.shape
+    _check("original", original)
+    _check("feedback", feedback, (rows, width))
+    _check("coefficients", coefficients, (width, width))
+    _check("output", output, (rows, width))
+    _check("scales", scales)
+    _check("codebook", codebook, (codebook_size + (256 if lattice else 0), dimension))
+    if encoded.dtype != torch.int32 or tuple(encoded.shape) != (rows, width // dimension) or not encoded.is_contiguous():
+        raise ValueError("encoded must be a contiguous int32 tensor with one code per block of columns")
+    native.check(native.library().mk_feedback_round_vector_tile(
+        original.data_ptr(), feedback.data_ptr(), coefficients.data_ptr(), scales.data_ptr(), codebook.data_ptr(),
+        output.data_ptr(), encoded.data_ptr(), rows, width, region_start, tile_start, tile_width, group,
+        scales.shape[1], dimension, codebook_size, int(lattice), native.current_stream(device),
+    ))

@@ -120,6 +120,13 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
         _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
         _c_int, _c_void_p,
     ]),
+    "mk_vector_nearest": (_c_int, [
+        _c_void_p, _c_longlong, _c_int, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
+    ]),
+    "mk_feedback_round_vector_tile": (_c_int, [
+        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+    ]),
 }
 
 _library: ctypes.CDLL | None = None

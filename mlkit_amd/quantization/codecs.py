@@ -3,6 +3,7 @@
 Mirrors, in /root/reference/src/mlkit/quantization/codecs:
   registry.py:1-46        codec, decoder, registered, row_parameters
   scaled.py:19-101        decode_grouped, decode_scaled ("scaled"), decode_feedback ("feedback")
+  scaled.py:104-128       decode_vector_scaled ("vector_scaled", "vector_feedback")
   composition.py:14-20    deterministic_signs
   composition.py:23-47    decode_basis ("basis")      composition.py:61-84   compose
   composition.py:87-116   concatenate_rows
@@ -108,6 +109,27 @@ def decode_feedback(codes: Tensor, *, scales: Tensor, values: Tensor, group: int
     return out if permutation is None else out[:, permutation.argsort()]
 
 
+@codec("vector_feedback", row_parameters=("scales", "zero"))
+@codec("vector_scaled", row_parameters=("scales", "zero"))
+def decode_vector_scaled(codes: Tensor, *, scales: Tensor, values: Tensor | None, group: int, dim: int,
+                         offset: int = 0, zero: Tensor | None = None, refit: int | None = None,
+                         permutation: Tensor | None = None) -> Tensor:
+    """One code per block of ``dim`` columns: the codeword (a row of ``values``, or the E8P
+    point of the code when ``values`` is None) laid out along the row, times the scale of each
+    column's group; groups restart at every ``refit`` columns."""
+    if values is None:
+        from mlkit_amd.quantization.lattice import device_points
+
+        values = device_points(codes.device)
+    width = codes.shape[1] * dim
+    columns = torch.arange(offset, offset + width, device=codes.device)
+    index = columns // group if refit is None else (columns // refit) * (-(-refit // group)) + (columns % refit) // group
+    out = values[codes.int()].reshape(codes.shape[0], width) * scales[:, index]
+    if zero is not None:
+        out = out + zero[:, index]
+    return out if permutation is None else out[:, permutation.argsort()]
+
+
 def deterministic_signs(width: int, seed: int, device: torch.device | str) -> Tensor:
     """Rademacher signs from an integer hash of ``index + seed``: identical on every device."""
     v = (torch.arange(width, device=device, dtype=torch.int64) + seed) & 0xFFFFFFFF
@@ -144,7 +166,7 @@ def compose(quantized: Q, name: str, parameters: dict[str, Any]) -> Q:
     metadata = dict(quantized.metadata)
     metadata["trainable"] = [f"inner_{key}" for key in metadata.get("trainable", [])]
     formats = dict(metadata.get("parameter_formats", {}))
-    if quantized.codec in {"scaled", "feedback"}:
+    if quantized.codec in {"scaled", "feedback", "vector_scaled", "vector_feedback"}:
         formats["scales"] = formats["zero"] = metadata.get("scale_fmt", "fp32")
     metadata["parameter_formats"] = {f"inner_{key}": value for key, value in formats.items()}
     metadata["parameter_bits"] = {f"inner_{key}": value for key, value in metadata.get("parameter_bits", {}).items()}

@@ -186,13 +186,31 @@ class ScalarRounding:
     metadata: dict[str, Any]
 
 
-class FittedRounder:
-    """``round(values, columns) -> Q`` for a fitted format, plus its scalar state if it has one."""
+@dataclasses.dataclass
+class VectorRounding:
+    """Fitted state of a scaled vector grid.  ``codebook`` holds the reconstruction of every
+    code; ``lattice`` marks the E8P table, in which the 256 magnitude patterns follow the
+    ``codebook_size`` points.  ``bits`` is the cost of the whole fitted region, scales included."""
 
-    def __init__(self, function: Callable[[Tensor, slice], Q], *, scalar: ScalarRounding | None = None) -> None:
+    grid: Any
+    scales: Tensor
+    group: int
+    codebook: Tensor
+    codebook_size: int
+    lattice: bool
+    bits: float
+    metadata: dict[str, Any]
+
+
+class FittedRounder:
+    """``round(values, columns) -> Q`` for a fitted format, plus the fitted state a rounding
+    kernel needs when the format is a scaled scalar or vector grid."""
+
+    def __init__(self, function: Callable[[Tensor, slice], Q], *, scalar: ScalarRounding | None = None,
+                 vector: VectorRounding | None = None) -> None:
         self.function = function
         self.scalar = scalar
-        self.vector = None
+        self.vector = vector
 
     @property
     def scalar_grid(self) -> Any:
@@ -207,10 +225,12 @@ class FittedRounder:
             result.metadata.update(metadata)
             return result
 
-        scalar = self.scalar
+        scalar, vector = self.scalar, self.vector
         if scalar is not None:
             scalar = dataclasses.replace(scalar, metadata={**scalar.metadata, **metadata})
-        return FittedRounder(tagged, scalar=scalar)
+        if vector is not None:
+            vector = dataclasses.replace(vector, metadata={**vector.metadata, **metadata})
+        return FittedRounder(tagged, scalar=scalar, vector=vector)
 
 
 class Quantizer:

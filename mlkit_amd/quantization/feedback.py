@@ -10,7 +10,9 @@ inverse.  Mirrors /root/reference/src/mlkit/quantization/algorithms/error_feedba
 On a HIP device, scalar grids with ``step == 1`` run entirely in kernels: per region one
 triangular solve (``mk_feedback_pending``), one scale fit, then per tile the column sweep
 (``mk_feedback_round_tile``) and the trailing update on the matrix cores
-(``mk_feedback_block_update``).  Other rounders take the block-by-block tensor path.
+(``mk_feedback_block_update``).  Vector grids (codebooks of 2-, 4-, 8- or 16-dimensional
+codewords, the E8P lattice) with ``step`` equal to their dimension run the same way with
+``mk_feedback_round_vector_tile``.  Other rounders take the block-by-block tensor path.
 """
 
 import math
@@ -20,14 +22,16 @@ from typing import Any
 import torch
 from torch import Tensor
 
-from mlkit_amd.quantization.codecs import decode_feedback
-from mlkit_amd.quantization.core import Ctx, FittedRounder, Q, Quantizer, ScalarRounding, as_q, fit_quantizer
+from mlkit_amd.quantization.codecs import decode_feedback, decode_vector_scaled
+from mlkit_amd.quantization.core import (Ctx, FittedRounder, Q, Quantizer, ScalarRounding, VectorRounding, as_q,
+                                         fit_quantizer)
 
 FUSED_CODEBOOK_LIMIT = 256
 FUSED_VECTOR_DIMENSIONS = {2, 4, 8, 16}
 FUSED_VECTOR_CODEBOOK_LIMIT = 65536
 UPPER_FACTORIZATION_WIDTH = 4096
 MAXIMUM_FUSED_TILE = 1024
+MAXIMUM_FUSED_VECTOR_TILE = 256
 DEFERRED_TILES = 4  # tiles whose far-column updates are applied in one pass on the device
 
 
@@ -209,18 +213,31 @@ class _Collected:
         self.count(scalar.bits)
         return self.codes
 
+    def open_vector_region(self, vector: VectorRounding) -> Tensor:
+        dimension = vector.grid.dim
+        if self.codes is None:
+            self.codes = torch.empty((self.rows, self.width // dimension), dtype=torch.int32, device=self.device)
+            self.shared = {"values": None if vector.lattice else vector.codebook, "group": vector.group,
+                           "dim": dimension}
+            self.metadata = vector.metadata
+        self.scales.append(vector.scales)
+        self.count(vector.bits)
+        return self.codes
+
     def add_block(self, quantized: Q, column: int, stop: int, region_start: int) -> None:
         self.count(quantized.bits)
         if not self.portable:
             return
-        if quantized.codec != "scaled" or quantized.codes is None:
+        if quantized.codec not in {"scaled", "vector_scaled"} or quantized.codes is None:
             self.portable = False
             return
+        dimension = quantized.params.get("dim", 1)
         if self.codes is None:
-            self.codes = torch.empty((self.rows, self.width), dtype=quantized.codes.dtype, device=self.device)
+            self.codes = torch.empty((self.rows, self.width // dimension), dtype=quantized.codes.dtype,
+                                     device=self.device)
             self.shared = quantized.params
             self.metadata = quantized.metadata
-        self.codes[:, column:stop] = quantized.codes
+        self.codes[:, column // dimension:stop // dimension] = quantized.codes
         if column == region_start:
             self.scales.append(quantized.params["scales"])
             if quantized.params["zero"] is not None:
@@ -233,6 +250,11 @@ class _Collected:
             params = {"scales": torch.cat(self.scales, dim=1), "values": self.shared["values"],
                       "group": self.shared["group"], "refit": refit_width,
                       "zero": torch.cat(self.zeros, dim=1) if self.zeros else None, "permutation": permutation}
+            dimension = self.shared.get("dim")
+            if dimension is not None:
+                params["dim"] = dimension
+                return Q(codes=self.codes, bits=self.bits, codec="vector_feedback", decode=decode_vector_scaled,
+                         params=params, metadata=self.metadata)
             return Q(codes=self.codes, bits=self.bits, codec="feedback", decode=decode_feedback, params=params,
                      metadata=self.metadata)
         if permutation is not None:
@@ -266,16 +288,23 @@ class ErrorFeedback(Quantizer):
 
     # -- pieces --------------------------------------------------------------------------
 
-    def _kernel_state(self, rounder: Callable[[Tensor, slice], Q], device: torch.device) -> ScalarRounding | None:
-        """The fitted scalar state when the HIP kernels can round this region."""
-        scalar = rounder.scalar if isinstance(rounder, FittedRounder) else None
-        usable = (scalar is not None and device.type == "cuda" and self.backend != "torch" and self.step == 1
-                  and scalar.grid.bits <= 8 and 1 <= scalar.values.numel() <= FUSED_CODEBOOK_LIMIT
-                  and self.block_size <= MAXIMUM_FUSED_TILE)
-        if usable:
+    def _kernel_state(self, rounder: Callable[[Tensor, slice], Q],
+                      device: torch.device) -> ScalarRounding | VectorRounding | None:
+        """The fitted state when the HIP kernels can round this region: scalar grids go column
+        by column, vector grids in blocks, which needs a step equal to the grid's dimension."""
+        fitted = rounder if isinstance(rounder, FittedRounder) and device.type == "cuda" and self.backend != "torch" else None
+        scalar = None if fitted is None else fitted.scalar
+        if (scalar is not None and self.step == 1 and scalar.grid.bits <= 8
+                and 1 <= scalar.values.numel() <= FUSED_CODEBOOK_LIMIT and self.block_size <= MAXIMUM_FUSED_TILE):
             return scalar
+        vector = None if fitted is None else fitted.vector
+        if (vector is not None and self.step == vector.grid.dim and vector.grid.dim in FUSED_VECTOR_DIMENSIONS
+                and vector.codebook_size <= FUSED_VECTOR_CODEBOOK_LIMIT and vector.scales.dtype == torch.float32
+                and self.block_size <= MAXIMUM_FUSED_VECTOR_TILE):
+            return vector
         if self.backend == "hip":
-            raise ValueError("fused error feedback requires a HIP device and a native scalar rounder with step=1")
+            raise ValueError("fused error feedback requires a HIP device and a native scalar rounder with step=1, "
+                             "or a native vector rounder with step equal to its dimension")
         return None
 
     def _whole_sweep(self, original: Tensor, feedback: Tensor, output: Tensor, coefficients: Tensor,
@@ -419,8 +448,14 @@ class ErrorFeedback(Quantizer):
             del targets
             if fitted_ctx is not ctx:
                 ctx.add_bits(fitted_ctx.additional_bits)
-            scalar = self._kernel_state(rounder, w.device)
-            encoded = None if scalar is None else collected.open_scalar_region(scalar)
+            state = self._kernel_state(rounder, w.device)
+            scalar = state if isinstance(state, ScalarRounding) else None
+            vector = state if isinstance(state, VectorRounding) else None
+            encoded = None
+            if scalar is not None:
+                encoded = collected.open_scalar_region(scalar)
+            elif vector is not None:
+                encoded = collected.open_vector_region(vector)
             for tile_start in range(region_start, region_stop, self.block_size):
                 tile_stop = min(region_stop, tile_start + self.block_size)
                 if scalar is not None:
@@ -429,6 +464,12 @@ class ErrorFeedback(Quantizer):
                                       region_start=region_start, tile_start=tile_start,
                                       tile_width=tile_stop - tile_start, group=scalar.group, bits=scalar.grid.bits,
                                       values=scalar.values, integer_grid=scalar.grid.integer)
+                elif vector is not None:
+                    kernel.round_vector_tile(original, feedback, coefficients, vector.scales.contiguous(),
+                                             vector.codebook, output, encoded, region_start=region_start,
+                                             tile_start=tile_start, tile_width=tile_stop - tile_start,
+                                             group=vector.group, dimension=vector.grid.dim,
+                                             codebook_size=vector.codebook_size, lattice=vector.lattice)
                 else:
                     self._round_tile_by_blocks(rounder, original, feedback, coefficients, output, collected,
                                                region_start, tile_start, tile_stop)

@@ -1,9 +1,10 @@
-"""Scalar grids: signed integers, explicit value tables and small floating-point formats.
+"""Grids: signed integers, explicit value tables, small floating-point formats, codebooks of
+vectors and the E8P lattice.
 
-Mirrors the scalar part of the reference's grid factory
-(/root/reference/src/mlkit/quantization/grids/factory.py:17-122,146-152): ``Grid``,
-``grid.int``, ``grid.values``, ``grid.fp`` and ``NF4_VALUES``.  Vector, lattice and trellis
-grids are outside this package's path.
+Mirrors the reference's grid factory
+(/root/reference/src/mlkit/quantization/grids/factory.py:17-125,146-152): ``Grid``,
+``grid.int``, ``grid.values``, ``grid.vector``, ``grid.fp``, ``grid.e8p`` and ``NF4_VALUES``.
+Trellis grids are outside this package's path.
 """
 
 import builtins
@@ -63,6 +64,29 @@ class GridFactory:
         if table.numel() > 2**width:
             raise ValueError("codebook size exceeds the declared bit capacity")
         return Grid(lambda x: _snap(x, table), width, values=table, name=name)
+
+    def vector(self, codebook: Tensor, *, bits: builtins.int | None = None) -> Grid:
+        """Round blocks of ``codebook.shape[1]`` values to the nearest row of ``codebook``."""
+        table = torch.as_tensor(codebook, dtype=torch.float32)
+        if table.ndim != 2 or min(table.shape) < 1 or not bool(torch.isfinite(table).all()):
+            raise ValueError("a vector codebook must be a nonempty finite matrix")
+        width = max(1, math.ceil(math.log2(table.shape[0]))) if bits is None else bits
+        if table.shape[0] > 2**width:
+            raise ValueError("codebook size exceeds the declared bit capacity")
+        dimension = table.shape[1]
+
+        def round_vectors(value: Tensor) -> Tensor:
+            from mlkit_amd.quantization.search import nearest
+
+            return nearest(value.reshape(-1, dimension), table).reshape_as(value)
+
+        return Grid(round_vectors, width, dimension, values=table, name="vector")
+
+    def e8p(self) -> Grid:
+        """The 16-bit, eight-dimensional E8P lattice codebook."""
+        from mlkit_amd.quantization.lattice import e8p_points, nearest_e8p
+
+        return Grid(nearest_e8p, 16, 8, values=e8p_points(), name="e8p")
 
     def fp(self, format: str) -> Grid:
         """Sign-magnitude minifloats without infinities or NaNs: e2m1, e3m2, e2m3, e4m3, e5m2."""

@@ -1,4 +1,5 @@
-"""Grouped scaling of scalar grids: ``scaled``, ``int``, ``nf4``, ``mxfp4`` and ``store_scale``.
+"""Grouped scaling of scalar and vector grids: ``scaled``, ``int``, ``nf4``, ``mxfp4`` and
+``store_scale``.
 
 Mirrors, in /root/reference/src/mlkit/quantization/formats:
   scale_storage.py:11-26        SCALE_FORMAT_BITS, store_scale
@@ -7,7 +8,8 @@ Mirrors, in /root/reference/src/mlkit/quantization/formats:
   standard.py:10-23             int, nf4, mxfp4
 Weights on a HIP device are fitted, searched and encoded by the kernels of
 ``mlkit_amd.kernels.scalar_encode`` (one launch each); host tensors go through the same
-arithmetic in tensor operations.  Vector grids are outside this package's path.
+arithmetic in tensor operations.  Vector grids (``grid.vector``, ``grid.e8p``) take their
+scales from the same fit kernel and their codes from ``mk_vector_nearest``.
 """
 
 import builtins
@@ -18,10 +20,10 @@ import torch
 import torch.nn.functional as functional
 from torch import Tensor
 
-from mlkit_amd.quantization.codecs import decode_scaled
-from mlkit_amd.quantization.core import Ctx, FittedRounder, Q, Quantizer, ScalarRounding
+from mlkit_amd.quantization.codecs import decode_scaled, decode_vector_scaled
+from mlkit_amd.quantization.core import Ctx, FittedRounder, Q, Quantizer, ScalarRounding, VectorRounding
 from mlkit_amd.quantization.grids import NF4_VALUES, Grid, grid
-from mlkit_amd.quantization.search import nearest_indices
+from mlkit_amd.quantization.search import nearest, nearest_indices
 
 SCALE_FORMAT_BITS = {"fp32": 32, "fp16": 16, "bf16": 16, "fp8": 8, "e8m0": 8}
 FUSED_CODEBOOK_LIMIT = 256
@@ -88,7 +90,8 @@ def nearest_codes(normalized: Tensor, values: Tensor) -> Tensor:
 
 
 class Scaled(Quantizer):
-    """A scalar grid applied to row groups that each carry a scale and, optionally, an offset."""
+    """A grid applied to row groups that each carry a scale and, for scalar grids, optionally
+    an offset."""
 
     row_separable = True
 
@@ -101,22 +104,21 @@ class Scaled(Quantizer):
             raise ValueError("scale must be absmax, mse, or callable")
         if search_steps < 1:
             raise ValueError("search_steps must be positive")
-        if grid.dim != 1:
-            raise ValueError("mlkit_amd implements scalar grids only (grid.dim must be 1)")
-        if asym and grid.values is None:
+        if asym and (grid.dim != 1 or grid.values is None):
             raise ValueError("asymmetric quantization requires an explicit scalar grid")
         if asym and (scale_fmt == "e8m0" or isinstance(scale_fmt, Grid)):
             raise ValueError("asymmetric offsets require a signed floating-point storage format")
         self.grid, self.group, self.scale, self.scale_fmt = grid, group, scale, scale_fmt
         self.asym, self.search_steps = asym, search_steps
         self._on_device: dict[torch.device, Tensor] = {}
-        table = None if grid.values is None else grid.values.detach().cpu()
+        table = None if grid.values is None or grid.dim != 1 else grid.values.detach().cpu()
         self._value_minimum = 0.0 if table is None else float(table.min())
         self._value_maximum = 0.0 if table is None else float(table.max())
         span = self._value_maximum - self._value_minimum
         if asym and span <= 0:
             raise ValueError("asymmetric quantization requires at least two distinct grid values")
-        self._magnitude_reciprocal = single_precision_reciprocal(1.0 if table is None else float(table.abs().max()))
+        self._magnitude_reciprocal = single_precision_reciprocal(
+            1.0 if grid.values is None else float(grid.values.abs().max()))
         self._range_reciprocal = single_precision_reciprocal(span) if asym else 1.0
 
     # -- description ---------------------------------------------------------------------
@@ -131,7 +133,8 @@ class Scaled(Quantizer):
     def reconstruct_activations(self, value: Tensor) -> Tensor:
         """Quantize-dequantize a two-dimensional activation tensor online (no codec state kept):
         one fused kernel on a HIP device, the rounder itself otherwise."""
-        fused = (value.is_cuda and value.dim() == 2 and value.dtype in (torch.float32, torch.float16, torch.bfloat16) and self.grid.values is not None and self.scale == "absmax"
+        fused = (value.is_cuda and value.dim() == 2 and value.dtype in (torch.float32, torch.float16, torch.bfloat16)
+                 and self.grid.dim == 1 and self.grid.values is not None and self.scale == "absmax"
                  and isinstance(self.scale_fmt, str) and self.scale_fmt in SCALE_FORMAT_BITS
                  and self.grid.values.numel() <= FUSED_CODEBOOK_LIMIT and self.grid.bits <= 8)
         if not fused:
@@ -161,9 +164,13 @@ class Scaled(Quantizer):
     # -- fitting -------------------------------------------------------------------------
 
     def _kernel_path(self, weight: Tensor, table: Tensor | None) -> bool:
-        """Whether the scales of ``weight`` can come from the fit / search kernels."""
-        return (weight.is_cuda and table is not None and table.numel() <= FUSED_CODEBOOK_LIMIT
-                and isinstance(self.scale_fmt, str) and not callable(self.scale))
+        """Whether the scales of ``weight`` can come from the fit / search kernels: scalar tables
+        of up to 256 values, and vector grids whose scales follow the range (no search)."""
+        if not (weight.is_cuda and isinstance(self.scale_fmt, str) and not callable(self.scale)):
+            return False
+        if self.grid.dim > 1:
+            return self.grid.values is not None and self.scale == "absmax"
+        return table is not None and table.numel() <= FUSED_CODEBOOK_LIMIT
 
     def _initial_scales(self, weight: Tensor, group: int) -> tuple[Tensor, Tensor | None]:
         rows, width = weight.shape
@@ -187,7 +194,12 @@ class Scaled(Quantizer):
         centered = blocks if zero is None else blocks - zero[..., None]
 
         def error_of(candidate: Tensor) -> Tensor:
-            rounded = self.grid(centered / candidate[..., None])
+            normalized = centered / candidate[..., None]
+            if self.grid.dim > 1:
+                blocks_of = normalized.reshape(*normalized.shape[:-1], -1, self.grid.dim)
+                rounded = self.grid(blocks_of).reshape_as(centered)
+            else:
+                rounded = self.grid(normalized)
             return ((rounded * candidate[..., None] - centered).square() * occupied).sum(-1)
 
         chosen, best = scales.clone(), error_of(scales)
@@ -203,13 +215,22 @@ class Scaled(Quantizer):
             raise ValueError("scaled requires a finite floating-point weight matrix")
         rows, width = w.shape
         group = width if self.group is None else min(self.group, width)
+        dimension, codebook = self.grid.dim, self.grid.values
+        if group % dimension:
+            raise ValueError("group width must be divisible by the vector grid dimension")
+        lattice = self.grid.name == "e8p"
+        if dimension > 1 and codebook is not None and not lattice:
+            counted = ctx.cache.setdefault("_mlkit_vector_codebooks", set())
+            if id(self.grid) not in counted:  # the codebook is side information, paid for once
+                ctx.add_bits(codebook.numel() * codebook.element_size() * 8)
+                counted.add(id(self.grid))
         weight = w.float()
-        table = None if self.grid.values is None else self.values_on(w.device)
+        table = None if codebook is None or dimension != 1 else self.values_on(w.device)
         on_kernels = self._kernel_path(weight, table)
         if on_kernels:
             from mlkit_amd.kernels import scalar_encode
 
-            assert isinstance(self.scale_fmt, str) and table is not None
+            assert isinstance(self.scale_fmt, str)
             weight = weight.contiguous()
             searching = self.scale == "mse"
             scales, zero = scalar_encode.fit_scales(
@@ -220,6 +241,7 @@ class Scaled(Quantizer):
                 raise ValueError("scaled requires a finite floating-point weight matrix")
             scale_bits = SCALE_FORMAT_BITS[self.scale_fmt]
             if searching:
+                assert table is not None
                 fractions = torch.linspace(0.5, 1.0, self.search_steps, device=w.device)
                 scales = scalar_encode.search_scales(
                     weight, scales, zero, table, fractions, group, None, self.scale_fmt,
@@ -241,11 +263,22 @@ class Scaled(Quantizer):
             scalar = ScalarRounding(grid=self.grid, scales=scales, zero=zero, group=group, values=table,
                                     bits=self.grid.bits * w.numel() + side_bits, metadata=metadata)
 
+        vector = None
+        vector_metadata = {"code_bits": self.grid.bits, "scale_fmt": self.scale_fmt, "trainable": ["scales"]}
+        if dimension > 1 and codebook is not None and w.is_cuda:
+            from mlkit_amd.quantization.lattice import device_table
+
+            vector = VectorRounding(grid=self.grid, scales=scales, group=group,
+                                    codebook=device_table(w.device) if lattice else self.values_on(w.device),
+                                    codebook_size=codebook.shape[0], lattice=lattice,
+                                    bits=self.grid.bits * w.numel() / dimension + side_bits,
+                                    metadata=vector_metadata)
+
         def round_columns(value: Tensor, columns: slice) -> Q:
             start, stop, stride = columns.indices(width)
             if stride != 1 or stop - start != value.shape[1]:
                 raise ValueError("rounder columns must describe a contiguous slice of its fitted region")
-            bits = self.grid.bits * value.numel() + side_bits * value.shape[1] / width
+            bits = self.grid.bits * value.numel() / dimension + side_bits * value.shape[1] / width
             if scalar is not None:
                 codes = self._scalar_codes(value, scalar, start, stop)
                 return Q(bits=bits, codes=codes, decode=decode_scaled, codec="scaled", metadata=scalar.metadata,
@@ -253,10 +286,29 @@ class Scaled(Quantizer):
                                  "zero": zero})
             index = torch.arange(start, stop, device=value.device) // group
             centered = value.float() if zero is None else value.float() - zero[:, index]
-            restored = self.grid(centered / scales[:, index]) * scales[:, index]
+            normalized = centered / scales[:, index]
+            if dimension == 1:
+                rounded = self.grid(normalized)
+            else:
+                if value.shape[1] % dimension:
+                    raise ValueError("column slices must align to the vector grid dimension")
+                blocks = normalized.reshape(-1, dimension)
+                if codebook is not None:
+                    if lattice:
+                        from mlkit_amd.quantization.lattice import nearest_e8p
+
+                        codes = nearest_e8p(blocks, return_indices=True)
+                    else:
+                        codes = nearest(blocks, codebook, return_indices=True)
+                    return Q(codes=codes.reshape(value.shape[0], -1).to(torch.int32), bits=bits,
+                             decode=decode_vector_scaled, codec="vector_scaled", metadata=vector_metadata,
+                             params={"scales": scales, "values": None if lattice else codebook.to(value.device),
+                                     "dim": dimension, "group": group, "offset": start, "zero": zero})
+                rounded = self.grid(blocks).reshape_as(value)
+            restored = rounded * scales[:, index]
             return Q(restored if zero is None else restored + zero[:, index], bits=bits)
 
-        return FittedRounder(round_columns, scalar=scalar)
+        return FittedRounder(round_columns, scalar=scalar, vector=vector)
 
     def _scalar_codes(self, value: Tensor, scalar: ScalarRounding, start: int, stop: int) -> Tensor:
         """Codes of the nearest grid values for columns ``start`` to ``stop`` of the fitted region."""
