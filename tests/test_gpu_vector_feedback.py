@@ -74,7 +74,7 @@ def test_lattice_table_on_device_is_the_oracle_point_set():
 
 
 @pytest.mark.parametrize("entries,dimension,count", [(256, 8, 5000), (600, 4, 5000), (37, 2, 3000), (1000, 16, 2000),
-                                                      (65536, 8, 96), (1, 4, 10)])
+                                                      (65536, 8, 96), (1, 4, 40)])
 def test_codebook_search_matches_oracle_codes(entries, dimension, count):
     from mlkit_amd.kernels import lattice_search
 
