@@ -320,6 +320,85 @@ def gptq_layer(device: torch.device, generator: torch.Generator, cpu_rows: int =
     return out
 
 
+def vector_ldlq_layer(device: torch.device, generator: torch.Generator, cpu_rows: int = 0) -> dict:
+    """LDLQ with vector grids at the shapes of the reference's own benchmark cases
+    (benchmarks/results: "algorithms/ldlq-e8p-step8/llama-attention-2048x2048",
+    "ldlq-vector8-256-step8", "kernels/lattice_search/e8p-2m-vectors", "operations/nearest/..."):
+    the E8P lattice and a 256-codeword 8-dimensional codebook, step 8, one region, one scale per
+    row.  With `cpu_rows` the CPU restatement sweeps that many rows with the device's
+    coefficient matrix and its codes are compared with the device's."""
+    import mlkit_amd as mk
+    from mlkit_amd.kernels import lattice_search
+    from mlkit_amd.quantization import feedback
+    from mlkit_amd.quantization.core import Ctx
+    from mlkit_amd.quantization.lattice import device_table
+
+    rows = width = 2048
+    target = (torch.randn((rows, width), device=device, generator=generator) * 0.02).half().float()
+    inputs = torch.randn((8192, width), device=device, generator=generator)
+    hessian = inputs.T @ inputs / inputs.shape[0]
+    del inputs
+    codebook = torch.randn((256, 8), device=device, generator=generator)
+
+    def wall_ms(function, repeats=5):
+        times = []
+        for _ in range(repeats):
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            function()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - started) * 1e3)
+        return sorted(times)[len(times) // 2]
+
+    out = {}
+    vectors = torch.randn((2_000_000, 8), device=device, generator=generator)
+    table = device_table(device)
+    ms = _time(lambda: lattice_search.search(vectors, table), repeats=10)
+    out["e8p search 2M vectors"] = {"ms": ms, "vectors_per_s": vectors.shape[0] / ms * 1e3}
+    ms = _time(lambda: lattice_search.nearest(vectors[:1_000_000], codebook), repeats=10)
+    out["nearest 1M vectors x 256 codewords"] = {"ms": ms, "vectors_per_s": 1e6 / ms * 1e3}
+    large = torch.randn((65536, 8), device=device, generator=generator)
+    ms = _time(lambda: lattice_search.nearest(vectors[:65536], large), repeats=5)
+    out["nearest 65k vectors x 65k codewords"] = {"ms": ms, "vectors_per_s": 65536 / ms * 1e3}
+    del vectors
+    ready = mk.feedback_coefficients(hessian.clone(), 8)
+    out["coefficients_ms"] = wall_ms(lambda: mk.feedback_coefficients(hessian.clone(), 8))
+    for label, inner, lattice in (("e8p", mk.scaled(mk.grid.e8p(), group=None), True),
+                                  ("vector8-256", mk.scaled(mk.grid.vector(codebook.cpu()), group=None), False)):
+        quantizer = mk.ldlq(inner, step=8, backend="hip")
+        result = quantizer(target, Ctx("warmup", H=hessian))
+        total_ms = wall_ms(lambda: quantizer(target, Ctx("attention", H=hessian)))
+        original = feedback.feedback_coefficients
+        feedback.feedback_coefficients = lambda *args, **kwargs: ready
+        try:
+            sweep_ms = wall_ms(lambda: quantizer(target, Ctx("attention", H=hessian)))
+        finally:
+            feedback.feedback_coefficients = original
+        direct = inner(target, Ctx("attention", H=hessian))
+        entry = {"total_ms": total_ms, "sweep_and_update_ms": sweep_ms, "weights_per_s": rows * width / (sweep_ms / 1e3),
+                 "proxy_loss": float(mk.proxy_loss(target, result.w, hessian)),
+                 "direct_rounding_proxy_loss": float(mk.proxy_loss(target, direct.w, hessian))}
+        if cpu_rows:
+            from oracle import lattice as oracle_lattice
+
+            picked = torch.linspace(0, rows - 1, cpu_rows, device=device).long()
+            points = oracle_lattice.e8p_points() if lattice else codebook.cpu().numpy()
+            host_coefficients, host_weight = ready[0].cpu().numpy(), target[picked].cpu().numpy()
+            started = time.perf_counter()
+            expected = oracle_lattice.vector_sweep(host_weight, host_coefficients, points, group=width, dimension=8,
+                                                   lattice=lattice, refit=None, block=128)
+            seconds = time.perf_counter() - started
+            entry["cpu_baseline"] = {
+                "value": cpu_rows * width / seconds, "unit": "weights/s", "cores": 1, "kind": "port",
+                "sample": f"{cpu_rows} rows spread over the layer, all {width} columns, the numpy restatement of the "
+                          f"sweep with the device's coefficient matrix: {seconds:.1f} s",
+                "code_mismatches_vs_device": int((result.codes[picked].cpu().numpy() != expected["codes"]).sum()),
+                "codes_compared": cpu_rows * width // 8,
+            }
+        out[f"ldlq {label} step 8, {rows}x{width}"] = entry
+    return out
+
+
 def rotated_layer(device: torch.device, generator: torch.Generator, values: torch.Tensor) -> dict:
     """Config 5: the rotated INT4-g128 layers at M = 1 and 8.  One step = the online rotation of
     the activations plus the packed matvec, enqueued by one mk_rotated_packed_matvec call; the
@@ -490,6 +569,8 @@ def main() -> None:
     parser.add_argument("--kernels", action="store_true", help="add the decoder-layer shapes, the tied head and wider codecs")
     parser.add_argument("--profile-gptq", action="store_true",
                         help="for rocprofv3: only run the GPTQ layer (4096 x 11008) and print its timings")
+    parser.add_argument("--profile-vector", action="store_true",
+                        help="for rocprofv3: only run the vector-grid searches and LDLQ layers (2048 x 2048) and print their record")
     parser.add_argument("--profile-launches", type=int, default=0,
                         help="for rocprofv3: only issue this many eager calls (grouped with --members > 1), plus three "
                              "256 MiB device copies whose counters calibrate FETCH_SIZE / WRITE_SIZE")
@@ -514,6 +595,9 @@ def main() -> None:
 
     if options.profile_gptq:
         print(json.dumps(gptq_layer(device, generator)))
+        return
+    if options.profile_vector:
+        print(json.dumps(vector_ldlq_layer(device, generator)))
         return
     if options.profile_launches:
         x = torch.randn((options.profile_rows, WIDTH), device=device, generator=generator).half()
@@ -607,6 +691,7 @@ def main() -> None:
         torch.cuda.empty_cache()
         kernels = other_kernels(device, options.kernels)
         kernels["gptq int4 g128 4096x11008"] = gptq_layer(device, generator, cpu_rows=0 if options.no_cpu_baseline else 32)
+        kernels["vector grids"] = vector_ldlq_layer(device, generator, cpu_rows=0 if options.no_cpu_baseline else 16)
         if not options.no_cpu_baseline:
             kernels["fwht_cpu_baseline"] = cpu_fwht_baseline()
         line["kernels"] = kernels
