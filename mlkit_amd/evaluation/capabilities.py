@@ -18,7 +18,7 @@ from mlkit_amd.inference.packed_linear import packed_compatible
 from mlkit_amd.kernels.packed_linear import layout_for
 from mlkit_amd.quantization.codecs import registered
 from mlkit_amd.quantization.core import Ctx, FittedRounder, FunctionQuantizer, Q, Quantizer, as_q
-from mlkit_amd.quantization.feedback import FUSED_CODEBOOK_LIMIT
+from mlkit_amd.quantization.feedback import FUSED_CODEBOOK_LIMIT, FUSED_VECTOR_CODEBOOK_LIMIT, FUSED_VECTOR_DIMENSIONS
 from mlkit_amd.quantization.scaled import SCALE_FORMAT_BITS, Scaled
 
 FUSED = "fused kernel"
@@ -48,11 +48,11 @@ class Capabilities:
         return "\n".join(f"{label:<{width}}  {text}" for label, text in rows)
 
 
-def _fitted_scalar(quantization: Quantizer, weight: Tensor):
-    """The scalar rounding state the quantizer fits on ``weight`` (None when it fits none)."""
+def _fitted_state(quantization: Quantizer, weight: Tensor):
+    """The scalar and vector rounding states the quantizer fits on ``weight`` (None where it fits none)."""
     with torch.no_grad():
         fitted = quantization.fit(weight, Ctx("capabilities", X=weight.new_zeros((1, weight.shape[1]))))
-    return fitted.scalar if isinstance(fitted, FittedRounder) else None
+    return (fitted.scalar, fitted.vector) if isinstance(fitted, FittedRounder) else (None, None)
 
 
 def error_feedback_path(quantization: Any, weight: Tensor) -> str:
@@ -61,9 +61,13 @@ def error_feedback_path(quantization: Any, weight: Tensor) -> str:
         return "reference rounding; the function is called on every column block"
     if type(quantization).fit is Quantizer.fit:
         return "not an inner format; it does not implement Quantizer.fit"
-    scalar = _fitted_scalar(quantization, weight)
-    kernel_ready = scalar is not None and scalar.grid.bits <= 8 and scalar.values.numel() <= FUSED_CODEBOOK_LIMIT
-    return "fused scalar kernel at step=1" if kernel_ready else "reference rounding with the fitted rounder"
+    scalar, vector = _fitted_state(quantization, weight)
+    if scalar is not None and scalar.grid.bits <= 8 and scalar.values.numel() <= FUSED_CODEBOOK_LIMIT:
+        return "fused scalar kernel at step=1"
+    if (vector is not None and vector.grid.dim in FUSED_VECTOR_DIMENSIONS
+            and vector.codebook_size <= FUSED_VECTOR_CODEBOOK_LIMIT):
+        return f"fused vector kernel at step={vector.grid.dim}"
+    return "reference rounding with the fitted rounder"
 
 
 def packed_inference_path(result: Q, input_width: int) -> str:

@@ -483,6 +483,13 @@ def test_capabilities_on_device():
     assert report.packed_inference == "fused kernel" and report.online_activations == "fused kernel"
     assert mk.capabilities(mk.gptq(mk.int(4))).packed_inference == "fused kernel"
     assert mk.capabilities(mk.int(3, group=50), shape=(16, 250)).packed_inference.startswith("packed storage with dense")
+    # vector grids (/root/reference/tests/evaluation/test_capability_report.py:47-72)
+    lattice = mk.capabilities(mk.scaled(mk.grid.e8p(), group=None))
+    assert lattice.error_feedback == "fused vector kernel at step=8" and lattice.packed_inference == "no; dense weights"
+    assert lattice.codec == "vector_scaled" and lattice.bits_per_weight == pytest.approx(2 + 16 / 256)
+    quadruples = mk.capabilities(mk.scaled(mk.grid.vector(torch.randn(600, 4)), group=16))
+    assert quadruples.error_feedback == "fused vector kernel at step=4"
+    assert mk.capabilities(mk.int(12)).error_feedback == "reference rounding with the fitted rounder"
 
 
 @pytest.mark.parametrize("rows,width", [(70, 1000), (256, 1024)])

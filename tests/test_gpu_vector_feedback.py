@@ -306,3 +306,37 @@ def test_scaled_vector_grid_on_device_matches_oracle_round_to_nearest():
             host(result.w), oracle_lattice.decode_vector_scaled(expected.reshape(rows, -1), scales, codebook, group, 8))
         assert result.params["values"] is None if lattice else result.params["values"].shape == (300, 8)
         assert context.additional_bits == (0 if lattice else 300 * 8 * 32)
+
+
+def test_vector_codecs_survive_a_checkpoint_and_stay_dense_under_optimize(tmp_path):
+    from torch import nn
+
+    torch.manual_seed(44)
+
+    def build():
+        return nn.Sequential(nn.Linear(64, 48), nn.ReLU(), nn.Linear(48, 16, bias=False))
+
+    codebook = torch.randn(64, 4)
+    for fmt, values_kept in ((mk.scaled(mk.grid.e8p(), group=32), False), (mk.scaled(mk.grid.vector(codebook), group=16), True)):
+        converted = mk.quantize(build(), fmt, calib=None)
+        assert converted.quantized["0"].codec == "vector_scaled"
+        inputs = torch.randn(4, 64)
+        expected = converted(inputs)
+        target = tmp_path / ("codebook" if values_kept else "lattice")
+        mk.save(converted, target)
+        restored = mk.load_checkpoint(target, model=build)
+        torch.testing.assert_close(restored(inputs), expected, rtol=0, atol=0)
+        entry = restored.quantized["0"]
+        # codes come back in the narrowest integer type that holds `code_bits`
+        assert entry.codec == "vector_scaled" and not entry.codes.is_floating_point() and entry.params["dim"] in (4, 8)
+        assert (entry.params["values"] is not None) == values_kept
+        assert entry.bits == converted.quantized["0"].bits
+        # vector codes have no packed kernel: the optimizer keeps such layers dense
+        packed = mk.optimize(restored)
+        assert packed.execution_backend == "packed:0"
+        with torch.inference_mode():
+            torch.testing.assert_close(packed(inputs), expected, rtol=1e-4, atol=1e-5)
+    # calibrated LDLQ over the lattice through the same driver
+    calibrated_model = mk.quantize(build(), mk.ldlq(mk.scaled(mk.grid.e8p(), group=None), step=8),
+                                   calib=[torch.randn(32, 64) for _ in range(4)])
+    assert calibrated_model.quantized["0"].codec == "vector_feedback"

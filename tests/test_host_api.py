@@ -333,3 +333,64 @@ def test_incoherent_identity_and_basis_codec(shape):
     assert torch.isfinite(with_feedback.w).all()
     with pytest.raises(ValueError, match="rht or None"):
         mk.incoherent(mk.int(4), left="dct")
+
+
+# ---- vector grids on host tensors -------------------------------------------------------------------
+
+
+def test_vector_grid_validation_and_nearest_on_the_host(rng):
+    from oracle import lattice as oracle_lattice
+
+    with pytest.raises(ValueError, match="nonempty finite matrix"):
+        mk.grid.vector(torch.zeros(0, 4))
+    with pytest.raises(ValueError, match="exceeds the declared bit capacity"):
+        mk.grid.vector(torch.randn(20, 4), bits=4)
+    grid = mk.grid.vector(torch.randn(20, 4))
+    assert (grid.bits, grid.dim, grid.name) == (5, 4, "vector")
+    lattice = mk.grid.e8p()
+    assert (lattice.bits, lattice.dim, lattice.name) == (16, 8, "e8p") and lattice.values.shape == (65536, 8)
+    codebook = rng.standard_normal((300, 8)).astype(np.float32)
+    codebook[200] = codebook[7]
+    samples = rng.standard_normal((500, 8)).astype(np.float32)
+    samples[0] = codebook[7]
+    found = mk.nearest(torch.from_numpy(samples), torch.from_numpy(codebook), return_indices=True, codebook_chunk=128)
+    expected = oracle_lattice.nearest_codes(samples, codebook)
+    assert (found.numpy() == expected).mean() > 0.99 and found[0] == 7
+    rounded = lattice(torch.from_numpy(samples))
+    codes = oracle_lattice.nearest_e8p_codes(samples)
+    np.testing.assert_array_equal(rounded.numpy(), oracle_lattice.e8p_points()[codes])
+    with pytest.raises(ValueError, match="eight-dimensional"):
+        lattice(torch.zeros(3, 4))
+    with pytest.raises(ValueError, match="asymmetric quantization requires an explicit scalar grid"):
+        mk.scaled(lattice, asym=True)
+    with pytest.raises(ValueError, match="divisible by the vector grid dimension"):
+        mk.scaled(lattice, group=12)(torch.randn(4, 48))
+
+
+def test_vector_grid_and_feedback_on_the_host():
+    # /root/reference/tests/quantization/test_algorithms.py:60-66, and the decoders
+    weights = torch.randn(16, 64)
+    codebook = torch.randn(32, 8)
+    quantization = mk.scaled(mk.grid.vector(codebook), group=None)
+    context = Ctx("layer", H=torch.eye(64))
+    result = mk.ldlq(quantization, step=8)(weights, context)
+    assert result.w.shape == weights.shape and result.codec == "vector_feedback"
+    assert result.bits == 5 * weights.numel() / 8 + 16 * weights.shape[0]
+    assert context.additional_bits == 32 * 8 * 32          # the codebook, counted once
+    assert quantization.logical_bits((16, 64)) == result.bits
+    torch.testing.assert_close(codecs.decoder("vector_feedback")(result.codes, **result.params), result.w, rtol=0, atol=0)
+    # with an identity Hessian no error is fed back: the sweep equals direct rounding
+    direct = quantization(weights, Ctx("layer"))
+    assert direct.codec == "vector_scaled" and direct.codes.dtype == torch.int32
+    assert torch.equal(direct.codes, result.codes)
+    lattice = mk.scaled(mk.grid.e8p(), group=32)(weights)
+    assert lattice.params["values"] is None and lattice.params["dim"] == 8
+    from oracle import lattice as oracle_lattice
+
+    expected = oracle_lattice.decode_vector_scaled(lattice.codes.numpy(), lattice.params["scales"].numpy(),
+                                                   oracle_lattice.e8p_points(), 32, 8)
+    np.testing.assert_array_equal(lattice.w.numpy(), expected)
+    joined = mk.concatenate_rows([mk.scaled(mk.grid.e8p(), group=32)(weights[:8]), mk.scaled(mk.grid.e8p(), group=32)(weights[8:])])
+    torch.testing.assert_close(joined.w, lattice.w, rtol=0, atol=0)
+    with pytest.raises(ValueError, match="step equal to its dimension"):
+        mk.ldlq(quantization, step=8, backend="hip")(weights, Ctx("layer", H=torch.eye(64)))
