@@ -489,12 +489,13 @@ def other_kernels(device: torch.device, full: bool) -> dict:
 
     # other matvec shapes and codecs, M = 1 and 8: HIP-graph launches through the C ABI over
     # enough distinct weight copies (> 512 MB) that the Infinity Cache cannot serve them
-    def matvec(rows, width, group, bits, table, uniform, asym, label, dtype=torch.float16, grouped=False):
+    def matvec(rows, width, group, bits, table, uniform, asym, label, dtype=torch.float16, grouped=False,
+               side_dtype=torch.float16):
         code_bytes = rows * width * bits // 8
         count = max(2, min(40, -(-MINIMUM_ROTATING_BYTES // code_bytes)))
         streams = [torch.randint(0, 256, (code_bytes,), dtype=torch.uint8, device=device, generator=generator)
                    for _ in range(count)]
-        side = (torch.rand((rows, width // group), device=device, generator=generator) * 0.004 + 0.005).half()
+        side = (torch.rand((rows, width // group), device=device, generator=generator) * 0.004 + 0.005).to(side_dtype)
         zeros = side.clone() if asym else None
         for samples in (1, 8):
             x = torch.randn((samples, width), device=device, generator=generator).to(dtype)
@@ -503,7 +504,8 @@ def other_kernels(device: torch.device, full: bool) -> dict:
                                   bits=bits, uniform=uniform, grid_min=float(table[0]),
                                   grid_step=float(table[1] - table[0])) for stream in streams]
             seconds = timed_graph(launchers, 200, 20, 20)[0]
-            nbytes = code_bytes + side.numel() * 2 * (2 if asym else 1) + samples * (width + rows) * 2
+            nbytes = (code_bytes + side.numel() * side.element_size() * (2 if asym else 1)
+                      + samples * (width + rows) * x.element_size())
             out[f"matvec {label} {rows}x{width} M={samples}"] = _entry(seconds * 1e3, nbytes, copies=count)
             if grouped and count >= 16:   # eight matrices per launch (mk_packed_matvec_group)
                 layout = packed_linear.layout_for(bits, width, group)
@@ -524,6 +526,9 @@ def other_kernels(device: torch.device, full: bool) -> dict:
     matvec(ROWS, WIDTH, 64, 3, torch.arange(-4, 4, dtype=torch.float32, device=device), True, False, "int3 g64", grouped=True)
     matvec(ROWS, WIDTH, 64, 4, nf4, False, False, "nf4 g64", grouped=True)
     matvec(ROWS, WIDTH, 64, 3, seven, False, False, "codebook7 g64", grouped=True)
+    # fp32 activations and fp32 scales (what the reference's own fp32 tests use): the generic word kernel
+    matvec(ROWS, WIDTH, 128, 4, values, True, False, "int4 g128, fp32 activations and scales", dtype=torch.float32,
+           side_dtype=torch.float32)
     if full:
         matvec(ROWS, WIDTH, 128, 4, values, True, False, "int4 g128, bf16 activations", dtype=torch.bfloat16)
         matvec(151936, 896, 128, 4, values, True, False, "int4 g128 (tied head)")

@@ -23,9 +23,12 @@
 
 #include "mk_common.h"
 
+#include <atomic>
+
 namespace {
 
 constexpr int kMaxThreads = 1024;
+constexpr long long kLeanRotationRows = 256;  // above this many outer rows mk_rotate_blocks streams with rotate_matrix_kernel
 
 struct FwhtArgs {
     const void *source;
@@ -276,6 +279,218 @@ int launch_fwht(FwhtArgs a, hipStream_t stream) {
     return launch_fwht_as<E, false>(a, threads, lds, stream);
 }
 
+// ---- Blocked rotation of weight-sized tensors: one pass, transform in registers -------------
+//
+// A workgroup owns one outer row of `order` blocks of `power` = 32 E values (E = 8 or 16) at a time
+// (two workgroups per CU, each taking every 512th row, the next row's values already on their
+// way into registers while the current one is mixed).  Half a wavefront holds a block: lane t of the half has elements (32 q + t) 4 + i of it (E / 4 coalesced
+// 16-byte loads), so index bits 0-1 and 7+ live in registers and bits 2-6 in the lane number.
+// The butterfly stages run in ascending stride as everywhere else: bits 0-1 between registers,
+// bits 2-6 between lanes (vector-ALU lane moves; the lane whose bit is set computes
+// partner - own, the other own + partner, both as one exactly rounded fma with +-1), the rest
+// between registers.  The transformed blocks are written to LDS once (16 bytes per lane, no
+// bank conflicts), and after one barrier every wavefront multiplies 32-column slices of them
+// by the basis on the fp32 matrix cores, exactly as fwht_kernel<.., TILES> does.  Per element:
+// about 20 vector instructions and 8 bytes of LDS traffic.
+
+struct MatrixArgs {
+    const float *source;
+    float *target;
+    const float *basis;
+    const float *signs_before, *signs_after;  // [order * power] or null
+    long long rows;  // outer rows
+    int order, power, transpose;
+    float scale;
+};
+
+// The value lane `lane ^ (1 << STAGE)` holds, STAGE 0 ... 4 (inside a half wavefront).
+template <int STAGE>
+__device__ __forceinline__ float half_wave_partner(float value) {
+    const int bits = __builtin_bit_cast(int, value);
+    int moved;
+    if constexpr (STAGE == 0) moved = __builtin_amdgcn_mov_dpp(bits, 0xB1, 0xf, 0xf, true);        // quad_perm [1,0,3,2]
+    else if constexpr (STAGE == 1) moved = __builtin_amdgcn_mov_dpp(bits, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+    else if constexpr (STAGE == 2) {
+        moved = __builtin_amdgcn_update_dpp(bits, bits, 0x104, 0xf, 0x5, false);    // row_shl:4 into lanes 0-3, 8-11
+        moved = __builtin_amdgcn_update_dpp(moved, bits, 0x114, 0xf, 0xa, false);   // row_shr:4 into lanes 4-7, 12-15
+    } else if constexpr (STAGE == 3) moved = __builtin_amdgcn_mov_dpp(bits, 0x128, 0xf, 0xf, true);  // row_ror:8
+    else {
+        const auto swapped = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+        moved = (threadIdx.x & 16) ? swapped[0] : swapped[1];
+    }
+    return __builtin_bit_cast(float, moved);
+}
+
+template <int E, int STAGE>
+__device__ __forceinline__ void lane_stage(float (&v)[E], int t) {
+    const float sign = (t >> STAGE) & 1 ? -1.0f : 1.0f;
+#pragma unroll
+    for (int j = 0; j < E; ++j) v[j] = __builtin_fmaf(v[j], sign, half_wave_partner<STAGE>(v[j]));
+}
+
+constexpr int kRotationWaves = 8;   // wavefronts per workgroup: two workgroups share a CU
+constexpr int kRotationUnits = 2;   // pairs of blocks per wavefront: up to 32 blocks per outer row
+
+template <int E>
+__global__ void __launch_bounds__(64 * kRotationWaves) rotate_matrix_kernel(const MatrixArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float tile[];  // [order][power], then the basis
+    constexpr int kQuads = E / 4;
+    constexpr int kPower = 32 * E;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int half = lane >> 5, t = lane & 31;
+    const size_t outer_floats = static_cast<size_t>(a.order) * kPower;
+
+    // In LDS behind the row: the basis as the left operand of the products, mix[out][in] at
+    // basis_tile[in * 32 + out], zero outside the basis.
+    float *basis_tile = tile + outer_floats;
+    for (int i = threadIdx.x; i < 32 * 32; i += blockDim.x) {
+        const int in = i >> 5, out = i & 31;
+        const bool inside = in < a.order && out < a.order;
+        const float held = a.basis[inside ? (a.transpose ? in * a.order + out : out * a.order + in) : 0];
+        basis_tile[i] = inside ? held : 0.0f;
+    }
+    const int pairs = (a.order + 1) >> 1;
+
+    // Wavefront w transforms the pairs of blocks w and w + 8 of every outer row the workgroup
+    // takes; their values are requested one row ahead.
+    float4 loaded[kRotationUnits][kQuads];
+    auto request = [&](long long row) __attribute__((always_inline)) {
+        if (row >= a.rows) return;
+        const float4 *source = reinterpret_cast<const float4 *>(a.source + static_cast<size_t>(row) * outer_floats);
+#pragma unroll
+        for (int u = 0; u < kRotationUnits; ++u) {
+            const int block = 2 * (wave + kRotationWaves * u) + half;
+            if (2 * (wave + kRotationWaves * u) >= a.order) continue;  // uniform
+            const uint32_t first = static_cast<uint32_t>(block < a.order ? block : 0) * (kPower / 4) + t;
+#pragma unroll
+            for (int q = 0; q < kQuads; ++q) loaded[u][q] = source[q * 32 + first];
+        }
+    };
+    request(blockIdx.x);
+    for (long long row = blockIdx.x; row < a.rows; row += gridDim.x) {
+#pragma unroll
+        for (int u = 0; u < kRotationUnits; ++u) {
+            const int block = 2 * (wave + kRotationWaves * u) + half;
+            if (2 * (wave + kRotationWaves * u) >= a.order) continue;  // uniform
+            const bool present = block < a.order;
+            const int offset = (present ? block : 0) * kPower;
+            float v[E];
+#pragma unroll
+            for (int q = 0; q < kQuads; ++q) {
+                v[4 * q] = loaded[u][q].x; v[4 * q + 1] = loaded[u][q].y;
+                v[4 * q + 2] = loaded[u][q].z; v[4 * q + 3] = loaded[u][q].w;
+            }
+            if (a.signs_before) {
+                const float4 *signs = reinterpret_cast<const float4 *>(a.signs_before + offset);
+#pragma unroll
+                for (int q = 0; q < kQuads; ++q) {
+                    const float4 sign = signs[q * 32 + t];
+                    v[4 * q] *= sign.x; v[4 * q + 1] *= sign.y; v[4 * q + 2] *= sign.z; v[4 * q + 3] *= sign.w;
+                }
+            }
+            // index bits 0 and 1: inside each group of four
+#pragma unroll
+            for (int bit = 0; bit < 2; ++bit)
+#pragma unroll
+                for (int j = 0; j < E; ++j) {
+                    if ((j >> bit) & 1) continue;
+                    const float first = v[j], second = v[j | (1 << bit)];
+                    v[j] = first + second;
+                    v[j | (1 << bit)] = first - second;
+                }
+            // bits 2 ... 6: between the lanes of the half wavefront
+            lane_stage<E, 0>(v, t);
+            lane_stage<E, 1>(v, t);
+            lane_stage<E, 2>(v, t);
+            lane_stage<E, 3>(v, t);
+            lane_stage<E, 4>(v, t);
+            // bits 7 and up: between the groups of four
+#pragma unroll
+            for (int bit = 2; (1 << bit) < E; ++bit)
+#pragma unroll
+                for (int j = 0; j < E; ++j) {
+                    if ((j >> bit) & 1) continue;
+                    const float first = v[j], second = v[j | (1 << bit)];
+                    v[j] = first + second;
+                    v[j | (1 << bit)] = first - second;
+                }
+            if (present) {
+                float4 *rows = reinterpret_cast<float4 *>(tile + offset);
+#pragma unroll
+                for (int q = 0; q < kQuads; ++q)
+                    rows[q * 32 + t] = make_float4(v[4 * q] * a.scale, v[4 * q + 1] * a.scale, v[4 * q + 2] * a.scale,
+                                                   v[4 * q + 3] * a.scale);
+            }
+        }
+        __syncthreads();
+        request(row + gridDim.x);
+
+        // target[f', p] = sum_f mix[f', f] * block f [p] over ascending f from zero (f in pairs on
+        // the matrix cores); lanes 0..31 read block f, lanes 32..63 block f + 1, at 32 adjacent p.
+        float *row_target = a.target + static_cast<size_t>(row) * outer_floats;
+        const float *mine = tile + half * kPower + t;          // + 2 q kPower + first
+        const float *basis_mine = basis_tile + half * 32 + t;  // + 64 q
+        for (int first = wave * 32; first < kPower; first += kRotationWaves * 32) {
+            const uint32_t store_lane = static_cast<uint32_t>(half * 4 * kPower + first + t);
+            mk_mix16 sums;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sums[r] = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                if (q < pairs) {  // uniform
+                    // (an odd order's last pair reads one block beyond the row: the basis tile, finite
+                    // values that meet the zeros of the basis' padding)
+                    const float right = mine[2 * q * kPower + first];
+                    sums = __builtin_amdgcn_mfma_f32_32x32x2f32(basis_mine[64 * q], right, sums, 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int out_uniform = (r >> 2) * 8 + (r & 3);   // + 4 for the upper half of the lanes
+                const bool both = out_uniform + 4 < a.order, lower = out_uniform < a.order;  // uniform
+                if (both || (lower && half == 0)) {
+                    float value = sums[r];
+                    if (a.signs_after) value *= (a.signs_after + out_uniform * kPower)[store_lane];
+                    (row_target + out_uniform * kPower)[store_lane] = value;
+                }
+            }
+        }
+        __syncthreads();  // the next row's blocks go into the same LDS
+    }
+}
+
+// Launches rotate_matrix_kernel when the shape fits it: fp32 in and out, 16-byte aligned,
+// power = 32 E with E in {8, 16} (blocks of 256 or 512 values), at most 32 blocks that fit
+// 76 KB of LDS together (two workgroups per CU).
+// Returns -1 when it does not apply.
+int launch_rotate_matrix(const FwhtArgs &f, long long outer_rows, hipStream_t stream) {
+    const auto aligned = [](const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15u) == 0; };
+    const int elements = f.width / 32;
+    const size_t lds = (static_cast<size_t>(f.order) * f.width + 32 * 32) * sizeof(float);
+    if (f.source_dtype != MK_F32 || f.target_dtype != MK_F32 || f.order > 32 ||
+        (elements != 8 && elements != 16) || lds > 80 * 1024 || !aligned(f.source) ||
+        !aligned(f.target) || !aligned(f.signs_before))
+        return -1;
+    MatrixArgs a{static_cast<const float *>(f.source), static_cast<float *>(f.target), f.basis, f.signs_before,
+                 f.signs_after, outer_rows, f.order, f.width, f.transpose, f.scale};
+    // Two workgroups of eight wavefronts per CU (registers and LDS allow no more), so that one's
+    // matrix-core phase overlaps the other's butterflies; each takes every 512th outer row.
+    const dim3 grid(static_cast<unsigned>(outer_rows < 512 ? outer_rows : 512)), block(64 * kRotationWaves);
+    static std::atomic<bool> raised{false};
+    if (lds > 48 * 1024 && !raised.load()) {
+        for (const void *kernel : {reinterpret_cast<const void *>(&rotate_matrix_kernel<8>),
+                                   reinterpret_cast<const void *>(&rotate_matrix_kernel<16>)}) {
+            const hipError_t status = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+            if (status != hipSuccess)
+                return mk_fail(MK_ERR_HIP, "mk_rotate_blocks: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(status));
+        }
+        raised.store(true);
+    }
+    if (elements == 8) hipLaunchKernelGGL(rotate_matrix_kernel<8>, grid, block, lds, stream, a);
+    else hipLaunchKernelGGL(rotate_matrix_kernel<16>, grid, block, lds, stream, a);
+    return MK_OK;
+}
+
 struct MixArgs {
     const float *source;
     float *target;
@@ -441,6 +656,13 @@ extern "C" int mk_rotate_blocks(const void *source, int source_dtype, void *targ
     a.log_width = 0;
     while ((1 << a.log_width) < power) ++a.log_width;
     int status = -1;
+    // Weight-sized tensors (more outer rows than the GPU has workgroup slots) take the lean one-pass kernel.
+    if (rows > kLeanRotationRows) status = launch_rotate_matrix(a, rows, stream);
+    if (status >= 0) {
+        if (status) return status;
+        MK_LAUNCH_CHECK("mk_rotate_blocks");
+        return MK_OK;
+    }
     if (order * (power / 16) <= kMaxThreads) {
         status = order <= 32 ? launch_blocked<16, 1>(a, stream)
                              : order <= 64 ? launch_blocked<16, 2>(a, stream) : launch_blocked<16, 3>(a, stream);

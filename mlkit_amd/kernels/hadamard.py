@@ -92,6 +92,14 @@ def fits_one_launch(order: int, power: int) -> bool:
     return order * (power // 16) <= 1024 or order * (power // 32) <= 1024
 
 
+def streams_in_one_pass(value: Tensor, order: int, power: int) -> bool:
+    """Whether ``rotate_blocks`` has its register-resident one-pass kernel for a weight-sized
+    ``value``: FP32, at most 32 blocks of 256 or 512 values that fit half a CU's LDS beside the
+    basis."""
+    return (value.dtype == torch.float32 and order <= 32 and power in (256, 512)
+            and (order * power + 1024) * 4 <= MAXIMUM_FUSED_LDS // 2 and value.data_ptr() % 16 == 0)
+
+
 def rotate_blocks(
     value: Tensor,
     basis: Tensor,

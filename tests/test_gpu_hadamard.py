@@ -127,6 +127,38 @@ def test_one_launch_blocked_transform_equals_the_two_calls(width, dtype):
             assert torch.equal(result, expected)
 
 
+@pytest.mark.parametrize("width", [14336, 7168, 5120, 6144])
+def test_one_pass_rotation_of_many_rows_equals_the_two_calls(width):
+    """More than 256 outer rows of fp32 take `rotate_matrix_kernel` (transform between registers
+    and lanes, one LDS exchange, basis product on the matrix cores): bit for bit what `mk_fwht` +
+    `mk_basis_mix` give, forward with the signs in front and inverse with the signs behind; and
+    `mk.rht` on a weight-sized tensor goes that way."""
+    from mlkit_amd.kernels import hadamard
+
+    order, power, basis = transforms.transform_factor(width)
+    rows = 301
+    generator = torch.Generator(device="cuda").manual_seed(width)
+    value = torch.randn((rows, order, power), device="cuda", generator=generator)
+    assert hadamard.streams_in_one_pass(value, order, power)
+    signs = dev(transforms.deterministic_signs(width, seed=9))
+    for inverse in (False, True):
+        before, after = (None, signs) if inverse else (signs, None)
+        staged = hadamard.transform(value, signs_before=before)
+        expected = hadamard.mix_blocks(staged, dev(basis), transpose=inverse, signs_after=after)
+        result = hadamard.rotate_blocks(value, dev(basis), transpose=inverse, signs_before=before, signs_after=after)
+        assert torch.equal(result, expected)
+        assert torch.equal(hadamard.rotate_blocks(value, dev(basis), transpose=inverse), 
+                           hadamard.mix_blocks(hadamard.transform(value), dev(basis), transpose=inverse))
+    import mlkit_amd as mk
+
+    flat = value.view(rows, width)
+    rotated = mk.rht(flat, seed=3)
+    torch.testing.assert_close(rotated.norm(dim=1), flat.norm(dim=1), rtol=1e-5, atol=0)
+    torch.testing.assert_close(mk.rht(rotated, seed=3, inverse=True), flat, rtol=1e-5, atol=2e-5)
+    np.testing.assert_allclose(host(mk.structured_transform(flat[:4].contiguous())),
+                               host(mk.structured_transform(flat))[:4], rtol=1e-5, atol=1e-5)  # few rows: the LDS kernel
+
+
 def test_one_launch_blocked_transform_declines_what_does_not_fit():
     from mlkit_amd.kernels import hadamard
 
