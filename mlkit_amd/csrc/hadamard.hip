@@ -303,21 +303,17 @@ struct MatrixArgs {
     float scale;
 };
 
-// The value lane `lane ^ (1 << STAGE)` holds, STAGE 0 ... 4 (inside a half wavefront).
+// The value lane `lane ^ (1 << STAGE)` holds, STAGE 0 ... 4 (inside a half wavefront): one DPP
+// move where a row permutation exists (lanes ^ 1, ^ 2, ^ 8), one swizzle through the LDS
+// crossbar (no memory access, no vector-ALU slot) for lanes ^ 4 and ^ 16.
 template <int STAGE>
 __device__ __forceinline__ float half_wave_partner(float value) {
     const int bits = __builtin_bit_cast(int, value);
     int moved;
     if constexpr (STAGE == 0) moved = __builtin_amdgcn_mov_dpp(bits, 0xB1, 0xf, 0xf, true);        // quad_perm [1,0,3,2]
     else if constexpr (STAGE == 1) moved = __builtin_amdgcn_mov_dpp(bits, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
-    else if constexpr (STAGE == 2) {
-        moved = __builtin_amdgcn_update_dpp(bits, bits, 0x104, 0xf, 0x5, false);    // row_shl:4 into lanes 0-3, 8-11
-        moved = __builtin_amdgcn_update_dpp(moved, bits, 0x114, 0xf, 0xa, false);   // row_shr:4 into lanes 4-7, 12-15
-    } else if constexpr (STAGE == 3) moved = __builtin_amdgcn_mov_dpp(bits, 0x128, 0xf, 0xf, true);  // row_ror:8
-    else {
-        const auto swapped = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
-        moved = (threadIdx.x & 16) ? swapped[0] : swapped[1];
-    }
+    else if constexpr (STAGE == 3) moved = __builtin_amdgcn_mov_dpp(bits, 0x128, 0xf, 0xf, true);  // row_ror:8
+    else moved = __builtin_amdgcn_ds_swizzle(bits, 0x1F | ((1 << STAGE) << 10));  // bit mode: and 31, or 0, xor 1 << STAGE
     return __builtin_bit_cast(float, moved);
 }
 
@@ -336,7 +332,7 @@ __global__ void __launch_bounds__(64 * kRotationWaves) rotate_matrix_kernel(cons
     extern __shared__ __attribute__((aligned(16))) float tile[];  // [order][power], then the basis
     constexpr int kQuads = E / 4;
     constexpr int kPower = 32 * E;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int half = lane >> 5, t = lane & 31;
     const size_t outer_floats = static_cast<size_t>(a.order) * kPower;
 
@@ -354,38 +350,43 @@ __global__ void __launch_bounds__(64 * kRotationWaves) rotate_matrix_kernel(cons
     // Wavefront w transforms the pairs of blocks w and w + 8 of every outer row the workgroup
     // takes; their values are requested one row ahead.
     float4 loaded[kRotationUnits][kQuads];
-    auto request = [&](long long row) __attribute__((always_inline)) {
-        if (row >= a.rows) return;
+    const int rows = static_cast<int>(a.rows), stride = gridDim.x;  // (rows * order < 2^31: checked by the caller)
+    auto request = [&](int u, int row) __attribute__((always_inline)) {
+        const int block = 2 * (wave + kRotationWaves * u) + half;
+        if (row >= rows || 2 * (wave + kRotationWaves * u) >= a.order) return;  // uniform
         const float4 *source = reinterpret_cast<const float4 *>(a.source + static_cast<size_t>(row) * outer_floats);
+        const uint32_t first = static_cast<uint32_t>(block < a.order ? block : 0) * (kPower / 4) + t;
 #pragma unroll
-        for (int u = 0; u < kRotationUnits; ++u) {
-            const int block = 2 * (wave + kRotationWaves * u) + half;
-            if (2 * (wave + kRotationWaves * u) >= a.order) continue;  // uniform
-            const uint32_t first = static_cast<uint32_t>(block < a.order ? block : 0) * (kPower / 4) + t;
-#pragma unroll
-            for (int q = 0; q < kQuads; ++q) loaded[u][q] = source[q * 32 + first];
-        }
+        for (int q = 0; q < kQuads; ++q) loaded[u][q] = source[q * 32 + first];
     };
-    request(blockIdx.x);
-    for (long long row = blockIdx.x; row < a.rows; row += gridDim.x) {
+#pragma unroll
+    for (int u = 0; u < kRotationUnits; ++u) request(u, blockIdx.x);
+    for (int row = blockIdx.x; row < rows; row += stride) {
 #pragma unroll
         for (int u = 0; u < kRotationUnits; ++u) {
             const int block = 2 * (wave + kRotationWaves * u) + half;
             if (2 * (wave + kRotationWaves * u) >= a.order) continue;  // uniform
             const bool present = block < a.order;
             const int offset = (present ? block : 0) * kPower;
+            // (the signs are requested before the next row's values: loads complete in order, and
+            // the butterflies must not wait for that row)
+            float4 sign[kQuads];
+            if (a.signs_before) {
+                const float4 *signs = reinterpret_cast<const float4 *>(a.signs_before + offset);
+#pragma unroll
+                for (int q = 0; q < kQuads; ++q) sign[q] = signs[q * 32 + t];
+            }
             float v[E];
 #pragma unroll
             for (int q = 0; q < kQuads; ++q) {
                 v[4 * q] = loaded[u][q].x; v[4 * q + 1] = loaded[u][q].y;
                 v[4 * q + 2] = loaded[u][q].z; v[4 * q + 3] = loaded[u][q].w;
             }
+            request(u, row + stride);  // the same blocks of the workgroup's next row, a whole turn ahead
             if (a.signs_before) {
-                const float4 *signs = reinterpret_cast<const float4 *>(a.signs_before + offset);
 #pragma unroll
                 for (int q = 0; q < kQuads; ++q) {
-                    const float4 sign = signs[q * 32 + t];
-                    v[4 * q] *= sign.x; v[4 * q + 1] *= sign.y; v[4 * q + 2] *= sign.z; v[4 * q + 3] *= sign.w;
+                    v[4 * q] *= sign[q].x; v[4 * q + 1] *= sign[q].y; v[4 * q + 2] *= sign[q].z; v[4 * q + 3] *= sign[q].w;
                 }
             }
             // index bits 0 and 1: inside each group of four
@@ -423,7 +424,6 @@ __global__ void __launch_bounds__(64 * kRotationWaves) rotate_matrix_kernel(cons
             }
         }
         __syncthreads();
-        request(row + gridDim.x);
 
         // target[f', p] = sum_f mix[f', f] * block f [p] over ascending f from zero (f in pairs on
         // the matrix cores); lanes 0..31 read block f, lanes 32..63 block f + 1, at 32 adjacent p.
@@ -431,7 +431,8 @@ __global__ void __launch_bounds__(64 * kRotationWaves) rotate_matrix_kernel(cons
         const float *mine = tile + half * kPower + t;          // + 2 q kPower + first
         const float *basis_mine = basis_tile + half * 32 + t;  // + 64 q
         for (int first = wave * 32; first < kPower; first += kRotationWaves * 32) {
-            const uint32_t store_lane = static_cast<uint32_t>(half * 4 * kPower + first + t);
+            // (byte offsets in 32 bits, so that a store takes a scalar base and one offset register)
+            const uint32_t store_bytes = static_cast<uint32_t>(half * 4 * kPower + first + t) * 4u;
             mk_mix16 sums;
 #pragma unroll
             for (int r = 0; r < 16; ++r) sums[r] = 0.0f;
@@ -450,8 +451,10 @@ __global__ void __launch_bounds__(64 * kRotationWaves) rotate_matrix_kernel(cons
                 const bool both = out_uniform + 4 < a.order, lower = out_uniform < a.order;  // uniform
                 if (both || (lower && half == 0)) {
                     float value = sums[r];
-                    if (a.signs_after) value *= (a.signs_after + out_uniform * kPower)[store_lane];
-                    (row_target + out_uniform * kPower)[store_lane] = value;
+                    if (a.signs_after)
+                        value *= *reinterpret_cast<const float *>(
+                            reinterpret_cast<const char *>(a.signs_after + out_uniform * kPower) + store_bytes);
+                    *reinterpret_cast<float *>(reinterpret_cast<char *>(row_target + out_uniform * kPower) + store_bytes) = value;
                 }
             }
         }
