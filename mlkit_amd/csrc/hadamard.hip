@@ -494,6 +494,106 @@ int launch_rotate_matrix(const FwhtArgs &f, long long outer_rows, hipStream_t st
     return MK_OK;
 }
 
+// ---- Plain transform of weight-sized fp32 tensors: one wavefront per row, registers only -----
+//
+// A row of 64 E values (E = 4 ... 64: 256 to 4096 values) lives in the registers of one
+// wavefront, lane t holding elements (64 q + t) 4 + i: index bits 0-1 and 8+ in registers, bits
+// 2-7 in the lane number.  Same stages in the same order as fwht_kernel, same sums, no LDS
+// memory and no barrier; lane exchanges are DPP moves (lanes ^ 1, ^ 2, ^ 8), swizzles through
+// the LDS crossbar (^ 4, ^ 16) and a crossbar permute (^ 32).
+
+// The value lane `lane ^ 32` holds.
+__device__ __forceinline__ float other_half_partner(float value, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, value)));
+}
+
+template <int E>
+__global__ void __launch_bounds__(256) fwht_rows_kernel(const FwhtArgs a) {
+    constexpr int kQuads = E / 4;
+    const int lane = threadIdx.x & 63;
+    const long long row = static_cast<long long>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (row >= a.rows) return;  // whole wavefronts leave; nothing below synchronises the workgroup
+    const size_t row_base = static_cast<size_t>(row) * a.width;
+    const int sign_base = a.sign_period ? static_cast<int>(row_base % static_cast<size_t>(a.sign_period)) : 0;
+    const float4 *source = reinterpret_cast<const float4 *>(static_cast<const float *>(a.source) + row_base);
+    float4 loaded[kQuads];
+#pragma unroll
+    for (int q = 0; q < kQuads; ++q) loaded[q] = source[q * 64 + lane];
+    float v[E];
+#pragma unroll
+    for (int q = 0; q < kQuads; ++q) {
+        v[4 * q] = loaded[q].x; v[4 * q + 1] = loaded[q].y; v[4 * q + 2] = loaded[q].z; v[4 * q + 3] = loaded[q].w;
+    }
+    if (a.signs_before) {
+        const float4 *signs = reinterpret_cast<const float4 *>(a.signs_before + sign_base);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) {
+            const float4 sign = signs[q * 64 + lane];
+            v[4 * q] *= sign.x; v[4 * q + 1] *= sign.y; v[4 * q + 2] *= sign.z; v[4 * q + 3] *= sign.w;
+        }
+    }
+#pragma unroll
+    for (int bit = 0; bit < 2; ++bit)
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            if ((j >> bit) & 1) continue;
+            const float first = v[j], second = v[j | (1 << bit)];
+            v[j] = first + second;
+            v[j | (1 << bit)] = first - second;
+        }
+    lane_stage<E, 0>(v, lane);
+    lane_stage<E, 1>(v, lane);
+    lane_stage<E, 2>(v, lane);
+    lane_stage<E, 3>(v, lane);
+    lane_stage<E, 4>(v, lane);
+    {
+        const float sign = lane & 32 ? -1.0f : 1.0f;
+#pragma unroll
+        for (int j = 0; j < E; ++j) v[j] = __builtin_fmaf(v[j], sign, other_half_partner(v[j], lane));
+    }
+#pragma unroll
+    for (int bit = 2; (1 << bit) < E; ++bit)
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            if ((j >> bit) & 1) continue;
+            const float first = v[j], second = v[j | (1 << bit)];
+            v[j] = first + second;
+            v[j | (1 << bit)] = first - second;
+        }
+    float4 *target = reinterpret_cast<float4 *>(static_cast<float *>(a.target) + row_base);
+    const float4 *signs_after = reinterpret_cast<const float4 *>(a.signs_after ? a.signs_after + sign_base : nullptr);
+#pragma unroll
+    for (int q = 0; q < kQuads; ++q) {
+        float4 out = make_float4(v[4 * q] * a.scale, v[4 * q + 1] * a.scale, v[4 * q + 2] * a.scale, v[4 * q + 3] * a.scale);
+        if (signs_after) {
+            const float4 sign = signs_after[q * 64 + lane];
+            out.x *= sign.x; out.y *= sign.y; out.z *= sign.z; out.w *= sign.w;
+        }
+        target[q * 64 + lane] = out;
+    }
+}
+
+// Launches fwht_rows_kernel when it applies (fp32 in and out, rows of 256 ... 4096 values,
+// 16-byte aligned, enough rows to fill the GPU with wavefronts); -1 otherwise.
+constexpr long long kRegisterTransformRows = 4096;
+
+int launch_fwht_rows(const FwhtArgs &a, hipStream_t stream) {
+    const auto aligned = [](const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15u) == 0; };
+    if (a.source_dtype != MK_F32 || a.target_dtype != MK_F32 || a.width < 256 || a.width > 4096 ||
+        a.rows < kRegisterTransformRows || !aligned(a.source) || !aligned(a.target) || !aligned(a.signs_before) ||
+        !aligned(a.signs_after))
+        return -1;
+    const dim3 grid(static_cast<unsigned>((a.rows + 3) / 4)), block(256);
+    switch (a.width / 64) {
+        case 4: hipLaunchKernelGGL(fwht_rows_kernel<4>, grid, block, 0, stream, a); break;
+        case 8: hipLaunchKernelGGL(fwht_rows_kernel<8>, grid, block, 0, stream, a); break;
+        case 16: hipLaunchKernelGGL(fwht_rows_kernel<16>, grid, block, 0, stream, a); break;
+        case 32: hipLaunchKernelGGL(fwht_rows_kernel<32>, grid, block, 0, stream, a); break;
+        default: hipLaunchKernelGGL(fwht_rows_kernel<64>, grid, block, 0, stream, a); break;
+    }
+    return MK_OK;
+}
+
 struct MixArgs {
     const float *source;
     float *target;
@@ -624,7 +724,11 @@ extern "C" int mk_fwht(const void *source, int source_dtype, void *target, int t
     a.sign_period = (signs_before || signs_after) ? sign_period : 0; a.scale = scale;
     a.log_width = 0;
     while ((1 << a.log_width) < width) ++a.log_width;
-    int status;
+    int status = launch_fwht_rows(a, stream);
+    if (status >= 0) {
+        MK_LAUNCH_CHECK("mk_fwht");
+        return MK_OK;
+    }
     if (width >= 32768) status = launch_fwht<32>(a, stream);
     else if (width >= 16) status = launch_fwht<16>(a, stream);
     else if (width == 8) status = launch_fwht<8>(a, stream);

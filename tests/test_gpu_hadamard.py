@@ -39,6 +39,33 @@ def test_transform_is_bit_exact(width, normalize):
         np.testing.assert_allclose(out, exact, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("width", [256, 512, 1024, 2048, 4096])
+def test_register_transform_of_many_rows_is_bit_exact(width):
+    """4096 fp32 rows and more take `fwht_rows_kernel` (a row in the registers of one wavefront, no
+    LDS): the stagewise oracle on sampled rows, and the workgroup kernel (fewer rows per call) on
+    all of them, bit for bit; with signs in front and behind whose period spans three rows."""
+    from mlkit_amd.kernels import hadamard
+
+    rows = 4098   # not a multiple of the four rows a workgroup takes
+    generator = torch.Generator(device="cuda").manual_seed(width)
+    value = torch.randn((rows, width), device="cuda", generator=generator)
+    out = hadamard.transform(value)
+    picked = [0, 1, 2, 3, 1000, 4095, 4096, 4097]
+    np.testing.assert_array_equal(host(out[picked]), transforms.fwht(host(value[picked])))
+    pieces = torch.cat([hadamard.transform(value[:2049].contiguous()), hadamard.transform(value[2049:].contiguous())])
+    assert torch.equal(out, pieces)
+    assert torch.equal(hadamard.transform(value, normalize=False)[:7], hadamard.transform(value[:7].contiguous(), normalize=False))
+    signs = dev(transforms.deterministic_signs(3 * width, seed=2))
+    blocks = value[: 4098 - 4098 % 3].view(-1, 3, width)
+    signed = hadamard.transform(blocks, signs_before=signs, signs_after=signs)
+    expected = torch.cat([hadamard.transform(blocks[:600].contiguous(), signs_before=signs, signs_after=signs),
+                          hadamard.transform(blocks[600:].contiguous(), signs_before=signs, signs_after=signs)])
+    assert torch.equal(signed, expected)
+    in_place = value.clone()
+    hadamard.transform(in_place, out=in_place)
+    assert torch.equal(in_place, out)
+
+
 def test_leading_dimensions_and_involution():
     from mlkit_amd.kernels import hadamard
 
