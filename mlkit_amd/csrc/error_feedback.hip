@@ -604,6 +604,9 @@ struct UpdateArgs {
     int chains;
     int column_begin, column_end;  // columns of feedback that are updated
     const float *deviation_t;      // null, or [width, rows] deviations written by the sweep
+    // The kernels that read `deviation_t` take a linear range of tiles (column tile fastest):
+    // workgroup b owns tile `tile_first + b` of a grid `column_tiles` wide.
+    int tile_first, column_tiles;
 };
 
 struct UpdateStage {
@@ -795,8 +798,10 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviation
     // the compiler keeps the bases in scalar registers.
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int row0 = blockIdx.y * kTileRows;
-    const int column0 = a.column_begin + blockIdx.x * kTileColumns;
+    const int tile = a.tile_first + blockIdx.x;
+    const int tile_row = tile / a.column_tiles;
+    const int row0 = tile_row * kTileRows;
+    const int column0 = a.column_begin + (tile - tile_row * a.column_tiles) * kTileColumns;
     const int wave_row = (wave >> 1) * 64, wave_column = (wave & 1) * 64;
     const int chunks_per_chain = a.chain_width / kDepthChunk;
     const int steps = a.chains * chunks_per_chain;
@@ -922,62 +927,98 @@ __global__ void __launch_bounds__(kUpdateThreads, 2) block_update_from_deviation
             for (int r = 0; r < 16; ++r) *cell(mi, ni, r) = totals[mi][ni][r];
 }
 
-// One chain of exactly 128 columns over a few tiles (the update of a super-block's own later
-// tiles right after a tile's sweep): at most 96 of the 128 x 128 tiles above, each a
-// wavefront-serial chain of 256 MFMAs (16 K cycles), on a GPU with 1024 SIMDs.  Here a
-// workgroup owns a 64 x 64 tile and a wavefront one 32 x 32 accumulator (64 MFMAs), so the
-// same update spreads over four times as many SIMDs; both whole 128-deep operands and the
-// feedback tile are requested at once and waited for once.  Sums are formed exactly as
-// above (ascending k from zero, then added to feedback).
+// Chains of exactly 128 columns on 64 x 64 tiles.  Two uses: the update of a super-block's own
+// later tiles right after a tile's sweep (one chain over at most 96 of the 128 x 128 tiles
+// above, each a wavefront-serial chain of 256 MFMAs, on a GPU with 1024 SIMDs), and the last,
+// partly filled round of a wide launch (a few 128 x 128 tiles would hold the whole GPU for a
+// full round; as quarter tiles they spread over four times as many SIMDs).  A workgroup owns
+// a 64 x 64 tile and a wavefront one 32 x 32 accumulator (64 MFMAs per chain); operands arrive
+// half a chain at a time in two LDS buffers, the next half on its way while the current one is
+// multiplied.  Sums are formed exactly as above (per chain: ascending k from zero, then added
+// to the running total).
 constexpr int kWholeChain = 128;
 constexpr int kSmallTile = 64;
 
+constexpr int kSmallDepth = 64;  // k rows per step: half a chain, two LDS buffers of 2 x 16 KB
+
 __global__ void __launch_bounds__(kUpdateThreads) block_update_small_tile_kernel(const UpdateArgs a) {
-    __shared__ __attribute__((aligned(16))) float deviation[kWholeChain][kSmallTile];     // [k][row]
-    __shared__ __attribute__((aligned(16))) float coefficient[kWholeChain][kSmallTile];   // [k][column]
+    __shared__ __attribute__((aligned(16))) float deviation_even[kSmallDepth][kSmallTile];     // [k][row]
+    __shared__ __attribute__((aligned(16))) float deviation_odd[kSmallDepth][kSmallTile];
+    __shared__ __attribute__((aligned(16))) float coefficient_even[kSmallDepth][kSmallTile];   // [k][column]
+    __shared__ __attribute__((aligned(16))) float coefficient_odd[kSmallDepth][kSmallTile];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int row0 = blockIdx.y * kSmallTile;
-    const int column0 = a.column_begin + blockIdx.x * kSmallTile;
+    // Quarter q of 128 x 128 tile `tile_first + b / 4` (the same linear order as the large kernel).
+    const int large = a.tile_first + (blockIdx.x >> 2), quarter = blockIdx.x & 3;
+    const int large_row = large / a.column_tiles;
+    const int row0 = large_row * kTileRows + (quarter >> 1) * kSmallTile;
+    const int column0 = a.column_begin + (large - large_row * a.column_tiles) * kTileColumns + (quarter & 1) * kSmallTile;
     const int wave_row = (wave >> 1) * 32, wave_column = (wave & 1) * 32;
 
     // One instruction moves four k rows of a tile (4 x 64 floats; lane l's 16 bytes land at
-    // 16 l from the uniform LDS address); a wavefront moves k rows 32 wave ... 32 wave + 31.
+    // 16 l from the uniform LDS address); per step a wavefront moves k rows 16 wave ... 16 wave + 15.
     const uint32_t left_lane = static_cast<uint32_t>(lane >> 4) * a.rows + (lane & 15) * 4;
     const uint32_t right_lane = static_cast<uint32_t>(lane >> 4) * a.width + (lane & 15) * 4;
-    const size_t k_base = static_cast<size_t>(a.first_column + wave * 32);
-    const float *left = a.deviation_t + row0 + k_base * a.rows;
-    const float *right = a.coeff + column0 + k_base * a.width;
+    auto fetch = [&](int step, auto odd) __attribute__((always_inline)) {
+        const size_t k_base = static_cast<size_t>(a.first_column + step * kSmallDepth + wave * 16);  // chains are adjacent
+        const float *left = a.deviation_t + row0 + k_base * a.rows;
+        const float *right = a.coeff + column0 + k_base * a.width;
 #pragma unroll
-    for (int four = 0; four < 8; ++four) {
-        rows_to_lds(left + static_cast<size_t>(4 * four) * a.rows + left_lane, &deviation[wave * 32 + 4 * four][0]);
-        rows_to_lds(right + static_cast<size_t>(4 * four) * a.width + right_lane, &coefficient[wave * 32 + 4 * four][0]);
-    }
+        for (int four = 0; four < 4; ++four) {
+            const int k = wave * 16 + 4 * four;
+            rows_to_lds(left + static_cast<size_t>(4 * four) * a.rows + left_lane,
+                        odd.value ? &deviation_odd[k][0] : &deviation_even[k][0]);
+            rows_to_lds(right + static_cast<size_t>(4 * four) * a.width + right_lane,
+                        odd.value ? &coefficient_odd[k][0] : &coefficient_even[k][0]);
+        }
+    };
+    const int steps = a.chains * (kWholeChain / kSmallDepth);
+    fetch(0, std::false_type{});
 
     // This lane's cells of the 32 x 32 tile: rows (lane / 32) * 4 + ..., column lane % 32.
     float *cells = a.feedback + static_cast<size_t>(row0 + wave_row + (lane >> 5) * 4) * a.width + column0 + wave_column + (lane & 31);
     mk_f32x16 totals, sums;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        totals[r] = cells[static_cast<size_t>((r >> 2) * 8 + (r & 3)) * a.width];
-        sums[r] = 0.0f;
-    }
-    wait_for_loads();
-    __syncthreads();
+    for (int r = 0; r < 16; ++r) totals[r] = cells[static_cast<size_t>((r >> 2) * 8 + (r & 3)) * a.width];
 
-    const float *left_rows = &deviation[0][0] + (lane >> 5) * kSmallTile + wave_row + (lane & 31);
-    const float *right_rows = &coefficient[0][0] + (lane >> 5) * kSmallTile + wave_column + (lane & 31);
-#pragma unroll 16
-    for (int kk = 0; kk < kWholeChain; kk += 2)
-        sums = __builtin_amdgcn_mfma_f32_32x32x2f32(left_rows[kk * kSmallTile], right_rows[kk * kSmallTile], sums, 0, 0, 0);
+    const uint32_t left_read = (lane >> 5) * kSmallTile + wave_row + (lane & 31);
+    const uint32_t right_read = (lane >> 5) * kSmallTile + wave_column + (lane & 31);
+    auto advance = [&](int step, auto odd) __attribute__((always_inline)) {
+        // The step's operands have landed for every wavefront, and every wavefront is done
+        // reading the other buffer (the step before): the next step's operands may overwrite it.
+        wait_for_loads();
+        __syncthreads();
+        if (step + 1 < steps) fetch(step + 1, std::bool_constant<!odd.value>{});
+        if ((step & 1) == 0) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r)
-        cells[static_cast<size_t>((r >> 2) * 8 + (r & 3)) * a.width] = __fadd_rn(totals[r], sums[r]);
+            for (int r = 0; r < 16; ++r) sums[r] = 0.0f;
+        }
+        const float *left_rows = (odd.value ? &deviation_odd[0][0] : &deviation_even[0][0]) + left_read;
+        const float *right_rows = (odd.value ? &coefficient_odd[0][0] : &coefficient_even[0][0]) + right_read;
+#pragma unroll 16
+        for (int kk = 0; kk < kSmallDepth; kk += 2)
+            sums = __builtin_amdgcn_mfma_f32_32x32x2f32(left_rows[kk * kSmallTile], right_rows[kk * kSmallTile], sums, 0, 0, 0);
+        if (step & 1) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) totals[r] = __fadd_rn(totals[r], sums[r]);
+        }
+    };
+    for (int step = 0; step < steps; step += 2) {  // a chain is two steps
+        advance(step, std::false_type{});
+        advance(step + 1, std::true_type{});
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) cells[static_cast<size_t>((r >> 2) * 8 + (r & 3)) * a.width] = totals[r];
 }
 
-int launch_update(const UpdateArgs &a, hipStream_t stream) {
+// Workgroup slots of block_update_from_deviations_kernel on the whole GPU (two per CU).
+constexpr int kUpdateSlots = 512;
+
+int launch_update(UpdateArgs a, hipStream_t stream) {
     MK_REQUIRE(mk_cdiv(a.rows, kTileRows) <= 65535, MK_ERR_UNSUPPORTED, "mk_feedback_block_update: too many rows");
     const dim3 grid(mk_cdiv(a.column_end - a.column_begin, kTileColumns), mk_cdiv(a.rows, kTileRows));
+    a.tile_first = 0;
+    a.column_tiles = static_cast<int>(grid.x);
     const auto aligned = [](const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15u) == 0; };
     const bool vec = a.width % 4 == 0 && a.first_column % 4 == 0 && a.chain_width % 4 == 0 && a.column_begin % 4 == 0 &&
                      aligned(a.original) && aligned(a.output) && aligned(a.coeff);
@@ -987,11 +1028,21 @@ int launch_update(const UpdateArgs &a, hipStream_t stream) {
                         (a.column_end - a.column_begin) % kTileColumns == 0 && a.chain_width % kDepthChunk == 0 &&
                         a.chain_width / kDepthChunk >= 4;   // the first chain spans the four steps that read feedback
     // (launches that leave most of the GPU idle with 128 x 128 tiles)
-    if (staged && a.chains == 1 && a.chain_width == kWholeChain && grid.x * grid.y <= 128)
-        hipLaunchKernelGGL(block_update_small_tile_kernel, dim3(grid.x * 2, grid.y * 2), dim3(kUpdateThreads), 0, stream, a);
-    else if (staged)
-        hipLaunchKernelGGL(block_update_from_deviations_kernel, grid, dim3(kUpdateThreads), 0, stream, a);
-    else if (vec)
+    const unsigned tiles = grid.x * grid.y;
+    if (staged && a.chains == 1 && a.chain_width == kWholeChain && tiles <= 128) {
+        hipLaunchKernelGGL(block_update_small_tile_kernel, dim3(tiles * 4), dim3(kUpdateThreads), 0, stream, a);
+    } else if (staged) {
+        // Whole rounds of workgroup slots on 128 x 128 tiles; a last round that would fill at most
+        // half of the slots runs as quarter tiles instead (chains of 128 columns only).
+        const unsigned tail = tiles % kUpdateSlots;
+        const bool split = a.chain_width == kWholeChain && tail > 0 && tail <= kUpdateSlots / 2;
+        const unsigned whole = split ? tiles - tail : tiles;
+        if (whole) hipLaunchKernelGGL(block_update_from_deviations_kernel, dim3(whole), dim3(kUpdateThreads), 0, stream, a);
+        if (split) {
+            a.tile_first = static_cast<int>(whole);
+            hipLaunchKernelGGL(block_update_small_tile_kernel, dim3(tail * 4), dim3(kUpdateThreads), 0, stream, a);
+        }
+    } else if (vec)
         hipLaunchKernelGGL((block_update_kernel<true>), grid, dim3(kUpdateThreads), 0, stream, a);
     else
         hipLaunchKernelGGL((block_update_kernel<false>), grid, dim3(kUpdateThreads), 0, stream, a);

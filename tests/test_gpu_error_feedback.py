@@ -132,6 +132,36 @@ def test_chained_block_update_equals_tile_after_tile(rows, width, first, chain, 
     np.testing.assert_array_equal(host(updated), expected)
 
 
+@pytest.mark.parametrize("rows,width,first,chain,chains,begin,end", [
+    (2048, 5120, 0, 128, 4, 512, 5120),     # 576 tiles: a whole round of 512 on large tiles, 64 as quarter tiles
+    (1024, 9216, 128, 128, 2, 384, 9216),   # 552 tiles, two chains
+    (2048, 5120, 0, 256, 2, 512, 5120),     # chains of 256 columns: large tiles throughout
+    (256, 1024, 0, 128, 4, 512, 1024),      # fewer tiles than slots
+    (256, 640, 128, 128, 1, 256, 512),      # one chain over a few tiles: quarter tiles only
+])
+def test_update_from_kept_deviations_equals_the_recomputing_update(rows, width, first, chain, chains, begin, end):
+    """mk_feedback_block_update_staged (deviations handed over column-major; whole rounds on
+    128 x 128 tiles, a short last round as 64 x 64 tiles) against mk_feedback_block_update_range,
+    which the test above pins to the oracle: the same sums, bit for bit."""
+    from mlkit_amd import native
+    from mlkit_amd.kernels import error_feedback
+
+    generator = torch.Generator(device="cuda").manual_seed(rows + width)
+    weight = torch.randn((rows, width), device="cuda", generator=generator) * 0.02
+    output = weight + torch.randn((rows, width), device="cuda", generator=generator) * 0.003
+    coeff = torch.randn((width, width), device="cuda", generator=generator).triu(1) * 0.05
+    feedback = torch.randn((rows, width), device="cuda", generator=generator) * 0.01
+    expected = feedback.clone()
+    error_feedback.block_update_range(expected, weight, output, coeff, first, chain, chains, begin, end)
+    deviations = (weight - output).T.contiguous()
+    updated = feedback.clone()
+    native.check(native.library().mk_feedback_block_update_staged(
+        updated.data_ptr(), deviations.data_ptr(), coeff.data_ptr(), rows, width, first, chain, chains, begin, end,
+        native.current_stream(updated.device)))
+    assert torch.equal(updated, expected)
+    assert torch.equal(updated[:, :begin], feedback[:, :begin])
+
+
 @pytest.mark.parametrize("width,step", [(1024, 1), (1100, 1), (1536, 8), (2304, 1)])
 def test_blocked_factorisation_matches_the_float64_coefficients(width, step):
     """`feedback_coefficients` on the device factors matrices of 1024 columns and more block by
