@@ -480,7 +480,7 @@ def other_kernels(device: torch.device, full: bool) -> dict:
     rotated = torch.empty_like(weight)
     fwht_ms = _time(lambda: hadamard.transform(weight.view(ROWS, 7, 2048), out=rotated.view(ROWS, 7, 2048)))
     out["fwht 4096x14336 fp32 as 7x2048 blocks"] = _entry(fwht_ms, elements * 8)
-    out["fwht_roofline"] = {"kernel": "fwht_kernel", "bound": "hbm", "achieved": elements * 8 / fwht_ms / 1e6,
+    out["fwht_roofline"] = {"kernel": "fwht_rows_kernel<32> (a row in the registers of one wavefront)", "bound": "hbm", "achieved": elements * 8 / fwht_ms / 1e6,
                             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": elements * 8 / fwht_ms / 1e6 / HBM_PEAK_GBPS,
                             "workload": "4096 x 14336 fp32 as 7 x 2048 blocks, read and written once"}
     tall = weight.view(WIDTH, ROWS)
