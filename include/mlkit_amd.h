@@ -346,6 +346,20 @@ int mk_feedback_sweep(const float *original, float *feedback, float *output, uin
                       float reciprocal, float value_minimum, int scale_format, int deferred_tiles,
                       void *stream);
 
+/* The matrix feedback_coefficients factors: target[a][b] = source[i(a)][i(b)] with
+ * i(a) = order[a] (int64 indices) or, with order NULL, width - 1 - a; on the diagonal a zero
+ * becomes one (a channel that was never activated) and *addend (one fp32 on the device: the
+ * damping) is added.  source, target: [width, width] fp32, distinct.
+ * Replaces: quantization/algorithms/error_feedback.py:55-66 (flip / index, masked_fill_, add_). */
+int mk_hessian_reversed(const float *source, float *target, int width, const long long *order,
+                        const float *addend, void *stream);
+
+/* Unit upper-triangular coefficients from the upper Cholesky factor U of the reversed matrix:
+ * out[a][b] = U[w-1-b][w-1-a] / U[w-1-b][w-1-b] (true division).  [width, width] fp32, distinct.
+ * Replaces: quantization/algorithms/error_feedback.py:72-75 for step == 1 (division of the
+ * lower factor's columns by its diagonal, flip back, contiguous copy). */
+int mk_unit_upper_from_factor(const float *factor, float *out, int width, void *stream);
+
 /* Index of the nearest codeword for `count` vectors of `dimension` (2, 4, 8 or 16) fp32
  * coordinates: the smallest sum over ascending coordinates of squared differences, the
  * lowest index on ties.  codebook: [codebook_size, dimension] fp32.  With lattice != 0 the

@@ -10,7 +10,9 @@
 //
 // Replaces the `torch.linalg.cholesky_ex` call of `feedback_coefficients`
 // (quantization/algorithms/error_feedback.py:37-83 in /root/reference/src/mlkit) for large
-// matrices on the device.
+// matrices on the device; mk_hessian_reversed and mk_unit_upper_from_factor are the tensor
+// operations in front of it and behind it (:55-66 index reversal and damping, :72-75 division
+// by the diagonal and reversal back), one pass over the matrix each.
 
 #include "mk_common.h"
 
@@ -47,8 +49,8 @@ constexpr int kRowFloats = 2 * kBlock;   // a published row: the block's columns
 //
 // ROW: the workgroup also carries 128 columns to the right of the block (`beside`), which take
 // the same row operations and so become U_jj^-T A_jr, the block row of the factor.
-template <int SIXTEEN, bool ROW>
-__device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[kTile][kTile], float (&beside)[kTile][kTile],
+template <int SIXTEEN, bool ROW, int BT>
+__device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[kTile][kTile], float (&beside)[kTile][BT],
                                               float (&pivot_rows)[2][2][kRowFloats], int tx, int ty) {
 #pragma unroll 1
     for (int lane = 0; lane < 16; lane += 2) {
@@ -82,10 +84,10 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
             columns_first[u] = first[k] * reciprocal;                                    // U[j][k]
             columns_second[u] = (second[k] - link * columns_first[u]) * next_reciprocal; // U[j+1][k]
         }
-        float beside_first[kTile], beside_second[kTile];
+        float beside_first[BT], beside_second[BT];
         if constexpr (ROW) {
 #pragma unroll
-            for (int v = 0; v < kTile; ++v) {
+            for (int v = 0; v < BT; ++v) {
                 const int c = kBlock + tx + 16 * v;
                 beside_first[v] = first[c] * reciprocal;
                 beside_second[v] = (second[c] - link * beside_first[v]) * next_reciprocal;
@@ -97,7 +99,7 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
             for (int v = SIXTEEN; v < kTile; ++v) mine[SIXTEEN][v] = columns_first[v];
             if constexpr (ROW) {
 #pragma unroll
-                for (int v = 0; v < kTile; ++v) beside[SIXTEEN][v] = beside_first[v];
+                for (int v = 0; v < BT; ++v) beside[SIXTEEN][v] = beside_first[v];
             }
         }
         if (ty == lane + 1) {
@@ -105,7 +107,7 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
             for (int v = SIXTEEN; v < kTile; ++v) mine[SIXTEEN][v] = columns_second[v];
             if constexpr (ROW) {
 #pragma unroll
-                for (int v = 0; v < kTile; ++v) beside[SIXTEEN][v] = beside_second[v];
+                for (int v = 0; v < BT; ++v) beside[SIXTEEN][v] = beside_second[v];
             }
         }
 #pragma unroll
@@ -115,7 +117,7 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
                 mine[u][v] -= rows_first[u] * columns_first[v] + rows_second[u] * columns_second[v];
             if constexpr (ROW) {
 #pragma unroll
-                for (int v = 0; v < kTile; ++v)
+                for (int v = 0; v < BT; ++v)
                     beside[u][v] -= rows_first[u] * beside_first[v] + rows_second[u] * beside_second[v];
             }
         }
@@ -127,7 +129,7 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
                 for (int v = SIXTEEN; v < kTile; ++v) next[ty - lane - 2][tx + 16 * v] = mine[SIXTEEN][v];   // columns < j are not read
                 if constexpr (ROW) {
 #pragma unroll
-                    for (int v = 0; v < kTile; ++v) next[ty - lane - 2][kBlock + tx + 16 * v] = beside[SIXTEEN][v];
+                    for (int v = 0; v < BT; ++v) next[ty - lane - 2][kBlock + tx + 16 * v] = beside[SIXTEEN][v];
                 }
             }
         } else if constexpr (SIXTEEN + 1 < kTile) {
@@ -136,7 +138,7 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
                 for (int v = SIXTEEN + 1; v < kTile; ++v) next[ty][tx + 16 * v] = mine[SIXTEEN + 1][v];
                 if constexpr (ROW) {
 #pragma unroll
-                    for (int v = 0; v < kTile; ++v) next[ty][kBlock + tx + 16 * v] = beside[SIXTEEN + 1][v];
+                    for (int v = 0; v < BT; ++v) next[ty][kBlock + tx + 16 * v] = beside[SIXTEEN + 1][v];
                 }
             }
         }
@@ -156,18 +158,20 @@ __device__ __forceinline__ bool sixteen_steps(const BlockArgs &a, float (&mine)[
 // reads the entries it needs, finishes the two rows for itself and subtracts their outer
 // products from its sub-block.  Rows up to the pivot rows are masked out of the update by
 // zero factors, so finished rows keep their values.
-template <bool ROW>
+// BT: sixteenths of 128 columns a workgroup carries beside the block (8: 128 columns, 4: 64).
+template <bool ROW, int BT>
 __global__ void __launch_bounds__(kThreads) cholesky_block_kernel(const BlockArgs a) {
     __shared__ float pivot_rows[2][2][kRowFloats];   // [buffer][row j, row j + 1][column]
     __shared__ int failed;
     const int n = a.size;
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     if (threadIdx.x == 0) failed = *a.status != 0;   // an earlier block already failed: do nothing
-    float mine[kTile][kTile], beside[kTile][kTile];
-    // ROW: workgroup b carries columns 128 b ... 128 b + 127 of the block row; every workgroup
+    float mine[kTile][kTile], beside[kTile][BT];
+    constexpr int kCarried = 16 * BT;
+    // ROW: workgroup b carries columns kCarried b ... kCarried (b + 1) - 1 of the block row; every workgroup
     // factors the block itself (from the matrix, which nobody overwrites: the factor goes to
     // `factor_out`), and the first one stores it.
-    const int beside_first_column = n + kBlock * blockIdx.x;
+    const int beside_first_column = n + kCarried * blockIdx.x;
 #pragma unroll
     for (int u = 0; u < kTile; ++u)
 #pragma unroll
@@ -177,32 +181,36 @@ __global__ void __launch_bounds__(kThreads) cholesky_block_kernel(const BlockArg
             const float loaded = a.matrix[(inside ? row : 0) * a.leading + (inside ? column : 0)];
             // Outside the block: an identity diagonal keeps every pivot of the padding at one.
             mine[u][v] = inside ? loaded : (row == column ? 1.0f : 0.0f);
-            beside[u][v] = 0.0f;
-            if constexpr (ROW) {
-                const bool present = row < n && kBlock * static_cast<int>(blockIdx.x) + column < a.row_columns;
-                const float carried = a.matrix[(present ? row : 0) * a.leading + (present ? beside_first_column + column : 0)];
-                beside[u][v] = present ? carried : 0.0f;
+            if (v < BT) {
+                beside[u][v] = 0.0f;
+                if constexpr (ROW) {
+                    const bool present = row < n && kCarried * static_cast<int>(blockIdx.x) + column < a.row_columns;
+                    const float carried = a.matrix[(present ? row : 0) * a.leading + (present ? beside_first_column + column : 0)];
+                    beside[u][v] = present ? carried : 0.0f;
+                }
             }
         }
     if (ty < 2) {
 #pragma unroll
         for (int v = 0; v < kTile; ++v) {
             pivot_rows[0][ty][tx + 16 * v] = mine[0][v];
-            if constexpr (ROW) pivot_rows[0][ty][kBlock + tx + 16 * v] = beside[0][v];
+            if constexpr (ROW) {
+                if (v < BT) pivot_rows[0][ty][kBlock + tx + 16 * v] = beside[0][v];
+            }
         }
     }
     __syncthreads();
     if (failed) return;
 
     // All 128 columns run (the padding is an identity): no data-dependent exit other than a bad pivot.
-    bool good = sixteen_steps<0, ROW>(a, mine, beside, pivot_rows, tx, ty);
-    good = good && sixteen_steps<1, ROW>(a, mine, beside, pivot_rows, tx, ty);
-    good = good && sixteen_steps<2, ROW>(a, mine, beside, pivot_rows, tx, ty);
-    good = good && sixteen_steps<3, ROW>(a, mine, beside, pivot_rows, tx, ty);
-    good = good && sixteen_steps<4, ROW>(a, mine, beside, pivot_rows, tx, ty);
-    good = good && sixteen_steps<5, ROW>(a, mine, beside, pivot_rows, tx, ty);
-    good = good && sixteen_steps<6, ROW>(a, mine, beside, pivot_rows, tx, ty);
-    good = good && sixteen_steps<7, ROW>(a, mine, beside, pivot_rows, tx, ty);
+    bool good = sixteen_steps<0, ROW, BT>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<1, ROW, BT>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<2, ROW, BT>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<3, ROW, BT>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<4, ROW, BT>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<5, ROW, BT>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<6, ROW, BT>(a, mine, beside, pivot_rows, tx, ty);
+    good = good && sixteen_steps<7, ROW, BT>(a, mine, beside, pivot_rows, tx, ty);
     if (!good) return;
     float *factor = ROW ? a.factor_out : a.matrix;
     const long long factor_leading = ROW ? kBlock : a.leading;
@@ -213,13 +221,96 @@ __global__ void __launch_bounds__(kThreads) cholesky_block_kernel(const BlockArg
             const int row = ty + 16 * u, column = tx + 16 * v;
             if (blockIdx.x == 0 && row < n && column < n) factor[row * factor_leading + column] = column >= row ? mine[u][v] : 0.0f;
             if constexpr (ROW) {
-                if (row < n && kBlock * static_cast<int>(blockIdx.x) + column < a.row_columns)
+                if (v < BT && row < n && kCarried * static_cast<int>(blockIdx.x) + column < a.row_columns)
                     a.matrix[row * a.leading + beside_first_column + column] = beside[u][v];
             }
         }
 }
 
 }  // namespace
+
+// ---- the matrix that goes into the factorisation, and the coefficients that come out ---------
+
+struct ReverseArgs {
+    const float *source;
+    float *target;
+    const long long *order;  // null: index a reads row / column width - 1 - a
+    const float *addend;     // one float: added to every diagonal entry (after zeros became ones)
+    int width;
+};
+
+// target[a][b] = source[i(a)][i(b)]; on the diagonal a zero becomes one and *addend is added.
+__global__ void __launch_bounds__(256) reversed_matrix_kernel(const ReverseArgs a) {
+    const int row = blockIdx.y;
+    const int column = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (column >= a.width) return;
+    const long long source_row = a.order ? a.order[row] : a.width - 1 - row;
+    const float *from = a.source + static_cast<size_t>(source_row) * a.width;
+    float values[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int b = column + i;
+        const bool inside = b < a.width;
+        const long long source_column = a.order ? a.order[inside ? b : 0] : a.width - 1 - (inside ? b : 0);
+        float value = from[source_column];
+        if (b == row) value = __fadd_rn(value == 0.0f ? 1.0f : value, *a.addend);
+        values[i] = value;
+    }
+    float *to = a.target + static_cast<size_t>(row) * a.width + column;
+    if (column + 3 < a.width && (a.width & 3) == 0) {
+        *reinterpret_cast<float4 *>(to) = make_float4(values[0], values[1], values[2], values[3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (column + i < a.width) to[i] = values[i];
+    }
+}
+
+// out[a][b] = U[w-1-b][w-1-a] / U[w-1-b][w-1-b]: the factor transposed, every column divided by
+// its diagonal entry, both index orders reversed; 32 x 32 tiles turned in LDS so that reads and
+// writes both run along rows.
+__global__ void __launch_bounds__(256) unit_upper_kernel(const float *factor, float *out, int width) {
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 8 rows of 32 threads
+    const int r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int r = r0 + ty + 8 * j, c = c0 + tx;
+        const bool inside = r < width && c < width;
+        const float value = factor[static_cast<size_t>(inside ? r : 0) * width + (inside ? c : 0)];
+        const float pivot = factor[static_cast<size_t>(inside ? r : 0) * (width + 1)];
+        tile[ty + 8 * j][tx] = inside ? __fdiv_rn(value, pivot) : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int c = c0 + ty + 8 * j, r = r0 + tx;   // tile[r - r0][c - c0] goes to out[w-1-c][w-1-r]
+        if (r < width && c < width)
+            out[static_cast<size_t>(width - 1 - c) * width + (width - 1 - r)] = tile[tx][ty + 8 * j];
+    }
+}
+
+extern "C" int mk_hessian_reversed(const float *source, float *target, int width, const long long *order,
+                                   const float *addend, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(source && target && addend, MK_ERR_INVALID, "mk_hessian_reversed: null pointer");
+    MK_REQUIRE(width >= 1 && width <= 65535, MK_ERR_INVALID, "mk_hessian_reversed: width out of range");
+    MK_REQUIRE(source != target, MK_ERR_INVALID, "mk_hessian_reversed: source and target must not alias");
+    ReverseArgs a{source, target, order, addend, width};
+    hipLaunchKernelGGL(reversed_matrix_kernel, dim3(mk_cdiv(width, 1024), width), dim3(256), 0, stream, a);
+    MK_LAUNCH_CHECK("mk_hessian_reversed");
+    return MK_OK;
+}
+
+extern "C" int mk_unit_upper_from_factor(const float *factor, float *out, int width, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MK_REQUIRE(factor && out, MK_ERR_INVALID, "mk_unit_upper_from_factor: null pointer");
+    MK_REQUIRE(width >= 1 && width <= 65535 * 32, MK_ERR_INVALID, "mk_unit_upper_from_factor: width out of range");
+    MK_REQUIRE(factor != out, MK_ERR_INVALID, "mk_unit_upper_from_factor: factor and out must not alias");
+    hipLaunchKernelGGL(unit_upper_kernel, dim3(mk_cdiv(width, 32), mk_cdiv(width, 32)), dim3(256), 0, stream, factor, out, width);
+    MK_LAUNCH_CHECK("mk_unit_upper_from_factor");
+    return MK_OK;
+}
 
 extern "C" int mk_cholesky_block(float *matrix, long long leading, int size, int first_column, int row_columns,
                                  float *factor_out, int *status, void *stream_) {
@@ -231,10 +322,14 @@ extern "C" int mk_cholesky_block(float *matrix, long long leading, int size, int
     MK_REQUIRE(row_columns == 0 || factor_out, MK_ERR_INVALID,
                "mk_cholesky_block: a block row needs a separate place for the factor");
     BlockArgs a{matrix, leading, size, first_column, status, row_columns, factor_out};
-    if (row_columns > 0)
-        hipLaunchKernelGGL(cholesky_block_kernel<true>, dim3(mk_cdiv(row_columns, kBlock)), dim3(kThreads), 0, stream, a);
+    // 64 columns per workgroup while that still fits one workgroup per CU (a step then costs a
+    // third less arithmetic); 128 beyond.
+    if (row_columns > 256 * 64)
+        hipLaunchKernelGGL((cholesky_block_kernel<true, 8>), dim3(mk_cdiv(row_columns, 128)), dim3(kThreads), 0, stream, a);
+    else if (row_columns > 0)
+        hipLaunchKernelGGL((cholesky_block_kernel<true, 4>), dim3(mk_cdiv(row_columns, 64)), dim3(kThreads), 0, stream, a);
     else
-        hipLaunchKernelGGL(cholesky_block_kernel<false>, dim3(1), dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL((cholesky_block_kernel<false, 4>), dim3(1), dim3(kThreads), 0, stream, a);
     MK_LAUNCH_CHECK("mk_cholesky_block");
     return MK_OK;
 }

@@ -120,6 +120,8 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
         _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
         _c_int, _c_void_p,
     ]),
+    "mk_hessian_reversed": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p]),
+    "mk_unit_upper_from_factor": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p]),
     "mk_vector_nearest": (_c_int, [
         _c_void_p, _c_longlong, _c_int, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
     ]),

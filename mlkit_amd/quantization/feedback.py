@@ -42,60 +42,87 @@ TRAILING_BAND = 1024                # rows per product of a trailing update (onl
 LOOK_AHEAD_WIDTH = 8192             # from here on the far part of a trailing update runs on a second stream
 
 
-def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
-    """``(U, status)`` with ``matrix = U^T U`` for a symmetric positive definite FP32 matrix on a
-    HIP device, factored in place.  Two levels of right-looking blocking: panels of 1024 columns
-    update the rest of the matrix (a rank-1024 product reads and writes the trailing matrix an
-    eighth as often as rank-128 ones would); inside a panel's diagonal block the same scheme
-    runs with 128-column blocks: ``mk_cholesky_block`` factors a diagonal block and carries the
-    rest of its rows, to the last column, through the same elimination, which makes them the
-    factor's block row; no triangular solve is left.
+def _factor_in_place(matrix: Tensor, status: Tensor, factored: Tensor) -> None:
+    """``matrix = U^T U`` for a symmetric positive definite FP32 matrix on a HIP device, factored
+    in place (``status``: an int32 device scalar holding zero; ``factored``: scratch for the
+    diagonal blocks, ``[ceil(width / 128), 128, 128]``).
 
-    Look-ahead: of a panel's trailing update only the band of rows the next panel consists of
-    runs on the current stream; the rest runs on a second stream while the next panel's
-    diagonal block, a chain of small dependent kernels, is factored.  Events fix the order in
-    which updates reach every entry, so results do not depend on timing.
+    Two levels of right-looking blocking: panels of 1024 columns update the rest of the matrix (a
+    rank-1024 product reads and writes the trailing matrix an eighth as often as rank-128 ones
+    would); inside a panel's diagonal block the same scheme runs with 128-column blocks:
+    ``mk_cholesky_block`` factors a diagonal block and carries the rest of its rows, to the last
+    column, through the same elimination, which makes them the factor's block row; no triangular
+    solve is left.  The factored diagonal blocks themselves are needed by nobody before the end
+    (updates read block rows only): they wait in ``factored`` and go into the matrix in one copy.
 
-    ``status`` is a device scalar: zero, or one plus the first column whose pivot is not
-    positive (as ``torch.linalg.cholesky_ex`` reports it)."""
+    Look-ahead, on two levels.  Inside a panel, a block's update of the rows of the *next* block
+    runs on the current stream and the next block kernel follows at once; its update of the
+    panel's remaining rows runs on a second stream meanwhile.  Between panels, only the band of
+    rows the next panel consists of is updated on the current stream; the rest runs on a third
+    stream while the next panel is factored.  Events fix the order in which updates reach every
+    entry, so results do not depend on timing (and are the same with all work on one stream).
+
+    ``status`` stays zero, or becomes one plus the first column whose pivot is not positive (as
+    ``torch.linalg.cholesky_ex`` reports it).  Nothing here allocates device memory or reads
+    anything back, so the whole sequence can be captured in a HIP graph."""
     from mlkit_amd import native
 
     width = matrix.shape[0]
     device = matrix.device
     library = native.library()
-    status = torch.zeros((), dtype=torch.int32, device=device)
-    factored = torch.empty((FACTORIZATION_BLOCK, FACTORIZATION_BLOCK), dtype=torch.float32, device=device)
     main = torch.cuda.current_stream(device)
     look_ahead = width >= LOOK_AHEAD_WIDTH   # narrower: the event traffic costs more than it hides
-    side = torch.cuda.Stream(device) if look_ahead else None
+    side = torch.cuda.Stream(device) if look_ahead else None    # far rows of a panel's update
+    inner = torch.cuda.Stream(device) if look_ahead else None   # remaining rows of a block's update inside its panel
 
-    def subtract_outer_product(start: int, stop: int, first_row: int, last_row: int, limit: int) -> None:
+    def subtract_outer_product(start: int, stop: int, first_row: int, last_row: int, limit: int, after_first_band=None):
         """A[r, c] -= sum_k U[k, r] U[k, c] for k in start:stop, rows first_row:last_row, columns from
         the row band's first column to ``limit``: bands of rows, so that little below the diagonal
-        is computed (what is, is never read)."""
+        is computed (what is, is never read).  ``after_first_band`` (a stream): returns an event
+        recorded on it behind the first band."""
+        event = None
         for band_start in range(first_row, last_row, TRAILING_BAND):
             band_stop = min(last_row, band_start + TRAILING_BAND)
             matrix[band_start:band_stop, band_start:limit].addmm_(
                 matrix[start:stop, band_start:band_stop].T, matrix[start:stop, band_start:limit], alpha=-1.0)
+            if after_first_band is not None and event is None:
+                event = after_first_band.record_event()
+        return event
 
-    side_done = None
+    side_done = band_done = None
     for panel_start in range(0, width, FACTORIZATION_PANEL):
         panel_stop = min(width, panel_start + FACTORIZATION_PANEL)
         raw_stream = native.current_stream(device)
+        inner_done = None
         for start in range(panel_start, panel_stop, FACTORIZATION_BLOCK):
             stop = min(panel_stop, start + FACTORIZATION_BLOCK)
             # the block kernel also carries the rest of rows start:stop, to the matrix's last column,
-            # through the elimination (their block row of the factor); the factored block comes back
-            # through `factored`, since every workgroup of that launch reads the block itself
+            # through the elimination (their block row of the factor); the factored block goes to
+            # `factored`, since every workgroup of that launch reads the block itself
             beside = width - stop
+            slot = factored[start // FACTORIZATION_BLOCK]
             native.check(library.mk_cholesky_block(matrix[start, start:].data_ptr(), width, stop - start, start, beside,
-                                                   factored.data_ptr() if beside else None, status.data_ptr(), raw_stream))
-            if beside:
-                matrix[start:stop, start:stop].copy_(factored[: stop - start, : stop - start])
-            if stop < panel_stop:
-                # the rest of the panel's rows, over all columns to the right: what a triangular
-                # solve with the panel's whole diagonal block would otherwise do for them
-                subtract_outer_product(start, stop, stop, panel_stop, width)
+                                                   slot.data_ptr() if beside else None, status.data_ptr(), raw_stream))
+            if stop >= panel_stop:
+                continue
+            # the rest of the panel's rows, over all columns to the right (what a triangular solve
+            # with the panel's whole diagonal block would otherwise do for them): the next block's
+            # rows now, after the earlier blocks' updates of them; the others beside the next block
+            next_stop = min(panel_stop, stop + FACTORIZATION_BLOCK)
+            if inner_done is not None:
+                main.wait_event(inner_done)
+            subtract_outer_product(start, stop, stop, next_stop, width)
+            if next_stop >= panel_stop:
+                continue
+            if not look_ahead:
+                subtract_outer_product(start, stop, next_stop, panel_stop, width)
+                continue
+            inner.wait_event(main.record_event())   # (also behind this block's update of the next rows: harmless)
+            with torch.cuda.stream(inner):
+                subtract_outer_product(start, stop, next_stop, panel_stop, width)
+                inner_done = inner.record_event()
+        if inner_done is not None:
+            main.wait_event(inner_done)
         # the diagonal block's lower triangle holds leftovers of the products above
         matrix[panel_start:panel_stop, panel_start:panel_stop].triu_()
         if panel_stop == width:
@@ -104,19 +131,85 @@ def _blocked_upper_factor(matrix: Tensor) -> tuple[Tensor, Tensor]:
             subtract_outer_product(panel_start, panel_stop, panel_stop, width, width)
             continue
         row_ready = main.record_event()
-        # the rows of the next panel: here, after the second stream's earlier update of them
-        next_stop = min(width, panel_stop + FACTORIZATION_PANEL)
-        if side_done is not None:
-            main.wait_event(side_done)
-        subtract_outer_product(panel_start, panel_stop, panel_stop, next_stop, width)
-        if next_stop < width:
+        # the rows of the next panel: here, after the third stream's earlier update of them (its
+        # first band: the stream works through the bands from the top, and through the panels in
+        # order, so that band being done means every earlier update of these rows is)
+        next_panel_stop = min(width, panel_stop + FACTORIZATION_PANEL)
+        if band_done is not None:
+            main.wait_event(band_done)
+        subtract_outer_product(panel_start, panel_stop, panel_stop, next_panel_stop, width)
+        if next_panel_stop < width:
             side.wait_event(row_ready)
             with torch.cuda.stream(side):
-                subtract_outer_product(panel_start, panel_stop, next_stop, width, width)
+                band_done = subtract_outer_product(panel_start, panel_stop, next_panel_stop, width, width, after_first_band=side)
                 side_done = side.record_event()
     if side_done is not None:
         main.wait_event(side_done)
+    # the factored diagonal blocks (all but a last block that has no columns beside it, factored in place)
+    whole = (width - 1) // FACTORIZATION_BLOCK
+    if whole:
+        diagonal = matrix.as_strided((whole, FACTORIZATION_BLOCK, FACTORIZATION_BLOCK),
+                                     (FACTORIZATION_BLOCK * (width + 1), width, 1))
+        diagonal.copy_(factored[:whole])
+
+
+def _factor_scratch(width: int, device: torch.device) -> Tensor:
+    return torch.empty((-(-width // FACTORIZATION_BLOCK), FACTORIZATION_BLOCK, FACTORIZATION_BLOCK), dtype=torch.float32,
+                       device=device)
+
+
+class _FactorGraph:
+    """The launches of ``_factor_in_place`` for one width, captured once: several hundred small
+    launches cost more to issue from Python than to run, and they are the same for every matrix
+    of that width.  The graph owns the buffer it factors in."""
+
+    def __init__(self, width: int, device: torch.device) -> None:
+        self.matrix = torch.empty((width, width), dtype=torch.float32, device=device)
+        self.status = torch.zeros((), dtype=torch.int32, device=device)
+        self.factored = _factor_scratch(width, device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.status.zero_()   # a fill kernel
+            _factor_in_place(self.matrix, self.status, self.factored)
+
+    def __call__(self, fill: Callable[[Tensor], None]) -> tuple[Tensor, Tensor]:
+        fill(self.matrix)
+        self.graph.replay()
+        return self.matrix, self.status
+
+
+FACTOR_GRAPHS = True        # capture the factorisation of a width the second time it is asked for
+FACTOR_GRAPH_LIMIT = 2      # graphs (and their width x width buffers) kept per process
+_factor_graphs: dict[tuple[int, int], "_FactorGraph | None"] = {}
+
+
+def clear_factor_graphs() -> None:
+    """Drop the captured factorisations and their buffers."""
+    _factor_graphs.clear()
+
+
+def _blocked_upper_factor(fill: Callable[[Tensor], None], width: int, device: torch.device) -> tuple[Tensor, Tensor]:
+    """``(U, status)`` with ``U^T U`` = the matrix that ``fill(target)`` writes into a
+    ``[width, width]`` FP32 tensor.  The first matrix of a width is factored launch by launch
+    (which also warms every kernel up); from the second on the captured graph of that width
+    runs.  The result may live in the graph's own buffer: it is valid until the next call."""
+    key = (device.index or 0, width)
+    if FACTOR_GRAPHS and key in _factor_graphs and not torch.cuda.is_current_stream_capturing():
+        graph = _factor_graphs[key]
+        if graph is None:
+            while sum(entry is not None for entry in _factor_graphs.values()) >= FACTOR_GRAPH_LIMIT:
+                oldest = next(k for k, entry in _factor_graphs.items() if entry is not None)
+                del _factor_graphs[oldest]
+            graph = _factor_graphs[key] = _FactorGraph(width, device)
+        return graph(fill)
+    _factor_graphs.setdefault(key, None)   # seen once
+    matrix = torch.empty((width, width), dtype=torch.float32, device=device)
+    fill(matrix)
+    status = torch.zeros((), dtype=torch.int32, device=device)
+    _factor_in_place(matrix, status, _factor_scratch(width, device))
     return matrix, status
+
+
 
 
 def feedback_coefficients(hessian: Tensor, step: int, *, damp: float = 0.01,
@@ -129,6 +222,8 @@ def feedback_coefficients(hessian: Tensor, step: int, *, damp: float = 0.01,
     reversed back, is the upper factor ``R``.
     """
     width = hessian.shape[0]
+    if width >= BLOCKED_FACTORIZATION_WIDTH and hessian.is_cuda and hessian.dtype == torch.float32:
+        return _coefficients_on_kernels(hessian, step, damp, permutation)
     if permutation is None:
         flipped = hessian.flip(0, 1)
     else:
@@ -137,18 +232,48 @@ def feedback_coefficients(hessian: Tensor, step: int, *, damp: float = 0.01,
     diagonal = flipped.diagonal()
     diagonal.masked_fill_(diagonal == 0, 1)
     diagonal.add_(damp * diagonal.mean().clamp_min(1e-12))
-    if width >= BLOCKED_FACTORIZATION_WIDTH and flipped.is_cuda and flipped.dtype == torch.float32:
-        flipped = flipped.contiguous()  # a fresh copy (flip / indexing never alias the caller's matrix)
-        factor, status = _blocked_upper_factor(flipped)
-        lower = factor.T
-    elif width >= UPPER_FACTORIZATION_WIDTH:
+    if width >= UPPER_FACTORIZATION_WIDTH:
         # column-major solvers factor the upper triangle faster; its transpose is the lower factor
         factor, status = torch.linalg.cholesky_ex(flipped, upper=True)
         lower = factor.T
     else:
         lower, status = torch.linalg.cholesky_ex(flipped)
+    return _coefficients_of(lower, status, step)
+
+
+def _coefficients_on_kernels(hessian: Tensor, step: int, damp: float, permutation: Tensor | None) -> tuple[Tensor, int]:
+    """The same on a HIP device for matrices of 1024 columns and more: one pass writes the
+    reversed, damped matrix where it is factored (``mk_hessian_reversed``), the blocked
+    factorisation runs, and for ``step == 1`` one pass turns the factor into the coefficients
+    (``mk_unit_upper_from_factor``)."""
+    from mlkit_amd import native
+
+    width, device = hessian.shape[0], hessian.device
+    source = hessian.contiguous()
+    order = None if permutation is None else permutation.flip(0).to(torch.int64).contiguous()
+    ones_for_zeros = source.diagonal().clone()
+    ones_for_zeros.masked_fill_(ones_for_zeros == 0, 1)
+    addend = (damp * ones_for_zeros.mean().clamp_min(1e-12)).reshape(1).float()
+    library = native.library()
+
+    def fill(target: Tensor) -> None:
+        native.check(library.mk_hessian_reversed(source.data_ptr(), target.data_ptr(), width, native.pointer(order),
+                                                 addend.data_ptr(), native.current_stream(device)))
+
+    factor, status = _blocked_upper_factor(fill, width, device)
+    if step == 1 and int(status.item()) == 0:
+        coefficients = torch.empty_like(factor)
+        native.check(library.mk_unit_upper_from_factor(factor.data_ptr(), coefficients.data_ptr(), width,
+                                                       native.current_stream(device)))
+        return coefficients, 0
+    return _coefficients_of(factor.T, status, step)
+
+
+def _coefficients_of(lower: Tensor, status: Tensor, step: int) -> tuple[Tensor, int]:
+    """``R blockdiag(R)^-1`` from the lower factor of the index-reversed matrix."""
+    width = lower.shape[0]
     if int(status.item()) != 0:
-        return lower, int(status.item())
+        return lower.clone(), int(status.item())
     if step == 1:
         lower = lower / lower.diagonal().clone()
         return lower.flip(0, 1).contiguous(), 0

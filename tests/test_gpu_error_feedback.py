@@ -202,6 +202,7 @@ def test_look_ahead_factorisation_equals_the_one_stream_order(width, monkeypatch
     inputs = rng.standard_normal((2 * width, width)).astype(np.float32)
     inputs[:, ::7] *= 4
     hessian = dev((inputs.T @ inputs / inputs.shape[0]).astype(np.float32))
+    monkeypatch.setattr(feedback, "FACTOR_GRAPHS", False)       # launch by launch, with the constants set here
     monkeypatch.setattr(feedback, "FACTORIZATION_PANEL", 256)   # several panels at these widths
     monkeypatch.setattr(feedback, "LOOK_AHEAD_WIDTH", 1 << 30)
     expected, status = mk.feedback_coefficients(hessian.clone(), 1)
@@ -211,6 +212,50 @@ def test_look_ahead_factorisation_equals_the_one_stream_order(width, monkeypatch
         result, status = mk.feedback_coefficients(hessian.clone(), 1)
         assert status == 0
         np.testing.assert_array_equal(np.triu(host(result), 1), np.triu(host(expected), 1))
+
+
+@pytest.mark.parametrize("look_ahead", [False, True])
+def test_captured_factorisation_equals_the_launch_by_launch_one(look_ahead, monkeypatch):
+    """From the second matrix of a width on, the factorisation replays a captured graph.  Five
+    different matrices of one width, with eager work and synchronisations between the replays and
+    another width in between: every result equals the one computed launch by launch, bit for bit
+    above the diagonal; an indefinite matrix reports its column through the graph as well."""
+    import mlkit_amd as mk
+    from mlkit_amd.quantization import feedback
+
+    feedback.clear_factor_graphs()
+    monkeypatch.setattr(feedback, "FACTORIZATION_PANEL", 512)
+    monkeypatch.setattr(feedback, "LOOK_AHEAD_WIDTH", 1024 if look_ahead else 1 << 30)
+    width = 1664
+    generator = torch.Generator(device="cuda").manual_seed(11)
+
+    def hessian_of(scale):
+        inputs = torch.randn((2 * width, width), device="cuda", generator=generator) * scale
+        inputs[:, ::9] *= 3
+        return inputs.T @ inputs / inputs.shape[0]
+
+    try:
+        matrices = [hessian_of(1.0 + 0.5 * index) for index in range(5)]
+        monkeypatch.setattr(feedback, "FACTOR_GRAPHS", False)
+        expected = [mk.feedback_coefficients(matrix.clone(), 1)[0] for matrix in matrices]
+        monkeypatch.setattr(feedback, "FACTOR_GRAPHS", True)
+        other = hessian_of(2.0)[:1280, :1280].contiguous()
+        for index, matrix in enumerate(matrices):
+            result, status = mk.feedback_coefficients(matrix.clone(), 1)
+            assert status == 0
+            assert torch.equal(result.triu(1), expected[index].triu(1)), index
+            busy = (matrix @ matrix).sum()            # eager work and a synchronisation between replays
+            torch.cuda.synchronize()
+            assert torch.isfinite(busy)
+            if index == 2:
+                mk.feedback_coefficients(other.clone(), 1)   # another width in between
+        assert feedback._factor_graphs[(0, width)] is not None
+        broken = matrices[0].clone()
+        broken[900, 900] = -1e6
+        assert mk.feedback_coefficients(broken, 1, damp=0.0)[1] != 0
+        assert mk.feedback_coefficients(matrices[1].clone(), 1)[1] == 0   # the status starts from zero again
+    finally:
+        feedback.clear_factor_graphs()
 
 
 def test_blocked_factorisation_reports_an_indefinite_matrix():
