@@ -261,6 +261,10 @@ def gptq_layer(device: torch.device, generator: torch.Generator, cpu_rows: int =
     feedback.feedback_coefficients = lambda *args, **kwargs: ready
     try:
         sweep_ms = wall_ms(lambda: quantizer(target, Ctx("down_proj", H=hessian)))
+        # the same sweep on a table of sixteen values (NF4, one scale per 64 columns)
+        table_quantizer = mk.gptq(mk.nf4(group=64))
+        table_quantizer(target, Ctx("warmup", H=hessian))
+        table_sweep_ms = wall_ms(lambda: table_quantizer(target, Ctx("down_proj", H=hessian)))
     finally:
         feedback.feedback_coefficients = original
     update_flops = sum(2 * rows * block * (width - stop) for stop in range(block, width, block))
@@ -268,6 +272,7 @@ def gptq_layer(device: torch.device, generator: torch.Generator, cpu_rows: int =
     out = {
         "total_ms": total_ms, "coefficients_ms": factor_ms, "sweep_and_update_ms": sweep_ms,
         "columns_per_s": width / (sweep_ms / 1e3), "weights_per_s": rows * width / (sweep_ms / 1e3),
+        "nf4_g64_sweep_and_update_ms": table_sweep_ms,
         "trailing_update_flops": update_flops,
         "proxy_loss": float(mk.proxy_loss(target, result.w, hessian)),
         "rtn_proxy_loss": float(mk.proxy_loss(target, rtn.w, hessian)),

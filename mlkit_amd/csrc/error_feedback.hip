@@ -292,10 +292,41 @@ __device__ __forceinline__ float row_value(float value, std::integral_constant<i
 // memory straight into LDS before the first step (row-major; one memory latency for the
 // whole kernel instead of one per slot).  Otherwise the sixteen steps of a slot are a loop
 // over coefficient rows staged slot by slot.
-template <int MODE, bool WHOLE>
+// The nearest of up to sixteen table values by (distance, index): every lane compares its own
+// value with all sixteen at once -- differences, then a tournament in which the entry with the
+// higher index wins only on a strictly smaller distance.  Entries beyond the table are NaN and
+// never win.  The same answer as a scan in ascending index order that keeps the first minimum.
+constexpr int kSmallTable = 16;
+
+struct Nearest {
+    float difference, value;
+    uint32_t index;
+};
+
+template <int COUNT>
+__device__ __forceinline__ Nearest nearest_of(const Nearest (&entries)[COUNT]) {
+    if constexpr (COUNT == 1) {
+        return entries[0];
+    } else {
+        Nearest winners[COUNT / 2];
+#pragma unroll
+        for (int i = 0; i < COUNT / 2; ++i) {
+            const Nearest &low = entries[2 * i], &high = entries[2 * i + 1];
+            const bool take = fabsf(high.difference) < fabsf(low.difference);
+            winners[i].difference = take ? high.difference : low.difference;
+            winners[i].value = take ? high.value : low.value;
+            winners[i].index = take ? high.index : low.index;
+        }
+        return nearest_of<COUNT / 2>(winners);
+    }
+}
+
+// TABLE: 0 rounds to an integer grid; kSmallTable rounds to a table of at most sixteen values.
+template <int MODE, bool WHOLE, int TABLE = 0>
 __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const SweepArgs a) {
     static_assert(MODE == kModeInteger || MODE == kModeSolve || (MODE == kModeRegion && WHOLE),
-                  "codebooks use the one-row-per-wavefront kernel; a fused region is one whole tile");
+                  "larger tables use the one-row-per-wavefront kernel; a fused region is one whole tile");
+    static_assert(TABLE == 0 || (TABLE == kSmallTable && MODE != kModeSolve), "a table of sixteen values, or none");
     constexpr int kStaged = WHOLE ? kNarrowTile * kNarrowTile : 2 * kRowLanes * kNarrowTile;
     __shared__ __attribute__((aligned(16))) float staged[kStaged];
     const int lane = threadIdx.x & 63;
@@ -305,6 +336,12 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
     const bool active = wanted_row < a.rows;
     const int row = active ? wanted_row : a.rows - 1;
     const size_t row_base = static_cast<size_t>(row) * a.width;
+
+    float table[TABLE > 0 ? TABLE : 1];
+    if constexpr (TABLE > 0) {
+#pragma unroll
+        for (int i = 0; i < TABLE; ++i) table[i] = i < a.n_values ? a.values[i < a.n_values ? i : 0] : __builtin_nanf("");
+    }
 
     float held[kNarrowHeld];
     if constexpr (WHOLE) {
@@ -371,8 +408,23 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
         } else {
             const float target = __fadd_rn(weight[t], running[t]);
             const float normalized = __fdiv_rn(__fsub_rn(target, zero[t]), scale[t]);
-            const float chosen = fminf(fmaxf(rintf(normalized), a.code_min), a.code_max);
-            const uint32_t index = static_cast<uint32_t>(static_cast<int>(__fsub_rn(chosen, a.code_min)));
+            float chosen;
+            uint32_t index;
+            if constexpr (TABLE > 0) {
+                Nearest entries[TABLE];
+#pragma unroll
+                for (int i = 0; i < TABLE; ++i) {
+                    entries[i].difference = __fsub_rn(normalized, table[i]);
+                    entries[i].value = table[i];
+                    entries[i].index = i;
+                }
+                const Nearest nearest = nearest_of<TABLE>(entries);
+                chosen = nearest.value;
+                index = nearest.index;
+            } else {
+                chosen = fminf(fmaxf(rintf(normalized), a.code_min), a.code_max);
+                index = static_cast<uint32_t>(static_cast<int>(__fsub_rn(chosen, a.code_min)));
+            }
             const float reconstruction = __fadd_rn(__fmul_rn(chosen, scale[t]), zero[t]);
             const bool mine = p == static_cast<int>(owner);
             finished[t] = mine ? reconstruction : finished[t];
@@ -542,14 +594,15 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
 
 // One kernel for a region that is a single whole tile of an integer grid: pending solve,
 // scale fit and column sweep.
-bool region_fusable(int span, int block, int fitted_group, bool integer_grid) {
-    return integer_grid && span == kNarrowTile && block >= kNarrowTile && fitted_group % kRowLanes == 0 &&
-           kNarrowTile % fitted_group == 0;
+bool region_fusable(int span, int block, int fitted_group, bool integer_grid, int n_values) {
+    return (integer_grid || n_values <= kSmallTable) && span == kNarrowTile && block >= kNarrowTile &&
+           fitted_group % kRowLanes == 0 && kNarrowTile % fitted_group == 0;
 }
 
-int launch_region(const SweepArgs &a, hipStream_t stream) {
-    hipLaunchKernelGGL((narrow_sweep_kernel<kModeRegion, true>), dim3(mk_cdiv(a.rows, kNarrowRows)), dim3(kSweepThreads), 0,
-                       stream, a);
+int launch_region(const SweepArgs &a, bool integer_grid, hipStream_t stream) {
+    const dim3 grid(mk_cdiv(a.rows, kNarrowRows)), block(kSweepThreads);
+    if (integer_grid) hipLaunchKernelGGL((narrow_sweep_kernel<kModeRegion, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((narrow_sweep_kernel<kModeRegion, true, kSmallTable>), grid, block, 0, stream, a);
     return MK_OK;
 }
 
@@ -565,6 +618,14 @@ int launch_sweep(const SweepArgs &a, hipStream_t stream) {
                 hipLaunchKernelGGL((narrow_sweep_kernel<MODE, false>), narrow_grid, block, 0, stream, a);
             return MK_OK;
         }
+    } else if (a.tile_width <= kNarrowTile && a.n_values <= kSmallTable) {
+        // small tables (NF4, FP4, ...): sixteen lanes per row, every lane searching the table for itself
+        const dim3 narrow_grid(mk_cdiv(a.rows, kNarrowRows));
+        if (a.tile_width == kNarrowTile)
+            hipLaunchKernelGGL((narrow_sweep_kernel<kModeInteger, true, kSmallTable>), narrow_grid, block, 0, stream, a);
+        else
+            hipLaunchKernelGGL((narrow_sweep_kernel<kModeInteger, false, kSmallTable>), narrow_grid, block, 0, stream, a);
+        return MK_OK;
     }
     if (a.tile_width <= 128)
         hipLaunchKernelGGL((sweep_kernel<2, MODE>), grid, block, 0, stream, a);
@@ -1231,7 +1292,7 @@ extern "C" int mk_feedback_sweep(const float *original, float *feedback, float *
         }
         float *region_scales = scales + group_offset;
         float *region_zeros = asym ? zeros + group_offset : nullptr;
-        const bool fused = region_fusable(span, block, fitted_group, integer_grid != 0) && scale_format >= 0 &&
+        const bool fused = region_fusable(span, block, fitted_group, integer_grid != 0, n_values) && scale_format >= 0 &&
                            scale_format <= 4;
         if (fused) {
             // fitted inside the sweep kernel below
@@ -1261,7 +1322,7 @@ extern "C" int mk_feedback_sweep(const float *original, float *feedback, float *
             if (fused) {
                 a.fit_scales = region_scales; a.fit_zeros = region_zeros; a.solve_first = region_start != 0;
                 a.asym = asym; a.scale_format = scale_format; a.reciprocal = reciprocal; a.value_minimum = value_minimum;
-                launch_region(a, stream);
+                launch_region(a, integer_grid != 0, stream);
             } else if (integer_grid) launch_sweep<kModeInteger>(a, stream);
             else launch_sweep<kModeCodebook>(a, stream);
             if (tile_stop >= width) continue;

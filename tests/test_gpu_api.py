@@ -81,6 +81,12 @@ def test_online_activation_reconstruction_equals_quantize_dequantize():
     (scaling.int_values(4), True, False, 16, 128, 128),
     (scaling.int_values(3), True, True, 32, 128, 256),
     (scaling.int_values(8), True, True, 128, 128, 128),
+    # tables of up to sixteen values in the same one-kernel-per-region path (NF4, FP4 and a ragged table)
+    (scaling.NF4_VALUES, False, False, 64, 128, 128),
+    (scaling.NF4_VALUES, False, True, 32, 128, 128),
+    (np.array([-6, -4, -3, -2, -1.5, -1, -0.5, 0, 0.5, 1, 1.5, 2, 3, 4, 6], dtype=np.float32), False, False, 32, 128, 256),
+    (np.array([-1, -0.5, -0.25, 0, 0.25, 0.5, 1], dtype=np.float32), False, False, 128, 128, 128),
+    (scaling.NF4_VALUES, False, False, 64, 96, 96),        # regions that are not whole tiles
 ])
 def test_gptq_on_device_matches_oracle_sweep(values, integer, asym, group, refit, block, rng):
     rows, width = 80, 512
