@@ -68,6 +68,11 @@ struct Stream4Args {
     const float *values;  // fp32 table (pair-table kernel, when uniform == 0)
     int n_values, uniform, bits;
     int x_dtype, scale_dtype;  // pair-table kernel: MK_F16 or MK_BF16 each
+    // stream4_launch_rotating only: the activations are multiplied by rotate_signs (or not, when
+    // null), Walsh-Hadamard transformed over the whole row and multiplied by rotate_scale inside
+    // the kernel, before they meet the codes.
+    const float *rotate_signs = nullptr;
+    float rotate_scale = 1.0f;
 };
 // Several weight matrices that share the activations, the row width and the codec, multiplied
 // by one launch: the grid's z index selects the member, x walks that member's tiles of rows
@@ -134,6 +139,10 @@ int pairs_launch_group(const Stream4Args &shared, Stream4Group &group, const int
                        hipStream_t stream);
 bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
+// One sample of fp16 activations, a power-of-two row of 2048 to 16384 codes and whole tiles of
+// rows only: the kernel rotates the activations itself (see Stream4Args).  Returns 0 when
+// launched, -1 when the runtime refused a launch attribute, -2 when the shape is not one of these.
+int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream);
 // The same for a group (Stream4Args carries what the members share; its packed / scales /
 // zeros / bias / y / rows are ignored).  `rows_per_tile` receives the tile height chosen for
 // all members: rows beyond the last whole tile of a member are left to the caller.

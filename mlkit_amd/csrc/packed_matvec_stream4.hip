@@ -89,12 +89,91 @@ __device__ __forceinline__ void chunk_dot_bf16(const CodeChunk<4> &codes, const 
     }
 }
 
+// ---- the input rotation inside the kernel -------------------------------------------------
+//
+// A rotated layer multiplies its codes with H(x * signs) * scale, H the Walsh-Hadamard
+// transform over the whole row.  With one sample the kernel has the row spread over its lanes
+// anyway (lane l of wavefront w holds elements 32 (64 w + l) ... + 31), and its first codes take
+// a microsecond to arrive: the transform runs in that shadow instead of in a launch of its own.
+// Stages in ascending stride as everywhere: index bits 0-4 between registers, bits 5-10
+// between lanes (DPP moves, swizzles and a permute through the LDS crossbar; the lane whose bit
+// is set computes partner - own as one exactly rounded fma with -1), bits 11 and up between
+// wavefronts through LDS.
+
+template <int STAGE>
+__device__ __forceinline__ float lane_partner(float value, int lane) {
+    const int bits = __builtin_bit_cast(int, value);
+    int moved;
+    if constexpr (STAGE == 0) moved = __builtin_amdgcn_mov_dpp(bits, 0xB1, 0xf, 0xf, true);        // quad_perm [1,0,3,2]
+    else if constexpr (STAGE == 1) moved = __builtin_amdgcn_mov_dpp(bits, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+    else if constexpr (STAGE == 3) moved = __builtin_amdgcn_mov_dpp(bits, 0x128, 0xf, 0xf, true);  // row_ror:8
+    else if constexpr (STAGE == 5) moved = __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, bits);
+    else moved = __builtin_amdgcn_ds_swizzle(bits, 0x1F | ((1 << STAGE) << 10));  // bit mode: xor 1 << STAGE within 32 lanes
+    return __builtin_bit_cast(float, moved);
+}
+
+template <int STAGE>
+__device__ __forceinline__ void rotation_lane_stage(float (&v)[kChunkCodes], int lane) {
+    const float sign = (lane >> STAGE) & 1 ? -1.0f : 1.0f;
+#pragma unroll
+    for (int k = 0; k < kChunkCodes; ++k) v[k] = __builtin_fmaf(v[k], sign, lane_partner<STAGE>(v[k], lane));
+}
+
+// x: this lane's 32 fp16 activations (elements 32 (64 wave + lane) ...), replaced by the
+// rotated ones.  `exchange`: waves * 8 KB of LDS that nothing else uses until the next barrier.
+__device__ __forceinline__ void rotate_activations(XChunk<MK_F16> &x, const float *signs, float scale, float *exchange,
+                                                   int wave, int waves, int lane) {
+    float v[kChunkCodes];
+#pragma unroll
+    for (int k = 0; k < kChunkCodes; ++k) v[k] = x_element(x, k);
+    if (signs) {
+        const float4 *mine = reinterpret_cast<const float4 *>(signs + (wave * 64 + lane) * kChunkCodes);
+#pragma unroll
+        for (int q = 0; q < kChunkCodes / 4; ++q) {
+            const float4 sign = mine[q];
+            v[4 * q] *= sign.x; v[4 * q + 1] *= sign.y; v[4 * q + 2] *= sign.z; v[4 * q + 3] *= sign.w;
+        }
+    }
+#pragma unroll
+    for (int bit = 0; bit < 5; ++bit)
+#pragma unroll
+        for (int k = 0; k < kChunkCodes; ++k) {
+            if ((k >> bit) & 1) continue;
+            const float first = v[k], second = v[k | (1 << bit)];
+            v[k] = first + second;
+            v[k | (1 << bit)] = first - second;
+        }
+    rotation_lane_stage<0>(v, lane);
+    rotation_lane_stage<1>(v, lane);
+    rotation_lane_stage<2>(v, lane);
+    rotation_lane_stage<3>(v, lane);
+    rotation_lane_stage<4>(v, lane);
+    rotation_lane_stage<5>(v, lane);
+    for (int stage = 1; stage < waves; stage <<= 1) {  // uniform
+        __syncthreads();  // the buffer's earlier readers are done
+#pragma unroll
+        for (int k = 0; k < kChunkCodes; ++k) exchange[(wave * kChunkCodes + k) * 64 + lane] = v[k];
+        __syncthreads();
+        const float sign = wave & stage ? -1.0f : 1.0f;
+        const float *partner = exchange + ((wave ^ stage) * kChunkCodes) * 64 + lane;
+#pragma unroll
+        for (int k = 0; k < kChunkCodes; ++k) v[k] = __builtin_fmaf(v[k], sign, partner[k * 64]);
+    }
+#pragma unroll
+    for (int i = 0; i < kChunkCodes / 2; ++i) {
+        const mk_h2 pair = {static_cast<_Float16>(v[2 * i] * scale), static_cast<_Float16>(v[2 * i + 1] * scale)};
+        x.r[i] = __builtin_bit_cast(uint32_t, pair);
+    }
+}
+
 // PARTS = 2: rows of at most 1024 codes, one wavefront per workgroup; lanes 0 - 31 take one
 // row and lanes 32 - 63 the next, so that a step covers two rows instead of leaving half the
 // wavefront without codes.
-template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS>
+// ROTATE: the activations are rotated in the kernel (one fp16 sample, whole power-of-two rows).
+template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS, bool ROTATE = false>
 __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4Group &members) {
     static_assert(ROWS * MT <= 64 && ROWS % PARTS == 0, "one transposed reduction per workgroup");
+    static_assert(!ROTATE || (MT == 1 && XT == MK_F16 && PARTS == 1), "the fused rotation takes one fp16 sample of long rows");
     __shared__ float partials[64 * 8];  // [row sum][wavefront]
     // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
     // must not hold LDS for eight).
@@ -183,6 +262,8 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         for (int i = 0; i < 4; ++i) park_piece(x_slice, i, lane, pieces[m][i]);
         chunk_from_slice(x[m], x_slice, lane & (kRowLanes - 1));
     }
+    if constexpr (ROTATE)
+        rotate_activations(x[0], a.rotate_signs, a.rotate_scale, reinterpret_cast<float *>(x_slices_storage), wave, waves, lane);
 
     // sum_k (min + step c_k) x_k = step * dot + min * sum(x) - step * (code-free part of dot).
 #pragma unroll
@@ -251,6 +332,11 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
 template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS>
 __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const Stream4Group members) {
     stream4_body<MT, HAS_ZERO, ROWS, XT, PARTS>(a, members);
+}
+
+template <bool HAS_ZERO, int ROWS>
+__global__ void __launch_bounds__(512) stream4_rotating_kernel(const Stream4Args a, const Stream4Group members) {
+    stream4_body<1, HAS_ZERO, ROWS, MK_F16, 1, true>(a, members);
 }
 
 // ---- two to eight samples: the dot products on the matrix cores ---------------------------
@@ -608,6 +694,35 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream) {
     }
     const int tiles = a.rows / kNarrowRows;
     return launch_rows<kNarrowRows>(a, none, tiles, stream) ? -1 : tiles * kNarrowRows;
+}
+
+int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream) {
+    const bool wide = a.rows / kWideRows >= kComputeUnits;
+    const int tile_rows = wide ? kWideRows : kNarrowRows;
+    const bool whole_rows = a.width == 2048 || a.width == 4096 || a.width == 8192 || a.width == 16384;
+    if (a.samples != 1 || a.x_dtype != MK_F16 || !whole_rows || a.rows % tile_rows != 0 ||
+        (reinterpret_cast<uintptr_t>(a.rotate_signs) & 15u) != 0)
+        return -2;
+    Stream4Group none;
+    none.count = 0;
+    none.widest_tiles = 0;
+    const int waves = a.width / 2048;
+    const dim3 grid(a.rows / tile_rows, 1, 1), block(waves * 64);
+    // the exchange between wavefronts (8 KB each) overlays the activation buffers (5 KB each)
+    const size_t lds = static_cast<size_t>(waves) * 64 * kChunkCodes * sizeof(float);
+    auto launch = [&](auto kernel) -> int {
+        static std::atomic<bool> raised{false};
+        if (lds > 48 * 1024 && !raised.load(std::memory_order_relaxed)) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    64 * 1024) != hipSuccess)
+                return -1;
+            raised.store(true, std::memory_order_relaxed);
+        }
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, a, none);
+        return 0;
+    };
+    if (wide) return a.zeros ? launch(stream4_rotating_kernel<true, kWideRows>) : launch(stream4_rotating_kernel<false, kWideRows>);
+    return a.zeros ? launch(stream4_rotating_kernel<true, kNarrowRows>) : launch(stream4_rotating_kernel<false, kNarrowRows>);
 }
 
 int stream4_launch_group(const Stream4Args &shared, Stream4Group &group, const int *member_rows, int *rows_per_tile,

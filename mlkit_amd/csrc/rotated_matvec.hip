@@ -7,13 +7,42 @@
 // activations are at most 8 x 16384 values: they are written to a small buffer by the
 // row-rotation kernel (mk_rotate_rows: order * samples short workgroups) and read back, from
 // L2, by the matvec kernel enqueued right behind it on the same stream.  One library call replaces a Python hook, an
-// allocation and two calls.
+// allocation and two calls.  One fp16 sample of an INT4 layer with a power-of-two row (2048 to
+// 16384 codes) needs neither the buffer nor the second launch: the matvec kernel transforms the
+// activations itself (rotate_inside_the_matvec).
 
 #include <mutex>
 
-#include "mk_common.h"
+#include "packed_matvec_impl.h"
 
 namespace {
+
+// One fp16 sample, INT4 codes on a uniform grid with 16-bit scales, a power-of-two row of 2048
+// to 16384 codes and whole tiles of rows: the matvec kernel rotates the activations itself while
+// its first codes are on their way (no second launch, no buffer).  Returns 1 when it took the
+// call, 0 when the shape is not one of these, a negative status on errors.
+int rotate_inside_the_matvec(const void *x, int x_dtype, const float *signs, float scale, const uint8_t *packed,
+                             const void *scales, int scale_dtype, const void *zeros, const void *bias, int bias_dtype,
+                             void *y, int samples, int output_width, int input_width, int group, int bits, int uniform,
+                             float grid_min, float grid_step, hipStream_t stream) {
+    if (samples != 1 || x_dtype != MK_F16 || !packed || !scales || !y || group < 1 || output_width < 1) return 0;
+    if (!mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0)) return 0;
+    const auto misaligned = [](const void *pointer, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(pointer) & mask) != 0; };
+    if (misaligned(packed, 3) || misaligned(scales, 3) || misaligned(zeros, 3) || misaligned(bias, 3) || misaligned(x, 15))
+        return 0;
+    if (bias && !mk_dtype_valid(bias_dtype)) return 0;
+    mk_matvec::Stream4Args a;
+    a.x = x; a.packed = packed; a.scales = scales; a.zeros = zeros; a.bias = bias; a.y = y;
+    a.samples = samples; a.rows = output_width; a.width = input_width; a.group = group;
+    a.groups = mk_cdiv(input_width, group); a.bias_dtype = bias_dtype; a.grid_min = grid_min; a.grid_step = grid_step;
+    a.values = nullptr; a.n_values = 0; a.uniform = uniform; a.bits = bits;
+    a.x_dtype = x_dtype; a.scale_dtype = scale_dtype;
+    a.rotate_signs = signs; a.rotate_scale = scale;
+    const int launched = mk_matvec::stream4_launch_rotating(a, stream);
+    if (launched == -2) return 0;
+    if (launched) return -mk_fail(MK_ERR_HIP, "mk_rotated_packed_matvec: the runtime refused the kernel's LDS size");
+    return 1;
+}
 
 int rotate_then_multiply(const void *x, int x_dtype, void *rotated, int order, int power, const float *basis,
                          const float *signs, float scale, const uint8_t *packed, const void *scales, int scale_dtype,
@@ -33,6 +62,14 @@ int rotate_then_multiply(const void *x, int x_dtype, void *rotated, int order, i
     if (order == 1) {
         MK_REQUIRE((input_width & (input_width - 1)) == 0 && input_width >= 32, MK_ERR_UNSUPPORTED,
                    "mk_rotated_packed_matvec: a Walsh-Hadamard rotation needs a power-of-two width of at least 32");
+        const int inside = rotate_inside_the_matvec(x, x_dtype, signs, scale, packed, scales, scale_dtype, zeros, bias, bias_dtype,
+                                                    y, samples, output_width, input_width, group, bits, uniform, grid_min,
+                                                    grid_step, static_cast<hipStream_t>(stream));
+        if (inside < 0) return -inside;
+        if (inside > 0) {
+            MK_LAUNCH_CHECK("mk_rotated_packed_matvec");
+            return MK_OK;
+        }
         int points = 32;
         while (points * points < input_width && points < 1024) points *= 2;
         status = mk_rotate_rows(x, x_dtype, rotated, x_dtype, samples, input_width / points, points, nullptr, signs, scale,
