@@ -121,18 +121,17 @@ __device__ __forceinline__ void rotation_lane_stage(float (&v)[kChunkCodes], int
 
 // x: this lane's 32 fp16 activations (elements 32 (64 wave + lane) ...), replaced by the
 // rotated ones.  `exchange`: waves * 8 KB of LDS that nothing else uses until the next barrier.
-__device__ __forceinline__ void rotate_activations(XChunk<MK_F16> &x, const float *signs, float scale, float *exchange,
-                                                   int wave, int waves, int lane) {
+// `sign`: the +-1 factors of this lane's 32 elements (all ones without a sign vector), requested
+// by the caller ahead of the codes: loads return in the order of their requests, and the
+// rotation is to run while the codes are still on their way.
+__device__ __forceinline__ void rotate_activations(XChunk<MK_F16> &x, const float4 (&sign)[kChunkCodes / 4], float scale,
+                                                   float *exchange, int wave, int waves, int lane) {
     float v[kChunkCodes];
 #pragma unroll
     for (int k = 0; k < kChunkCodes; ++k) v[k] = x_element(x, k);
-    if (signs) {
-        const float4 *mine = reinterpret_cast<const float4 *>(signs + (wave * 64 + lane) * kChunkCodes);
 #pragma unroll
-        for (int q = 0; q < kChunkCodes / 4; ++q) {
-            const float4 sign = mine[q];
-            v[4 * q] *= sign.x; v[4 * q + 1] *= sign.y; v[4 * q + 2] *= sign.z; v[4 * q + 3] *= sign.w;
-        }
+    for (int q = 0; q < kChunkCodes / 4; ++q) {
+        v[4 * q] *= sign[q].x; v[4 * q + 1] *= sign[q].y; v[4 * q + 2] *= sign[q].z; v[4 * q + 3] *= sign[q].w;
     }
 #pragma unroll
     for (int bit = 0; bit < 5; ++bit)
@@ -180,7 +179,7 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
     uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
     constexpr int kStreamRows = ROWS / PARTS;            // steps: PARTS rows each
-    constexpr int kStreamAhead = rows_ahead_of<kStreamRows>();
+    constexpr int kStreamAhead = rows_ahead_of<kStreamRows>();  // (with ROTATE too: all 16 rows ahead measured slower)
     constexpr int kSums = kStreamRows * MT;
     constexpr int kRowLanes = 64 / PARTS;
 
@@ -215,6 +214,15 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         }
     };
     request_activations();
+    float4 rotation_sign[ROTATE ? kChunkCodes / 4 : 1];
+    if constexpr (ROTATE) {
+#pragma unroll
+        for (int q = 0; q < kChunkCodes / 4; ++q) {
+            rotation_sign[q] = float4{1.0f, 1.0f, 1.0f, 1.0f};
+            if (a.rotate_signs)  // uniform
+                rotation_sign[q] = reinterpret_cast<const float4 *>(a.rotate_signs + (wave * 64 + lane) * kChunkCodes)[q];
+        }
+    }
     // The scale (and offset) of this lane's chunk in every row, 2 bytes each.
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
     const uint32_t group_offset = static_cast<uint32_t>(part) * scale_row_bytes +
@@ -263,7 +271,7 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         chunk_from_slice(x[m], x_slice, lane & (kRowLanes - 1));
     }
     if constexpr (ROTATE)
-        rotate_activations(x[0], a.rotate_signs, a.rotate_scale, reinterpret_cast<float *>(x_slices_storage), wave, waves, lane);
+        rotate_activations(x[0], rotation_sign, a.rotate_scale, reinterpret_cast<float *>(x_slices_storage), wave, waves, lane);
 
     // sum_k (min + step c_k) x_k = step * dot + min * sum(x) - step * (code-free part of dot).
 #pragma unroll
@@ -398,26 +406,74 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
 
     __syncthreads();  // aligns the workgroup's wavefronts before their first loads
 
+    // Scales and the first codes of a tile (defined here, because long rows ask for them before
+    // the activations are in place).
+    uint16_t scale_raw[kSteps], zero_raw[HAS_ZERO ? kSteps : 1];
+    CodeChunk<4> codes[kSteps];
+    auto request_tile = [&](int tile) __attribute__((always_inline)) {
+        const int row_base = tile * ROWS;
+        const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
+        const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
+        const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
+        // Scale (and offset) of row 4 q + t at every sub-slice, 2 bytes each.
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q)
+#pragma unroll
+            for (int s = 0; s < kSlices; ++s) {
+                const size_t quad_offset = static_cast<size_t>(4 * q) * scale_row_bytes;
+                scale_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(scale_base + quad_offset + group_offset[s]);
+                if constexpr (HAS_ZERO)
+                    zero_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(zero_base + quad_offset + group_offset[s]);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int step = 0; step < kAhead; ++step) {
+            load_codes<4>(codes[step], codes_base + static_cast<size_t>(4 * (step / kSlices)) * row_bytes + code_offset[step % kSlices]);
+            __builtin_amdgcn_sched_barrier(0);  // in order
+        }
+    };
+
     // Activations of sample t (and t + 4) for this lane's four chunks, 16 fp16 pairs each:
     // the wavefront reads the slices of a set's four samples coalesced, parks them side by
-    // side in LDS, and every lane picks its sample's chunks.
+    // side in LDS, and every lane picks its sample's chunks.  Long rows (one tile per
+    // workgroup): all activations are requested first and the tile's first codes right behind
+    // them, before any activation is waited for -- eight samples are 28 KB per wavefront, and
+    // the codes should stream while those arrive and are laid out.
     XChunk<XT> x[SETS][kSlices];
+    {
+        mk_u32x4 pieces[SETS][4][kSlices];
+        auto request_set = [&](int set) __attribute__((always_inline)) {
 #pragma unroll
-    for (int set = 0; set < SETS; ++set) {
-        mk_u32x4 pieces[4][kSlices];
+            for (int j = 0; j < 4; ++j) {
+                const int wanted_sample = blockIdx.y * 4 * SETS + 4 * set + j;
+                const int sample = wanted_sample < a.samples ? wanted_sample : a.samples - 1;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int wanted_sample = blockIdx.y * 4 * SETS + 4 * set + j;
-            const int sample = wanted_sample < a.samples ? wanted_sample : a.samples - 1;
+                for (int i = 0; i < kSlices; ++i)
+                    pieces[set][j][i] = request_piece(source.x, a.width, sample, wave * (512 * kSlices), i, lane);
+            }
+        };
+        auto place_set = [&](int set) __attribute__((always_inline)) {
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(source.x, a.width, sample, wave * (512 * kSlices), i, lane);
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < kSlices; ++i) park_piece_swizzled(x_slice + j * kSampleWords, i, lane, pieces[set][j][i]);
+#pragma unroll
+            for (int s = 0; s < kSlices; ++s) chunk_from_swizzled_slice(x[set][s], x_slice + t * kSampleWords, s * 16 + block);
+        };
+        if constexpr (kStrided) {
+#pragma unroll
+            for (int set = 0; set < SETS; ++set) {
+                request_set(set);
+                place_set(set);
+            }
+        } else {
+#pragma unroll
+            for (int set = 0; set < SETS; ++set) request_set(set);
+            __builtin_amdgcn_sched_barrier(0);
+            request_tile(blockIdx.x);
+#pragma unroll
+            for (int set = 0; set < SETS; ++set) place_set(set);
         }
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int i = 0; i < kSlices; ++i) park_piece_swizzled(x_slice + j * kSampleWords, i, lane, pieces[j][i]);
-#pragma unroll
-        for (int s = 0; s < kSlices; ++s) chunk_from_swizzled_slice(x[set][s], x_slice + t * kSampleWords, s * 16 + block);
     }
     float x_sum[SETS][kSlices], grid_term[SETS][kSlices];
 #pragma unroll
@@ -449,27 +505,7 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     do {
     const int row_base = tile * ROWS;
     const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
-    const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
-    const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
-    // Scale (and offset) of row 4 q + t at every sub-slice, 2 bytes each.
-    uint16_t scale_raw[kSteps], zero_raw[HAS_ZERO ? kSteps : 1];
-#pragma unroll
-    for (int q = 0; q < kQuads; ++q)
-#pragma unroll
-        for (int s = 0; s < kSlices; ++s) {
-            const size_t quad_offset = static_cast<size_t>(4 * q) * scale_row_bytes;
-            scale_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(scale_base + quad_offset + group_offset[s]);
-            if constexpr (HAS_ZERO)
-                zero_raw[q * kSlices + s] = *reinterpret_cast<const uint16_t *>(zero_base + quad_offset + group_offset[s]);
-        }
-    __builtin_amdgcn_sched_barrier(0);
-
-    CodeChunk<4> codes[kSteps];
-#pragma unroll
-    for (int step = 0; step < kAhead; ++step) {
-        load_codes<4>(codes[step], codes_base + static_cast<size_t>(4 * (step / kSlices)) * row_bytes + code_offset[step % kSlices]);
-        __builtin_amdgcn_sched_barrier(0);  // in order
-    }
+    if constexpr (kStrided) request_tile(tile);
 
     float sums[SETS][kSums];
 #pragma unroll
