@@ -407,15 +407,17 @@ def vector_ldlq_layer(device: torch.device, generator: torch.Generator, cpu_rows
 def rotated_layer(device: torch.device, generator: torch.Generator, values: torch.Tensor) -> dict:
     """Config 5: the rotated INT4-g128 layers at M = 1 and 8.  One step = the online rotation of
     the activations plus the packed matvec, enqueued by one mk_rotated_packed_matvec call; the
-    unrotated matvec of the same layer is timed beside it."""
+    unrotated matvec of the same layer is timed beside it.  The 14336-wide layer is rotated as
+    the reference does it (a 28 x 28 Paley basis over blocks of 512) and as seven separate
+    blocks of 2048."""
     from mlkit_amd import native
     from mlkit_amd.quantization.transforms import OnlineRotation
 
     library = native.library()
     out = {}
-    for rows, width in ((ROWS, WIDTH), (WIDTH, 4096)):
+    for rows, width, block in ((ROWS, WIDTH, None), (WIDTH, 4096, None), (ROWS, WIDTH, 2048)):
         copies = make_copies(max(2, -(-MINIMUM_ROTATING_BYTES // (rows * width // 2))), device, rows=rows, width=width)
-        order, power, basis, signs, scale, keep = OnlineRotation(17).launch_arguments(width, device)
+        order, power, basis, signs, scale, keep = OnlineRotation(17, block).launch_arguments(width, device)
         for samples in (1, 8):
             x = torch.randn((samples, width), device=device, generator=generator).half()
             y = torch.empty((samples, rows), device=device, dtype=torch.float16)
@@ -431,8 +433,9 @@ def rotated_layer(device: torch.device, generator: torch.Generator, values: torc
             plain = [Launcher(x, packed, scales, values, y, rows=rows, width=width) for packed, scales in copies]
             rotated_s = timed_graph(with_rotation, 200, 20, 20)[0]
             plain_s = timed_graph(plain, 200, 20, 20)[0]
-            out[f"{rows}x{width} M={samples}"] = {
-                "rotation": f"{order} x {power}" if order > 1 else f"fwht {power}",
+            label = f"{rows}x{width} M={samples}" + (f", separate blocks of {block}" if block else "")
+            out[label] = {
+                "rotation": (f"{order} separate fwht {power}" if block else f"{order} x {power}") if order > 1 else f"fwht {power}",
                 "rotated_us": rotated_s * 1e6, "unrotated_us": plain_s * 1e6, "rotation_costs_us": (rotated_s - plain_s) * 1e6,
             }
         del copies

@@ -86,17 +86,20 @@ int mk_packed_matvec_group(const void *const *x, int x_dtype, int count, const u
 /* The online input rotation of a rotated layer and its packed matvec from one call:
  * rotated = T(x * signs), T = (basis (x) H_power) * scale along the input width
  * (input_width = order * power, power a power of two; order == 1: a plain Walsh-Hadamard
- * transform, basis unused), written to `rotated` ([samples, input_width] of x_dtype, a
+ * transform, basis unused; order > 1 with basis NULL: the `order` blocks of `power` values are
+ * transformed one by one, T = (I (x) H_power) * scale, through mk_fwht), written to `rotated`
+ * ([samples, input_width] of x_dtype, a
  * buffer of the caller's that must not alias x), then mk_packed_matvec on `rotated` with the
  * remaining arguments.  signs: NULL (or [input_width] fp32 of +-1, 16-byte aligned for the
  * one-launch form).  Results equal mk_rotate_rows followed by mk_packed_matvec bit for bit;
  * MK_ERR_UNSUPPORTED when mk_rotate_rows does not take (order, power).  One exception, taken
- * whenever it applies: one fp16 sample, order == 1, input_width 2048 / 4096 / 8192 / 16384,
- * INT4 codes with 16-bit scales and whole tiles of rows (16, or 4 below 4096 rows) run as ONE
- * launch in which every workgroup transforms the activations in its registers; `rotated` is
- * then left untouched, and the result equals mk_packed_matvec on mk_fwht's (stagewise) output
- * rounded to fp16 bit for bit -- the same linear map as mk_rotate_rows, summed in the order of
- * the stages.
+ * whenever it applies: one fp16 sample, no basis (a plain transform of 2048 / 4096 / 8192 /
+ * 16384 values, or separate blocks of 64 to 16384 values that tile a row of whole 2048-value
+ * slices, 14336 = 7 x 2048 for one), INT4 codes with 16-bit scales and whole tiles of rows (16,
+ * or 4 below 4096 rows) run as ONE launch in which every workgroup transforms the activations
+ * in its registers; `rotated` is then left untouched, and the result equals mk_packed_matvec on
+ * mk_fwht's (stagewise) output rounded to fp16 bit for bit -- for a plain transform the same
+ * linear map as mk_rotate_rows, summed in the order of the stages.
  * Replaces: the rotate_inputs forward pre-hook (conversion/model_transforms.py:116-128) in
  * front of PackedLinear.forward (inference/packed_linear.py:148-245). */
 int mk_rotated_packed_matvec(const void *x, int x_dtype, void *rotated, int order, int power,

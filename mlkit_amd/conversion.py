@@ -47,7 +47,7 @@ def install_transform(model: nn.Module, descriptor: dict[str, Any]) -> None:
     if descriptor["kind"] != "rotation":
         raise ValueError(f"unknown model transform {descriptor['kind']!r}")
     layer = model.get_submodule(descriptor["name"])
-    hook = RotateInputs(OnlineRotation(descriptor["seed"]))
+    hook = RotateInputs(OnlineRotation(descriptor["seed"], descriptor.get("block")))
     absorb = getattr(layer, "absorb_input_rotation", None)
     if absorb is not None and not layer._forward_pre_hooks:
         absorb(hook.rotation)  # a packed layer runs the rotation inside its own launch sequence
@@ -61,6 +61,7 @@ class Rotate:
 
     seed: int = 0
     names: tuple[str, ...] = ROTATED_LAYER_NAMES
+    block: int | None = None   # rotate blocks of this many input features one by one (None: the whole row, as the reference)
 
     def __call__(self, model: "Model | nn.Module", calib: Any = None) -> None:
         module = model.module if isinstance(model, Model) else model
@@ -69,11 +70,14 @@ class Rotate:
                 if not isinstance(layer, nn.Linear) or name.split(".")[-1] not in self.names:
                     continue
                 seed = layer_seed(name, self.seed)
-                layer.weight.copy_(rht(layer.weight.float(), seed=seed).to(layer.weight.dtype))
+                block = self.block if self.block and layer.in_features % self.block == 0 and layer.in_features > self.block else None
+                layer.weight.copy_(rht(layer.weight.float(), seed=seed, block=block).to(layer.weight.dtype))
                 descriptor = {"kind": "rotation", "name": name, "seed": seed}
+                if block is not None:
+                    descriptor["block"] = block
                 install_transform(module, descriptor)
                 record_transform(module, descriptor)
 
 
-def rotate(seed: int = 0, names: tuple[str, ...] = ROTATED_LAYER_NAMES) -> Rotate:
-    return Rotate(seed, tuple(names))
+def rotate(seed: int = 0, names: tuple[str, ...] = ROTATED_LAYER_NAMES, block: int | None = None) -> Rotate:
+    return Rotate(seed, tuple(names), block)

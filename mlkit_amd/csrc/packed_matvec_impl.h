@@ -73,6 +73,7 @@ struct Stream4Args {
     // the kernel, before they meet the codes.
     const float *rotate_signs = nullptr;
     float rotate_scale = 1.0f;
+    int rotate_log_block = 0;  // the transform spans blocks of 1 << rotate_log_block values (the whole row, or equal parts of it)
 };
 // Several weight matrices that share the activations, the row width and the codec, multiplied
 // by one launch: the grid's z index selects the member, x walks that member's tiles of rows
@@ -139,8 +140,9 @@ int pairs_launch_group(const Stream4Args &shared, Stream4Group &group, const int
                        hipStream_t stream);
 bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
-// One sample of fp16 activations, a power-of-two row of 2048 to 16384 codes and whole tiles of
-// rows only: the kernel rotates the activations itself (see Stream4Args).  Returns 0 when
+// One sample of fp16 activations, a row of whole 2048-code slices made of power-of-two blocks
+// (one block: a power-of-two row) and whole tiles of rows only: the kernel rotates the
+// activations itself (see Stream4Args).  Returns 0 when
 // launched, -1 when the runtime refused a launch attribute, -2 when the shape is not one of these.
 int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream);
 // The same for a group (Stream4Args carries what the members share; its packed / scales /

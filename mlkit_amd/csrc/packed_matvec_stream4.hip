@@ -124,8 +124,10 @@ __device__ __forceinline__ void rotation_lane_stage(float (&v)[kChunkCodes], int
 // `sign`: the +-1 factors of this lane's 32 elements (all ones without a sign vector), requested
 // by the caller ahead of the codes: loads return in the order of their requests, and the
 // rotation is to run while the codes are still on their way.
+// `log_block`: the transform spans aligned blocks of 1 << log_block elements (64 at least): the
+// stages of higher index bits are left out (uniform branches).
 __device__ __forceinline__ void rotate_activations(XChunk<MK_F16> &x, const float4 (&sign)[kChunkCodes / 4], float scale,
-                                                   float *exchange, int wave, int waves, int lane) {
+                                                   float *exchange, int wave, int waves, int lane, int log_block) {
     float v[kChunkCodes];
 #pragma unroll
     for (int k = 0; k < kChunkCodes; ++k) v[k] = x_element(x, k);
@@ -143,12 +145,14 @@ __device__ __forceinline__ void rotate_activations(XChunk<MK_F16> &x, const floa
             v[k | (1 << bit)] = first - second;
         }
     rotation_lane_stage<0>(v, lane);
-    rotation_lane_stage<1>(v, lane);
-    rotation_lane_stage<2>(v, lane);
-    rotation_lane_stage<3>(v, lane);
-    rotation_lane_stage<4>(v, lane);
-    rotation_lane_stage<5>(v, lane);
-    for (int stage = 1; stage < waves; stage <<= 1) {  // uniform
+    if (log_block > 6) rotation_lane_stage<1>(v, lane);
+    if (log_block > 7) rotation_lane_stage<2>(v, lane);
+    if (log_block > 8) rotation_lane_stage<3>(v, lane);
+    if (log_block > 9) rotation_lane_stage<4>(v, lane);
+    if (log_block > 10) rotation_lane_stage<5>(v, lane);
+    const int wave_stages = log_block > 11 ? 1 << (log_block - 11) : 1;  // wavefronts a block spans
+    (void)waves;
+    for (int stage = 1; stage < wave_stages; stage <<= 1) {  // uniform
         __syncthreads();  // the buffer's earlier readers are done
 #pragma unroll
         for (int k = 0; k < kChunkCodes; ++k) exchange[(wave * kChunkCodes + k) * 64 + lane] = v[k];
@@ -271,7 +275,8 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         chunk_from_slice(x[m], x_slice, lane & (kRowLanes - 1));
     }
     if constexpr (ROTATE)
-        rotate_activations(x[0], rotation_sign, a.rotate_scale, reinterpret_cast<float *>(x_slices_storage), wave, waves, lane);
+        rotate_activations(x[0], rotation_sign, a.rotate_scale, reinterpret_cast<float *>(x_slices_storage), wave, waves, lane,
+                           a.rotate_log_block);
 
     // sum_k (min + step c_k) x_k = step * dot + min * sum(x) - step * (code-free part of dot).
 #pragma unroll
@@ -735,7 +740,10 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream) {
 int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream) {
     const bool wide = a.rows / kWideRows >= kComputeUnits;
     const int tile_rows = wide ? kWideRows : kNarrowRows;
-    const bool whole_rows = a.width == 2048 || a.width == 4096 || a.width == 8192 || a.width == 16384;
+    // whole 2048-code slices (every lane of every wavefront holds activations), whole blocks
+    const long long block_length = 1ll << a.rotate_log_block;
+    const bool whole_rows = a.width % 2048 == 0 && a.width >= 2048 && a.width <= 16384 && a.rotate_log_block >= 6 &&
+                            a.rotate_log_block <= 14 && a.width % block_length == 0;
     if (a.samples != 1 || a.x_dtype != MK_F16 || !whole_rows || a.rows % tile_rows != 0 ||
         (reinterpret_cast<uintptr_t>(a.rotate_signs) & 15u) != 0)
         return -2;
@@ -744,8 +752,9 @@ int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream) {
     none.widest_tiles = 0;
     const int waves = a.width / 2048;
     const dim3 grid(a.rows / tile_rows, 1, 1), block(waves * 64);
-    // the exchange between wavefronts (8 KB each) overlays the activation buffers (5 KB each)
-    const size_t lds = static_cast<size_t>(waves) * 64 * kChunkCodes * sizeof(float);
+    // the exchange between the wavefronts of a block (8 KB each) overlays the activation buffers (5 KB each)
+    const size_t lds = static_cast<size_t>(waves) * (a.rotate_log_block > 11 ? 64 * kChunkCodes * sizeof(float)
+                                                                                : kSliceWords * sizeof(uint32_t));
     auto launch = [&](auto kernel) -> int {
         static std::atomic<bool> raised{false};
         if (lds > 48 * 1024 && !raised.load(std::memory_order_relaxed)) {

@@ -21,7 +21,7 @@ namespace {
 // to 16384 codes and whole tiles of rows: the matvec kernel rotates the activations itself while
 // its first codes are on their way (no second launch, no buffer).  Returns 1 when it took the
 // call, 0 when the shape is not one of these, a negative status on errors.
-int rotate_inside_the_matvec(const void *x, int x_dtype, const float *signs, float scale, const uint8_t *packed,
+int rotate_inside_the_matvec(const void *x, int x_dtype, int block, const float *signs, float scale, const uint8_t *packed,
                              const void *scales, int scale_dtype, const void *zeros, const void *bias, int bias_dtype,
                              void *y, int samples, int output_width, int input_width, int group, int bits, int uniform,
                              float grid_min, float grid_step, hipStream_t stream) {
@@ -38,6 +38,7 @@ int rotate_inside_the_matvec(const void *x, int x_dtype, const float *signs, flo
     a.values = nullptr; a.n_values = 0; a.uniform = uniform; a.bits = bits;
     a.x_dtype = x_dtype; a.scale_dtype = scale_dtype;
     a.rotate_signs = signs; a.rotate_scale = scale;
+    while ((1 << a.rotate_log_block) < block) ++a.rotate_log_block;
     const int launched = mk_matvec::stream4_launch_rotating(a, stream);
     if (launched == -2) return 0;
     if (launched) return -mk_fail(MK_ERR_HIP, "mk_rotated_packed_matvec: the runtime refused the kernel's LDS size");
@@ -54,22 +55,31 @@ int rotate_then_multiply(const void *x, int x_dtype, void *rotated, int order, i
     MK_REQUIRE(order >= 1 && power >= 1 && static_cast<long long>(order) * power == input_width, MK_ERR_INVALID,
                "mk_rotated_packed_matvec: order * power must equal the input width (%d * %d != %d)", order, power,
                input_width);
-    MK_REQUIRE(order == 1 || basis, MK_ERR_INVALID, "mk_rotated_packed_matvec: a blocked rotation needs its basis");
+    // Without a basis: Walsh-Hadamard transforms of the row's `order` blocks, each for itself.
+    const bool block_diagonal = order > 1 && !basis;
+    MK_REQUIRE(!block_diagonal || (power >= 32 && (power & (power - 1)) == 0), MK_ERR_UNSUPPORTED,
+               "mk_rotated_packed_matvec: blocks transformed one by one need a power-of-two length of at least 32 (got %d)",
+               power);
     // The rotation runs on order * samples short workgroups (mk_rotate_rows); a plain
     // power-of-two width is split as H_width = H_blocks (x) H_points with about sqrt(width)
     // points per block.
     int status;
-    if (order == 1) {
-        MK_REQUIRE((input_width & (input_width - 1)) == 0 && input_width >= 32, MK_ERR_UNSUPPORTED,
+    if (order == 1 || block_diagonal) {
+        MK_REQUIRE(block_diagonal || ((input_width & (input_width - 1)) == 0 && input_width >= 32), MK_ERR_UNSUPPORTED,
                    "mk_rotated_packed_matvec: a Walsh-Hadamard rotation needs a power-of-two width of at least 32");
-        const int inside = rotate_inside_the_matvec(x, x_dtype, signs, scale, packed, scales, scale_dtype, zeros, bias, bias_dtype,
-                                                    y, samples, output_width, input_width, group, bits, uniform, grid_min,
-                                                    grid_step, static_cast<hipStream_t>(stream));
+        const int inside = rotate_inside_the_matvec(x, x_dtype, power, signs, scale, packed, scales, scale_dtype, zeros, bias,
+                                                    bias_dtype, y, samples, output_width, input_width, group, bits, uniform,
+                                                    grid_min, grid_step, static_cast<hipStream_t>(stream));
         if (inside < 0) return -inside;
         if (inside > 0) {
             MK_LAUNCH_CHECK("mk_rotated_packed_matvec");
             return MK_OK;
         }
+    }
+    if (block_diagonal) {
+        status = mk_fwht(x, x_dtype, rotated, x_dtype, static_cast<long long>(samples) * order, power, signs, nullptr,
+                         input_width, scale, stream);
+    } else if (order == 1) {
         int points = 32;
         while (points * points < input_width && points < 1024) points *= 2;
         status = mk_rotate_rows(x, x_dtype, rotated, x_dtype, samples, input_width / points, points, nullptr, signs, scale,

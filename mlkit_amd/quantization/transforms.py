@@ -116,9 +116,36 @@ ONE_LAUNCH_ROWS = 256
 ROW_KERNEL_ROWS = 64   # activation rows the per-block rotation kernel takes (mk_rotate_rows)
 
 
-def rotate(value: Tensor, *, inverse: bool = False, signs: Tensor | None = None) -> Tensor:
+def _rotate_blocks_separately(value: Tensor, block: int, inverse: bool, signs: Tensor | None) -> Tensor:
+    """The final dimension as blocks of ``block`` values (a power of two), each
+    Walsh-Hadamard-transformed for itself: ``(I (x) H_block) / sqrt(block)``, its own inverse."""
+    width = value.shape[-1]
+    if block < 2 or block & (block - 1) or width % block:
+        raise ValueError(f"blocks of {block} values do not tile a width of {width} as powers of two")
+    before, after = (None, signs) if inverse else (signs, None)
+    blocks = value.reshape(*value.shape[:-1], width // block, block)
+    if _on_kernel(value) and block <= MAXIMUM_KERNEL_WIDTH:
+        from mlkit_amd.kernels import hadamard as kernel
+
+        def as_kernel_signs(vector):
+            return None if vector is None else vector.to(device=value.device, dtype=torch.float32).contiguous()
+
+        out = kernel.transform(blocks.contiguous(), signs_before=as_kernel_signs(before), signs_after=as_kernel_signs(after))
+        return out.reshape(value.shape)
+    if before is not None:
+        blocks = (value * before).reshape(blocks.shape)
+    out = hadamard(blocks).reshape(value.shape)
+    return out * after if after is not None else out
+
+
+def rotate(value: Tensor, *, inverse: bool = False, signs: Tensor | None = None, block: int | None = None) -> Tensor:
     """``structured_transform`` with optional fused sign flips: forward ``T(value * signs)``,
-    inverse ``T^-1(value) * signs``.  Two launches at most on a HIP device."""
+    inverse ``T^-1(value) * signs``.  Two launches at most on a HIP device.  ``block``: T
+    transforms blocks of that many values one by one instead (no counterpart in the reference,
+    whose T always spans the row; a row of whole 2048-value blocks is what a packed layer can
+    rotate inside its own matvec launch)."""
+    if block is not None:
+        return _rotate_blocks_separately(value, block, inverse, signs)
     order, power, basis = transform_factor(value.shape[-1])
     if not (_on_kernel(value) and power <= MAXIMUM_KERNEL_WIDTH and order <= MAXIMUM_KERNEL_ORDER):
         if signs is not None and not inverse:
@@ -176,12 +203,12 @@ def random_signs(width: int, seed: int, device: torch.device | str, dtype: torch
     return _cached_signs(width, seed, torch.device(device)).to(dtype)
 
 
-def randomized_transform(value: Tensor, *, seed: int = 0, inverse: bool = False) -> Tensor:
+def randomized_transform(value: Tensor, *, seed: int = 0, inverse: bool = False, block: int | None = None) -> Tensor:
     # the cached FP32 vector itself: +-1 is exact in every dtype and the kernels take FP32 signs
     signs = _cached_signs(value.shape[-1], seed, value.device)
     if not _on_kernel(value):
         signs = signs.to(value.dtype)
-    return rotate(value, inverse=inverse, signs=signs)
+    return rotate(value, inverse=inverse, signs=signs, block=block)
 
 
 class OnlineRotation:
@@ -189,8 +216,9 @@ class OnlineRotation:
     with the per-call work reduced to one allocation and one library call (the launch
     arguments of a width, device and dtype are prepared once)."""
 
-    def __init__(self, seed: int):
+    def __init__(self, seed: int, block: int | None = None):
         self.seed = seed
+        self.block = block   # None: the transform spans the row; else blocks of that many values, one by one
         self._plans: dict = {}
 
     def __call__(self, value: Tensor) -> Tensor:
@@ -205,10 +233,15 @@ class OnlineRotation:
         ``mk_rotate_rows`` / ``mk_rotated_packed_matvec``, or None when the row-rotation kernel
         does not take this width (``keep`` holds the tensors the pointers belong to).  A plain
         power-of-two width is ``(1, width, None, ...)``."""
-        order, power, basis = transform_factor(width)
         from mlkit_amd.kernels import hadamard as kernel
 
         signs = _cached_signs(width, self.seed, device)
+        if self.block is not None:   # no basis and several blocks: each block for itself
+            block = self.block
+            if block < 32 or block & (block - 1) or width % block or block > MAXIMUM_KERNEL_WIDTH or width == block:
+                return None
+            return width // block, block, None, signs.data_ptr(), kernel.normaliser(block), (signs,)
+        order, power, basis = transform_factor(width)
         if basis is None:
             if width < 32 or width > MAXIMUM_KERNEL_WIDTH:
                 return None
@@ -225,10 +258,12 @@ class OnlineRotation:
         seed = self.seed
         width = value.shape[-1]
 
-        def general(tensor: Tensor) -> Tensor:
-            return randomized_transform(tensor, seed=seed)
+        block = self.block
 
-        arguments = self.launch_arguments(width, value.device) if _on_kernel(value) else None
+        def general(tensor: Tensor) -> Tensor:
+            return randomized_transform(tensor, seed=seed, block=block)
+
+        arguments = self.launch_arguments(width, value.device) if _on_kernel(value) and block is None else None
         if arguments is None:
             return general
         from mlkit_amd import native
@@ -258,5 +293,5 @@ class OnlineRotation:
         return by_rows
 
 
-def rht(value: Tensor, *, seed: int = 0, inverse: bool = False) -> Tensor:
-    return randomized_transform(value, seed=seed, inverse=inverse)
+def rht(value: Tensor, *, seed: int = 0, inverse: bool = False, block: int | None = None) -> Tensor:
+    return randomized_transform(value, seed=seed, inverse=inverse, block=block)

@@ -673,6 +673,47 @@ def test_packed_layer_absorbs_its_online_rotation(rows, width):
         assert torch.equal(duplicate(x), fused(x))
 
 
+def test_rotation_of_separate_blocks_end_to_end(tmp_path):
+    """mk.rotate(seed, block=2048): the down projection's 14336 input features are rotated as
+    seven blocks of 2048 (offline on the weight columns, online on the activations).  The
+    rotated float layer reproduces the original outputs; quantised and packed, one fp16 row
+    goes through one launch and equals the pre-hook followed by the unrotated packed layer bit
+    for bit; the block length travels through the checkpoint manifest."""
+    from mlkit_amd.conversion import RotateInputs
+    from mlkit_amd.quantization.transforms import OnlineRotation
+
+    torch.manual_seed(50)
+    rows, width = 256, 14336
+    module = nn.ModuleDict({"down_proj": nn.Linear(width, rows, bias=True, dtype=torch.float16)}).cuda()
+    x = torch.randn(3, width, device="cuda").half()
+    with torch.inference_mode():
+        expected = module["down_proj"](x)
+    mk.rotate(seed=4, block=2048)(module)
+    assert module._mlkit_transforms[0]["block"] == 2048
+    hooks = [hook for hook in module["down_proj"]._forward_pre_hooks.values() if isinstance(hook, RotateInputs)]
+    assert len(hooks) == 1 and hooks[0].rotation.block == 2048
+    with torch.inference_mode():
+        rotated_output = module["down_proj"](x)
+    assert (rotated_output.float() - expected.float()).abs().max() <= 2e-2 * expected.float().abs().max()
+    converted = mk.quantize(module, mk.int(4, group=128), calib=None)
+    packed = mk.optimize(converted, backend="packed")
+    fused = packed.module["down_proj"]
+    assert isinstance(fused, mk.PackedLinear) and fused._rotation is not None and fused._rotation.block == 2048
+    plain = copy.deepcopy(fused)
+    plain._rotation = None
+    hook = OnlineRotation(mk.layer_seed("down_proj", 4), 2048)
+    for samples in (1, 2, 8, 20):
+        inputs = torch.randn(samples, width, device="cuda").half()
+        with torch.inference_mode():
+            assert torch.equal(fused(inputs), plain(hook(inputs))), samples
+    converted.save(tmp_path / "blocks")
+    restored = mk.load_checkpoint(tmp_path / "blocks",
+                                  model=lambda: nn.ModuleDict({"down_proj": nn.Linear(width, rows, dtype=torch.float16)}))
+    assert restored.transforms[0]["block"] == 2048
+    with torch.inference_mode():
+        assert torch.equal(restored.module["down_proj"](x), converted.module["down_proj"](x))
+
+
 def test_checkpoint_mirrors_of_the_reference_tests(tmp_path):
     import json
 

@@ -509,3 +509,50 @@ def test_rotation_inside_the_matvec_kernel(rows, width, asym, with_bias, with_si
     host_signs = np.ones(width, dtype=np.float32) if signs is None else signs.cpu().numpy()
     expected_x = torch.from_numpy(oracle_transforms.randomized(x.float().cpu().numpy(), host_signs)).half().float()
     check(outputs[0].float().cpu().numpy(), layer, expected_x, None if bias is None else bias.cpu(), relative=2e-3)
+
+
+@pytest.mark.parametrize("rows,width,block,asym,with_bias,with_signs", [
+    (4096, 14336, 2048, False, True, True),     # seven blocks, one per wavefront: no exchange between wavefronts
+    (512, 14336, 512, True, False, True),       # four blocks per wavefront: the last lane stages are left out
+    (4096, 12288, 4096, False, False, False),   # three blocks of two wavefronts each
+    (256, 6144, 64, True, True, True),          # the shortest block: one lane stage
+])
+def test_rotation_of_separate_blocks_inside_the_matvec_kernel(rows, width, block, asym, with_bias, with_signs):
+    """order > 1 without a basis: every block of `power` values is Walsh-Hadamard transformed for
+    itself.  One fp16 sample of whole 2048-code slices runs in ONE launch, the transform inside
+    the matvec kernel with the stages above the block length left out: bit for bit
+    mk_packed_matvec on mk_fwht's output (rows of `block` values) rounded to fp16, the buffer
+    untouched.  Two samples take mk_fwht and mk_packed_matvec behind each other and equal the same."""
+    from mlkit_amd import native
+    from mlkit_amd.kernels import hadamard
+    from oracle import transforms as oracle_transforms
+
+    weight = helpers.normal_weight(rows, width, seed=rows + width)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True, asym=asym)
+    tensors = helpers.to_device(layer, torch.float16)
+    signs = torch.from_numpy(oracle_transforms.deterministic_signs(width, seed=3)).cuda() if with_signs else None
+    bias = helpers.activations(1, rows, seed=6)[0].cuda() if with_bias else None
+    lib = native.library()
+    matvec = (tensors["packed"].data_ptr(), tensors["scales"].data_ptr(), native.dtype_code(tensors["scales"]),
+              tensors["values"].data_ptr(), 16, native.pointer(tensors["zeros"]), native.pointer(bias), native.MK_F16)
+    for samples in (1, 2):
+        x = helpers.activations(samples, width, seed=5 + samples).cuda()
+        rotated = hadamard.transform(x.float().view(samples, width // block, block), signs_before=signs).half().view(samples, width)
+        outputs = [torch.full((samples, rows), float("nan"), dtype=torch.float16, device="cuda") for _ in range(2)]
+        workspace = torch.full((samples, width), float("nan"), dtype=torch.float16, device="cuda")
+        shape = (samples, rows, width, 128, 4, 1, -8.0, 1.0, native.current_stream(x.device))
+        native.check(lib.mk_rotated_packed_matvec(x.data_ptr(), native.MK_F16, workspace.data_ptr(), width // block, block,
+                                                  None, native.pointer(signs), hadamard.normaliser(block), *matvec,
+                                                  outputs[0].data_ptr(), *shape))
+        native.check(lib.mk_packed_matvec(rotated.data_ptr(), native.MK_F16, *matvec, outputs[1].data_ptr(), *shape))
+        torch.cuda.synchronize()
+        if samples == 1:
+            assert torch.isnan(workspace).all()      # one launch: the buffer was not needed
+        else:
+            assert torch.equal(workspace, rotated)   # mk_fwht wrote the rotated activations there
+        assert torch.equal(outputs[0], outputs[1])
+        host_signs = np.ones(width, dtype=np.float32) if signs is None else signs.cpu().numpy()
+        blocks = (x.float().cpu().numpy() * host_signs).reshape(samples, width // block, block)
+        expected_x = torch.from_numpy(oracle_transforms.fwht(blocks).reshape(samples, width)).half().float()
+        check(outputs[0].float().cpu().numpy(), layer, expected_x, None if bias is None else bias.cpu(), relative=2e-3)
+
