@@ -394,3 +394,34 @@ def test_vector_grid_and_feedback_on_the_host():
     torch.testing.assert_close(joined.w, lattice.w, rtol=0, atol=0)
     with pytest.raises(ValueError, match="step equal to its dimension"):
         mk.ldlq(quantization, step=8, backend="hip")(weights, Ctx("layer", H=torch.eye(64)))
+
+
+def test_rotation_of_separate_blocks_on_the_host():
+    """``rht(value, seed, block=b)`` transforms blocks of b values one by one: per block the
+    oracle's stagewise transform of value * signs, its own inverse, and an error for blocks
+    that do not tile the width as powers of two.  ``mk.rotate(seed, block=b)`` records the
+    block length with the layer and leaves layers the blocks do not tile to the whole-row
+    transform."""
+    from oracle import transforms as oracle_transforms
+    from mlkit_amd.conversion import RotateInputs
+
+    torch.manual_seed(3)
+    value = torch.randn(5, 768)
+    rotated = mk.rht(value, seed=9, block=256)
+    signs = host_transforms.random_signs(768, 9, "cpu").numpy()
+    expected = oracle_transforms.fwht((value.numpy() * signs).reshape(5, 3, 256)).reshape(5, 768)
+    np.testing.assert_allclose(rotated.numpy(), expected, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(mk.rht(rotated, seed=9, inverse=True, block=256).numpy(), value.numpy(), rtol=1e-5, atol=1e-5)
+    with pytest.raises(ValueError, match="do not tile"):
+        mk.rht(value, seed=9, block=512)
+    with pytest.raises(ValueError, match="do not tile"):
+        mk.rht(value, seed=9, block=96)
+    module = nn.ModuleDict({"down_proj": nn.Linear(768, 8), "o_proj": nn.Linear(96, 8)})
+    inputs = torch.randn(2, 768)
+    before = module["down_proj"](inputs)
+    mk.rotate(seed=1, block=256)(module)
+    descriptors = {entry["name"]: entry for entry in module._mlkit_transforms}
+    assert descriptors["down_proj"]["block"] == 256 and "block" not in descriptors["o_proj"]
+    hook, = (h for h in module["down_proj"]._forward_pre_hooks.values() if isinstance(h, RotateInputs))
+    assert hook.rotation.block == 256
+    torch.testing.assert_close(module["down_proj"](inputs), before, rtol=1e-4, atol=1e-5)
