@@ -93,12 +93,12 @@ int mk_packed_matvec_group(const void *const *x, int x_dtype, int count, const u
  * remaining arguments.  signs: NULL (or [input_width] fp32 of +-1, 16-byte aligned for the
  * one-launch form).  Results equal mk_rotate_rows followed by mk_packed_matvec bit for bit;
  * MK_ERR_UNSUPPORTED when mk_rotate_rows does not take (order, power).  One exception, taken
- * whenever it applies: one fp16 sample, no basis (a plain transform of 2048 / 4096 / 8192 /
+ * whenever it applies: one fp16 or bf16 sample, no basis (a plain transform of 2048 / 4096 / 8192 /
  * 16384 values, or separate blocks of 64 to 16384 values that tile a row of whole 2048-value
  * slices, 14336 = 7 x 2048 for one), INT4 codes with 16-bit scales and whole tiles of rows (16,
  * or 4 below 4096 rows) run as ONE launch in which every workgroup transforms the activations
  * in its registers; `rotated` is then left untouched, and the result equals mk_packed_matvec on
- * mk_fwht's (stagewise) output rounded to fp16 bit for bit -- for a plain transform the same
+ * mk_fwht's (stagewise) output rounded to x_dtype bit for bit -- for a plain transform the same
  * linear map as mk_rotate_rows, summed in the order of the stages.
  * Replaces: the rotate_inputs forward pre-hook (conversion/model_transforms.py:116-128) in
  * front of PackedLinear.forward (inference/packed_linear.py:148-245). */

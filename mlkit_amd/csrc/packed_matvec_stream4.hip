@@ -126,11 +126,13 @@ __device__ __forceinline__ void rotation_lane_stage(float (&v)[kChunkCodes], int
 // rotation is to run while the codes are still on their way.
 // `log_block`: the transform spans aligned blocks of 1 << log_block elements (64 at least): the
 // stages of higher index bits are left out (uniform branches).
-__device__ __forceinline__ void rotate_activations(XChunk<MK_F16> &x, const float4 (&sign)[kChunkCodes / 4], float scale,
+template <int XT>
+__device__ __forceinline__ void rotate_activations(XChunk<XT> &x, const float4 (&sign)[kChunkCodes / 4], float scale,
                                                    float *exchange, int wave, int waves, int lane, int log_block) {
+    static_assert(XT == MK_F16 || XT == MK_BF16, "16-bit activations");
     float v[kChunkCodes];
 #pragma unroll
-    for (int k = 0; k < kChunkCodes; ++k) v[k] = x_element(x, k);
+    for (int k = 0; k < kChunkCodes; ++k) v[k] = x_element<XT>(x, k);
 #pragma unroll
     for (int q = 0; q < kChunkCodes / 4; ++q) {
         v[4 * q] *= sign[q].x; v[4 * q + 1] *= sign[q].y; v[4 * q + 2] *= sign[q].z; v[4 * q + 3] *= sign[q].w;
@@ -164,19 +166,24 @@ __device__ __forceinline__ void rotate_activations(XChunk<MK_F16> &x, const floa
     }
 #pragma unroll
     for (int i = 0; i < kChunkCodes / 2; ++i) {
-        const mk_h2 pair = {static_cast<_Float16>(v[2 * i] * scale), static_cast<_Float16>(v[2 * i + 1] * scale)};
-        x.r[i] = __builtin_bit_cast(uint32_t, pair);
+        if constexpr (XT == MK_F16) {
+            const mk_h2 pair = {static_cast<_Float16>(v[2 * i] * scale), static_cast<_Float16>(v[2 * i + 1] * scale)};
+            x.r[i] = __builtin_bit_cast(uint32_t, pair);
+        } else {
+            x.r[i] = static_cast<uint32_t>(mk_float_to_bf16(v[2 * i] * scale)) |
+                     (static_cast<uint32_t>(mk_float_to_bf16(v[2 * i + 1] * scale)) << 16);
+        }
     }
 }
 
 // PARTS = 2: rows of at most 1024 codes, one wavefront per workgroup; lanes 0 - 31 take one
 // row and lanes 32 - 63 the next, so that a step covers two rows instead of leaving half the
 // wavefront without codes.
-// ROTATE: the activations are rotated in the kernel (one fp16 sample, whole power-of-two rows).
+// ROTATE: the activations are rotated in the kernel (one sample, rows of whole 2048-code slices).
 template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS, bool ROTATE = false>
 __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4Group &members) {
     static_assert(ROWS * MT <= 64 && ROWS % PARTS == 0, "one transposed reduction per workgroup");
-    static_assert(!ROTATE || (MT == 1 && XT == MK_F16 && PARTS == 1), "the fused rotation takes one fp16 sample of long rows");
+    static_assert(!ROTATE || (MT == 1 && PARTS == 1), "the fused rotation takes one sample of long rows");
     __shared__ float partials[64 * 8];  // [row sum][wavefront]
     // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
     // must not hold LDS for eight).
@@ -275,7 +282,7 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         chunk_from_slice(x[m], x_slice, lane & (kRowLanes - 1));
     }
     if constexpr (ROTATE)
-        rotate_activations(x[0], rotation_sign, a.rotate_scale, reinterpret_cast<float *>(x_slices_storage), wave, waves, lane,
+        rotate_activations<XT>(x[0], rotation_sign, a.rotate_scale, reinterpret_cast<float *>(x_slices_storage), wave, waves, lane,
                            a.rotate_log_block);
 
     // sum_k (min + step c_k) x_k = step * dot + min * sum(x) - step * (code-free part of dot).
@@ -347,9 +354,9 @@ __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const
     stream4_body<MT, HAS_ZERO, ROWS, XT, PARTS>(a, members);
 }
 
-template <bool HAS_ZERO, int ROWS>
+template <bool HAS_ZERO, int ROWS, int XT>
 __global__ void __launch_bounds__(512) stream4_rotating_kernel(const Stream4Args a, const Stream4Group members) {
-    stream4_body<1, HAS_ZERO, ROWS, MK_F16, 1, true>(a, members);
+    stream4_body<1, HAS_ZERO, ROWS, XT, 1, true>(a, members);
 }
 
 // ---- two to eight samples: the dot products on the matrix cores ---------------------------
@@ -744,7 +751,7 @@ int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream) {
     const long long block_length = 1ll << a.rotate_log_block;
     const bool whole_rows = a.width % 2048 == 0 && a.width >= 2048 && a.width <= 16384 && a.rotate_log_block >= 6 &&
                             a.rotate_log_block <= 14 && a.width % block_length == 0;
-    if (a.samples != 1 || a.x_dtype != MK_F16 || !whole_rows || a.rows % tile_rows != 0 ||
+    if (a.samples != 1 || (a.x_dtype != MK_F16 && a.x_dtype != MK_BF16) || !whole_rows || a.rows % tile_rows != 0 ||
         (reinterpret_cast<uintptr_t>(a.rotate_signs) & 15u) != 0)
         return -2;
     Stream4Group none;
@@ -766,8 +773,13 @@ int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream) {
         hipLaunchKernelGGL(kernel, grid, block, lds, stream, a, none);
         return 0;
     };
-    if (wide) return a.zeros ? launch(stream4_rotating_kernel<true, kWideRows>) : launch(stream4_rotating_kernel<false, kWideRows>);
-    return a.zeros ? launch(stream4_rotating_kernel<true, kNarrowRows>) : launch(stream4_rotating_kernel<false, kNarrowRows>);
+    auto of_type = [&](auto xt) -> int {
+        constexpr int XT = decltype(xt)::value;
+        if (wide) return a.zeros ? launch(stream4_rotating_kernel<true, kWideRows, XT>) : launch(stream4_rotating_kernel<false, kWideRows, XT>);
+        return a.zeros ? launch(stream4_rotating_kernel<true, kNarrowRows, XT>) : launch(stream4_rotating_kernel<false, kNarrowRows, XT>);
+    };
+    if (a.x_dtype == MK_F16) return of_type(std::integral_constant<int, MK_F16>{});
+    return of_type(std::integral_constant<int, MK_BF16>{});
 }
 
 int stream4_launch_group(const Stream4Args &shared, Stream4Group &group, const int *member_rows, int *rows_per_tile,

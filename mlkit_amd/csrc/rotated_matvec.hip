@@ -7,9 +7,10 @@
 // activations are at most 8 x 16384 values: they are written to a small buffer by the
 // row-rotation kernel (mk_rotate_rows: order * samples short workgroups) and read back, from
 // L2, by the matvec kernel enqueued right behind it on the same stream.  One library call replaces a Python hook, an
-// allocation and two calls.  One fp16 sample of an INT4 layer with a power-of-two row (2048 to
-// 16384 codes) needs neither the buffer nor the second launch: the matvec kernel transforms the
-// activations itself (rotate_inside_the_matvec).
+// allocation and two calls.  One fp16 or bf16 sample of an INT4 layer whose transform has no
+// basis (a power-of-two row of 2048 to 16384 codes, or separate power-of-two blocks of a row of
+// whole 2048-code slices) needs neither the buffer nor the second launch: the matvec kernel
+// transforms the activations itself (rotate_inside_the_matvec).
 
 #include <mutex>
 
@@ -17,15 +18,17 @@
 
 namespace {
 
-// One fp16 sample, INT4 codes on a uniform grid with 16-bit scales, a power-of-two row of 2048
-// to 16384 codes and whole tiles of rows: the matvec kernel rotates the activations itself while
-// its first codes are on their way (no second launch, no buffer).  Returns 1 when it took the
+// One fp16 or bf16 sample, INT4 codes on a uniform grid with 16-bit scales, a row of whole
+// 2048-code slices transformed in blocks of `block` values (the whole row: one block) and whole
+// tiles of rows: the matvec kernel rotates the activations itself while its first codes are on
+// their way (no second launch, no buffer).  Returns 1 when it took the
 // call, 0 when the shape is not one of these, a negative status on errors.
 int rotate_inside_the_matvec(const void *x, int x_dtype, int block, const float *signs, float scale, const uint8_t *packed,
                              const void *scales, int scale_dtype, const void *zeros, const void *bias, int bias_dtype,
                              void *y, int samples, int output_width, int input_width, int group, int bits, int uniform,
                              float grid_min, float grid_step, hipStream_t stream) {
-    if (samples != 1 || x_dtype != MK_F16 || !packed || !scales || !y || group < 1 || output_width < 1) return 0;
+    if (samples != 1 || (x_dtype != MK_F16 && x_dtype != MK_BF16) || !packed || !scales || !y || group < 1 || output_width < 1)
+        return 0;
     if (!mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0)) return 0;
     const auto misaligned = [](const void *pointer, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(pointer) & mask) != 0; };
     if (misaligned(packed, 3) || misaligned(scales, 3) || misaligned(zeros, 3) || misaligned(bias, 3) || misaligned(x, 15))

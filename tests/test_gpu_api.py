@@ -632,7 +632,7 @@ def test_packed_layer_absorbs_its_online_rotation(rows, width):
     """mk.optimize turns the rotate_inputs pre-hook of a rotated layer into a rotation inside
     PackedLinear.forward: one library call (rotation kernel + matvec) for up to eight rows.
     The result equals hook-then-matvec bit for bit (the same two kernels), for fp16 and bf16,
-    for more than eight rows (dense path) and after deepcopy / state reload.  One fp16 sample
+    for more than eight rows (dense path) and after deepcopy / state reload.  One sample
     of a power-of-two width is rotated inside the matvec kernel, with the sums of the stagewise
     transform: there the result equals the matvec of that transform's output, and the hook's
     (the same sums in another order) to rounding."""
@@ -658,12 +658,12 @@ def test_packed_layer_absorbs_its_online_rotation(rows, width):
             if samples > 8 and dtype != layer.weight.dtype:
                 continue   # the dense path multiplies in the layer's own dtype (bias included)
             x = torch.randn(samples, width, device="cuda").to(dtype)
-            inside = dtype == torch.float16 and samples == 1 and width & (width - 1) == 0
+            inside = samples == 1 and width & (width - 1) == 0
             with torch.inference_mode():
                 rotated = hook(x)
                 if inside:
-                    stagewise = hadamard.transform(x.float(), signs_before=random_signs(width, seed, "cuda")).half()
-                    assert (stagewise.float() - rotated.float()).abs().max() <= 2e-3 * rotated.float().abs().max()
+                    stagewise = hadamard.transform(x.float(), signs_before=random_signs(width, seed, "cuda")).to(dtype)
+                    assert (stagewise.float() - rotated.float()).abs().max() <= 1.6e-2 * rotated.float().abs().max()
                     rotated = stagewise
                 assert torch.equal(fused(x), plain(rotated)), (dtype, samples)
                 assert torch.equal(fused(x.view(1, samples, width)), plain(rotated).view(1, samples, rows))

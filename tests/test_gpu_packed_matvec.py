@@ -477,38 +477,41 @@ def test_grouped_launch_with_activations_per_matrix():
     (512, 8192, False, True, False),       # four wavefronts: two exchange stages; no sign vector
     (4096, 16384, True, False, True),      # eight wavefronts, the widest row
 ])
-def test_rotation_inside_the_matvec_kernel(rows, width, asym, with_bias, with_signs):
-    """One fp16 sample of an INT4 layer with a power-of-two row: mk_rotated_packed_matvec runs
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_rotation_inside_the_matvec_kernel(rows, width, asym, with_bias, with_signs, dtype):
+    """One fp16 or bf16 sample of an INT4 layer with a power-of-two row: mk_rotated_packed_matvec runs
     the Walsh-Hadamard rotation inside the matvec kernel.  Its stages and sums are the stagewise
     transform's, so the result equals, bit for bit, mk_packed_matvec on activations rotated by
-    mk_fwht and rounded to fp16; and it is the rotated layer of the oracle within tolerance."""
+    mk_fwht and rounded to the activation type; and it is the rotated layer of the oracle within tolerance."""
     from mlkit_amd import native
     from mlkit_amd.kernels import hadamard
     from oracle import transforms as oracle_transforms
 
     weight = helpers.normal_weight(rows, width, seed=rows + width)
     layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True, asym=asym)
-    tensors = helpers.to_device(layer, torch.float16)
-    x = helpers.activations(1, width, seed=5).cuda()
+    tensors = helpers.to_device(layer, dtype)
+    code = native.DTYPE_CODES[dtype]
+    x = helpers.activations(1, width, seed=5, dtype=dtype).cuda()
     signs = torch.from_numpy(oracle_transforms.deterministic_signs(width, seed=3)).cuda() if with_signs else None
-    bias = helpers.activations(1, rows, seed=6)[0].cuda() if with_bias else None
+    bias = helpers.activations(1, rows, seed=6, dtype=dtype)[0].cuda() if with_bias else None
     scale = hadamard.normaliser(width)
-    rotated = hadamard.transform(x.float(), signs_before=signs).half()        # stagewise, scaled, rounded once
+    rotated = hadamard.transform(x.float(), signs_before=signs).to(dtype)     # stagewise, scaled, rounded once
     lib = native.library()
-    outputs = [torch.full((1, rows), float("nan"), dtype=torch.float16, device="cuda") for _ in range(2)]
-    workspace = torch.full((1, width), float("nan"), dtype=torch.float16, device="cuda")
+    outputs = [torch.full((1, rows), float("nan"), dtype=dtype, device="cuda") for _ in range(2)]
+    workspace = torch.full((1, width), float("nan"), dtype=dtype, device="cuda")
     matvec = (tensors["packed"].data_ptr(), tensors["scales"].data_ptr(), native.dtype_code(tensors["scales"]),
-              tensors["values"].data_ptr(), 16, native.pointer(tensors["zeros"]), native.pointer(bias), native.MK_F16)
+              tensors["values"].data_ptr(), 16, native.pointer(tensors["zeros"]), native.pointer(bias), code)
     shape = (1, rows, width, 128, 4, 1, -8.0, 1.0, native.current_stream(x.device))
-    native.check(lib.mk_rotated_packed_matvec(x.data_ptr(), native.MK_F16, workspace.data_ptr(), 1, width, None,
+    native.check(lib.mk_rotated_packed_matvec(x.data_ptr(), code, workspace.data_ptr(), 1, width, None,
                                               native.pointer(signs), scale, *matvec, outputs[0].data_ptr(), *shape))
-    native.check(lib.mk_packed_matvec(rotated.data_ptr(), native.MK_F16, *matvec, outputs[1].data_ptr(), *shape))
+    native.check(lib.mk_packed_matvec(rotated.data_ptr(), code, *matvec, outputs[1].data_ptr(), *shape))
     torch.cuda.synchronize()
     assert torch.isnan(workspace).all()          # the buffer was not needed
     assert torch.equal(outputs[0], outputs[1])
     host_signs = np.ones(width, dtype=np.float32) if signs is None else signs.cpu().numpy()
-    expected_x = torch.from_numpy(oracle_transforms.randomized(x.float().cpu().numpy(), host_signs)).half().float()
-    check(outputs[0].float().cpu().numpy(), layer, expected_x, None if bias is None else bias.cpu(), relative=2e-3)
+    expected_x = torch.from_numpy(oracle_transforms.randomized(x.float().cpu().numpy(), host_signs)).to(dtype).float()
+    check(outputs[0].float().cpu().numpy(), layer, expected_x, None if bias is None else bias.cpu(),
+          relative=2e-3 if dtype == torch.float16 else 1.6e-2)
 
 
 @pytest.mark.parametrize("rows,width,block,asym,with_bias,with_signs", [
