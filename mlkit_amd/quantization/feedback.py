@@ -47,20 +47,22 @@ def _factor_in_place(matrix: Tensor, status: Tensor, factored: Tensor) -> None:
     in place (``status``: an int32 device scalar holding zero; ``factored``: scratch for the
     diagonal blocks, ``[ceil(width / 128), 128, 128]``).
 
-    Two levels of right-looking blocking: panels of 1024 columns update the rest of the matrix (a
+    Two levels of blocking.  Panels of 1024 columns update the rest of the matrix, right-looking (a
     rank-1024 product reads and writes the trailing matrix an eighth as often as rank-128 ones
-    would); inside a panel's diagonal block the same scheme runs with 128-column blocks:
-    ``mk_cholesky_block`` factors a diagonal block and carries the rest of its rows, to the last
-    column, through the same elimination, which makes them the factor's block row; no triangular
-    solve is left.  The factored diagonal blocks themselves are needed by nobody before the end
-    (updates read block rows only): they wait in ``factored`` and go into the matrix in one copy.
+    would).  Inside a panel 128-column blocks are factored left-looking: a block's rows first take
+    the updates of all earlier blocks of the panel in one product, then ``mk_cholesky_block``
+    factors the diagonal block and carries the rest of its rows, to the last column, through the
+    same elimination, which makes them the factor's block row; no triangular solve is left.  (The
+    chain block kernel -> product -> block kernel is what bounds the run time; right-looking blocks
+    with the far rows of each update on a stream of their own made it 7 % longer: every block then
+    waited for two products.)  The factored diagonal blocks themselves are needed by nobody before
+    the end (updates read block rows only): they wait in ``factored`` and go into the matrix in one
+    copy.
 
-    Look-ahead, on two levels.  Inside a panel, a block's update of the rows of the *next* block
-    runs on the current stream and the next block kernel follows at once; its update of the
-    panel's remaining rows runs on a second stream meanwhile.  Between panels, only the band of
-    rows the next panel consists of is updated on the current stream; the rest runs on a third
-    stream while the next panel is factored.  Events fix the order in which updates reach every
-    entry, so results do not depend on timing (and are the same with all work on one stream).
+    Look-ahead between panels: only the band of rows the next panel consists of is updated on the
+    current stream; the rest runs on a second stream while the next panel is factored.  Events fix
+    the order in which updates reach every entry, so results do not depend on timing (and are the
+    same with all work on one stream).
 
     ``status`` stays zero, or becomes one plus the first column whose pivot is not positive (as
     ``torch.linalg.cholesky_ex`` reports it).  Nothing here allocates device memory or reads
@@ -73,7 +75,6 @@ def _factor_in_place(matrix: Tensor, status: Tensor, factored: Tensor) -> None:
     main = torch.cuda.current_stream(device)
     look_ahead = width >= LOOK_AHEAD_WIDTH   # narrower: the event traffic costs more than it hides
     side = torch.cuda.Stream(device) if look_ahead else None    # far rows of a panel's update
-    inner = torch.cuda.Stream(device) if look_ahead else None   # remaining rows of a block's update inside its panel
 
     def subtract_outer_product(start: int, stop: int, first_row: int, last_row: int, limit: int, after_first_band=None):
         """A[r, c] -= sum_k U[k, r] U[k, c] for k in start:stop, rows first_row:last_row, columns from
@@ -93,9 +94,14 @@ def _factor_in_place(matrix: Tensor, status: Tensor, factored: Tensor) -> None:
     for panel_start in range(0, width, FACTORIZATION_PANEL):
         panel_stop = min(width, panel_start + FACTORIZATION_PANEL)
         raw_stream = native.current_stream(device)
-        inner_done = None
         for start in range(panel_start, panel_stop, FACTORIZATION_BLOCK):
             stop = min(panel_stop, start + FACTORIZATION_BLOCK)
+            if start > panel_start:
+                # the block's rows take the updates of every earlier block of the panel at once: one
+                # product of rank start - panel_start, over all columns to the right (what a triangular
+                # solve with the panel's whole diagonal block would otherwise do for them)
+                matrix[start:stop, start:width].addmm_(matrix[panel_start:start, start:stop].T,
+                                                       matrix[panel_start:start, start:width], alpha=-1.0)
             # the block kernel also carries the rest of rows start:stop, to the matrix's last column,
             # through the elimination (their block row of the factor); the factored block goes to
             # `factored`, since every workgroup of that launch reads the block itself
@@ -103,26 +109,6 @@ def _factor_in_place(matrix: Tensor, status: Tensor, factored: Tensor) -> None:
             slot = factored[start // FACTORIZATION_BLOCK]
             native.check(library.mk_cholesky_block(matrix[start, start:].data_ptr(), width, stop - start, start, beside,
                                                    slot.data_ptr() if beside else None, status.data_ptr(), raw_stream))
-            if stop >= panel_stop:
-                continue
-            # the rest of the panel's rows, over all columns to the right (what a triangular solve
-            # with the panel's whole diagonal block would otherwise do for them): the next block's
-            # rows now, after the earlier blocks' updates of them; the others beside the next block
-            next_stop = min(panel_stop, stop + FACTORIZATION_BLOCK)
-            if inner_done is not None:
-                main.wait_event(inner_done)
-            subtract_outer_product(start, stop, stop, next_stop, width)
-            if next_stop >= panel_stop:
-                continue
-            if not look_ahead:
-                subtract_outer_product(start, stop, next_stop, panel_stop, width)
-                continue
-            inner.wait_event(main.record_event())   # (also behind this block's update of the next rows: harmless)
-            with torch.cuda.stream(inner):
-                subtract_outer_product(start, stop, next_stop, panel_stop, width)
-                inner_done = inner.record_event()
-        if inner_done is not None:
-            main.wait_event(inner_done)
         # the diagonal block's lower triangle holds leftovers of the products above
         matrix[panel_start:panel_stop, panel_start:panel_stop].triu_()
         if panel_stop == width:
@@ -131,7 +117,7 @@ def _factor_in_place(matrix: Tensor, status: Tensor, factored: Tensor) -> None:
             subtract_outer_product(panel_start, panel_stop, panel_stop, width, width)
             continue
         row_ready = main.record_event()
-        # the rows of the next panel: here, after the third stream's earlier update of them (its
+        # the rows of the next panel: here, after the second stream's earlier update of them (its
         # first band: the stream works through the bands from the top, and through the panels in
         # order, so that band being done means every earlier update of these rows is)
         next_panel_stop = min(width, panel_stop + FACTORIZATION_PANEL)
