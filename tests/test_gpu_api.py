@@ -706,6 +706,10 @@ def test_rotation_of_separate_blocks_end_to_end(tmp_path):
         inputs = torch.randn(samples, width, device="cuda").half()
         with torch.inference_mode():
             assert torch.equal(fused(inputs), plain(hook(inputs))), samples
+    for samples in (1, 3):   # bf16 activations into the fp16 layer: the same launches in the other type
+        inputs = torch.randn(samples, width, device="cuda").bfloat16()
+        with torch.inference_mode():
+            assert torch.equal(fused(inputs), plain(hook(inputs))), samples
     converted.save(tmp_path / "blocks")
     restored = mk.load_checkpoint(tmp_path / "blocks",
                                   model=lambda: nn.ModuleDict({"down_proj": nn.Linear(width, rows, dtype=torch.float16)}))
