@@ -238,3 +238,44 @@ def test_row_rotation_kernel_matches_oracle(width, dtype):
             assert (host(rotated.float()) == rounded).mean() > 0.99          # one rounding: only near-ties move
     first = rotation(value[:1].cuda())
     assert torch.equal(first, rotated[:1])
+
+
+def test_known_answers_of_the_bases_on_the_device():
+    """The device path applies the known Paley sign patterns and scipy's DCT-II to the outer axis
+    (tests/golden/transform_known_answers.json, worked out with Python integers): a unit vector e_f comes out
+    as column f of the basis, and with a power-of-two factor as that column times the Sylvester block."""
+    import json
+    import pathlib
+
+    import scipy.fft
+
+    from mlkit_amd.quantization import codecs, transforms as device_transforms
+
+    known = json.loads((pathlib.Path(__file__).resolve().parent / "golden" / "transform_known_answers.json").read_text())
+    for order in (12, 20, 28, 44):
+        pattern = np.array(known["paley"][str(order)], dtype=np.float64) / np.sqrt(order)
+        out = host(device_transforms.structured_transform(torch.eye(order, device="cuda")))
+        np.testing.assert_allclose(out, pattern.T, atol=1e-6)
+        back = host(device_transforms.structured_transform(torch.eye(order, device="cuda"), inverse=True))
+        np.testing.assert_allclose(back, pattern, atol=1e-6)
+    pattern = np.array(known["paley"]["28"], dtype=np.float64) / np.sqrt(28)
+    for power in (2, 32, 512):                                        # 56, 896, 14336 = 28 x power
+        width = 28 * power
+        rows = torch.zeros(3, width, device="cuda")
+        picks = [(0, 0), (1, power + 1), (2, 14 * power + power - 1)]  # e_(f, p) at rows 0, 1, 2
+        for row, index in picks:
+            rows[row, index] = 1.0
+        out = host(device_transforms.structured_transform(rows)).reshape(3, 28, power)
+        sylvester = transforms.sylvester(power) / np.sqrt(power)
+        for row, index in picks:
+            f, p = divmod(index, power)
+            np.testing.assert_allclose(out[row], np.outer(pattern[:, f], sylvester[:, p]), atol=1e-6)
+    for width, order in ((7, 7), (43, 43), (86, 43), (11008, 43)):
+        power = width // order
+        dct = scipy.fft.dct(np.eye(order), type=2, norm="ortho", axis=0)
+        rows = torch.zeros(order, width, device="cuda")
+        rows[torch.arange(order), torch.arange(order) * power] = 1.0   # e_(f, 0)
+        out = host(device_transforms.structured_transform(rows)).reshape(order, order, power)
+        np.testing.assert_allclose(out[:, :, 0], dct.T / np.sqrt(power), atol=1e-6)
+    for case in known["signs"]:
+        assert codecs.deterministic_signs(16, case["seed"], "cuda").tolist() == case["first"]
