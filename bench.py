@@ -1,12 +1,12 @@
 """Headline benchmark: INT4-g128 packed matvec, weight 4096x14336 (N x K), M=1, on one MI355X.
 
-One step = one call of ``mk_packed_matvec_group`` over ``--members`` (default 8) distinct
-4096x14336 weight matrices that read one activation row each: the shape of a
-mixture-of-experts layer's expert down-projections, or of sibling projections fed by one
-tensor.  Every member is a complete INT4-g128 matvec whose output equals the single-matrix
-call bit for bit; the single-matrix chain (one ``mk_packed_matvec`` per step) is timed beside
-it and reported in ``config.by_rows``.  Weight sets rotate so that more than 512 MB of distinct
-weights pass between two uses of a set and the 256 MB Infinity Cache cannot serve the stream.
+One step = one ``mk_packed_matvec`` call on one 4096x14336 weight matrix and one activation
+row: the launch ``PackedLinear.forward`` issues per layer.  ``config`` also carries the same
+call at M = 2, 4, 8 (``us_M*``, ``frac_M*``) and the grouped launch (``mk_packed_matvec_group``
+over eight such matrices that read one activation row each, as the experts of a
+mixture-of-experts layer or sibling projections do; ``--members 8`` makes that the step).
+Weight copies rotate so that more than 512 MB of distinct weights pass between two uses of a
+copy and the 256 MB Infinity Cache cannot serve the stream.
 
 The timed region is a HIP graph of ``--steps`` calls; ``ms_per_step`` is the median over
 ``--replays`` timed replays (HIP events on the stream the graph runs on).  Prints ONE JSON line:
@@ -38,10 +38,14 @@ MFMA_FP32_PEAK_TFLOPS = 157.3
 MINIMUM_ROTATING_BYTES = 512 * 2**20
 # HBM bytes per matrix of a launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; recorded, not
 # measured by this script.
-RECORDED_TRAFFIC = {"bytes_per_matrix": 30_331_800,
-                    "source": "profiles/packed_matvec_stream4_int4_g128_4096x14336_m1_group8.md (rocprofv3 --pmc "
-                              "FETCH_SIZE, WRITE_SIZE of the 8-matrix launch, per matrix); recorded there, not measured in "
-                              "this run"}
+RECORDED_TRAFFIC = {
+    "single": {"bytes_per_launch": 30_638_000,
+               "source": "profiles/packed_matvec_stream4_int4_g128_4096x14336_m1.md (rocprofv3 --pmc FETCH_SIZE, then "
+                         "WRITE_SIZE); recorded there, not measured in this run"},
+    "group_of_8": {"bytes_per_launch": 8 * 30_331_800,
+                   "source": "profiles/packed_matvec_stream4_int4_g128_4096x14336_m1_group8.md (rocprofv3 --pmc FETCH_SIZE, "
+                             "then WRITE_SIZE of the 8-matrix launch); recorded there, not measured in this run"},
+}
 
 
 def algorithmic_bytes(samples: int) -> int:
@@ -149,10 +153,11 @@ def _blas_threads(limit: int | None):
 
 
 def cpu_matvec_baseline() -> dict:
-    """The CPU restatement of reconstruct-then-matmul (unpack -> values[codes] * scale -> fp32
-    matmul) on the whole 4096x14336 layer at M=1, one thread: at least 10 timed repetitions of
-    the matmul on the reconstructed weight after 2 warm-ups, and as many whole passes
-    (reconstruction included) as fit in about 12 s."""
+    """The CPU restatement of the reference's CPU path, reconstruct-then-matmul (unpack ->
+    values[codes] * scale -> fp32 matmul), on the whole 4096x14336 layer at M=1: as tensor
+    operations on all of the host's cores (the reported value), and as numpy on one thread beside
+    it.  Whole passes (reconstruction included) for about 10 s and 6 s, the first of each untimed;
+    then the product alone on the reconstructed weight."""
     from oracle import matvec as oracle_matvec, scaling
 
     rng = np.random.default_rng(7)
@@ -160,37 +165,45 @@ def cpu_matvec_baseline() -> dict:
     scales = (rng.random((ROWS, WIDTH // GROUP), dtype=np.float32) * 0.004 + 0.005).astype(np.float16).astype(np.float32)
     values = scaling.int_values(4)
     x = rng.standard_normal((1, WIDTH), dtype=np.float32).astype(np.float16).astype(np.float32)
+
+    def passes(function, seconds, most):
+        times = []
+        budget = time.perf_counter() + seconds
+        while len(times) < most and (len(times) < 2 or time.perf_counter() < budget):
+            started = time.perf_counter()
+            function()
+            times.append(time.perf_counter() - started)
+        return float(np.median(times[1:]))      # the first pass warms the caches
+
+    tensors = [torch.from_numpy(array) for array in (x, packed, scales, values)]
+    threads = torch.get_num_threads()
+    whole_torch = passes(lambda: oracle_matvec.reconstruct_then_matmul_torch(
+        tensors[0], tensors[1], BITS, (ROWS, WIDTH), tensors[2], tensors[3], GROUP), 10.0, 12)
+    _, dense = oracle_matvec.reconstruct_then_matmul_torch(tensors[0], tensors[1], BITS, (ROWS, WIDTH), tensors[2],
+                                                           tensors[3], GROUP)
+    product_torch = passes(lambda: oracle_matvec.reconstruct_then_matmul_torch(
+        tensors[0], None, BITS, (ROWS, WIDTH), None, None, GROUP, dense=dense), 2.0, 12)
+    del dense
     limiter = _blas_threads(1)
     try:
-        whole = []
-        budget = time.perf_counter() + 12.0
-        dense = None
-        while len(whole) < 10 and (len(whole) < 2 or time.perf_counter() < budget):
-            started = time.perf_counter()
-            dense = oracle_matvec.dequantise(packed, BITS, (ROWS, WIDTH), scales, values, GROUP)
-            oracle_matvec.reconstruct_then_matmul(x, None, BITS, (ROWS, WIDTH), scales, values, GROUP, dense=dense)
-            whole.append(time.perf_counter() - started)
-        for _ in range(2):
-            oracle_matvec.reconstruct_then_matmul(x, None, BITS, (ROWS, WIDTH), scales, values, GROUP, dense=dense)
-        matmul = []
-        for _ in range(10):
-            started = time.perf_counter()
-            oracle_matvec.reconstruct_then_matmul(x, None, BITS, (ROWS, WIDTH), scales, values, GROUP, dense=dense)
-            matmul.append(time.perf_counter() - started)
+        whole_numpy = passes(lambda: oracle_matvec.reconstruct_then_matmul(
+            x, packed, BITS, (ROWS, WIDTH), scales, values, GROUP), 6.0, 5)
     finally:
         if limiter is not None and hasattr(limiter, "restore_original_limits"):
             limiter.restore_original_limits()
-    timed = whole[1:] if len(whole) > 1 else whole   # the first pass warms the caches
-    seconds = float(np.median(timed))
     return {
-        "value": WEIGHT_BYTES / seconds / 1e9,
+        "value": WEIGHT_BYTES / whole_torch / 1e9,
         "unit": "GB/s effective weight bandwidth",
-        "cores": 1,
+        "cores": threads,
         "kind": "port",
-        "sample": f"{len(timed)} timed passes (after 1 warm-up) over the whole 4096x14336 INT4-g128 layer at M=1: numpy unpack + "
-                  f"dequantise + fp32 matmul, one thread, median {seconds * 1e3:.0f} ms; the matmul alone on the reconstructed "
-                  f"weight, 10 repetitions after 2 warm-ups, median {float(np.median(matmul)) * 1e3:.2f} ms "
-                  f"({WEIGHT_BYTES / float(np.median(matmul)) / 1e9:.1f} GB/s of packed bytes); os.cpu_count()={os.cpu_count()}",
+        "us_per_call": whole_torch * 1e6,
+        "matmul_only_us_per_call": product_torch * 1e6,
+        "one_thread_numpy_GBps": WEIGHT_BYTES / whole_numpy / 1e9,
+        "os_cpu_count": os.cpu_count(),
+        "sample": f"whole 4096x14336 INT4-g128 layer, M=1, reconstruct-then-matmul as torch tensor operations on "
+                  f"{threads} threads (torch.get_num_threads()), median of the passes that fit 10 s: {whole_torch * 1e3:.0f} ms "
+                  f"per call; the fp32 product alone on the reconstructed weight {product_torch * 1e3:.2f} ms; the numpy "
+                  f"restatement on one thread {whole_numpy * 1e3:.0f} ms per call; os.cpu_count()={os.cpu_count()}",
     }
 
 
@@ -573,7 +586,11 @@ def main() -> None:
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=100)
     parser.add_argument("--warmup", type=int, default=20)
-    parser.add_argument("--members", type=int, default=8, help="weight matrices per mk_packed_matvec_group call (1..8)")
+    parser.add_argument("--members", type=int, default=1,
+                        help="weight matrices per step: 1 = one mk_packed_matvec call (the metric's configuration), 2..8 = one "
+                             "mk_packed_matvec_group call over that many matrices")
+    parser.add_argument("--gptq-cpu-rows", type=int, default=4096,
+                        help="rows of the 4096 x 11008 layer that the CPU restatement of the GPTQ sweep covers (all by default)")
     parser.add_argument("--replays", type=int, default=60, help="timed replays of the graph; the median is reported")
     parser.add_argument("--copies", type=int, default=0, help="distinct weight copies in rotation (default: enough for 512 MB "
                                                                "between two uses of a copy)")
@@ -602,7 +619,7 @@ def main() -> None:
     # Between two uses of a weight set at least 512 MB of other weights are streamed.
     sets = -(-MINIMUM_ROTATING_BYTES // (members * WEIGHT_BYTES)) + 1
     copy_count = max(options.copies, sets * members, 18)
-    copy_count = -(-copy_count // members) * members
+    copy_count = -(-copy_count // 8) * 8 if 8 % members == 0 else -(-copy_count // (8 * members)) * 8 * members
     copies = make_copies(copy_count, device)
     generator = torch.Generator(device=device).manual_seed(5)
 
@@ -630,37 +647,47 @@ def main() -> None:
         return
 
     results = {}
+    flat = {}
     head_step = None
     for samples in (1, 2, 4, 8):
         x = torch.randn((samples, WIDTH), device=device, generator=generator).half()
         y = torch.empty((samples, ROWS), device=device, dtype=torch.float16)
         single = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
         row = {}
-        median, low, high, batch = timed_graph(single, max(options.steps, 50), options.warmup, max(20, options.replays // 2))
+        head = samples == 1 and members == 1
+        steps = options.steps if head else max(options.steps, 50)
+        replays = options.replays if head else max(20, options.replays // 2)
+        median, low, high, batch = timed_graph(single, steps, options.warmup, replays)
+        if head:
+            head_step = (median, low, high, batch, steps, replays)
         row["single_call"] = {"us_per_matrix": median * 1e6, "min_us": low * 1e6, "max_us": high * 1e6,
                               "hbm_frac": algorithmic_bytes(samples) / median / 1e9 / HBM_PEAK_GBPS}
         resident = timed_graph([single[0]], max(options.steps, 50), options.warmup, 10)[0]
         row["single_call"]["cache_resident_us"] = resident * 1e6
-        for count in sorted({2, 4, members} - {1}):
+        flat[f"us_M{samples}"] = median * 1e6
+        flat[f"frac_M{samples}"] = row["single_call"]["hbm_frac"]
+        flat[f"cache_resident_us_M{samples}"] = resident * 1e6
+        for count in sorted({2, 4, 8, members} - {1}):
             grouped = [GroupLauncher(x, copies[index:index + count], values) for index in range(0, copy_count - count + 1, count)]
-            steps = options.steps if (samples == 1 and count == members) else max(options.steps // 2, 25)
-            replays = options.replays if (samples == 1 and count == members) else max(20, options.replays // 3)
+            head = samples == 1 and count == members
+            steps = options.steps if head else max(options.steps // 2, 25)
+            replays = options.replays if head else max(20, options.replays // 3)
             median, low, high, batch = timed_graph(grouped, steps, options.warmup, replays)
             row[f"group_of_{count}"] = {"us_per_call": median * 1e6, "us_per_matrix": median * 1e6 / count,
                                         "min_us_per_matrix": low * 1e6 / count, "max_us_per_matrix": high * 1e6 / count,
                                         "hbm_frac": algorithmic_bytes(samples) * count / median / 1e9 / HBM_PEAK_GBPS}
-            if samples == 1 and count == members:
+            if count == 8:
+                flat[f"group_of_8_us_per_matrix_M{samples}"] = median * 1e6 / count
+                flat[f"group_of_8_frac_M{samples}"] = row["group_of_8"]["hbm_frac"]
+            if head:
                 head_step = (median, low, high, batch, steps, replays)
             del grouped
         results[samples] = row
-    if members == 1:
-        x = torch.randn((1, WIDTH), device=device, generator=generator).half()
-        y = torch.empty((1, ROWS), device=device, dtype=torch.float16)
-        single = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
-        median, low, high, batch = timed_graph(single, options.steps, options.warmup, options.replays)
-        head_step = (median, low, high, batch, options.steps, options.replays)
     per_step, low, high, batch, steps, replays = head_step
     achieved = algorithmic_bytes(1) * members / per_step / 1e9
+    traffic = RECORDED_TRAFFIC["group_of_8" if members == 8 else "single"] if members in (1, 8) else None
+    one_step = ("one mk_packed_matvec call (one launch of one matrix, what PackedLinear.forward issues per layer)" if members == 1
+                else f"one mk_packed_matvec_group call over {members} such matrices (one launch)")
     line = {
         "metric": "effective weight GB/s, INT4-g128 packed matvec 4096x14336, M=1",
         "value": WEIGHT_BYTES * members / per_step / 1e9,
@@ -675,16 +702,14 @@ def main() -> None:
         "dtype": "f16 activations, u4 codes, f32 accumulate",
         "data": "synthetic seeded codes and fp16 scales",
         "config": {
-            "workload": f"INT4 symmetric g128 packed matvec, weight 4096x14336 (N x K), M=1; one step = one "
-                        f"mk_packed_matvec_group call over {members} such matrices (one launch); "
+            "workload": f"INT4 symmetric g128 packed matvec, weight 4096x14336 (N x K), M=1; one step = {one_step}; "
                         f"{copy_count} distinct weight copies ({copy_count * WEIGHT_BYTES / 2**20:.0f} MiB) in rotation",
             "matrices_per_step": members,
-            "us_per_matrix": per_step * 1e6 / members,
-            "single_call_us_per_matrix": results[1]["single_call"]["us_per_matrix"],
+            "us_per_call": per_step * 1e6,
             "launch": "HIP graph of `steps` back-to-back calls on one stream",
-            "timing": {"replays": replays, "graph_launches_per_timed_replay": batch, "statistic": "median",
-                       "min_ms_per_step": low * 1e3, "max_ms_per_step": high * 1e3},
-            "by_rows": {str(k): v for k, v in results.items()},
+            "replays": replays, "graph_launches_per_timed_replay": batch, "statistic": "median",
+            "min_ms_per_step": low * 1e3, "max_ms_per_step": high * 1e3,
+            **flat,
         },
         "roofline": {
             "kernel": "stream4_kernel<1,false,16,f16,1> (one launch per step)",
@@ -694,21 +719,62 @@ def main() -> None:
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
             "algorithmic_bytes_per_launch": algorithmic_bytes(1) * members,
-            "traffic": RECORDED_TRAFFIC["bytes_per_matrix"] * members,
-            "traffic_source": RECORDED_TRAFFIC["source"],
+            "traffic": None if traffic is None else traffic["bytes_per_launch"],
+            "traffic_source": None if traffic is None else traffic["source"],
         },
         "cpu_baseline": None if options.no_cpu_baseline else cpu_matvec_baseline(),
+        "by_rows": {str(k): v for k, v in results.items()},
     }
     if not options.skip_kernels:
         del copies, single
         torch.cuda.empty_cache()
         kernels = other_kernels(device, options.kernels)
-        kernels["gptq int4 g128 4096x11008"] = gptq_layer(device, generator, cpu_rows=0 if options.no_cpu_baseline else 32)
+        kernels["gptq int4 g128 4096x11008"] = gptq_layer(device, generator, cpu_rows=0 if options.no_cpu_baseline else options.gptq_cpu_rows)
         kernels["vector grids"] = vector_ldlq_layer(device, generator, cpu_rows=0 if options.no_cpu_baseline else 16)
         if not options.no_cpu_baseline:
             kernels["fwht_cpu_baseline"] = cpu_fwht_baseline()
         line["kernels"] = kernels
-    print(json.dumps(line))
+        line["config"].update(kernel_summary(kernels))
+    # the record's first fields are the contract's; nested detail follows, floats cut to five digits
+    print(json.dumps(compact(line)))
+
+
+def kernel_summary(kernels: dict) -> dict:
+    """Flat scalars of the other kernels' figures, for records that keep scalars only."""
+    flat = {}
+    for label, entry in kernels.items():
+        if label.startswith("matvec ") and isinstance(entry, dict) and "ms" in entry:
+            key = label[len("matvec "):].replace(" ", "_").replace(",", "")
+            flat[f"us:{key}"] = entry.get("us_per_matrix", entry["ms"] * 1e3)
+            flat[f"frac:{key}"] = entry["hbm_frac"]
+        elif isinstance(entry, dict) and "hbm_frac" in entry:
+            flat[f"frac:{label.replace(' ', '_')}"] = entry["hbm_frac"]
+    gptq = kernels.get("gptq int4 g128 4096x11008", {})
+    if gptq:
+        flat["gptq_sweep_and_update_ms"] = gptq["sweep_and_update_ms"]
+        flat["gptq_coefficients_ms"] = gptq["coefficients_ms"]
+        flat["gptq_trailing_update_mfma_frac"] = gptq["trailing_update_roofline"]["frac"]
+        flat["gptq_proxy_loss"] = gptq["proxy_loss"]
+        if "cpu_baseline" in gptq:
+            flat["gptq_cpu_weights_per_s"] = gptq["cpu_baseline"]["value"]
+            flat["gptq_cpu_cores"] = gptq["cpu_baseline"]["cores"]
+            flat["gptq_codes_compared"] = gptq["cpu_baseline"]["codes_compared"]
+            flat["gptq_code_mismatches"] = gptq["cpu_baseline"]["code_mismatches_vs_device"]
+    for label, entry in kernels.get("rotated layers (config 5)", {}).items():
+        key = label.replace(" ", "_").replace(",", "")
+        flat[f"rotated_us:{key}"] = entry["rotated_us"]
+        flat[f"unrotated_us:{key}"] = entry["unrotated_us"]
+    return flat
+
+
+def compact(value):
+    if isinstance(value, float):
+        return float(f"{value:.5g}")
+    if isinstance(value, dict):
+        return {key: compact(item) for key, item in value.items()}
+    if isinstance(value, (list, tuple)):
+        return [compact(item) for item in value]
+    return value
 
 
 if __name__ == "__main__":

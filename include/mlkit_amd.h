@@ -135,7 +135,9 @@ int mk_packed_decode(const uint8_t *packed, const void *scales, int scale_dtype,
 
 /* Rows rows[0 .. n_rows) of the [output_width, input_width] packed matrix, decoded as by
  * mk_packed_decode into out [n_rows, input_width]: the embedding lookup of a tied output
- * projection.  rows: device int64; an index outside [0, output_width) decodes row 0.
+ * projection.  rows: device int64; a negative index i means output_width + i, as in the
+ * reference's tensor indexing; an index still outside [0, output_width) decodes row 0 (the
+ * reference raises there; the kernel stays within the matrix and reports nothing).
  * Replaces: the gather + unpack + decode_scaled of PackedEmbedding.forward
  * (inference/packed_linear.py:273-287). */
 int mk_packed_decode_rows(const uint8_t *packed, const void *scales, int scale_dtype, const float *values,

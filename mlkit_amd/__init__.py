@@ -18,7 +18,7 @@ from mlkit_amd.models import Model, QModel, quantize
 from mlkit_amd.quantization.bitstream import pack, unpack
 from mlkit_amd.quantization.codecs import codec, concatenate_rows, deterministic_signs
 from mlkit_amd.quantization.core import Ctx, Q, Quantizer, layer_seed, quantizer
-from mlkit_amd.quantization.feedback import feedback_coefficients, gptq, ldlq, proxy_loss
+from mlkit_amd.quantization.feedback import clear_factor_graphs, feedback_coefficients, gptq, ldlq, proxy_loss
 from mlkit_amd.quantization.grids import NF4_VALUES, Grid, grid
 from mlkit_amd.quantization.incoherence import Incoherent, incoherent
 from mlkit_amd.quantization.scaled import Scaled, int, mxfp4, nf4, scaled, store_scale  # noqa: A004
@@ -36,7 +36,7 @@ def rtn(w, ctx=None, *, fmt=None):
 
 __all__ = [
     "Capabilities", "Ctx", "Grid", "Model", "NF4_VALUES", "PackedEmbedding", "PackedLinear", "Q", "QModel",
-    "Quantizer", "Rotate", "Scaled", "capabilities", "codec", "concatenate_rows", "deterministic_signs",
+    "Quantizer", "Rotate", "Scaled", "capabilities", "clear_factor_graphs", "codec", "concatenate_rows", "deterministic_signs",
     "feedback_coefficients", "gptq", "grid", "hadamard", "incoherent", "install_transform", "int", "layer_seed", "ldlq", "load_checkpoint", "mxfp4",
     "nearest", "nf4", "optimize", "pack", "packed_compatible", "paley_matrix", "proxy_loss", "quantize", "quantizer", "rht",
     "rotate", "rtn", "save", "scaled", "snap", "store_scale", "structured_transform", "transform_factor", "unpack",

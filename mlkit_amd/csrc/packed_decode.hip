@@ -26,13 +26,14 @@ struct DecodeArgs {
     float grid_min, grid_step;
     int chunks_per_group_shift;   // log2(group / 32) when that is a power of two (31: one group per row), else -1
     const long long *row_index;   // null, or the source row of every output row (a gather of rows)
-    int source_rows;              // rows of the packed matrix; an index outside [0, source_rows) reads row 0
+    int source_rows;              // rows of the packed matrix; index i < 0 means source_rows + i; one still outside reads row 0
 };
 
 // The row of the packed matrix that output row `row` decodes.
 __device__ __forceinline__ size_t source_row_of(const DecodeArgs &a, size_t row) {
     if (!a.row_index) return row;
-    const long long wanted = a.row_index[row];
+    long long wanted = a.row_index[row];
+    if (wanted < 0) wanted += a.source_rows;   // -1 is the last row, as in tensor indexing
     return wanted >= 0 && wanted < a.source_rows ? static_cast<size_t>(wanted) : 0;
 }
 

@@ -108,6 +108,14 @@ __device__ __forceinline__ int nearest_lattice_code(const float (&v)[8], const L
                                                     int lane, float (&point)[8]) {
     float best_cost = __builtin_inff();
     int best_code = 0;
+    {   // Code 0 (pattern 0, no sign bits, the +1/4 coset): the answer when no cost compares below infinity (NaN).
+        float total = 0.0f;
+#pragma unroll
+        for (int d = 0; d < 8; ++d) total += patterns[d];
+        const int parity = static_cast<int>(total) & 1;
+#pragma unroll
+        for (int d = 0; d < 8; ++d) point[d] = __fadd_rn((d == 7 && parity) ? -patterns[d] : patterns[d], 0.25f);
+    }
 #pragma unroll
     for (int coset = 0; coset < 2; ++coset) {
         const float shift = coset == 0 ? -0.25f : 0.25f;

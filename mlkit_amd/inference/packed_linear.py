@@ -171,6 +171,13 @@ class PackedLinear(nn.Module):
                 self.__dict__["_siblings"].reset()
         super().register_buffer(name, tensor, persistent)
 
+    def __getstate__(self) -> dict:
+        """Bound launch arguments hold raw device addresses: a pickled or deep-copied layer (both go through
+        here) binds its own on first use."""
+        state = self.__dict__.copy()
+        state["_launch"] = state["_rotation_launch"] = None
+        return state
+
     def _apply(self, fn: Callable[[Tensor], Tensor], recurse: bool = True) -> "PackedLinear":
         self._launch = self._rotation_launch = None
         self._dense_weight = None
@@ -273,6 +280,13 @@ class PackedLinear(nn.Module):
         this device and input dtype, or None when the rotation kernels do not take the width."""
         key = (inputs.device, inputs.dtype)
         bound = self._rotation_launch
+        if bound is not None and bound[0] == key and bound[1] is not None:
+            # the bound pointers are addresses of the `keep` tensors: a copied or reloaded layer carries copies
+            # of those tensors (or none), never the addresses
+            _, _, basis, signs, _ = bound[2]
+            keep = bound[3]
+            if keep[0].data_ptr() != signs or (basis is not None and (len(keep) < 2 or keep[1].data_ptr() != basis)):
+                bound = None
         if bound is None or bound[0] != key:
             arguments = self._rotation.launch_arguments(self.in_features, inputs.device)
             if arguments is None:
@@ -311,7 +325,8 @@ class SiblingLaunch:
     version counter where one exists (not under ``torch.inference_mode``: there the model must
     not modify the shared input between the sibling calls).  Anything else -- another input, a
     member called twice -- simply starts a new grouped launch, so results never depend on the
-    cache being hit."""
+    cache being hit.  A member that is called with another input while its output of the last
+    grouped launch still waits does not share its siblings' input: it leaves the group."""
 
     MAXIMUM = 8
 
@@ -325,6 +340,23 @@ class SiblingLaunch:
     def reset(self) -> None:
         self._launch = None
         self._pending = None
+
+    def __getstate__(self) -> dict:
+        return {"layers": self.layers, "_launch": None, "_pending": None}
+
+    def _release(self, layer: "PackedLinear") -> None:
+        """Take ``layer`` out of the group; a group of one is dissolved."""
+        layer._siblings = None
+        self.layers = tuple(member for member in self.layers if member is not layer)
+        self._launch = None
+        if self._pending is not None:
+            self._pending[2].pop(id(layer), None)
+            if not self._pending[2]:
+                self._pending = None
+        if len(self.layers) == 1:
+            self.layers[0]._siblings = None
+            self.layers = ()
+            self._pending = None
 
     def __deepcopy__(self, memo: dict) -> "SiblingLaunch":
         """A copy links the copied layers and binds its own launch arguments on first use."""
@@ -364,6 +396,14 @@ class SiblingLaunch:
                 output = outputs.pop(id(layer))
                 if not outputs:
                     self._pending = None
+                return output
+            if id(layer) in outputs and kept is not original and kept.data_ptr() != original.data_ptr():
+                # an output of this layer is still waiting and it is called with a tensor that lives elsewhere: it
+                # does not read what its siblings read (an output projection beside q / k / v).  It leaves the
+                # group; its share of every grouped launch was wasted work.
+                self._release(layer)
+                output = flat.new_empty((flat.shape[0], layer.out_features))
+                layer._matvec(flat, output, flat.shape[0])
                 return output
         rows = flat.shape[0]
         results = [flat.new_empty((rows, member.out_features)) for member in self.layers]

@@ -146,4 +146,9 @@ def quantize(model: "Model | nn.Module", quantization: Callable[..., "Q | Tensor
         if result.bits is not None:
             result.bits = result.bits + context.additional_bits
         converted.quantized[name] = result
+    # captured factorisations (a width x width buffer each) served this pass; the model that is served next
+    # should not find their memory taken
+    from mlkit_amd.quantization.feedback import clear_factor_graphs
+
+    clear_factor_graphs()
     return converted

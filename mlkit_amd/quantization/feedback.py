@@ -153,10 +153,33 @@ class _FactorGraph:
         self.matrix = torch.empty((width, width), dtype=torch.float32, device=device)
         self.status = torch.zeros((), dtype=torch.int32, device=device)
         self.factored = _factor_scratch(width, device)
-        self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        current = torch.cuda.current_stream(device)
+        torch.cuda.synchronize(device)
+        stream = torch.cuda.Stream(device)
+        stream.wait_stream(current)
+        with torch.cuda.stream(stream):
+            try:
+                self.graph = self._captured()
+            except RuntimeError as error:
+                # The random generator's capture state belongs to the mode in which the process made its first
+                # capture.  If that was inference mode (a compiled model's first call under it), beginning a
+                # capture writes that state in place, which only inference mode may do: capture there.  The
+                # refused capture had not begun; its graph object is dropped.
+                if "nference tensor" not in str(error):
+                    raise
+                with torch.inference_mode():
+                    self.graph = self._captured()
+        current.wait_stream(stream)
+
+    def _captured(self) -> "torch.cuda.CUDAGraph":
+        graph = torch.cuda.CUDAGraph()
+        graph.capture_begin()
+        try:
             self.status.zero_()   # a fill kernel
             _factor_in_place(self.matrix, self.status, self.factored)
+        finally:
+            graph.capture_end()
+        return graph
 
     def __call__(self, fill: Callable[[Tensor], None]) -> tuple[Tensor, Tensor]:
         fill(self.matrix)
@@ -170,7 +193,9 @@ _factor_graphs: dict[tuple[int, int], "_FactorGraph | None"] = {}
 
 
 def clear_factor_graphs() -> None:
-    """Drop the captured factorisations and their buffers."""
+    """Drop the captured factorisations and their buffers (up to FACTOR_GRAPH_LIMIT graphs, each holding a
+    width x width fp32 matrix plus scratch: about 0.5 GB at 11008 columns).  ``mk.quantize`` calls this at
+    the end of a pass; callers that drive ``mk.gptq`` layer by layer themselves call it when they are done."""
     _factor_graphs.clear()
 
 
@@ -179,7 +204,7 @@ def _blocked_upper_factor(fill: Callable[[Tensor], None], width: int, device: to
     ``[width, width]`` FP32 tensor.  The first matrix of a width is factored launch by launch
     (which also warms every kernel up); from the second on the captured graph of that width
     runs.  The result may live in the graph's own buffer: it is valid until the next call."""
-    key = (device.index or 0, width)
+    key = (torch.cuda.current_device() if device.index is None else device.index, width)
     if FACTOR_GRAPHS and key in _factor_graphs and not torch.cuda.is_current_stream_capturing():
         graph = _factor_graphs[key]
         if graph is None:

@@ -221,6 +221,13 @@ class OnlineRotation:
         self.block = block   # None: the transform spans the row; else blocks of that many values, one by one
         self._plans: dict = {}
 
+    def __getstate__(self) -> dict:
+        """Prepared plans are closures over raw device addresses: a copy prepares its own."""
+        return {"seed": self.seed, "block": self.block, "_plans": {}}
+
+    def __deepcopy__(self, memo: dict) -> "OnlineRotation":
+        return OnlineRotation(self.seed, self.block)
+
     def __call__(self, value: Tensor) -> Tensor:
         key = (value.shape[-1], value.device, value.dtype)
         plan = self._plans.get(key)

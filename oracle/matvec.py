@@ -45,3 +45,26 @@ def reconstruct_then_matmul_f64(x, dense, bias=None) -> np.ndarray:
     if bias is not None:
         y = y + np.asarray(bias, dtype=np.float64)[None, :]
     return y
+
+
+def reconstruct_then_matmul_torch(x, packed, bits, shape, scales, values, group, zero=None, dense=None):
+    """The same path as tensor operations on the host's cores, as the reference's own CPU path
+    runs it (unpack: quantization/operations/bit_packing.py:80-99 for widths that divide a byte;
+    decode: codecs/scaled.py:55-60; then ``x @ w.T`` in fp32).  All arguments are CPU tensors;
+    returns ``(y, dense)`` so that a caller can time the product alone on the reconstruction."""
+    import torch
+
+    if dense is None:
+        if 8 % bits:
+            raise ValueError("the tensor restatement covers code widths that divide a byte")
+        rows, width = shape
+        stream = packed.flatten()
+        mask = 2**bits - 1
+        fields = [(stream >> shift) & mask for shift in range(0, 8, bits)]
+        codes = torch.stack(fields, dim=1).flatten()[: rows * width].reshape(rows, width)
+        reconstruction = values[codes.int()]
+        grouped = reconstruction.reshape(rows, -1, group) * scales.float()[:, :, None]
+        if zero is not None:
+            grouped = grouped + zero.float()[:, :, None]
+        dense = grouped.reshape(rows, width)
+    return x.float() @ dense.T, dense

@@ -79,3 +79,43 @@ def uniform_grid(values):
     steps = values.diff()
     uniform = bool(len(steps) and torch.allclose(steps, steps[0].expand_as(steps)))
     return uniform, float(values[0]), float(steps[0]) if len(steps) else 1.0
+
+
+ROTATED_NEAR_TIE_FRACTION = 0.02
+
+
+def check_rotated_layer(y, layer, device_rotated, oracle_rotated, dtype, bias=None):
+    """A rotated layer's output against the oracle, in two parts that together say what a single looser
+    output tolerance would blur:
+
+    * the matvec: ``y`` against the float64 product of the dense reconstruction with the activations the
+      DEVICE rotated (already rounded to ``dtype``), at the unrotated layers' tolerance: 1e-3 of the output
+      range for fp16, 8e-3 for bf16;
+    * the rotation: the device's rounded activations against the oracle's rotated activations rounded the same
+      way.  They are the same sums (in another order for the row-rotation kernel): no value may differ by more
+      than one unit in the last place of ``dtype`` (plus the fp32 summation noise, 1e-5 of the row's largest
+      value, which matters for values near zero only), and at most ROTATED_NEAR_TIE_FRACTION of them may
+      differ at all (values whose exact sum lies next to a rounding boundary).
+
+    Returns ``(output error, fraction of differing activations)``."""
+    from oracle import matvec as oracle_matvec
+
+    device_rotated = device_rotated.detach().float().cpu()
+    rounded_oracle = torch.as_tensor(np.asarray(oracle_rotated, dtype=F32)).to(dtype).float()
+    reference = oracle_matvec.reconstruct_then_matmul_f64(
+        device_rotated.numpy(), layer["dense"], None if bias is None else bias.float().cpu().numpy())
+    error = np.abs(np.asarray(y, dtype=np.float64) - reference).max() / np.abs(reference).max()
+    bound = 1e-3 if dtype == torch.float16 else 8e-3
+    assert error <= bound, f"max error {error:.3e} of the output range"
+    mantissa = 10 if dtype == torch.float16 else 7
+    smallest = -14 if dtype == torch.float16 else -126
+    magnitude = torch.maximum(device_rotated.abs(), rounded_oracle.abs()).clamp_min(2.0 ** smallest)
+    unit = torch.exp2(torch.floor(torch.log2(magnitude)) - mantissa)
+    difference = (device_rotated - rounded_oracle).abs()
+    # before rounding the two fp32 sums agree to 1e-5 of the row's largest value, which for values near zero is more
+    # than their own unit in the last place
+    noise = 1e-5 * rounded_oracle.abs().amax(dim=-1, keepdim=True)
+    assert bool((difference <= unit + noise).all()), "a rotated activation is more than one unit in the last place away"
+    fraction = float((difference > 0).float().mean())
+    assert fraction <= ROTATED_NEAR_TIE_FRACTION, f"{fraction:.4f} of the rotated activations differ"
+    return error, fraction

@@ -32,9 +32,18 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert result["n_gpus"] == 1 and result["steps"] == 4 and result["warmup"] == 2
     assert result["higher_is_better"] is True and result["vs_baseline"] is None and result["unit"] == "GB/s"
     assert "workload" in result["config"] and "model" not in result["config"]
+    # the step is the metric's configuration: ONE mk_packed_matvec call on one 4096 x 14336 matrix at M=1, and
+    # the other row counts of the metric ride in the same record as flat scalars
+    config = result["config"]
+    assert config["matrices_per_step"] == 1 and "one mk_packed_matvec call" in config["workload"]
+    assert abs(config["us_M1"] - result["ms_per_step"] * 1e3) < 1e-3 * config["us_M1"]
+    assert result["roofline"]["algorithmic_bytes_per_launch"] == 30_314_496
+    for samples in (1, 2, 4, 8):
+        assert config[f"us_M{samples}"] > 0 and 0 < config[f"frac_M{samples}"] < 1
+        assert config[f"group_of_8_us_per_matrix_M{samples}"] > 0
     roofline = result["roofline"]
     assert roofline["bound"] == "hbm" and roofline["peak"] == 8000.0 and roofline["unit"] == "GB/s"
-    assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-9
+    assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-4      # the line keeps five digits
     assert 0.2 < roofline["frac"] < 1.0
     # whole-job throughput: algorithmic bytes per step over the step time
     assert abs(result["value"] - roofline["algorithmic_bytes_per_launch"] / (result["ms_per_step"] * 1e-3) / 1e9) < 0.02 * result["value"]

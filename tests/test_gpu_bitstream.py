@@ -87,7 +87,8 @@ def test_row_gather_decode_equals_rows_of_the_oracle_decode(name, values, bits, 
                                         integer=integer, asym=asym)
         tensors = helpers.to_device(layer)
         uniform, minimum, step = helpers.uniform_grid(layer["values"])
-        tokens = torch.tensor([0, 299, 5, 5, 17, 128, 1, 299, 64], device="cuda")
+        # -1 and -300 index from the end as tensor indexing does; 300 and -301 lie outside the table: row 0
+        tokens = torch.tensor([0, 299, 5, 5, 17, 128, 1, 299, 64, -1, -300, -7, 300, -301], device="cuda")
         out = torch.empty((tokens.numel(), width), dtype=out_dtype, device="cuda")
         native.check(native.library().mk_packed_decode_rows(
             tensors["packed"].data_ptr(), tensors["scales"].data_ptr(), native.dtype_code(tensors["scales"]),
@@ -95,5 +96,7 @@ def test_row_gather_decode_equals_rows_of_the_oracle_decode(name, values, bits, 
             tokens.numel(), out.data_ptr(), native.dtype_code(out), 300, width, layer["group"], bits, int(uniform), minimum,
             step, None))
         torch.cuda.synchronize()
-        expected = torch.from_numpy(layer["dense"][tokens.cpu().numpy()]).to(out_dtype)
+        wrapped = np.array([0, 299, 5, 5, 17, 128, 1, 299, 64, 299, 0, 293, 0, 0])
+        assert (layer["dense"][np.array([-1, -300, -7])] == layer["dense"][wrapped[9:12]]).all()
+        expected = torch.from_numpy(layer["dense"][wrapped]).to(out_dtype)
         assert torch.equal(out.cpu(), expected)

@@ -178,6 +178,33 @@ def test_round_vector_tile_matches_oracle(name, rows, width, tile_start, tile_wi
     np.testing.assert_array_equal(host(output), expected_out)
 
 
+def test_round_vector_tile_answers_code_zero_for_values_that_are_not_numbers():
+    """No distance of a NaN vector compares below infinity: the code is 0 and the reconstruction is code 0's
+    table point times the scale (the reference reconstructs ``table[0]`` there), in the first block of a row
+    and, through the corrections, in every later block of that row; other rows are untouched."""
+    from mlkit_amd.kernels import error_feedback
+    from mlkit_amd.quantization.lattice import device_table
+
+    rows, width = 6, 64
+    weight, hessian = calibrated(rows, width, seed=77, step=8)
+    weight[2, 3] = np.nan
+    coefficients, status = mk.feedback_coefficients(dev(hessian).clone(), 8)
+    assert int(status) == 0
+    scales = np.full((rows, 1), 0.01, dtype=F32)
+    points = oracle_lattice.e8p_points()
+    for lattice, table, entries in ((True, device_table(torch.device("cuda", 0)), 65536),
+                                    (False, dev(codebook_of(256, 8, seed=1)), 256)):
+        output = torch.full((rows, width), 7.0, device="cuda")
+        encoded = torch.full((rows, width // 8), 9, device="cuda", dtype=torch.int32)
+        error_feedback.round_vector_tile(dev(weight), torch.zeros((rows, width), device="cuda"), coefficients, dev(scales),
+                                         table, output, encoded, region_start=0, tile_start=0, tile_width=width, group=width,
+                                         dimension=8, codebook_size=entries, lattice=lattice)
+        first = points[0] if lattice else codebook_of(256, 8, seed=1)[0]
+        assert host(encoded)[2].tolist() == [0] * (width // 8)
+        np.testing.assert_array_equal(host(output)[2].reshape(-1, 8), np.tile(first * F32(0.01), (width // 8, 1)))
+        assert np.isfinite(host(output)).all() and (host(encoded)[[0, 1, 3, 4, 5]] != 9).all()
+
+
 def test_round_vector_tile_refuses_what_the_kernel_does_not_cover():
     from mlkit_amd.kernels import error_feedback
 

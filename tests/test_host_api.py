@@ -425,3 +425,19 @@ def test_rotation_of_separate_blocks_on_the_host():
     hook, = (h for h in module["down_proj"]._forward_pre_hooks.values() if isinstance(h, RotateInputs))
     assert hook.rotation.block == 256
     torch.testing.assert_close(module["down_proj"](inputs), before, rtol=1e-4, atol=1e-5)
+
+
+def test_copies_of_an_online_rotation_prepare_their_own_plans():
+    """Prepared plans close over device addresses; copies and pickles carry the seed and block only."""
+    import copy
+    import pickle
+
+    from mlkit_amd.quantization.transforms import OnlineRotation
+
+    rotation = OnlineRotation(5, 2048)
+    value = torch.randn(2, 4096)
+    expected = rotation(value)
+    assert rotation._plans
+    for other in (copy.deepcopy(rotation), pickle.loads(pickle.dumps(rotation))):
+        assert (other.seed, other.block) == (5, 2048) and not other._plans
+        assert torch.equal(other(value), expected)
