@@ -260,6 +260,15 @@ __device__ __forceinline__ void park_piece(uint32_t *slice, int i, int lane, mk_
     *reinterpret_cast<mk_u32x4 *>(slice + (16 * i + (lane >> 2)) * kChunkStrideWords + (lane & 3) * 4) = piece;
 }
 
+// Between a wavefront's parking of pieces in its own LDS buffer and its lanes' reads of what OTHER lanes
+// parked: the hardware completes a wavefront's LDS operations in order, and this pins the compiler to the
+// same order (writes before the barrier, reads after it; wavefront scope, no wait beyond the LDS counter).
+__device__ __forceinline__ void wave_exchange_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 template <int XT>
 __device__ __forceinline__ void chunk_from_slice(XChunk<XT> &x, const uint32_t *slice, int chunk_in_slice) {
 #pragma unroll

@@ -273,12 +273,14 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
     request_codes();
 
     if (first_tile) {  // uniform
-    // Each lane's chunk of every sample, through the wavefront's LDS buffer (LDS operations
-    // of a wavefront complete in order, so no barrier is needed).
+    // Each lane's chunk of every sample, through the wavefront's own LDS buffer (no workgroup barrier:
+    // nobody else touches the buffer).
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
+        if (m > 0) wave_exchange_fence();   // the last sample's readers before this one's pieces
 #pragma unroll
         for (int i = 0; i < 4; ++i) park_piece(x_slice, i, lane, pieces[m][i]);
+        wave_exchange_fence();
         chunk_from_slice(x[m], x_slice, lane & (kRowLanes - 1));
     }
     if constexpr (ROTATE)
@@ -469,8 +471,10 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int i = 0; i < kSlices; ++i) park_piece_swizzled(x_slice + j * kSampleWords, i, lane, pieces[set][j][i]);
+            wave_exchange_fence();
 #pragma unroll
             for (int s = 0; s < kSlices; ++s) chunk_from_swizzled_slice(x[set][s], x_slice + t * kSampleWords, s * 16 + block);
+            wave_exchange_fence();   // the next set's pieces go to the same buffers
         };
         if constexpr (kStrided) {
 #pragma unroll

@@ -15,10 +15,12 @@ package).
 import copy
 from collections import defaultdict
 
+import torch
 from torch import nn
 
 from mlkit_amd.inference.packed_linear import PackedEmbedding, PackedLinear, SiblingLaunch, packed_compatible
 from mlkit_amd.models import Model, QModel
+from mlkit_amd.quantization.bitstream import check_overflow
 
 BACKENDS = ("auto", "dense", "packed")
 
@@ -27,11 +29,24 @@ def _planned_replacements(model: QModel, cache_dense: bool) -> tuple[dict[str, n
     """``{module name: packed module}`` for every layer that can execute its codes, and the
     number of packed linear layers among them."""
     module = model.module
+    # one range check of the codes per device for the whole model instead of one read-back per layer
+    flags: dict[torch.device, torch.Tensor] = {}
+
+    def flag_on(device: torch.device) -> "torch.Tensor | None":
+        if device.type != "cuda":
+            return None
+        if device not in flags:
+            flags[device] = torch.zeros(1, dtype=torch.int32, device=device)
+        return flags[device]
+
     planned: dict[str, nn.Module] = {
-        name: PackedLinear(module.get_submodule(name), state, cache_dense=cache_dense)
+        name: PackedLinear(module.get_submodule(name), state, cache_dense=cache_dense,
+                           overflow=flag_on(module.get_submodule(name).weight.device))
         for name, state in model.quantized.items()
         if isinstance(module.get_submodule(name), nn.Linear) and packed_compatible(state)
     }
+    for flag in flags.values():
+        check_overflow(flag)
     linear_layers = len(planned)
     # An input embedding that shares the weight of a packed head reads the head's codes.
     for parameter, head_name in model.tied_weights.items():

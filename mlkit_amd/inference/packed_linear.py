@@ -95,7 +95,11 @@ class PackedLinear(nn.Module):
     bias: Tensor | None
     _dense_weight: Tensor | None
 
-    def __init__(self, original: nn.Linear, quantized: Q, *, cache_dense: bool = False) -> None:
+    def __init__(self, original: nn.Linear, quantized: Q, *, cache_dense: bool = False,
+                 overflow: Tensor | None = None) -> None:
+        """``overflow``: a one-element int32 tensor on the layer's device that collects the range check of
+        the codes (see ``pack``); the caller looks at it once for all the layers it builds.  Without it the
+        check is made here, which synchronises."""
         super().__init__()
         if not packed_compatible(quantized):
             raise ValueError(
@@ -117,7 +121,9 @@ class PackedLinear(nn.Module):
         def resident(tensor: Tensor | None, dtype: torch.dtype) -> Tensor | None:
             return None if tensor is None else tensor.detach().to(device=device, dtype=dtype).contiguous()
 
-        self.register_buffer("packed", pack(quantized.codes.to(device), self.code_bits))
+        if overflow is not None and overflow.device != device:
+            overflow = None
+        self.register_buffer("packed", pack(quantized.codes.to(device), self.code_bits, overflow=overflow))
         self.register_buffer("scales", resident(parameters["scales"], side_dtype))
         self.register_buffer("values", resident(parameters["values"], torch.float32))
         self.register_buffer("zeros", resident(parameters.get("zero"), side_dtype))

@@ -25,8 +25,13 @@ def _bit_planes(values: Tensor, bits: int) -> Tensor:
     return ((values.to(torch.int32).unsqueeze(1) >> shifts) & 1).to(torch.uint8)
 
 
-def pack(codes: Tensor, bits: int) -> Tensor:
-    """A flat uint8 tensor of ``ceil(codes.numel() * bits / 8)`` bytes."""
+def pack(codes: Tensor, bits: int, *, overflow: Tensor | None = None) -> Tensor:
+    """A flat uint8 tensor of ``ceil(codes.numel() * bits / 8)`` bytes.
+
+    ``overflow`` (device tensors only): a one-element int32 tensor on the codes' device that the
+    kernel sets to one when a code does not fit ``bits`` bits.  With it the call does not read
+    the flag back (no synchronisation): a caller that packs many tensors hands the same flag to
+    all of them and looks at it once (``check_overflow``)."""
     if not 1 <= bits <= 16:
         raise ValueError("packing supports one through sixteen bits")
     if codes.is_floating_point() or codes.is_complex():
@@ -41,12 +46,19 @@ def pack(codes: Tensor, bits: int) -> Tensor:
             flat = flat.to(torch.int32)
         flat = flat.contiguous()
         packed = torch.empty(size, dtype=torch.uint8, device=flat.device)
-        overflow = torch.zeros(1, dtype=torch.int32, device=flat.device)
+        deferred = overflow is not None
+        if deferred:
+            if overflow.dtype != torch.int32 or overflow.numel() != 1 or overflow.device != flat.device:
+                raise ValueError("overflow must be a one-element int32 tensor on the codes' device")
+        elif flat.dtype == torch.uint8 and bits >= 8:
+            overflow = None    # every uint8 value fits: nothing to report, nothing to read back
+        else:
+            overflow = torch.zeros(1, dtype=torch.int32, device=flat.device)
         native.check(native.library().mk_pack(flat.data_ptr(), _KERNEL_CODE_BYTES[flat.dtype], count, bits,
-                                              packed.data_ptr(), overflow.data_ptr(),
+                                              packed.data_ptr(), native.pointer(overflow),
                                               native.current_stream(flat.device)))
-        if int(overflow.item()):
-            raise ValueError(f"codes exceed the unsigned capacity of {bits} bits")
+        if not deferred and overflow is not None:
+            check_overflow(overflow, bits)
         return packed
     if count and (int(flat.min()) < 0 or int(flat.max()) >= 1 << bits):
         raise ValueError(f"codes exceed the unsigned capacity of {bits} bits")
@@ -55,6 +67,13 @@ def pack(codes: Tensor, bits: int) -> Tensor:
         stream = torch.cat([stream, stream.new_zeros(8 - stream.numel() % 8)])
     weights = (1 << torch.arange(8, dtype=torch.int32)).to(torch.uint8)
     return (stream.view(-1, 8) * weights).sum(dim=1, dtype=torch.int32).to(torch.uint8)[:size]
+
+
+def check_overflow(overflow: Tensor, bits: "int | None" = None) -> None:
+    """Raises the error of ``pack`` when a deferred overflow flag is set (reads it back: one synchronisation)."""
+    if int(overflow.item()):
+        width = "the declared width" if bits is None else f"{bits} bits"
+        raise ValueError(f"codes exceed the unsigned capacity of {width}")
 
 
 def unpack(packed: Tensor, bits: int, shape: tuple[int, ...]) -> Tensor:

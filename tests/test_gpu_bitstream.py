@@ -69,6 +69,33 @@ def test_pack_error_cases_on_device():
         mk.unpack(torch.zeros(3, dtype=torch.uint8, device="cuda"), 4, (7,))
 
 
+def test_deferred_overflow_flag_collects_the_range_checks():
+    """pack(..., overflow=flag) does not read the flag back; one flag serves many calls and is checked once;
+    optimize checks the codes of a whole model that way and still raises the reference's error."""
+    import mlkit_amd as mk
+    from mlkit_amd.quantization.bitstream import check_overflow
+    from torch import nn
+
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    good = torch.tensor([0, 7, 15, 3], dtype=torch.uint8, device="cuda")
+    packed = mk.pack(good, 4, overflow=flag)
+    assert packed.tolist() == [0x70, 0x3F]
+    check_overflow(flag, 4)
+    mk.pack(torch.tensor([1, 16], dtype=torch.uint8, device="cuda"), 4, overflow=flag)   # no error here
+    mk.pack(good, 4, overflow=flag)                                                           # the flag stays set
+    with pytest.raises(ValueError, match="capacity"):
+        check_overflow(flag, 4)
+    with pytest.raises(ValueError, match="one-element int32"):
+        mk.pack(good, 4, overflow=torch.zeros(2, dtype=torch.int32, device="cuda"))
+    assert mk.pack(torch.arange(256, dtype=torch.uint8, device="cuda"), 8).tolist() == list(range(256))
+    # a model whose codes do not fit their declared width is refused by optimize
+    module = nn.Sequential(nn.Linear(256, 32, dtype=torch.float16)).cuda()
+    converted = mk.quantize(module, mk.int(4, group=128), calib=None)
+    converted.quantized["0"].codes[3, 5] = 16
+    with pytest.raises(ValueError, match="capacity"):
+        mk.optimize(converted, backend="packed")
+
+
 @pytest.mark.parametrize("name,values,bits,integer,group", [
     ("int4", scaling.int_values(4), 4, True, 128), ("int3", scaling.int_values(3), 3, True, 64),
     ("nf4", scaling.NF4_VALUES, 4, False, 64), ("int8", scaling.int_values(8), 8, True, 128),

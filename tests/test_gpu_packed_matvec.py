@@ -561,3 +561,48 @@ def test_rotation_of_separate_blocks_inside_the_matvec_kernel(rows, width, block
                                                    oracle_transforms.fwht(blocks).reshape(samples, width), torch.float16, bias)
         assert differing == 0.0
 
+
+
+@pytest.mark.parametrize("rows,width,asym,with_bias,scale_dtype", [
+    (64, 14336, False, True, torch.float16),
+    (4096 + 23, 4096, True, False, torch.float16),   # 7 rows beyond the last whole tile
+    (48, 4864, False, True, torch.bfloat16),      # 38 groups of 128 codes
+    (32, 16384, True, True, torch.float16),       # the widest row of the streaming kernels
+    (16, 2048, False, False, torch.float16),
+    (80, 8192, False, False, torch.float16),
+    (32, 8320, False, False, torch.float16),      # 65 groups
+])
+def test_two_to_eight_samples_on_rows_of_many_lengths(rows, width, asym, with_bias, scale_dtype):
+    """INT4 with one scale per 128 codes, fp16 activations, every sample count from two to eight, on rows from
+    2048 to 16384 codes (ragged tiles of rows, odd numbers of 128-code groups): against the float64 product of
+    the oracle's reconstruction at 1e-3 of the output range and the reference's own fp16 bound."""
+    weight = helpers.normal_weight(rows, width, seed=rows + width)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True, asym=asym)
+    bias = helpers.activations(1, rows, seed=8)[0] if with_bias else None
+    for samples in (2, 3, 4, 5, 7, 8):
+        x = helpers.activations(samples, width, seed=40 + samples)
+        y = run_matvec(layer, x, bias, scale_dtype=scale_dtype)
+        if scale_dtype == torch.float16:
+            check(y, layer, x, bias)
+            fp32_reference = oracle_matvec.reconstruct_then_matmul(
+                x.float().numpy(), layer["packed"], 4, layer["shape"], layer["scales"], layer["values"], 128, layer["zero"],
+                None if bias is None else bias.float().numpy())
+            np.testing.assert_allclose(y, fp32_reference, rtol=2e-3, atol=2e-3)
+        else:   # the oracle's scales rounded to bf16: compare with the kernel for one sample, which they also serve
+            single = np.concatenate([run_matvec(layer, x[m:m + 1], bias, scale_dtype=scale_dtype) for m in range(samples)])
+            assert np.abs(y - single).max() <= 1e-3 * np.abs(single).max()
+
+
+def test_small_and_large_activations_keep_the_tolerance():
+    """Rows of activations a hundred times smaller or two thousand times larger than the usual ones, and a row
+    with every second value small: the error stays within the tolerance of each row's output range."""
+    weight = helpers.normal_weight(64, 4096, seed=77)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
+    x = helpers.activations(4, 4096, seed=3).float()
+    x[0] *= 1e-2
+    x[1] *= 2000.0
+    x[2, ::2] *= 1e-3
+    x = x.half()
+    y = run_matvec(layer, x)
+    for m in range(4):
+        check(y[m:m + 1], layer, x[m:m + 1])
