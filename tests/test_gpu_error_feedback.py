@@ -72,6 +72,51 @@ def test_round_tile_matches_oracle(rows, width, tile_start, tile_width, group, v
     np.testing.assert_array_equal(host(output), expected_out)
 
 
+@pytest.mark.parametrize("asym", [False, True])
+@pytest.mark.parametrize("tile_width", [128, 96])
+def test_round_tile_on_quotients_next_to_half_integers(asym, tile_width):
+    """Every target of the tile divides by its scale to k + 1/2 exactly, or to the fp32 numbers right next to
+    it on either side: the cases in which the correctly rounded quotient, and not a product with the scale's
+    reciprocal, decides the code (a sweep that multiplied by reciprocals would miss a few per cent of these
+    codes, as the last assertion shows).  No feedback and no coefficients, so that every column is such a
+    case; codes and reconstructions equal the oracle's (true division, round half to even)."""
+    from mlkit_amd.kernels import error_feedback
+
+    rows, width, group = 192, 256, 64
+    rng = np.random.default_rng(31 + tile_width)
+    scales = (rng.random((rows, width // group)) * 0.05 + 0.002).astype(np.float16).astype(F32)
+    scales[::3] = (2.0 ** rng.integers(-9, -3, (len(scales[::3]), width // group))).astype(F32)     # exact ties
+    zeros = (rng.standard_normal((rows, width // group)) * 0.01).astype(np.float16).astype(F32) if asym else None
+    halves = rng.integers(-9, 9, (rows, width)).astype(F32) + F32(0.5)
+    wide = np.repeat(scales, group, axis=1)
+    weight = (halves * wide).astype(F32)
+    if asym:
+        weight = (weight + np.repeat(zeros, group, axis=1)).astype(F32)
+    nudge = rng.integers(-2, 3, (rows, width))
+    weight = np.where(nudge < 0, np.nextafter(weight, F32(-np.inf)), np.where(nudge > 0, np.nextafter(weight, F32(np.inf)), weight)).astype(F32)
+    weight[5, 7] = np.nan                                             # a value that is not a number takes the division, too
+    feedback = np.zeros_like(weight)
+    coeff = np.eye(width, dtype=F32)
+    expected_out = np.zeros_like(weight)
+    expected_codes = np.zeros(weight.shape, dtype=np.uint8)
+    oracle_feedback.round_tile(weight, feedback, coeff, scales, zeros, INT4, expected_out, expected_codes,
+                               region_start=0, tile_start=64, tile_width=tile_width, group=group, integer=True)
+    output = torch.zeros((rows, width), device="cuda")
+    encoded = torch.zeros((rows, width), device="cuda", dtype=torch.uint8)
+    error_feedback.round_tile(dev(weight), dev(feedback), dev(coeff), dev(scales), None if zeros is None else dev(zeros), output,
+                              encoded, region_start=0, tile_start=64, tile_width=tile_width, group=group, bits=4,
+                              values=dev(INT4), integer_grid=True)
+    keep = np.ones(weight.shape, dtype=bool)
+    keep[5, 7] = False
+    np.testing.assert_array_equal(host(encoded)[keep], expected_codes[keep])
+    np.testing.assert_array_equal(host(output)[keep], expected_out[keep])
+    # the crafted cases really sit at the boundaries: a product with the reciprocal alone would miss some codes
+    inside = slice(64, 64 + tile_width)
+    centered = weight[:, inside] - (np.repeat(zeros, group, axis=1)[:, inside] if asym else 0)
+    by_reciprocal = np.clip(np.rint((centered.astype(F32) * (F32(1) / wide[:, inside])).astype(F32)), -8, 7) + 8
+    assert (by_reciprocal[keep[:, inside]] != expected_codes[:, inside][keep[:, inside]]).sum() > 0
+
+
 @pytest.mark.parametrize("rows,width,start,stop", [(64, 384, 128, 256), (37, 512, 192, 492), (16, 1024, 0, 1024)])
 def test_pending_continuation_matches_oracle(rows, width, start, stop):
     from mlkit_amd.kernels import error_feedback
