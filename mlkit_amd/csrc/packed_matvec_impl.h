@@ -235,6 +235,25 @@ __device__ __forceinline__ float pair_for_nibbles(XChunk<MK_F16> &x, float *stor
     return 1024.0f * (plain + reduced);
 }
 
+// The same pairing without the factor 1/16: (x0,x4) (x1,x5) (x2,x6) (x3,x7) for every eight codes, for codes
+// that enter as fp16 subnormals (chunk_dot_subnormal).  Returns the sum of the chunk's activations.
+__device__ __forceinline__ float pair_for_subnormal_nibbles(XChunk<MK_F16> &x) {
+    const mk_h2 ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+    float total = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const uint32_t p0 = x.r[4 * g + 0], p1 = x.r[4 * g + 1];
+        const uint32_t p2 = x.r[4 * g + 2], p3 = x.r[4 * g + 3];
+        x.r[4 * g + 0] = __builtin_amdgcn_perm(p2, p0, 0x05040100u);
+        x.r[4 * g + 1] = __builtin_amdgcn_perm(p2, p0, 0x07060302u);
+        x.r[4 * g + 2] = __builtin_amdgcn_perm(p3, p1, 0x05040100u);
+        x.r[4 * g + 3] = __builtin_amdgcn_perm(p3, p1, 0x07060302u);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) total = __builtin_amdgcn_fdot2(ones, __builtin_bit_cast(mk_h2, x.r[4 * g + i]), total, false);
+    }
+    return total;
+}
+
 // ---- activations: coalesced loads, then each lane's chunk out of LDS ------------------------
 //
 // A lane needs the 32 activations (64 bytes) of a chunk.  Sixty-four lanes reading 16 bytes
@@ -243,6 +262,13 @@ __device__ __forceinline__ float pair_for_nibbles(XChunk<MK_F16> &x, float *stor
 // reads the 4 KB of one sample's 2048-code slice as four 1 KB instructions (lane l: bytes
 // 16 l), parks them in its own LDS buffer and reads chunks back.  Chunks are 80 bytes apart
 // in LDS so that sixteen lanes reading 16 bytes of sixteen chunks hit different banks.
+
+// The value of the lane whose index differs in bit 0 (XOR = 1) or bit 1 (XOR = 2): DPP quad permutations.
+template <int XOR>
+__device__ __forceinline__ float quad_value_of_lane(float value) {
+    constexpr int control = XOR == 1 ? 0xB1 : 0x4E;   // quad_perm [1,0,3,2] / [2,3,0,1]
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, value), control, 0xf, 0xf, true));
+}
 
 constexpr int kChunkStrideWords = 20;
 constexpr int kSliceWords = 64 * kChunkStrideWords;  // one wavefront's buffer: 5 KB
@@ -254,6 +280,103 @@ __device__ __forceinline__ mk_u32x4 request_piece(const void *x, int width, int 
     const int element = slice_start + (16 * i + (lane >> 2)) * kChunkCodes + (lane & 3) * 8;
     const size_t offset = static_cast<size_t>(sample) * width + (element < width ? element : (lane & 3) * 8);
     return *reinterpret_cast<const mk_u32x4 *>(static_cast<const uint8_t *>(x) + offset * 2);
+}
+
+// The same eight elements of an fp32 row as two loads of four floats (`second`: elements 4 - 7).
+__device__ __forceinline__ mk_u32x4 request_wide_piece(const void *x, int width, int sample, int slice_start, int i, int lane, int second) {
+    const int element = slice_start + (16 * i + (lane >> 2)) * kChunkCodes + (lane & 3) * 8;
+    const size_t offset = static_cast<size_t>(sample) * width + (element < width ? element : (lane & 3) * 8) + 4 * second;
+    return *reinterpret_cast<const mk_u32x4 *>(static_cast<const uint8_t *>(x) + offset * 4);
+}
+
+// fp32 activations enter the dot products as integers: a chunk's 32 values are scaled by a power of two 2^k of
+// the chunk's own (largest magnitude into [2^21, 2^22)), rounded to integers X and cut into six signed 4-bit
+// digits, X = sum_d t_d 16^d with t_d in [-8, 7].  Plane d of a chunk is four words that hold digit d of its 32
+// values in the nibble order of the packed codes, so that one v_dot8_i32_i4 multiplies eight codes (as c - 8, one
+// XOR away from the packed word) by eight digits, exactly.  Six such instructions per eight codes replace eight
+// v_dot2 and four masks of a split into two fp16 halves, and the only roundings left are the one to X (half a
+// unit in 2^22 of the chunk's largest value) and those of the fp32 sums over the chunks.
+constexpr int kPlaneDigits = 6;
+constexpr int kPlaneStrideWords = 28;   // 24 plane words, 2^-k, the sum of the X; 112 bytes apart: eight lanes reading
+                                        // 16 bytes of eight adjacent chunks touch every LDS bank once
+constexpr int kPlaneSliceWords = 64 * kPlaneStrideWords;  // one wavefront's buffer: 7 KB
+
+// Eight fp32 activations of a chunk (this lane's quarter of it; the four lanes of a quad hold the chunk): digit d
+// of the eight in plane[d], their sum (of the integers X) in `total`; returns 2^-k.  Chunks of zeros keep k = 0,
+// chunks below 2^-106 the largest usable k; a chunk with a value that is not finite returns NaN.
+__device__ __forceinline__ float planes_of_piece(mk_u32x4 first, mk_u32x4 second, uint32_t (&plane)[kPlaneDigits], int &total) {
+    const uint32_t bits[8] = {first.x, first.y, first.z, first.w, second.x, second.y, second.z, second.w};
+    uint32_t largest = 0;   // as magnitude bits: NaN above infinity above everything finite
+#pragma unroll
+    for (int k = 0; k < 8; ++k) largest = max(largest, bits[k] & 0x7fffffffu);
+    largest = max(largest, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(largest), 0xB1, 0xf, 0xf, true)));
+    largest = max(largest, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(largest), 0x4E, 0xf, 0xf, true)));
+    // biased exponent e of the largest value; the factor 2^(148 - e) has biased exponent 275 - e (at least 21)
+    const int exponent = static_cast<int>(largest >> 23);
+    const int wanted = 275 - exponent;
+    const int biased = exponent == 0 ? 127 : (wanted > 253 ? 253 : wanted);
+    const float factor = __uint_as_float(static_cast<uint32_t>(biased) << 23);
+    const float inverse = __uint_as_float(exponent == 255 ? 0x7fc00000u : static_cast<uint32_t>(254 - biased) << 23);
+    // x 2^k + 1.5 * 2^23 holds X + 2^22 in its low 23 bits (rounded to nearest even); adding 8 to every digit makes
+    // them unsigned nibbles, and flipping each nibble's top bit afterwards makes those two's complement again.
+    constexpr uint32_t kEights = 0x888888u;
+    uint32_t y[8];
+    int sum = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        y[k] = __float_as_uint(__builtin_fmaf(__uint_as_float(bits[k]), factor, 12582912.0f)) + (kEights - 0x4B400000u);
+        sum += static_cast<int>(y[k]);
+    }
+    total = sum - 8 * static_cast<int>(kEights);
+    uint32_t even[4], odd[4];   // byte b of even[p]: digit 2 b of value 2 p (low nibble) and of value 2 p + 1 (high nibble)
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t a = y[2 * p], b = y[2 * p + 1];
+        even[p] = (a & 0x0f0f0fu) | ((b & 0x0f0f0fu) << 4);
+        odd[p] = ((a >> 4) & 0x0f0f0fu) | (b & 0xf0f0f0u);
+    }
+    auto gather = [](const uint32_t (&w)[4], uint32_t &d0, uint32_t &d1, uint32_t &d2) __attribute__((always_inline)) {
+        const uint32_t t01 = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);   // w0.b0 w1.b0 w0.b1 w1.b1
+        const uint32_t t23 = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u);
+        d0 = __builtin_amdgcn_perm(t23, t01, 0x05040100u) ^ 0x88888888u;
+        d1 = __builtin_amdgcn_perm(t23, t01, 0x07060302u) ^ 0x88888888u;
+        const uint32_t u01 = __builtin_amdgcn_perm(w[1], w[0], 0x0c0c0602u);   // w0.b2 w1.b2 0 0
+        const uint32_t u23 = __builtin_amdgcn_perm(w[3], w[2], 0x0c0c0602u);
+        d2 = __builtin_amdgcn_perm(u23, u01, 0x05040100u) ^ 0x88888888u;
+    };
+    gather(even, plane[0], plane[2], plane[4]);
+    gather(odd, plane[1], plane[3], plane[5]);
+    return inverse;
+}
+
+// Parks a piece's planes (and, from the quad's first lane, 2^-k and the chunk's sum) in the wavefront's buffer.
+__device__ __forceinline__ void park_planes(uint32_t *slice, int i, int lane, const uint32_t (&plane)[kPlaneDigits], float inverse, int total) {
+    uint32_t *const slot = slice + (16 * i + (lane >> 2)) * kPlaneStrideWords;
+#pragma unroll
+    for (int d = 0; d < kPlaneDigits; ++d) slot[4 * d + (lane & 3)] = plane[d];
+    total += __builtin_amdgcn_mov_dpp(total, 0xB1, 0xf, 0xf, true);
+    total += __builtin_amdgcn_mov_dpp(total, 0x4E, 0xf, 0xf, true);
+    if ((lane & 3) == 0) {
+        slot[24] = __float_as_uint(inverse);
+        slot[25] = static_cast<uint32_t>(total);
+    }
+}
+
+// A lane's chunk out of the buffer: planes[4 d + j] is digit d of code word j; masked by `keep`.
+__device__ __forceinline__ void planes_from_slice(uint32_t (&planes)[4 * kPlaneDigits], float &inverse, float &sum,
+                                                  const uint32_t *slice, int chunk_in_slice, uint32_t keep) {
+    const uint32_t *const slot = slice + chunk_in_slice * kPlaneStrideWords;
+#pragma unroll
+    for (int d = 0; d < kPlaneDigits; ++d) {
+        const mk_u32x4 v = *reinterpret_cast<const mk_u32x4 *>(slot + 4 * d);
+        planes[4 * d + 0] = v.x & keep;
+        planes[4 * d + 1] = v.y & keep;
+        planes[4 * d + 2] = v.z & keep;
+        planes[4 * d + 3] = v.w & keep;
+    }
+    const mk_u32x2 tail = *reinterpret_cast<const mk_u32x2 *>(slot + 24);
+    inverse = __uint_as_float(tail.x);
+    sum = static_cast<float>(static_cast<int>(tail.y & keep));
 }
 
 __device__ __forceinline__ void park_piece(uint32_t *slice, int i, int lane, mk_u32x4 piece) {
@@ -433,6 +556,65 @@ __device__ __forceinline__ void chunk_dot(const CodeChunk<BITS> &codes, const XC
 #pragma unroll
             for (int m = 0; m < MT; ++m) dot[m] = __builtin_fmaf(value, x_element<XT>(x[m], k), dot[m]);
         }
+    }
+}
+
+// sum_k code_k x_k of a chunk of 4-bit codes for MT samples, times 2^-24.  A nibble left where it is in the low
+// bits of a half word is the fp16 subnormal c * 2^-24 (16 c * 2^-24 for the upper nibble of a byte), which
+// v_dot2_f32_f16 multiplies exactly: no exponent is inserted, nothing code-free has to be removed afterwards and
+// the activations are used as they are.  The upper nibbles have their own sum, divided by 16 at the end.
+template <int MT>
+__device__ __forceinline__ void chunk_dot_subnormal(const CodeChunk<4> &codes, const XChunk<MK_F16> (&x)[MT], float (&dot)[MT]) {
+    float lower[MT], upper[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) lower[m] = upper[m] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w = codes.w[i], w8 = w >> 8;
+        const mk_h2 h0 = __builtin_bit_cast(mk_h2, w & 0x000f000fu), h1 = __builtin_bit_cast(mk_h2, w & 0x00f000f0u);
+        const mk_h2 h2 = __builtin_bit_cast(mk_h2, w8 & 0x000f000fu), h3 = __builtin_bit_cast(mk_h2, w8 & 0x00f000f0u);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            lower[m] = __builtin_amdgcn_fdot2(h0, __builtin_bit_cast(mk_h2, x[m].r[4 * i + 0]), lower[m], false);
+            upper[m] = __builtin_amdgcn_fdot2(h1, __builtin_bit_cast(mk_h2, x[m].r[4 * i + 1]), upper[m], false);
+            lower[m] = __builtin_amdgcn_fdot2(h2, __builtin_bit_cast(mk_h2, x[m].r[4 * i + 2]), lower[m], false);
+            upper[m] = __builtin_amdgcn_fdot2(h3, __builtin_bit_cast(mk_h2, x[m].r[4 * i + 3]), upper[m], false);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) dot[m] = __builtin_fmaf(upper[m], 0.0625f, lower[m]);
+}
+
+// A chunk of 32 codes against the digit planes of MT fp32 samples (planes_of_piece): sum_k (c_k - 8) X_k, exact
+// in integers and rounded once on its way to fp32.  (Codes as fp16 subnormals would not do for fp32 outputs:
+// v_dot2_f32_f16 aligns its terms by the exponent FIELDS of its inputs and keeps about 24 bits below the largest,
+// so a subnormal code, whose value lies far below its field's 2^-14, costs the running sum up to ten low bits.)
+template <int MT>
+__device__ __forceinline__ void chunk_dot_planes(const CodeChunk<4> &codes, const uint32_t (&planes)[MT][4 * kPlaneDigits], float (&dot)[MT]) {
+    int signed_codes[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) signed_codes[j] = static_cast<int>(codes.w[j] ^ 0x88888888u);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        int digit_sum[kPlaneDigits];
+#pragma unroll
+        for (int d = 0; d < kPlaneDigits; ++d) {
+            // the first of a chain in the three-operand form with a literal zero (the builtin's two-operand form
+            // wants its accumulator cleared by a move of its own)
+            asm("v_dot8_i32_i4 %0, %1, %2, 0" : "=v"(digit_sum[d]) : "v"(signed_codes[0]), "v"(planes[m][4 * d]));
+#pragma unroll
+            for (int j = 1; j < 4; ++j)
+                digit_sum[d] = __builtin_amdgcn_sdot8(signed_codes[j], static_cast<int>(planes[m][4 * d + j]), digit_sum[d], false);
+        }
+        // |digit sum| <= 32 * 64: three of them combine within 20 bits (two shift-and-adds each)
+        auto sixteen_times_plus = [](int upper, int lower) __attribute__((always_inline)) {
+            int result;   // (spelled out: the compiler turns the two-step form into three shifts and a three-way add)
+            asm("v_lshl_add_u32 %0, %1, 4, %2" : "=v"(result) : "v"(upper), "v"(lower));
+            return result;
+        };
+        const int low = sixteen_times_plus(sixteen_times_plus(digit_sum[2], digit_sum[1]), digit_sum[0]);
+        const int high = sixteen_times_plus(sixteen_times_plus(digit_sum[5], digit_sum[4]), digit_sum[3]);
+        dot[m] = __builtin_fmaf(static_cast<float>(high), 4096.0f, static_cast<float>(low));
     }
 }
 

@@ -1,5 +1,6 @@
-// 4-bit uniform-grid packed matvec with fp16 activations and fp16 scales: the decode-time
-// kernel for INT4 layers whose rows are whole multiples of 32 codes (K = 32 ... 16384).
+// 4-bit uniform-grid packed matvec with fp16 or bf16 activations (fp32 ones as pairs of fp16
+// halves, for one or two samples) and 16-bit or fp32 scales: the decode-time kernel for INT4
+// layers whose rows are whole multiples of 32 codes (K = 32 ... 16384).
 //
 // The kernel is bound by whichever is larger: the HBM stream of the codes, or the vector
 // ALU time of the busiest SIMD (a wavefront issues one vector instruction per four
@@ -180,15 +181,33 @@ __device__ __forceinline__ void rotate_activations(XChunk<XT> &x, const float4 (
 // row and lanes 32 - 63 the next, so that a step covers two rows instead of leaving half the
 // wavefront without codes.
 // ROTATE: the activations are rotated in the kernel (one sample, rows of whole 2048-code slices).
-template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS, bool ROTATE = false>
+// SPLIT: the activations are fp32 and the outputs too.  Every chunk of 32 is scaled by a power of two 2^k of its
+// own, rounded to integers of 22 bits and a sign and cut into six planes of signed 4-bit digits (planes_of_piece);
+// v_dot8_i32_i4 multiplies them with the codes as c - 8 exactly, and a lane's sums are multiplied by 2^-k.
+// WIDE_SIDES: scales and offsets are fp32.
+template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS, bool ROTATE = false, bool SPLIT = false, bool WIDE_SIDES = false>
 __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4Group &members) {
     static_assert(ROWS * MT <= 64 && ROWS % PARTS == 0, "one transposed reduction per workgroup");
     static_assert(!ROTATE || (MT == 1 && PARTS == 1), "the fused rotation takes one sample of long rows");
+    static_assert(!SPLIT || (XT == MK_F16 && !ROTATE), "fp32 activations: XT only names the unused fp16 chunk type");
+    using SideRaw = std::conditional_t<WIDE_SIDES, uint32_t, uint16_t>;
+    constexpr uint32_t kSideBytes = WIDE_SIDES ? 4u : 2u;
+    auto side_of = [&](SideRaw raw) __attribute__((always_inline)) {
+        if constexpr (WIDE_SIDES) return __uint_as_float(raw);
+        else return side_as_float(raw, a.scale_dtype);
+    };
+    // fp16 activations: codes enter the dot products as fp16 subnormals (c * 2^-24; no exponent is inserted and the
+    // activations stay unscaled, measured as fast as the exponent trick: 7.43 against 7.45 us).  The factor 2^24
+    // goes into the grid's step.  bf16 has too few mantissa bits and too small subnormals for that.
+    // fp32 activations (SPLIT) enter as planes of signed 4-bit digits against the codes as c - 8 (chunk_dot_planes).
+    constexpr bool kSubnormalCodes = XT == MK_F16;
+    const float code_step = kSubnormalCodes && !SPLIT ? a.grid_step * 16777216.0f : a.grid_step;
+    const float sum_factor = SPLIT ? __builtin_fmaf(8.0f, a.grid_step, a.grid_min) : a.grid_min;
     __shared__ float partials[64 * 8];  // [row sum][wavefront]
     // One 5 KB activation buffer per wavefront, sized at launch (a workgroup of one wavefront
     // must not hold LDS for eight).
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
-    uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
+    uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * (SPLIT ? kPlaneSliceWords : kSliceWords);
     constexpr int kStreamRows = ROWS / PARTS;            // steps: PARTS rows each
     constexpr int kStreamAhead = rows_ahead_of<kStreamRows>();  // (with ROTATE too: all 16 rows ahead measured slower)
     constexpr int kSums = kStreamRows * MT;
@@ -215,13 +234,20 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
     __syncthreads();
 
     // Activations: 32 per sample, as 16 fp16 pairs (L2 hits), requested first.
-    mk_u32x4 pieces[MT][4];
+    mk_u32x4 pieces[SPLIT ? 2 * MT : MT][4];   // SPLIT: [2 m] and [2 m + 1] hold the first and second four floats of a lane's eight
     auto request_activations = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             const int sample = sample_base + m < a.samples ? sample_base + m : a.samples - 1;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) pieces[m][i] = request_piece(source.x, a.width, sample, wave * 2048, i, lane);
+            for (int i = 0; i < 4; ++i) {
+                if constexpr (SPLIT) {
+                    pieces[2 * m][i] = request_wide_piece(source.x, a.width, sample, wave * 2048, i, lane, 0);
+                    pieces[2 * m + 1][i] = request_wide_piece(source.x, a.width, sample, wave * 2048, i, lane, 1);
+                } else {
+                    pieces[m][i] = request_piece(source.x, a.width, sample, wave * 2048, i, lane);
+                }
+            }
         }
     };
     request_activations();
@@ -235,15 +261,17 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         }
     }
     // The scale (and offset) of this lane's chunk in every row, 2 bytes each.
-    const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
+    const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * kSideBytes;
     const uint32_t group_offset = static_cast<uint32_t>(part) * scale_row_bytes +
-                                  ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
+                                  ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * kSideBytes;
     // Short rows (two per wavefront step): a workgroup takes every gridDim.x-th tile of ROWS
     // rows and prepares its activations once, during the first tile's loads; tall matrices
     // then pay for that preparation once per workgroup instead of once per tile.
     constexpr bool kStrided = PARTS == 2;
-    XChunk<XT> x[MT];
+    XChunk<XT> x[SPLIT ? 1 : MT];
+    uint32_t planes[SPLIT ? MT : 1][4 * kPlaneDigits];   // SPLIT: this lane's chunk of every sample as digit planes
     float x_sum[MT], grid_term[MT];
+    float unscale[SPLIT ? MT : 1];   // SPLIT: 2^-k of this lane's chunk, per sample
     int tile = blockIdx.x;
     bool first_tile = true;
     do {
@@ -251,14 +279,14 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
     const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
     const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
     const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
-    uint16_t scale_raw[kStreamRows], zero_raw[HAS_ZERO ? kStreamRows : 1];
+    SideRaw scale_raw[kStreamRows], zero_raw[HAS_ZERO ? kStreamRows : 1];
     CodeChunk<4> codes[kStreamRows];
     auto request_sides = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < kStreamRows; ++r) {
-            scale_raw[r] = *reinterpret_cast<const uint16_t *>(scale_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
+            scale_raw[r] = *reinterpret_cast<const SideRaw *>(scale_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
             if constexpr (HAS_ZERO)
-                zero_raw[r] = *reinterpret_cast<const uint16_t *>(zero_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
+                zero_raw[r] = *reinterpret_cast<const SideRaw *>(zero_base + static_cast<size_t>(PARTS * r) * scale_row_bytes + group_offset);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -275,6 +303,23 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
     if (first_tile) {  // uniform
     // Each lane's chunk of every sample, through the wavefront's own LDS buffer (no workgroup barrier:
     // nobody else touches the buffer).
+    if constexpr (SPLIT) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            if (m > 0) wave_exchange_fence();   // the last sample's readers before this one's planes
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint32_t plane[kPlaneDigits];
+                int total;
+                const float inverse = planes_of_piece(pieces[2 * m][i], pieces[2 * m + 1][i], plane, total);
+                park_planes(x_slice, i, lane, plane, inverse, total);
+            }
+            wave_exchange_fence();
+            const uint32_t keep = in_row && sample_base + m < a.samples ? 0xffffffffu : 0u;
+            planes_from_slice(planes[m], unscale[m], x_sum[m], x_slice, lane & (kRowLanes - 1), keep);
+            grid_term[m] = sum_factor * x_sum[m];
+        }
+    } else {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         if (m > 0) wave_exchange_fence();   // the last sample's readers before this one's pieces
@@ -283,24 +328,30 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         wave_exchange_fence();
         chunk_from_slice(x[m], x_slice, lane & (kRowLanes - 1));
     }
+    }
     if constexpr (ROTATE)
         rotate_activations<XT>(x[0], rotation_sign, a.rotate_scale, reinterpret_cast<float *>(x_slices_storage), wave, waves, lane,
                            a.rotate_log_block);
 
     // sum_k (min + step c_k) x_k = step * dot + min * sum(x) - step * (code-free part of dot).
+    if constexpr (!SPLIT) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const uint32_t keep = in_row && sample_base + m < a.samples ? 0xffffffffu : 0u;
 #pragma unroll
         for (int i = 0; i < 16; ++i) x[m].r[i] &= keep;
         float code_free;
-        if constexpr (XT == MK_F16) {
+        if constexpr (kSubnormalCodes) {
+            x_sum[m] = pair_for_subnormal_nibbles(x[m]);
+            code_free = 0.0f;
+        } else if constexpr (XT == MK_F16) {
             code_free = pair_for_nibbles(x[m], &x_sum[m]);
         } else {
             x_sum[m] = pair_for_nibbles_bf16(x[m]);
             code_free = 128.0f * x_sum[m];
         }
-        grid_term[m] = a.grid_min * x_sum[m] - a.grid_step * code_free;
+        grid_term[m] = sum_factor * x_sum[m] - a.grid_step * code_free;
+    }
     }
     }
     first_tile = false;
@@ -309,17 +360,20 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
 #pragma unroll
     for (int r = 0; r < kStreamRows; ++r) {
         float dot[MT];
-        if constexpr (XT == MK_F16) chunk_dot<4, MK_F16, MT, true>(codes[r], x, nullptr, dot);
+        if constexpr (SPLIT) chunk_dot_planes<MT>(codes[r], planes, dot);
+        else if constexpr (kSubnormalCodes) chunk_dot_subnormal<MT>(codes[r], x, dot);
+        else if constexpr (XT == MK_F16) chunk_dot<4, MK_F16, MT, true>(codes[r], x, nullptr, dot);
         else chunk_dot_bf16<MT>(codes[r], x, dot);
         if (r + kStreamAhead < kStreamRows)
             load_codes<4>(codes[r + kStreamAhead],
                           codes_base + static_cast<size_t>(PARTS * (r + kStreamAhead)) * row_bytes + code_offset);
-        const float scale = side_as_float(scale_raw[r], a.scale_dtype);
+        const float scale = side_of(scale_raw[r]);
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-            float value = scale * __builtin_fmaf(a.grid_step, dot[m], grid_term[m]);
+            float value = scale * __builtin_fmaf(code_step, dot[m], grid_term[m]);
             if constexpr (HAS_ZERO)
-                value = __builtin_fmaf(side_as_float(zero_raw[r], a.scale_dtype), x_sum[m], value);
+                value = __builtin_fmaf(side_of(zero_raw[r]), x_sum[m], value);
+            if constexpr (SPLIT) value *= unscale[m];
             sums[r * MT + m] = value;
         }
         // Keeps the rows in arrival order and their temporaries short-lived.
@@ -341,7 +395,8 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         const int sample = sample_base + m;
         if (sample < a.samples) {
             if (source.bias) total += mk_load_as_float(source.bias, row, a.bias_dtype);
-            store_output<XT>(source.y, static_cast<size_t>(sample) * source.rows + row, total);
+            if constexpr (SPLIT) static_cast<float *>(source.y)[static_cast<size_t>(sample) * source.rows + row] = total;
+            else store_output<XT>(source.y, static_cast<size_t>(sample) * source.rows + row, total);
         }
     }
     if constexpr (!kStrided) break;
@@ -351,9 +406,9 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
     } while (true);
 }
 
-template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS>
+template <int MT, bool HAS_ZERO, int ROWS, int XT, int PARTS, bool SPLIT = false, bool WIDE_SIDES = false>
 __global__ void __launch_bounds__(512) stream4_kernel(const Stream4Args a, const Stream4Group members) {
-    stream4_body<MT, HAS_ZERO, ROWS, XT, PARTS>(a, members);
+    stream4_body<MT, HAS_ZERO, ROWS, XT, PARTS, false, SPLIT, WIDE_SIDES>(a, members);
 }
 
 template <bool HAS_ZERO, int ROWS, int XT>
@@ -683,7 +738,7 @@ template <int MT, int ROWS, int PARTS>
 int launch_tile_parts(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1);
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
-    const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
+    const size_t slices = static_cast<size_t>(block.x / 64) * (a.x_dtype == MK_F32 ? kPlaneSliceWords : kSliceWords) * sizeof(uint32_t);
     auto launch = [&](auto kernel) -> int {
         if constexpr (PARTS == 2) {  // short rows: one wavefront per workgroup, which walks the tiles
             static std::atomic<int> known{0};
@@ -693,17 +748,39 @@ int launch_tile_parts(const Stream4Args &a, const Stream4Group &members, int til
         hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
         return 0;
     };
+    const bool wide_sides = a.scale_dtype == MK_F32;
+    if (a.x_dtype != MK_F32 && MT > 2) return -1;   // four samples at once only as digit planes
+    if (a.x_dtype == MK_F32) {   // digit planes
+        if (wide_sides) {
+            if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_F16, PARTS, true, true>);
+            return launch(stream4_kernel<MT, false, ROWS, MK_F16, PARTS, true, true>);
+        }
+        if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_F16, PARTS, true, false>);
+        return launch(stream4_kernel<MT, false, ROWS, MK_F16, PARTS, true, false>);
+    }
+    if constexpr (MT <= 2) {
+    if (wide_sides) {
+        if (a.x_dtype == MK_F16) {
+            if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_F16, PARTS, false, true>);
+            return launch(stream4_kernel<MT, false, ROWS, MK_F16, PARTS, false, true>);
+        }
+        if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_BF16, PARTS, false, true>);
+        return launch(stream4_kernel<MT, false, ROWS, MK_BF16, PARTS, false, true>);
+    }
     if (a.x_dtype == MK_F16) {
         if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_F16, PARTS>);
         return launch(stream4_kernel<MT, false, ROWS, MK_F16, PARTS>);
     }
     if (a.zeros) return launch(stream4_kernel<MT, true, ROWS, MK_BF16, PARTS>);
     return launch(stream4_kernel<MT, false, ROWS, MK_BF16, PARTS>);
+    }
+    return -1;
 }
 
 template <int MT, int ROWS>
 int launch_tile(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
-    if (a.width <= 1024) return launch_tile_parts<MT, ROWS, 2>(a, members, tiles, stream);
+    // (short rows keep two samples per pass: the tile loop has no registers for four samples' planes)
+    if (a.width <= 1024) return launch_tile_parts<(MT > 2 ? 2 : MT), ROWS, 2>(a, members, tiles, stream);
     return launch_tile_parts<MT, ROWS, 1>(a, members, tiles, stream);
 }
 
@@ -715,6 +792,8 @@ int launch_rows(const Stream4Args &a, const Stream4Group &members, int tiles, hi
     // One or two samples: v_dot2 kernel.  Three and more: matrix-core blocks (measured at
     // 4096 x 14336: 9.5 against 10.8 us for four samples, 13.3 against 17.6 us for eight).
     if (a.samples >= 3) {
+        // fp32 activations: four samples' digit planes per lane, samples 5 - 8 in a second pass over the codes
+        if (a.x_dtype == MK_F32) return launch_tile<4, ROWS>(a, members, tiles, stream);
         if (a.samples <= 4) return launch_blocks<1, ROWS>(a, members, tiles, stream);
         return launch_blocks<2, ROWS>(a, members, tiles, stream);
     }
@@ -727,10 +806,10 @@ constexpr int kComputeUnits = 256;
 }  // namespace
 
 bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform) {
-    const bool sixteen_bit_sides = scale_dtype == MK_F16 || scale_dtype == MK_BF16;
-    (void)samples;
-    const bool activations = x_dtype == MK_F16 || x_dtype == MK_BF16;
-    return bits == 4 && uniform && activations && sixteen_bit_sides && width % kChunkCodes == 0 && width <= 16384 &&
+    // fp32 activations run as digit planes at any sample count; fp32 scales under 16-bit activations: the v_dot2
+    // kernel, one or two samples
+    const bool by_pairs = x_dtype != MK_F32 && scale_dtype == MK_F32;   // fp32 scales with 16-bit activations
+    return bits == 4 && uniform && (!by_pairs || samples <= 2) && width % kChunkCodes == 0 && width <= 16384 &&
            (group % kChunkCodes == 0 || group >= width);
 }
 

@@ -27,7 +27,8 @@ int rotate_inside_the_matvec(const void *x, int x_dtype, int block, const float 
                              const void *scales, int scale_dtype, const void *zeros, const void *bias, int bias_dtype,
                              void *y, int samples, int output_width, int input_width, int group, int bits, int uniform,
                              float grid_min, float grid_step, hipStream_t stream) {
-    if (samples != 1 || (x_dtype != MK_F16 && x_dtype != MK_BF16) || !packed || !scales || !y || group < 1 || output_width < 1)
+    if (samples != 1 || (x_dtype != MK_F16 && x_dtype != MK_BF16) || (scale_dtype != MK_F16 && scale_dtype != MK_BF16) || !packed ||
+        !scales || !y || group < 1 || output_width < 1)
         return 0;
     if (!mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0)) return 0;
     const auto misaligned = [](const void *pointer, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(pointer) & mask) != 0; };

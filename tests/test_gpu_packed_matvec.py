@@ -595,7 +595,9 @@ def test_two_to_eight_samples_on_rows_of_many_lengths(rows, width, asym, with_bi
 
 def test_small_and_large_activations_keep_the_tolerance():
     """Rows of activations a hundred times smaller or two thousand times larger than the usual ones, and a row
-    with every second value small: the error stays within the tolerance of each row's output range."""
+    with every second value small: the error stays within the tolerance of each row's output range.  One
+    sample at a time the activations meet the codes unscaled, and a row ten thousand times smaller than usual
+    (fp16 values near the end of the normal range) keeps the tolerance as well."""
     weight = helpers.normal_weight(64, 4096, seed=77)
     layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
     x = helpers.activations(4, 4096, seed=3).float()
@@ -606,3 +608,65 @@ def test_small_and_large_activations_keep_the_tolerance():
     y = run_matvec(layer, x)
     for m in range(4):
         check(y[m:m + 1], layer, x[m:m + 1])
+    tiny = (helpers.activations(2, 4096, seed=4).float() * 1e-4).half()
+    for samples in (1, 2):
+        y = run_matvec(layer, tiny[:samples])
+        for m in range(samples):
+            check(y[m:m + 1], layer, tiny[m:m + 1])
+
+
+@pytest.mark.parametrize("rows,width,group,asym,with_bias", [
+    (4096, 14336, 128, False, False),   # the metric shape
+    (4096 + 5, 4096, 128, True, True),
+    (64, 896, 128, False, True),        # two rows per wavefront step
+    (48, 2080, 32, True, False),        # a ragged last slice, one scale per chunk
+    (32, 256, 256, False, False),       # one scale per row
+])
+@pytest.mark.parametrize("scale_format", ["fp32", "fp16"])
+def test_fp32_activations_on_the_streaming_kernel(rows, width, group, asym, with_bias, scale_format):
+    """INT4 with fp32 activations, one to eight samples (what the reference's own matvec tests run,
+    tests/inference/test_packed_linear.py:91-98): chunks of 32 activations are scaled by a power of two, rounded
+    to 22-bit integers and multiplied with the codes exactly, as planes of 4-bit digits.  Against the float64
+    product within 1.5e-7 of sum |w| |x| (an fp32 dot product of these lengths measures 2e-8 to 4.5e-8 of it on the
+    CPU, this path 1.5e-8 to 8.5e-8), and against the oracle's fp32 reconstruct-then-matmul at the reference's own
+    bound (rtol 1e-4, atol 1e-5); with fp32 and with fp16 scales; activations spanning sixty
+    times 1e-30 and 1e30, and rows of zeros, keep the bound; activations spanning sixty powers of two inside a
+    chunk (which keeps 22 bits of its LARGEST value) keep 1e-6 of the outputs' range."""
+    weight = helpers.normal_weight(rows, width, seed=rows + width)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=group, integer=True, asym=asym, fmt=scale_format)
+    bias = helpers.activations(1, rows, seed=8, dtype=torch.float32)[0] if with_bias else None
+    for samples in (1, 2, 3, 4, 5, 8):
+        x = helpers.activations(samples, width, seed=60 + samples, dtype=torch.float32)
+        spread = torch.ones(width)
+        spread[: width // 2] = 2.0 ** torch.randint(-30, 30, (width // 2,), generator=torch.Generator().manual_seed(3)).float()
+        for scaled in (x, x * 1e-30, x * 1e30, torch.zeros_like(x), x * spread):
+            y = run_matvec(layer, scaled, bias, scale_dtype=torch.float32 if scale_format == "fp32" else torch.float16)
+            reference = oracle_matvec.reconstruct_then_matmul_f64(
+                scaled.double().numpy(), layer["dense"], None if bias is None else bias.double().numpy())
+            budget = 1.5e-7 * (np.abs(scaled.double().numpy()) @ np.abs(layer["dense"]).T.astype(np.float64)) + 1e-7 * np.abs(reference) + 1e-30
+            if torch.equal(scaled, x * spread) and not torch.equal(scaled, x):
+                # the error is bounded against the outputs' range, which the large values make
+                assert np.abs(y - reference).max() <= 1e-6 * np.abs(reference).max()
+                continue
+            worst = float((np.abs(y - reference) / budget).max())
+            assert worst <= 1.0, (samples, worst)
+            if scaled is x:
+                fp32_reference = oracle_matvec.reconstruct_then_matmul(
+                    x.numpy(), layer["packed"], 4, layer["shape"], layer["scales"], layer["values"], group, layer["zero"],
+                    None if bias is None else bias.numpy())
+                np.testing.assert_allclose(y, fp32_reference, rtol=1e-4, atol=1e-5)
+
+
+def test_fp32_activations_that_are_not_finite_stay_so():
+    """The reference's fp32 matmul answers an infinite or NaN activation with outputs that are not finite; the digit
+    planes answer with NaN for every row (the chunk's factor becomes NaN), and other samples are not touched."""
+    weight = helpers.normal_weight(64, 4096, seed=9)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True, asym=False, fmt="fp16")
+    for samples in (1, 2, 4):
+        for poison in (float("inf"), float("-inf"), float("nan")):
+            x = helpers.activations(samples, 4096, seed=70 + samples, dtype=torch.float32)
+            clean = run_matvec(layer, x, None, scale_dtype=torch.float16)
+            x[0, 1234] = poison
+            y = run_matvec(layer, x, None, scale_dtype=torch.float16)
+            assert not np.isfinite(y[0]).any()
+            np.testing.assert_array_equal(y[1:], clean[1:])
