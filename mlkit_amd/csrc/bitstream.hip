@@ -49,9 +49,52 @@ __device__ __forceinline__ uint32_t code_at(const void *codes, long long index, 
     }
 }
 
+// A whole run of 32 codes as unsigned values.  WIDE: the codes start on a 16-byte boundary (a run of one-byte
+// codes is then two 16-byte loads, of four-byte codes eight, instead of 32 scalar ones at a stride that wastes
+// most of every cache line a wavefront touches).
+template <int CODE_BYTES, bool WIDE>
+__device__ __forceinline__ void run_at(const void *codes, long long first, int bits, uint32_t (&value)[kRun], uint32_t &bad) {
+    if constexpr (WIDE && CODE_BYTES == 1) {
+        const uint4 *source = reinterpret_cast<const uint4 *>(static_cast<const uint8_t *>(codes) + first);
+        const uint4 halves[2] = {source[0], source[1]};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t words[4] = {halves[h].x, halves[h].y, halves[h].z, halves[h].w};
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const uint32_t code = (words[w] >> (8 * b)) & 0xffu;
+                    value[16 * h + 4 * w + b] = code;
+                    bad |= code >> bits;
+                }
+        }
+    } else if constexpr (WIDE && CODE_BYTES == 4) {
+        const uint4 *source = reinterpret_cast<const uint4 *>(static_cast<const int32_t *>(codes) + first);
+#pragma unroll
+        for (int q = 0; q < kRun / 4; ++q) {
+            const uint4 four = source[q];
+            const uint32_t words[4] = {four.x, four.y, four.z, four.w};
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                value[4 * q + w] = words[w];
+                bad |= words[w] >> bits;   // a negative value has high bits set
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kRun; ++i) value[i] = code_at<CODE_BYTES>(codes, first + i, bits, bad);
+    }
+}
+
 // ALIGNED: the stream starts on a 4-byte boundary and whole runs are stored as dwords.
-template <int CODE_BYTES, bool ALIGNED>
-__global__ void __launch_bounds__(256) pack_kernel(const StreamArgs a) {
+// WIDE: see run_at.
+// BITS: the code width when the launch knows it (the shift register then resolves at compile time and a run's
+// dwords leave as one or two wide stores), or 0 for a.bits.
+template <int CODE_BYTES, bool ALIGNED, bool WIDE = false, int BITS = 0>
+__global__ void __launch_bounds__(256) pack_kernel(const StreamArgs a_) {
+    StreamArgs a = a_;
+    if constexpr (BITS != 0) a.bits = BITS;
     const long long whole_runs = a.count / kRun;
     const long long runs = whole_runs + (a.count % kRun ? 1 : 0);
     const uint32_t mask = (1u << a.bits) - 1u;
@@ -63,9 +106,23 @@ __global__ void __launch_bounds__(256) pack_kernel(const StreamArgs a) {
         if (run < whole_runs) {
             uint64_t window = 0;
             int filled = 0, word = 0;
+            uint32_t value[kRun];
+            run_at<CODE_BYTES, WIDE>(a.codes_in, first, a.bits, value, bad);
+            if constexpr (BITS == 4 && ALIGNED) {   // 16-byte aligned: the stream is, and a run is 16 bytes
+                uint32_t words[4];
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    words[w] = 0;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) words[w] |= (value[8 * w + i] & 15u) << (4 * i);
+                }
+                typedef uint32_t u4 __attribute__((ext_vector_type(4), aligned(4)));
+                *reinterpret_cast<u4 *>(target) = u4{words[0], words[1], words[2], words[3]};
+                continue;
+            }
 #pragma unroll
             for (int i = 0; i < kRun; ++i) {
-                window |= static_cast<uint64_t>(code_at<CODE_BYTES>(a.codes_in, first + i, a.bits, bad) & mask) << filled;
+                window |= static_cast<uint64_t>(value[i] & mask) << filled;
                 filled += a.bits;
                 if (filled >= 32) {
                     const uint32_t out = static_cast<uint32_t>(window);
@@ -98,8 +155,10 @@ __global__ void __launch_bounds__(256) pack_kernel(const StreamArgs a) {
     if (bad && a.overflow) atomicOr(a.overflow, 1);
 }
 
-template <bool WIDE_CODES, bool ALIGNED>
-__global__ void __launch_bounds__(256) unpack_kernel(const StreamArgs a) {
+template <bool WIDE_CODES, bool ALIGNED, int BITS = 0>
+__global__ void __launch_bounds__(256) unpack_kernel(const StreamArgs a_) {
+    StreamArgs a = a_;
+    if constexpr (BITS != 0) a.bits = BITS;   // known at the launch: the shift register resolves at compile time
     const long long whole_runs = a.count / kRun;
     const long long runs = whole_runs + (a.count % kRun ? 1 : 0);
     const long long stream_bytes = (a.count * a.bits + 7) / 8;
@@ -139,10 +198,13 @@ __global__ void __launch_bounds__(256) unpack_kernel(const StreamArgs a) {
         } else {
             uint8_t *target = static_cast<uint8_t *>(a.codes_out) + first;
             if (left == kRun && (reinterpret_cast<uintptr_t>(target) & 3u) == 0) {
+                uint32_t words[kRun / 4];
 #pragma unroll
                 for (int q = 0; q < kRun / 4; ++q)
-                    reinterpret_cast<uint32_t *>(target)[q] =
-                        out[4 * q] | (out[4 * q + 1] << 8) | (out[4 * q + 2] << 16) | (out[4 * q + 3] << 24);
+                    words[q] = out[4 * q] | (out[4 * q + 1] << 8) | (out[4 * q + 2] << 16) | (out[4 * q + 3] << 24);
+                typedef uint32_t u4 __attribute__((ext_vector_type(4), aligned(4)));   // two wide stores per run
+                reinterpret_cast<u4 *>(target)[0] = u4{words[0], words[1], words[2], words[3]};
+                reinterpret_cast<u4 *>(target)[1] = u4{words[4], words[5], words[6], words[7]};
             } else {
 #pragma unroll
                 for (int i = 0; i < kRun; ++i)
@@ -173,7 +235,23 @@ extern "C" int mk_pack(const void *codes, int code_bytes, long long count, int b
     StreamArgs a{};
     a.codes_in = codes; a.packed = packed; a.count = count; a.bits = bits; a.overflow = overflow;
     const bool aligned = (reinterpret_cast<uintptr_t>(packed) & 3u) == 0;
+    const bool wide = aligned && (reinterpret_cast<uintptr_t>(codes) & 15u) == 0 && (code_bytes == 1 || code_bytes == 4);
     const dim3 grid(grid_for(count)), block(256);
+    if (wide) {
+        if (code_bytes == 1) {
+            switch (bits) {
+                case 2: hipLaunchKernelGGL((pack_kernel<1, true, true, 2>), grid, block, 0, stream, a); break;
+                case 3: hipLaunchKernelGGL((pack_kernel<1, true, true, 3>), grid, block, 0, stream, a); break;
+                case 4: hipLaunchKernelGGL((pack_kernel<1, true, true, 4>), grid, block, 0, stream, a); break;
+                case 8: hipLaunchKernelGGL((pack_kernel<1, true, true, 8>), grid, block, 0, stream, a); break;
+                default: hipLaunchKernelGGL((pack_kernel<1, true, true>), grid, block, 0, stream, a); break;
+            }
+        } else {
+            hipLaunchKernelGGL((pack_kernel<4, true, true>), grid, block, 0, stream, a);
+        }
+        MK_LAUNCH_CHECK("mk_pack");
+        return MK_OK;
+    }
     auto launch = [&](auto aligned_tag) {
         constexpr bool A = decltype(aligned_tag)::value;
         switch (code_bytes) {
@@ -203,8 +281,17 @@ extern "C" int mk_unpack(const uint8_t *packed, long long count, int bits, void 
         if (aligned) hipLaunchKernelGGL((unpack_kernel<true, true>), grid, block, 0, stream, a);
         else hipLaunchKernelGGL((unpack_kernel<true, false>), grid, block, 0, stream, a);
     } else {
-        if (aligned) hipLaunchKernelGGL((unpack_kernel<false, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((unpack_kernel<false, false>), grid, block, 0, stream, a);
+        if (aligned) {
+            switch (bits) {
+                case 2: hipLaunchKernelGGL((unpack_kernel<false, true, 2>), grid, block, 0, stream, a); break;
+                case 3: hipLaunchKernelGGL((unpack_kernel<false, true, 3>), grid, block, 0, stream, a); break;
+                case 4: hipLaunchKernelGGL((unpack_kernel<false, true, 4>), grid, block, 0, stream, a); break;
+                case 8: hipLaunchKernelGGL((unpack_kernel<false, true, 8>), grid, block, 0, stream, a); break;
+                default: hipLaunchKernelGGL((unpack_kernel<false, true>), grid, block, 0, stream, a); break;
+            }
+        } else {
+            hipLaunchKernelGGL((unpack_kernel<false, false>), grid, block, 0, stream, a);
+        }
     }
     MK_LAUNCH_CHECK("mk_unpack");
     return MK_OK;
