@@ -547,7 +547,7 @@ def other_kernels(device: torch.device, full: bool) -> dict:
     matvec(ROWS, WIDTH, 64, 3, torch.arange(-4, 4, dtype=torch.float32, device=device), True, False, "int3 g64", grouped=True)
     matvec(ROWS, WIDTH, 64, 4, nf4, False, False, "nf4 g64", grouped=True)
     matvec(ROWS, WIDTH, 64, 3, seven, False, False, "codebook7 g64", grouped=True)
-    # fp32 activations and fp32 scales (what the reference's own fp32 tests use): the generic word kernel
+    # fp32 activations and fp32 scales (what the reference's own fp32 tests use): digit planes against v_dot8_i32_i4
     matvec(ROWS, WIDTH, 128, 4, values, True, False, "int4 g128, fp32 activations and scales", dtype=torch.float32,
            side_dtype=torch.float32)
     if full:
@@ -559,6 +559,34 @@ def other_kernels(device: torch.device, full: bool) -> dict:
     del weight, rotated, dense, codes
     out["rotated layers (config 5)"] = rotated_layer(device, generator, values)
     return out
+
+
+# name -> (group, bits, table, uniform grid, activation and scale dtype)
+PROFILE_CODECS = {
+    "int4": None,
+    "int2": (64, 2, [-2, -1, 0, 1], True, torch.float16),
+    "int3": (64, 3, [-4, -3, -2, -1, 0, 1, 2, 3], True, torch.float16),
+    "nf4": (64, 4, None, False, torch.float16),
+    "codebook7": (64, 3, [-1, -0.5, -0.25, 0, 0.25, 0.5, 1], False, torch.float16),
+    "int4-fp32": (128, 4, list(range(-8, 8)), True, torch.float32),
+}
+
+
+def codec_launchers(name: str, samples: int, device: torch.device, generator: torch.Generator) -> list:
+    """Eager-call launchers of one of the other codecs at 4096 x 14336 over rotating weight copies (what
+    other_kernels() times), for counter runs."""
+    import mlkit_amd as mk
+
+    group, bits, table, uniform, dtype = PROFILE_CODECS[name]
+    table = mk.NF4_VALUES.to(device) if table is None else torch.tensor(table, dtype=torch.float32, device=device)
+    code_bytes = ROWS * WIDTH * bits // 8
+    count = max(2, min(40, -(-MINIMUM_ROTATING_BYTES // code_bytes)))
+    streams = [torch.randint(0, 256, (code_bytes,), dtype=torch.uint8, device=device, generator=generator) for _ in range(count)]
+    side = (torch.rand((ROWS, WIDTH // group), device=device, generator=generator) * 0.004 + 0.005).to(dtype)
+    x = torch.randn((samples, WIDTH), device=device, generator=generator).to(dtype)
+    y = torch.empty((samples, ROWS), device=device, dtype=dtype)
+    return [Launcher(x, stream, side, table, y, rows=ROWS, width=WIDTH, group=group, bits=bits, uniform=uniform,
+                     grid_min=float(table[0]), grid_step=float(table[1] - table[0])) for stream in streams]
 
 
 def cpu_fwht_baseline() -> dict:
@@ -596,6 +624,9 @@ def main() -> None:
                                                                "between two uses of a copy)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--skip-kernels", action="store_true", help="only the headline matvec (no GPTQ / FWHT / codec legs)")
+    parser.add_argument("--headline-only", action="store_true",
+                        help="for rocprofv3 --kernel-trace --stats: only the headline leg (M=1, one call per step, rotating copies), "
+                             "so that every launch of the kernel in the trace is one of the timed workload")
     parser.add_argument("--kernels", action="store_true", help="add the decoder-layer shapes, the tied head and wider codecs")
     parser.add_argument("--profile-gptq", action="store_true",
                         help="for rocprofv3: only run the GPTQ layer (4096 x 11008) and print its timings")
@@ -605,7 +636,12 @@ def main() -> None:
                         help="for rocprofv3: only issue this many eager calls (grouped with --members > 1), plus three "
                              "256 MiB device copies whose counters calibrate FETCH_SIZE / WRITE_SIZE")
     parser.add_argument("--profile-rows", type=int, default=1, help="activation rows M of the --profile-launches calls")
+    parser.add_argument("--profile-codec", default="int4", choices=sorted(PROFILE_CODECS),
+                        help="codec of the --profile-launches calls (4096 x 14336; int4 = the metric's INT4-g128)")
     options = parser.parse_args()
+    if options.headline_only:
+        options.skip_kernels = options.no_cpu_baseline = True
+        options.members = 1
     if options.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
     if not torch.cuda.is_available():
@@ -631,7 +667,9 @@ def main() -> None:
         return
     if options.profile_launches:
         x = torch.randn((options.profile_rows, WIDTH), device=device, generator=generator).half()
-        if members > 1:
+        if options.profile_codec != "int4":
+            launchers = codec_launchers(options.profile_codec, options.profile_rows, device, generator)
+        elif members > 1:
             launchers = [GroupLauncher(x, copies[index:index + members], values) for index in range(0, copy_count, members)]
         else:
             y = torch.empty((options.profile_rows, ROWS), device=device, dtype=torch.float16)
@@ -649,7 +687,7 @@ def main() -> None:
     results = {}
     flat = {}
     head_step = None
-    for samples in (1, 2, 4, 8):
+    for samples in ((1,) if options.headline_only else (1, 2, 4, 8)):
         x = torch.randn((samples, WIDTH), device=device, generator=generator).half()
         y = torch.empty((samples, ROWS), device=device, dtype=torch.float16)
         single = [Launcher(x, packed, scales, values, y) for packed, scales in copies]
@@ -662,6 +700,11 @@ def main() -> None:
             head_step = (median, low, high, batch, steps, replays)
         row["single_call"] = {"us_per_matrix": median * 1e6, "min_us": low * 1e6, "max_us": high * 1e6,
                               "hbm_frac": algorithmic_bytes(samples) / median / 1e9 / HBM_PEAK_GBPS}
+        if options.headline_only:
+            results[samples] = row
+            flat[f"us_M{samples}"] = median * 1e6
+            flat[f"frac_M{samples}"] = row["single_call"]["hbm_frac"]
+            break
         resident = timed_graph([single[0]], max(options.steps, 50), options.warmup, 10)[0]
         row["single_call"]["cache_resident_us"] = resident * 1e6
         flat[f"us_M{samples}"] = median * 1e6
