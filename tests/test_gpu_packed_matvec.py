@@ -421,15 +421,21 @@ def test_grouped_launch_of_table_codecs(name, width, rows):
             check(grouped[0].float().cpu().numpy(), layers[0], x)
 
 
-def test_grouped_launch_of_layouts_without_a_group_kernel():
-    """fp32 activations (the generic kernel) go through the same entry point as one launch per
-    matrix: same results as mk_packed_matvec."""
-    layers = [helpers.quantised_layer(helpers.normal_weight(n, 256, seed=77 + i), INT4, bits=4, group=64, integer=True,
-                                      fmt="fp32") for i, n in enumerate((37, 21))]
-    x = helpers.activations(2, 256, seed=78, dtype=torch.float32)
-    grouped = run_group(layers, x, scale_dtype=torch.float32)
-    for index, layer in enumerate(layers):
-        assert np.array_equal(grouped[index].cpu().numpy(), run_matvec(layer, x, scale_dtype=torch.float32))
+def test_grouped_launch_with_fp32_activations():
+    """fp32 activations through the grouped entry point: INT4 uniform grids run as one launch of the digit-plane
+    kernel (members of different heights, rows past a member's last whole tile, every sample count), other
+    layouts (3-bit codes here) as one launch of the generic kernel per matrix; both equal mk_packed_matvec bit for
+    bit, and the first member is held against the float64 product."""
+    for values, bits, width, group in ((INT4, 4, 2048, 128), (INT4, 4, 256, 64), (scaling.int_values(3), 3, 256, 64)):
+        layers = [helpers.quantised_layer(helpers.normal_weight(n, width, seed=77 + i), values, bits=bits, group=group,
+                                          integer=True, fmt="fp32") for i, n in enumerate((37, 21, 64))]
+        for samples in (1, 2, 3, 5, 8):
+            x = helpers.activations(samples, width, seed=78 + samples, dtype=torch.float32)
+            grouped = run_group(layers, x, scale_dtype=torch.float32)
+            for index, layer in enumerate(layers):
+                assert np.array_equal(grouped[index].cpu().numpy(), run_matvec(layer, x, scale_dtype=torch.float32)), (bits, width, samples, index)
+            reference = oracle_matvec.reconstruct_then_matmul_f64(x.double().numpy(), layers[0]["dense"], None)
+            np.testing.assert_allclose(grouped[0].cpu().numpy(), reference, rtol=1e-4, atol=1e-5)
 
 
 def test_grouped_launch_validation():
