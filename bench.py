@@ -278,6 +278,10 @@ def gptq_layer(device: torch.device, generator: torch.Generator, cpu_rows: int =
         table_quantizer = mk.gptq(mk.nf4(group=64))
         table_quantizer(target, Ctx("warmup", H=hessian))
         table_sweep_ms = wall_ms(lambda: table_quantizer(target, Ctx("down_proj", H=hessian)))
+        # and on a table of 253 values (the e4m3 minifloat grid, one scale per 64 columns)
+        wide_quantizer = mk.gptq(mk.scaled(mk.grid.fp("e4m3"), group=64))
+        wide_quantizer(target, Ctx("warmup", H=hessian))
+        wide_sweep_ms = wall_ms(lambda: wide_quantizer(target, Ctx("down_proj", H=hessian)))
     finally:
         feedback.feedback_coefficients = original
     update_flops = sum(2 * rows * block * (width - stop) for stop in range(block, width, block))
@@ -286,6 +290,7 @@ def gptq_layer(device: torch.device, generator: torch.Generator, cpu_rows: int =
         "total_ms": total_ms, "coefficients_ms": factor_ms, "sweep_and_update_ms": sweep_ms,
         "columns_per_s": width / (sweep_ms / 1e3), "weights_per_s": rows * width / (sweep_ms / 1e3),
         "nf4_g64_sweep_and_update_ms": table_sweep_ms,
+        "e4m3_g64_sweep_and_update_ms": wide_sweep_ms,
         "trailing_update_flops": update_flops,
         "proxy_loss": float(mk.proxy_loss(target, result.w, hessian)),
         "rtn_proxy_loss": float(mk.proxy_loss(target, rtn.w, hessian)),

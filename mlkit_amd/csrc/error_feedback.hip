@@ -321,12 +321,65 @@ __device__ __forceinline__ Nearest nearest_of(const Nearest (&entries)[COUNT]) {
     }
 }
 
-// TABLE: 0 rounds to an integer grid; kSmallTable rounds to a table of at most sixteen values.
+// Tables of 17 to 256 values: the sixteen lanes of a row search for the value of the column that is being rounded
+// (the step's owner) together.  Lane p holds entries p, 16 + p, 32 + p, ... (entries beyond the table are NaN and
+// never win: every lane holds at least one real entry), finds the nearest of its own by the tournament above
+// and the sixteen winners meet in four DPP exchanges (lane ^ 1, lane ^ 2, mirrored halves of eight, mirrored
+// row), in each of which the other lane's entry wins on a strictly smaller distance, or on an equal distance and
+// a lower index: the smallest (distance, index) of the table, in every lane of the row.
+constexpr int kLargeTable = 256;
+
+template <int CONTROL>
+__device__ __forceinline__ Nearest nearer_of_lane_pair(const Nearest &mine) {
+    Nearest other;
+    other.difference = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(mine.difference), CONTROL, 0xf, 0xf, true));
+    other.value = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(mine.value), CONTROL, 0xf, 0xf, true));
+    other.index = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(mine.index), CONTROL, 0xf, 0xf, true));
+    const float own_distance = fabsf(mine.difference), other_distance = fabsf(other.difference);
+    const bool take = other_distance < own_distance || (other_distance == own_distance && other.index < mine.index);
+    Nearest winner;
+    winner.difference = take ? other.difference : mine.difference;
+    winner.value = take ? other.value : mine.value;
+    winner.index = take ? other.index : mine.index;
+    return winner;
+}
+
+__device__ __forceinline__ Nearest nearest_over_row(float wanted, const float (&table)[kLargeTable / 16], int p) {
+    constexpr int kOwn = kLargeTable / 16;
+    // This lane's entries in ascending index order, keeping the first minimum (a scan rather than the tournament:
+    // one comparison result alive at a time; the fully unrolled sweep around it has no registers to spare).
+    __builtin_amdgcn_sched_barrier(0);
+    float best_difference = __fsub_rn(wanted, table[0]), best_value = table[0];
+    int best_slot = 0;
+#pragma unroll
+    for (int i = 1; i < kOwn; ++i) {
+        const float difference = __fsub_rn(wanted, table[i]);
+        const bool take = fabsf(difference) < fabsf(best_difference);
+        best_difference = take ? difference : best_difference;
+        best_value = take ? table[i] : best_value;
+        best_slot = take ? i : best_slot;
+    }
+    Nearest best;
+    best.difference = best_difference;
+    best.value = best_value;
+    best.index = static_cast<uint32_t>(16 * best_slot + p);
+    best = nearer_of_lane_pair<0xB1>(best);    // quad_perm [1,0,3,2]
+    best = nearer_of_lane_pair<0x4E>(best);    // quad_perm [2,3,0,1]
+    best = nearer_of_lane_pair<0x141>(best);   // row_half_mirror: lane i <-> 7 - i of each eight
+    best = nearer_of_lane_pair<0x140>(best);   // row_mirror: lane i <-> 15 - i of the row
+    __builtin_amdgcn_sched_barrier(0);
+    return best;
+}
+
+// TABLE: 0 rounds to an integer grid; kSmallTable rounds to a table of at most sixteen values, kLargeTable to one of
+// at most 256.
 template <int MODE, bool WHOLE, int TABLE = 0>
 __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const SweepArgs a) {
     static_assert(MODE == kModeInteger || MODE == kModeSolve || (MODE == kModeRegion && WHOLE),
                   "larger tables use the one-row-per-wavefront kernel; a fused region is one whole tile");
-    static_assert(TABLE == 0 || (TABLE == kSmallTable && MODE != kModeSolve), "a table of sixteen values, or none");
+    static_assert(TABLE == 0 || ((TABLE == kSmallTable || TABLE == kLargeTable) && MODE != kModeSolve),
+                  "a table of at most sixteen or at most 256 values, or none");
+    constexpr int kHeldEntries = TABLE == kLargeTable ? kLargeTable / 16 : TABLE;
     constexpr int kStaged = WHOLE ? kNarrowTile * kNarrowTile : 2 * kRowLanes * kNarrowTile;
     __shared__ __attribute__((aligned(16))) float staged[kStaged];
     const int lane = threadIdx.x & 63;
@@ -337,8 +390,14 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
     const int row = active ? wanted_row : a.rows - 1;
     const size_t row_base = static_cast<size_t>(row) * a.width;
 
-    float table[TABLE > 0 ? TABLE : 1];
-    if constexpr (TABLE > 0) {
+    float table[TABLE > 0 ? kHeldEntries : 1];
+    if constexpr (TABLE == kLargeTable) {
+#pragma unroll
+        for (int i = 0; i < kHeldEntries; ++i) {
+            const int entry = 16 * i + p;
+            table[i] = entry < a.n_values ? a.values[entry < a.n_values ? entry : 0] : __builtin_nanf("");
+        }
+    } else if constexpr (TABLE > 0) {
 #pragma unroll
         for (int i = 0; i < TABLE; ++i) table[i] = i < a.n_values ? a.values[i < a.n_values ? i : 0] : __builtin_nanf("");
     }
@@ -410,7 +469,11 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
             const float normalized = __fdiv_rn(__fsub_rn(target, zero[t]), scale[t]);
             float chosen;
             uint32_t index;
-            if constexpr (TABLE > 0) {
+            if constexpr (TABLE == kLargeTable) {
+                const Nearest nearest = nearest_over_row(row_value(normalized, owner, row_in_wave), table, p);
+                chosen = nearest.value;
+                index = nearest.index;
+            } else if constexpr (TABLE > 0) {
                 Nearest entries[TABLE];
 #pragma unroll
                 for (int i = 0; i < TABLE; ++i) {
@@ -467,7 +530,25 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
     };
     auto slot_of_steps = [&](auto slot, auto solving) __attribute__((always_inline)) {
         constexpr int t = decltype(slot)::value;
-        if constexpr (WHOLE) {
+        if constexpr (WHOLE && TABLE == kLargeTable) {
+            // The search of a large table is some 150 instructions per step: unrolled 128 times it neither fits the
+            // registers nor the instruction cache.  The sixteen steps of a slot are a loop; the owner's value
+            // comes through v_readlane and the next step's coefficient row is read from LDS a step ahead.
+            float row_now[kSlots], row_next[kSlots];
+            auto read_row = [&](int index, float (&row)[kSlots]) __attribute__((always_inline)) {
+                const float *coefficients = staged + index * kNarrowTile + p;
+#pragma unroll
+                for (int later = t; later < kSlots; ++later) row[later] = coefficients[kRowLanes * later];
+            };
+            read_row(kRowLanes * t, row_now);
+            for (int owner = 0; owner < kRowLanes; ++owner) {
+                const int following = kRowLanes * t + owner + 1;
+                read_row(following < kNarrowTile ? following : kNarrowTile - 1, row_next);
+                advance(slot, owner, nullptr, solving, row_now);
+#pragma unroll
+                for (int later = t; later < kSlots; ++later) row_now[later] = row_next[later];
+            }
+        } else if constexpr (WHOLE) {
             step_of_whole(slot, std::integral_constant<int, 0>{}, solving);
             step_of_whole(slot, std::integral_constant<int, 1>{}, solving);
             step_of_whole(slot, std::integral_constant<int, 2>{}, solving);
@@ -495,7 +576,7 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
         }
     };
     auto all_slots = [&](auto solving) __attribute__((always_inline)) {
-        if constexpr (WHOLE) load_row(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, row_even);
+        if constexpr (WHOLE && TABLE != kLargeTable) load_row(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, row_even);
         slot_of_steps(std::integral_constant<int, 0>{}, solving);
         slot_of_steps(std::integral_constant<int, 1>{}, solving);
         slot_of_steps(std::integral_constant<int, 2>{}, solving);
@@ -595,14 +676,15 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
 // One kernel for a region that is a single whole tile of an integer grid: pending solve,
 // scale fit and column sweep.
 bool region_fusable(int span, int block, int fitted_group, bool integer_grid, int n_values) {
-    return (integer_grid || n_values <= kSmallTable) && span == kNarrowTile && block >= kNarrowTile &&
+    return (integer_grid || n_values <= kLargeTable) && span == kNarrowTile && block >= kNarrowTile &&
            fitted_group % kRowLanes == 0 && kNarrowTile % fitted_group == 0;
 }
 
 int launch_region(const SweepArgs &a, bool integer_grid, hipStream_t stream) {
     const dim3 grid(mk_cdiv(a.rows, kNarrowRows)), block(kSweepThreads);
     if (integer_grid) hipLaunchKernelGGL((narrow_sweep_kernel<kModeRegion, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((narrow_sweep_kernel<kModeRegion, true, kSmallTable>), grid, block, 0, stream, a);
+    else if (a.n_values <= kSmallTable) hipLaunchKernelGGL((narrow_sweep_kernel<kModeRegion, true, kSmallTable>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((narrow_sweep_kernel<kModeRegion, true, kLargeTable>), grid, block, 0, stream, a);
     return MK_OK;
 }
 
@@ -625,6 +707,14 @@ int launch_sweep(const SweepArgs &a, hipStream_t stream) {
             hipLaunchKernelGGL((narrow_sweep_kernel<kModeInteger, true, kSmallTable>), narrow_grid, block, 0, stream, a);
         else
             hipLaunchKernelGGL((narrow_sweep_kernel<kModeInteger, false, kSmallTable>), narrow_grid, block, 0, stream, a);
+        return MK_OK;
+    } else if (a.tile_width <= kNarrowTile && a.n_values <= kLargeTable) {
+        // larger tables (minifloat grids, codebooks): the sixteen lanes of a row search the table together
+        const dim3 narrow_grid(mk_cdiv(a.rows, kNarrowRows));
+        if (a.tile_width == kNarrowTile)
+            hipLaunchKernelGGL((narrow_sweep_kernel<kModeInteger, true, kLargeTable>), narrow_grid, block, 0, stream, a);
+        else
+            hipLaunchKernelGGL((narrow_sweep_kernel<kModeInteger, false, kLargeTable>), narrow_grid, block, 0, stream, a);
         return MK_OK;
     }
     if (a.tile_width <= 128)

@@ -87,6 +87,11 @@ def test_online_activation_reconstruction_equals_quantize_dequantize():
     (np.array([-6, -4, -3, -2, -1.5, -1, -0.5, 0, 0.5, 1, 1.5, 2, 3, 4, 6], dtype=np.float32), False, False, 32, 128, 256),
     (np.array([-1, -0.5, -0.25, 0, 0.25, 0.5, 1], dtype=np.float32), False, False, 128, 128, 128),
     (scaling.NF4_VALUES, False, False, 64, 96, 96),        # regions that are not whole tiles
+    # tables of 17 to 256 values take the one-kernel-per-region path too (a row's sixteen lanes search together)
+    (np.sinh(np.linspace(-3, 3, 256)).astype(np.float32), False, False, 64, 128, 128),
+    (np.sinh(np.linspace(-3, 3, 256)).astype(np.float32), False, True, 128, 128, 256),
+    ((np.linspace(-1, 1, 40) ** 3).astype(np.float32), False, False, 32, 128, 128),
+    ((np.linspace(-1, 1, 40) ** 3).astype(np.float32), False, False, 64, 96, 96),   # tiles of 96 columns
 ])
 def test_gptq_on_device_matches_oracle_sweep(values, integer, asym, group, refit, block, rng):
     rows, width = 80, 512
@@ -95,7 +100,7 @@ def test_gptq_on_device_matches_oracle_sweep(values, integer, asym, group, refit
     inputs[:, ::9] *= 5
     inputs[:, 100] = 0
     hessian = (inputs.T @ inputs / 1536).astype(F32)
-    grid = mk.grid.int(int(np.log2(len(values)))) if integer else mk.grid.values(values, bits=4)
+    grid = mk.grid.int(int(np.log2(len(values)))) if integer else mk.grid.values(values, bits=max(4, int(np.ceil(np.log2(len(values))))))
     inner = mk.scaled(grid, group=group, asym=asym)
     quantizer = mk.gptq(inner, refit=refit, block_size=block)
     context = Ctx("layer", H=dev(hessian))

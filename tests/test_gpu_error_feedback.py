@@ -47,6 +47,11 @@ def problem(rows, width, seed, samples=None):
     (19, 640, 64, 300, 50, INT4, True, True),        # sixteen-slot kernel, ragged groups
     (64, 256, 128, 128, 64, scaling.NF4_VALUES, False, False),
     (33, 128, 0, 100, 128, SEVEN, False, True),
+    # tables of 17 to 256 values: the sixteen lanes of a row search the table together
+    (64, 256, 128, 128, 64, np.sinh(np.linspace(-3, 3, 256)).astype(F32), False, False),
+    (37, 256, 0, 128, 32, np.sinh(np.linspace(-3, 3, 256)).astype(F32), False, True),
+    (50, 384, 128, 100, 128, (np.linspace(-1, 1, 40) ** 3).astype(F32), False, False),   # ragged tile, 40 values
+    (16, 128, 0, 128, 128, np.linspace(-1, 1, 17).astype(F32), False, True),              # 17 values: ties to the lower entry
 ])
 def test_round_tile_matches_oracle(rows, width, tile_start, tile_width, group, values, integer, asym):
     from mlkit_amd.kernels import error_feedback
