@@ -31,7 +31,7 @@ namespace {
 // Rows per workgroup: 16 when that still gives every compute unit a workgroup, 4 for
 // layers with fewer rows (more, shorter workgroups).  Up to 8 rows of codes are in flight
 // per wavefront (both values swept on the GPU together with 8 / 32 rows and 4 - 16 ahead).
-constexpr int kWideRows = 16, kNarrowRows = 4;
+constexpr int kWideRows = 16, kMidRows = 8, kNarrowRows = 4;
 
 template <int ROWS>
 constexpr int rows_ahead_of() {
@@ -651,7 +651,8 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     for (int set = 0; set < SETS; ++set) {
         transposed_wave_sum<kSums, 2>(sums[set], lane);
         // With four sums per lane the last two stages leave every total in four lanes.
-        const bool writer = ((lane >> 2) >> (kSums == 16 ? 4 : 2)) == 0;
+        static_assert(kSums == 16 || kSums == 8 || kSums == 4, "one, two or four lanes per total");
+        const bool writer = ((lane >> 2) >> (kSums == 16 ? 4 : kSums == 8 ? 3 : 2)) == 0;
         if (writer)
             partials[((set * ROWS + transposed_value_of_lane<kSums>(lane >> 2)) * 4 + t) * 8 + wave] = sums[set][0];
     }
@@ -820,6 +821,14 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream) {
     none.count = 0;
     none.widest_tiles = 0;
     if (a.rows / kWideRows >= kComputeUnits) {
+        // Three and more samples are bound by instruction issue.  Rows of one wavefront (at most 2048 codes) in
+        // fewer than 512 tiles of sixteen rows leave SIMDs without a wavefront: tiles of eight rows fill them
+        // (4096 x 2048 at eight samples: 6.2 -> 5.2 us; with two and more wavefronts per row the activation
+        // preparation repeated per tile costs more than the idle SIMDs: 4096 x 4096 6.4 -> 7.0 us).
+        if (a.samples >= 3 && a.x_dtype != MK_F32 && a.width <= 2048 && a.rows / kWideRows < 2 * kComputeUnits) {
+            const int tiles = a.rows / kMidRows;
+            return launch_rows<kMidRows>(a, none, tiles, stream) ? -1 : tiles * kMidRows;
+        }
         const int tiles = a.rows / kWideRows;
         return launch_rows<kWideRows>(a, none, tiles, stream) ? -1 : tiles * kWideRows;
     }

@@ -577,6 +577,8 @@ def test_rotation_of_separate_blocks_inside_the_matvec_kernel(rows, width, block
     (16, 2048, False, False, torch.float16),
     (80, 8192, False, False, torch.float16),
     (32, 8320, False, False, torch.float16),      # 65 groups
+    (4096 + 13, 2048, True, True, torch.float16),    # tiles of eight rows (one wavefront per row, many rows), 5 rows beyond
+    (4096 + 8, 896, False, False, torch.float16),    # the same with two rows per wavefront step
 ])
 def test_two_to_eight_samples_on_rows_of_many_lengths(rows, width, asym, with_bias, scale_dtype):
     """INT4 with one scale per 128 codes, fp16 activations, every sample count from two to eight, on rows from
