@@ -320,6 +320,29 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const S
     const float shifted_step = a.grid_step * 16777216.0f;
 
     const uint8_t *table_bytes = reinterpret_cast<const uint8_t *>(table);
+    // The table entries of a row are read one row ahead of their use: the reads of row r + 1 are in flight (and
+    // queue behind each other in the banks they share) while the dot products of row r are issued.
+    constexpr int kLookups = kLookup == 1 ? 16 : 32 / kLookup;
+    uint32_t looked_up[SHIFTED ? 1 : kLookups][kEntryWords], looked_up_next[SHIFTED ? 1 : kLookups][kEntryWords];
+    auto look_up = [&](int r, uint32_t (&entry)[SHIFTED ? 1 : kLookups][kEntryWords]) __attribute__((always_inline)) {
+        if constexpr (!SHIFTED) {
+#pragma unroll
+            for (int i = 0; i < kLookups; ++i) {
+                if constexpr (kLookup == 4) {
+                    const mk_u32x2 both = *reinterpret_cast<const mk_u32x2 *>(table_bytes + lookup_offset<BITS, 4>(codes[r], i));
+                    entry[i][0] = both.x;
+                    entry[i][1] = both.y;
+                } else if constexpr (kLookup == 2) {
+                    entry[i][0] = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, 2>(codes[r], i));
+                } else {
+                    const uint32_t even = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[r], 2 * i));
+                    const uint32_t odd = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[r], 2 * i + 1));
+                    entry[i][0] = even | (odd << 16);
+                }
+            }
+        }
+    };
+    look_up(0, looked_up_next);
 #pragma unroll
     for (int pass = 0; pass < kPairRows / kReduceRows; ++pass) {
         float sums[kSums];
@@ -335,32 +358,25 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const S
                 for (int m = 0; m < MT; ++m) dot[m] = __builtin_fmaf(shifted_step, dot[m], grid_term[m]);
             } else {
 #pragma unroll
-            for (int i = 0; i < (kLookup == 1 ? 16 : 32 / kLookup); ++i) {
-                uint32_t entry[kEntryWords];
-                if constexpr (kLookup == 4) {
-                    const mk_u32x2 both = *reinterpret_cast<const mk_u32x2 *>(table_bytes + lookup_offset<BITS, 4>(codes[r], i));
-                    entry[0] = both.x;
-                    entry[1] = both.y;
-                } else if constexpr (kLookup == 2) {
-                    entry[0] = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, 2>(codes[r], i));
-                } else {
-                    const uint32_t even = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[r], 2 * i));
-                    const uint32_t odd = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[r], 2 * i + 1));
-                    entry[0] = even | (odd << 16);
-                }
+                for (int i = 0; i < kLookups; ++i)
 #pragma unroll
-                for (int h = 0; h < kEntryWords; ++h)
+                    for (int h = 0; h < kEntryWords; ++h) looked_up[i][h] = looked_up_next[i][h];
+                if (r + 1 < kPairRows) look_up(r + 1, looked_up_next);
+                __builtin_amdgcn_sched_barrier(0);   // the next row's reads are issued before this row's products
 #pragma unroll
-                    for (int m = 0; m < MT; ++m) {
-                        const uint32_t inputs = x[m].r[kEntryWords * i + h];
-                        if constexpr (XT == MK_F16)
-                            dot[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(mk_h2, entry[h]),
-                                                            __builtin_bit_cast(mk_h2, inputs), dot[m], false);
-                        else
-                            dot[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mk_bf2, entry[h]),
-                                                                     __builtin_bit_cast(mk_bf2, inputs), dot[m], false);
-                    }
-            }
+                for (int i = 0; i < kLookups; ++i)
+#pragma unroll
+                    for (int h = 0; h < kEntryWords; ++h)
+#pragma unroll
+                        for (int m = 0; m < MT; ++m) {
+                            const uint32_t inputs = x[m].r[kEntryWords * i + h];
+                            if constexpr (XT == MK_F16)
+                                dot[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(mk_h2, looked_up[i][h]),
+                                                                __builtin_bit_cast(mk_h2, inputs), dot[m], false);
+                            else
+                                dot[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mk_bf2, looked_up[i][h]),
+                                                                         __builtin_bit_cast(mk_bf2, inputs), dot[m], false);
+                        }
             }
             if (r + kPairAhead < kPairRows)
                 load_codes<BITS>(codes[r + kPairAhead],
@@ -521,6 +537,27 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
     };
     const uint8_t *table_bytes = reinterpret_cast<const uint8_t *>(table);
 
+    // The table entries of a step are read one step ahead of their use (as in pairs_kernel).
+    uint32_t looked_up[8][2], looked_up_next[8][2];
+    auto look_up = [&](int step, uint32_t (&entry)[8][2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {  // codes 4 i ... 4 i + 3
+            if constexpr (LOOKUP == 4) {
+                const mk_u32x2 both = *reinterpret_cast<const mk_u32x2 *>(table_bytes + lookup_offset<BITS, 4>(codes[step], i));
+                entry[i][0] = both.x, entry[i][1] = both.y;
+            } else if constexpr (LOOKUP == 2) {
+                entry[i][0] = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, 2>(codes[step], 2 * i));
+                entry[i][1] = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, 2>(codes[step], 2 * i + 1));
+            } else {
+                const uint32_t v0 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i));
+                const uint32_t v1 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i + 1));
+                const uint32_t v2 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i + 2));
+                const uint32_t v3 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i + 3));
+                entry[i][0] = v0 | (v1 << 16), entry[i][1] = v2 | (v3 << 16);
+            }
+        }
+    };
+    look_up(0, looked_up_next);
 #pragma unroll
     for (int step = 0; step < kSteps; ++step) {
         const int q = step / kSlices, s = step % kSlices;
@@ -528,25 +565,14 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
 #pragma unroll
         for (int set = 0; set < SETS; ++set) dot[set] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {  // codes 4 i ... 4 i + 3
-            uint32_t low, high;
-            if constexpr (LOOKUP == 4) {
-                const mk_u32x2 both = *reinterpret_cast<const mk_u32x2 *>(table_bytes + lookup_offset<BITS, 4>(codes[step], i));
-                low = both.x, high = both.y;
-            } else if constexpr (LOOKUP == 2) {
-                low = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, 2>(codes[step], 2 * i));
-                high = *reinterpret_cast<const uint32_t *>(table_bytes + lookup_offset<BITS, 2>(codes[step], 2 * i + 1));
-            } else {
-                const uint32_t v0 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i));
-                const uint32_t v1 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i + 1));
-                const uint32_t v2 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i + 2));
-                const uint32_t v3 = *reinterpret_cast<const uint16_t *>(table_bytes + lookup_offset<BITS, 1>(codes[step], 4 * i + 3));
-                low = v0 | (v1 << 16), high = v2 | (v3 << 16);
-            }
+        for (int i = 0; i < 8; ++i) looked_up[i][0] = looked_up_next[i][0], looked_up[i][1] = looked_up_next[i][1];
+        if (step + 1 < kSteps) look_up(step + 1, looked_up_next);
+        __builtin_amdgcn_sched_barrier(0);   // the next step's reads are issued before this step's products
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
 #pragma unroll
             for (int set = 0; set < SETS; ++set)
-                dot[set] = blocks(low, high, x[set][s].r[2 * i], x[set][s].r[2 * i + 1], dot[set]);
-        }
+                dot[set] = blocks(looked_up[i][0], looked_up[i][1], x[set][s].r[2 * i], x[set][s].r[2 * i + 1], dot[set]);
         if (step + kAhead < kSteps)
             load_codes<BITS>(codes[step + kAhead], codes_base + static_cast<size_t>(4 * ((step + kAhead) / kSlices)) * row_bytes +
                                                        code_offset[(step + kAhead) % kSlices]);
@@ -702,14 +728,8 @@ void launch_bits(const Stream4Args &a, const Stream4Group &members, int tiles, h
         else launch_blocks<BITS, 2>(a, members, tiles, stream);
         return;
     }
-    int tile = 1;
-    while (tile < a.samples && tile < 8) tile <<= 1;
-    switch (tile) {
-        case 1: launch_tile<BITS, 1>(a, members, tiles, stream); break;
-        case 2: launch_tile<BITS, 2>(a, members, tiles, stream); break;
-        case 4: launch_tile<BITS, 4>(a, members, tiles, stream); break;
-        default: launch_tile<BITS, 8>(a, members, tiles, stream); break;
-    }
+    if (a.samples == 1) launch_tile<BITS, 1>(a, members, tiles, stream);
+    else launch_tile<BITS, 2>(a, members, tiles, stream);
 }
 
 }  // namespace
