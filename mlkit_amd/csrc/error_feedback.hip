@@ -329,13 +329,16 @@ __device__ __forceinline__ Nearest nearest_of(const Nearest (&entries)[COUNT]) {
 // a lower index: the smallest (distance, index) of the table, in every lane of the row.
 constexpr int kLargeTable = 256;
 
+// (Distances compare as the bit patterns of their magnitudes: the same order for numbers, and a NaN -- an entry
+// beyond the table -- is larger than every number, so it loses to any real entry.)
 template <int CONTROL>
 __device__ __forceinline__ Nearest nearer_of_lane_pair(const Nearest &mine) {
     Nearest other;
     other.difference = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(mine.difference), CONTROL, 0xf, 0xf, true));
     other.value = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(mine.value), CONTROL, 0xf, 0xf, true));
     other.index = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(mine.index), CONTROL, 0xf, 0xf, true));
-    const float own_distance = fabsf(mine.difference), other_distance = fabsf(other.difference);
+    const uint32_t own_distance = __float_as_uint(mine.difference) & 0x7fffffffu;
+    const uint32_t other_distance = __float_as_uint(other.difference) & 0x7fffffffu;
     const bool take = other_distance < own_distance || (other_distance == own_distance && other.index < mine.index);
     Nearest winner;
     winner.difference = take ? other.difference : mine.difference;
@@ -371,6 +374,20 @@ __device__ __forceinline__ Nearest nearest_over_row(float wanted, const float (&
     return best;
 }
 
+// Up to sixteen values with a compile-time owner (the unrolled whole-tile kernels): lane p holds entry p alone and
+// the sixteen lanes meet as above; the owner's value arrives as a DPP row broadcast folded into the subtraction.
+__device__ __forceinline__ Nearest nearest_one_per_lane(float wanted, float entry, int p) {
+    Nearest best;
+    best.difference = __fsub_rn(wanted, entry);
+    best.value = entry;
+    best.index = static_cast<uint32_t>(p);
+    best = nearer_of_lane_pair<0xB1>(best);
+    best = nearer_of_lane_pair<0x4E>(best);
+    best = nearer_of_lane_pair<0x141>(best);
+    best = nearer_of_lane_pair<0x140>(best);
+    return best;
+}
+
 // TABLE: 0 rounds to an integer grid; kSmallTable rounds to a table of at most sixteen values, kLargeTable to one of
 // at most 256.
 template <int MODE, bool WHOLE, int TABLE = 0>
@@ -397,6 +414,8 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
             const int entry = 16 * i + p;
             table[i] = entry < a.n_values ? a.values[entry < a.n_values ? entry : 0] : __builtin_nanf("");
         }
+    } else if constexpr (TABLE > 0 && WHOLE) {
+        table[0] = p < a.n_values ? a.values[p < a.n_values ? p : 0] : __builtin_nanf("");   // this lane's entry
     } else if constexpr (TABLE > 0) {
 #pragma unroll
         for (int i = 0; i < TABLE; ++i) table[i] = i < a.n_values ? a.values[i < a.n_values ? i : 0] : __builtin_nanf("");
@@ -471,6 +490,10 @@ __global__ void __launch_bounds__(kSweepThreads) narrow_sweep_kernel(const Sweep
             uint32_t index;
             if constexpr (TABLE == kLargeTable) {
                 const Nearest nearest = nearest_over_row(row_value(normalized, owner, row_in_wave), table, p);
+                chosen = nearest.value;
+                index = nearest.index;
+            } else if constexpr (TABLE > 0 && WHOLE) {
+                const Nearest nearest = nearest_one_per_lane(row_value(normalized, owner, row_in_wave), table[0], p);
                 chosen = nearest.value;
                 index = nearest.index;
             } else if constexpr (TABLE > 0) {
