@@ -466,6 +466,7 @@ def other_kernels(device: torch.device, full: bool) -> dict:
     shapes, the tied head and the wider codecs."""
     import mlkit_amd as mk
     from mlkit_amd.kernels import hadamard, packed_linear, scalar_decode, scalar_encode
+    from mlkit_amd.quantization import bitstream
 
     out = {}
     generator = torch.Generator(device=device).manual_seed(1)
@@ -483,7 +484,10 @@ def other_kernels(device: torch.device, full: bool) -> dict:
     out["encode int4 4096x14336 g128"] = _entry(_time(encode), elements * 5 + scales.numel() * 4)
     out["decode codes 4096x14336 g128"] = _entry(
         _time(lambda: scalar_decode.decode(codes, scales, values, None, GROUP)), elements * 5 + scales.numel() * 4)
-    out["pack int4 4096x14336"] = _entry(_time(lambda: mk.pack(codes, 4), repeats=10), elements + elements // 2)
+    # (the range check of the codes is collected in a device flag and read once afterwards, as mk.optimize does)
+    overflow = torch.zeros(1, dtype=torch.int32, device=device)
+    out["pack int4 4096x14336"] = _entry(_time(lambda: mk.pack(codes, 4, overflow=overflow), repeats=10), elements + elements // 2)
+    bitstream.check_overflow(overflow, 4)
     stream = mk.pack(codes, 4)
     out["unpack int4 4096x14336"] = _entry(_time(lambda: mk.unpack(stream, 4, (ROWS, WIDTH)), repeats=10),
                                            elements + elements // 2)
