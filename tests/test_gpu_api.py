@@ -953,3 +953,56 @@ def test_online_rotation_hook_equals_rht(width, dtype):
     batched = torch.randn((2, 3, width), device="cuda", generator=generator).to(dtype)
     assert close(rotation(batched), mk.rht(batched, seed=11))
     assert rotation(batched).shape == batched.shape
+
+
+class GatedBlock(nn.Module):
+    """q / k / v on one input, an output projection, and a gated MLP whose down projection is rotated."""
+
+    def __init__(self, hidden: int = 896, inner: int = 2048) -> None:
+        super().__init__()
+        self.q_proj = nn.Linear(hidden, hidden, bias=True)
+        self.k_proj = nn.Linear(hidden, 128, bias=True)
+        self.v_proj = nn.Linear(hidden, 128, bias=True)
+        self.o_proj = nn.Linear(hidden, hidden, bias=False)
+        self.gate_proj = nn.Linear(hidden, inner, bias=False)
+        self.up_proj = nn.Linear(hidden, inner, bias=False)
+        self.down_proj = nn.Linear(inner, hidden, bias=False)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+        mixed = self.o_proj(q * (k.sum(-1, keepdim=True) + v.mean(-1, keepdim=True)))
+        hidden = x + mixed
+        return hidden + self.down_proj(torch.nn.functional.silu(self.gate_proj(hidden)) * self.up_proj(hidden))
+
+
+@pytest.mark.parametrize("group_siblings", [False, True])
+@pytest.mark.parametrize("rows", [1, 4])
+def test_forward_of_packed_layers_captured_in_a_hip_graph(group_siblings, rows):
+    """Serving code captures a decoder block once and replays it.  A block of seven packed layers (three
+    siblings on one input, gate / up on another, a down projection with an online rotation of 2048 points) is
+    captured with torch.cuda.graph; every replay, with new values in the static input and eager work and
+    synchronisations between the replays, equals the eager forward of the same values bit for bit."""
+    torch.manual_seed(61)
+    module = GatedBlock().half().cuda()
+    mk.rotate(seed=5)(nn.ModuleDict({"down_proj": module.down_proj}))
+    converted = mk.quantize(module, mk.int(4, group=128), calib=None)
+    packed = mk.optimize(converted, backend="packed", group_siblings=group_siblings)
+    block = packed.module
+    assert isinstance(block.down_proj, mk.PackedLinear) and block.down_proj._rotation is not None
+    static = torch.randn(rows, 896, device="cuda").half()
+    with torch.inference_mode():
+        for _ in range(3):   # binds the launch arguments and the rotation buffers before the capture
+            block(static)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = block(static)
+        for trial in range(4):
+            fresh = torch.randn(rows, 896, device="cuda").half() * (1 + trial)
+            static.copy_(fresh)
+            graph.replay()
+            torch.cuda.synchronize()
+            result = captured.clone()
+            eager = block(fresh.clone())     # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(result, eager), (group_siblings, rows, trial)
