@@ -69,10 +69,11 @@ int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packed, const vo
  * either every matrix has offsets or none has.  x, packed, scales, zeros (NULL = none), bias
  * (NULL = none; single entries may be NULL) and y are HOST arrays of `count` device pointers,
  * output_widths a host array of `count` ints; the arrays are read before the call returns.
- * Layouts the streaming and table kernels take (2- to 8-bit codes of any grid, 16-bit
- * activations and scales, input_width a multiple of 32 up to 16384, scale groups of whole
- * multiples of 32 codes) run as ONE launch whose grid covers all the matrices; every other
- * layout runs as `count` launches of mk_packed_matvec.  Results equal
+ * Layouts the streaming and table kernels take (2- to 8-bit codes of any grid with 16-bit
+ * activations and scales, or 4-bit codes of a uniform grid with fp32 activations and scales of
+ * any type; input_width a multiple of 32 up to 16384, scale groups of whole multiples of 32
+ * codes) run as ONE launch whose grid covers all the matrices; every other layout runs as
+ * `count` launches of mk_packed_matvec.  Results equal
  * those of `count` separate calls bit for bit.
  * Replaces: the consecutive launches of kernels/packed_linear.py:181-226 that a model makes
  * for such layers (it calls PackedLinear.forward, inference/packed_linear.py:148-245, once
