@@ -1,6 +1,7 @@
-// 4-bit uniform-grid packed matvec with fp16 or bf16 activations (fp32 ones as pairs of fp16
-// halves, for one or two samples) and 16-bit or fp32 scales: the decode-time kernel for INT4
-// layers whose rows are whole multiples of 32 codes (K = 32 ... 16384).
+// 4-bit uniform-grid packed matvec with fp16 or bf16 activations (codes as fp16 subnormals or with the exponent of
+// 128 inserted, v_dot2; 4 x 4 x 4 matrix-core blocks from three samples on) or fp32 activations (planes of 4-bit
+// digits against v_dot8_i32_i4) and 16-bit or fp32 scales: the decode-time kernel for INT4 layers whose rows are
+// whole multiples of 32 codes (K = 32 ... 16384).
 //
 // The kernel is bound by whichever is larger: the HBM stream of the codes, or the vector
 // ALU time of the busiest SIMD (a wavefront issues one vector instruction per four
@@ -29,7 +30,7 @@ namespace mk_matvec {
 namespace {
 
 // Rows per workgroup: 16 when that still gives every compute unit a workgroup, 4 for
-// layers with fewer rows (more, shorter workgroups).  Up to 8 rows of codes are in flight
+// layers with fewer rows (more, shorter workgroups); 8 for three and more samples on short rows (stream4_launch).  Up to 8 rows of codes are in flight
 // per wavefront (both values swept on the GPU together with 8 / 32 rows and 4 - 16 ahead).
 constexpr int kWideRows = 16, kMidRows = 8, kNarrowRows = 4;
 constexpr int kComputeUnits = 256;
@@ -341,12 +342,10 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         const uint32_t keep = in_row && sample_base + m < a.samples ? 0xffffffffu : 0u;
 #pragma unroll
         for (int i = 0; i < 16; ++i) x[m].r[i] &= keep;
-        float code_free;
+        float code_free;   // what the dot products accumulate for all-zero codes (bf16: the inserted exponent of 128)
         if constexpr (kSubnormalCodes) {
             x_sum[m] = pair_for_subnormal_nibbles(x[m]);
             code_free = 0.0f;
-        } else if constexpr (XT == MK_F16) {
-            code_free = pair_for_nibbles(x[m], &x_sum[m]);
         } else {
             x_sum[m] = pair_for_nibbles_bf16(x[m]);
             code_free = 128.0f * x_sum[m];
@@ -363,7 +362,6 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         float dot[MT];
         if constexpr (SPLIT) chunk_dot_planes<MT>(codes[r], planes, dot);
         else if constexpr (kSubnormalCodes) chunk_dot_subnormal<MT>(codes[r], x, dot);
-        else if constexpr (XT == MK_F16) chunk_dot<4, MK_F16, MT, true>(codes[r], x, nullptr, dot);
         else chunk_dot_bf16<MT>(codes[r], x, dot);
         if (r + kStreamAhead < kStreamRows)
             load_codes<4>(codes[r + kStreamAhead],
