@@ -143,6 +143,17 @@ def timed_graph(launchers, steps, warmup, replays, minimum_span_ms=1.0):
     return statistics.median(samples), min(samples), max(samples), batch
 
 
+def launch_floor(device: torch.device, values: torch.Tensor) -> float:
+    """Seconds per call of the same entry point on a 16 x 32 layer (512 codes: no work to speak of), in the same
+    kind of graph of back-to-back calls: what a dependent launch costs before any weight streams."""
+    packed = torch.zeros(16 * 32 // 2, dtype=torch.uint8, device=device)
+    scales = torch.ones((16, 1), dtype=torch.float16, device=device)
+    x = torch.ones((1, 32), dtype=torch.float16, device=device)
+    y = torch.empty((1, 16), dtype=torch.float16, device=device)
+    tiny = Launcher(x, packed, scales, values, y, rows=16, width=32, group=32)
+    return timed_graph([tiny], 200, 20, 20)[0]
+
+
 def _blas_threads(limit: int | None):
     try:
         import threadpoolctl
@@ -735,6 +746,9 @@ def main() -> None:
                 head_step = (median, low, high, batch, steps, replays)
             del grouped
         results[samples] = row
+    floor = launch_floor(device, values)
+    flat["launch_floor_us"] = floor * 1e6
+    flat["us_M1_above_launch_floor"] = flat["us_M1"] - floor * 1e6
     per_step, low, high, batch, steps, replays = head_step
     achieved = algorithmic_bytes(1) * members / per_step / 1e9
     traffic = RECORDED_TRAFFIC["group_of_8" if members == 8 else "single"] if members in (1, 8) else None
