@@ -507,10 +507,12 @@ def other_kernels(device: torch.device, full: bool) -> dict:
     square = weight[:, :4096].contiguous()
     base, _ = scalar_encode.fit_scales(square, 64, asym=False, reciprocal=1.0, value_minimum=-1.0,
                                        scale_format="fp16", store_zero=False)
-    out["search_scales codebook7 4096x4096 g64, 21 candidates"] = _entry(
-        _time(lambda: scalar_encode.search_scales(square, base, None, seven, fractions, 64, None, "fp16",
-                                                  integer=False, minimum=-1.0, maximum=1.0), repeats=5),
-        4096 * 4096 * 4 + 2 * base.numel() * 4)
+    search_ms = _time(lambda: scalar_encode.search_scales(square, base, None, seven, fractions, 64, None, "fp16",
+                                                          integer=False, minimum=-1.0, maximum=1.0), repeats=5)
+    # bound by vector-ALU work (an IEEE division and a table search per element and candidate), not by HBM
+    out["search_scales codebook7 4096x4096 g64, 21 candidates"] = {
+        "ms": search_ms, "bound": "valu", "bytes": 4096 * 4096 * 4 + 2 * base.numel() * 4,
+        "candidate_elements_per_s": 21 * 4096 * 4096 / (search_ms / 1e3)}
     dense = torch.empty((ROWS, WIDTH), device=device, dtype=torch.float16)
     layout = packed_linear.layout_for(BITS, WIDTH, GROUP)
     half_scales = scales.half()
@@ -815,6 +817,9 @@ def kernel_summary(kernels: dict) -> dict:
             flat[f"frac:{key}"] = entry["hbm_frac"]
         elif isinstance(entry, dict) and "hbm_frac" in entry:
             flat[f"frac:{label.replace(' ', '_')}"] = entry["hbm_frac"]
+    search = kernels.get("search_scales codebook7 4096x4096 g64, 21 candidates")
+    if search:
+        flat["search_scales_ms"] = search["ms"]
     gptq = kernels.get("gptq int4 g128 4096x11008", {})
     if gptq:
         flat["gptq_sweep_and_update_ms"] = gptq["sweep_and_update_ms"]

@@ -300,8 +300,96 @@ __global__ void __launch_bounds__(kThreads) search_kernel(const SearchArgs a) {
     }
 }
 
+// The same sums with four (or two) adjacent partial sums of a group in one lane: a team of LANES / V lanes owns a
+// group, lane q the partial sums 4 q ... 4 q + 3 (elements 4 q ... 4 q + 3, + LANES, + 2 LANES, ...: one vector load
+// each).  The butterfly's first stages (partners 1 and 2 apart) are then additions inside a lane, in the same
+// order, and the rest runs over the team: bit for bit the result of search_kernel<LANES>, with the group's values
+// held in registers across the candidates and a quarter of the exchanges, scale roundings and comparisons per
+// element.  For groups of at most 256 values (at most sixteen registers of them per lane).
+template <int LANES, int V>
+__global__ void __launch_bounds__(kThreads) search_kernel_in_registers(const SearchArgs a) {
+    static_assert(LANES % V == 0 && (V == 4 || V == 2), "two or four partial sums per lane");
+    constexpr int kTeam = LANES / V;
+    constexpr int kMaxTrips = 256 / LANES;   // elements per partial sum
+    __shared__ float table[kMaxTable];
+    __shared__ float fraction[64];
+    if (!a.integer) stage_table(table, a.values, a.n_values);
+    for (int i = threadIdx.x; i < a.n_fractions; i += blockDim.x) fraction[i] = a.fractions[i];
+    __syncthreads();
+    const int steps = bisection_steps(a.n_values);
+    constexpr int kTeams = kThreads / kTeam;
+    const int lane_in_team = threadIdx.x % kTeam;
+    const int trips = a.group / LANES;   // uniform; at most kMaxTrips
+    for (int first = blockIdx.x * kTeams; first < a.total_groups; first += gridDim.x * kTeams) {
+        const int wanted = first + threadIdx.x / kTeam;
+        const int identifier = wanted < a.total_groups ? wanted : a.total_groups - 1;
+        const int row = identifier / a.groups_per_row;
+        const int group_start = (identifier - row * a.groups_per_row) * a.group;
+        const float *row_value = a.value + static_cast<size_t>(row) * a.width;
+        const float base = a.scales[identifier];
+        const float zero = a.zeros ? a.zeros[identifier] : 0.0f;
+        float centered[kMaxTrips][V];
+        bool valid[kMaxTrips][V];
+#pragma unroll
+        for (int k = 0; k < kMaxTrips; ++k)
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                const int column = group_start + k * LANES + lane_in_team * V + v;
+                valid[k][v] = k < trips && column < a.width;
+                centered[k][v] = __fsub_rn(valid[k][v] ? row_value[column] : 0.0f, zero);
+            }
+        auto error_of = [&](float scale) __attribute__((always_inline)) {
+            float partial[V];
+#pragma unroll
+            for (int v = 0; v < V; ++v) partial[v] = 0.0f;
+#pragma unroll
+            for (int k = 0; k < kMaxTrips; ++k) {
+                if (k < trips) {   // uniform
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        const float normalized = __fdiv_rn(centered[k][v], scale);
+                        float rounded;
+                        if (a.integer)
+                            rounded = nearest_integer(normalized, a.minimum, a.maximum);
+                        else
+                            rounded = table[nearest_entry(normalized, table, a.n_values, steps)];
+                        const float difference = valid[k][v] ? __fsub_rn(__fmul_rn(rounded, scale), centered[k][v]) : 0.0f;
+                        partial[v] = __fadd_rn(partial[v], __fmul_rn(difference, difference));
+                    }
+                }
+            }
+            float folded;
+            if constexpr (V == 4)
+                folded = __fadd_rn(__fadd_rn(partial[0], partial[1]), __fadd_rn(partial[2], partial[3]));
+            else
+                folded = __fadd_rn(partial[0], partial[1]);
+            return mk_segment_sum<kTeam>(folded);
+        };
+        float best_scale = base;
+        float best_error = error_of(base);
+        for (int c = 0; c < a.n_fractions; ++c) {
+            const float scale = mk_rounded_scale(__fmul_rn(base, fraction[c]), a.format);
+            const float error = error_of(scale);
+            const bool improved = error < best_error;
+            best_scale = improved ? scale : best_scale;
+            best_error = fminf(best_error, error);
+        }
+        if (lane_in_team == 0 && wanted < a.total_groups) a.selected[identifier] = best_scale;
+    }
+}
+
 template <int LANES>
 void launch_search(const SearchArgs &a, hipStream_t stream) {
+    if constexpr (LANES >= 32) {
+        if (a.group <= 256) {
+            constexpr int kV = LANES == 64 ? 4 : 2;
+            const int teams = kThreads / (LANES / kV);
+            int blocks = mk_cdiv(a.total_groups, teams);
+            if (blocks > 256 * 64) blocks = 256 * 64;
+            hipLaunchKernelGGL((search_kernel_in_registers<LANES, kV>), dim3(blocks), dim3(kThreads), 0, stream, a);
+            return;
+        }
+    }
     const int teams = kThreads / LANES;
     int blocks = mk_cdiv(a.total_groups, teams);
     if (blocks > 256 * 64) blocks = 256 * 64;
