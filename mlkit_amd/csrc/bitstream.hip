@@ -169,6 +169,44 @@ __global__ void __launch_bounds__(256) unpack_kernel(const StreamArgs a_) {
         const long long source_byte = run * (4 * a.bits);
         const uint8_t *source = a.stream + source_byte;
         const int left = run < whole_runs ? kRun : static_cast<int>(a.count - first);
+        if constexpr (BITS != 0 && ALIGNED && !WIDE_CODES) {
+            // A whole run of a known width onto an aligned target: the run's BITS dwords in one go, every code by a
+            // constant shift, two 16-byte stores.
+            uint8_t *target = static_cast<uint8_t *>(a.codes_out) + first;
+            if (run < whole_runs && (reinterpret_cast<uintptr_t>(target) & 3u) == 0) {
+                uint32_t words[BITS];
+                typedef uint32_t chunk __attribute__((ext_vector_type(BITS == 3 ? 3 : (BITS >= 4 ? 4 : BITS)), aligned(4)));
+                if constexpr (BITS <= 4) {
+                    const chunk loaded = *reinterpret_cast<const chunk *>(source);
+#pragma unroll
+                    for (int w = 0; w < BITS; ++w) words[w] = loaded[w];
+                } else {
+#pragma unroll
+                    for (int q = 0; q < BITS / 4; ++q) {
+                        const chunk loaded = reinterpret_cast<const chunk *>(source)[q];
+#pragma unroll
+                        for (int w = 0; w < 4; ++w) words[4 * q + w] = loaded[w];
+                    }
+                }
+                uint32_t packed[kRun / 4];
+#pragma unroll
+                for (int q = 0; q < kRun / 4; ++q) {
+                    packed[q] = 0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        constexpr uint32_t kMask = (1u << BITS) - 1u;
+                        const int position = (4 * q + j) * BITS, index = position >> 5, shift = position & 31;
+                        uint32_t code = words[index] >> shift;
+                        if (shift + BITS > 32) code |= words[(index + 1) % BITS] << (32 - shift);
+                        packed[q] |= (code & kMask) << (8 * j);
+                    }
+                }
+                typedef uint32_t u4 __attribute__((ext_vector_type(4), aligned(4)));
+                reinterpret_cast<u4 *>(target)[0] = u4{packed[0], packed[1], packed[2], packed[3]};
+                reinterpret_cast<u4 *>(target)[1] = u4{packed[4], packed[5], packed[6], packed[7]};
+                continue;
+            }
+        }
         uint64_t window = 0;
         int filled = 0, word = 0;
         uint32_t out[kRun];
