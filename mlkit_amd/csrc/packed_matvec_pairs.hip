@@ -43,9 +43,9 @@ __device__ __forceinline__ float side_value(uint16_t raw, int dtype) {
 // (two per CU at 4096 rows); short rows keep sixteen rows per table fill.
 constexpr int kShortTileRows = 8;
 constexpr int kShortTileWidth = 4096;
-// Uniform 2- and 3-bit grids with fp16 activations, one or two samples: decoded by shifts and masks.
+// Uniform 2-, 3- and 8-bit grids with fp16 activations, one or two samples: decoded by shifts and masks.
 inline bool shifted_decoding(const Stream4Args &a) {
-    return a.uniform && a.x_dtype == MK_F16 && (a.bits == 2 || a.bits == 3) && a.samples <= 2;
+    return a.uniform && a.x_dtype == MK_F16 && (a.bits == 2 || a.bits == 3 || a.bits == 8) && a.samples <= 2;
 }
 
 // (Without lookups to wait on, sixteen rows per workgroup measure faster: 5.8 against 6.0 us for two bits, 6.5
@@ -161,6 +161,18 @@ struct ShiftedPlan<3> {
     static constexpr bool halve_low = true;
 };
 
+// Eight bits: a byte left in the low byte of a half word is the subnormal c * 2^-24 as it stands (eight of the ten
+// mantissa bits).  A word holds codes 4 j ... 4 j + 3; the word and the word shifted by 8, each masked with
+// 0x00ff00ff, are the pairs (4 j, 4 j + 2) and (4 j + 1, 4 j + 3): one shift, two ANDs and two v_dot2 per four codes,
+// one class.
+template <>
+struct ShiftedPlan<8> {
+    static constexpr int kPairs = 16, kClasses = 2;   // (two sums only to shorten the dependent chains)
+    static constexpr int low_code(int pair) { return 4 * (pair / 2) + (pair % 2); }
+    static constexpr int high_code(int pair) { return low_code(pair) + 2; }
+    static constexpr bool halve_low = false;
+};
+
 // The activations of a chunk as the pairs of the plan, from their natural order (x.r[k] = elements 2 k, 2 k + 1).
 template <int BITS>
 __device__ __forceinline__ void pair_for_shifted_codes(const XChunk<MK_F16> &x, uint32_t (&pairs)[ShiftedPlan<BITS>::kPairs]) {
@@ -196,7 +208,16 @@ __device__ __forceinline__ void shifted_chunk_dot(const CodeChunk<BITS> &codes, 
         for (int m = 0; m < MT; ++m)
             sums[cls][m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(mk_h2, fields), __builtin_bit_cast(mk_h2, pairs[m][pair]), sums[cls][m], false);
     };
-    if constexpr (BITS == 2) {
+    if constexpr (BITS == 8) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t word = codes.w[j];
+            add(0, word & 0x00ff00ffu, 2 * j);
+            add(1, (word >> 8) & 0x00ff00ffu, 2 * j + 1);
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) dot[m] = sums[0][m] + sums[1][m];
+    } else if constexpr (BITS == 2) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const uint32_t word = codes.w[j], shifted = word >> 8;
@@ -238,7 +259,7 @@ __device__ __forceinline__ void shifted_chunk_dot(const CodeChunk<BITS> &codes, 
 // SHIFTED: a uniform 2- or 3-bit grid with fp16 activations, decoded by shifts and masks (no table).
 template <int BITS, int MT, bool HAS_ZERO, int XT, int LOOKUP, int ROWS, bool SHIFTED = false>
 __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const Stream4Group members) {
-    static_assert(!SHIFTED || ((BITS == 2 || BITS == 3) && XT == MK_F16), "shifted decoding: 2 or 3 bits, fp16 activations");
+    static_assert(!SHIFTED || ((BITS == 2 || BITS == 3 || BITS == 8) && XT == MK_F16), "shifted decoding: 2, 3 or 8 bits, fp16 activations");
     constexpr int kLookup = LOOKUP;
     constexpr int kPairRows = ROWS;
     constexpr int kPairAhead = rows_in_flight<BITS>();
@@ -307,7 +328,7 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const S
     }
     // shifted decoding: the activations as the plan's pairs; the affine map of the grid applies to a chunk's sum:
     // sum (min + step c) x = (step 2^24) (2^-24 sum c x) + min sum x
-    constexpr int kPlanPairs = SHIFTED ? ShiftedPlan<SHIFTED ? BITS : 2>::kPairs : 1;
+    constexpr int kPlanPairs = SHIFTED ? ShiftedPlan<SHIFTED ? BITS : 2>::kPairs : 1;   // (BITS has a plan whenever SHIFTED)
     uint32_t shifted_pairs[MT][kPlanPairs];
     float grid_term[MT];
     if constexpr (SHIFTED) {
@@ -647,7 +668,7 @@ template <int BITS, int MT, int XT, int LOOKUP>
 void launch_tile_with(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1);
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
-    if constexpr ((BITS == 2 || BITS == 3) && XT == MK_F16 && MT <= 2) {
+    if constexpr ((BITS == 2 || BITS == 3 || BITS == 8) && XT == MK_F16 && MT <= 2) {
         if (shifted_decoding(a)) {
             if (a.zeros) {
                 hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP, kPairRows, true>), grid, block, 0, stream, a, members);
