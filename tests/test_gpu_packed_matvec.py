@@ -74,6 +74,13 @@ def test_config2_tied_output_head():
     for samples in (1, 2, 4, 8):
         x = helpers.activations(samples, 896, seed=6 + samples)
         check(run_matvec(layer, x), layer, x)
+    # fp32 activations on the same layer: 9496 tiles of rows, more than the GPU holds workgroups, so a workgroup
+    # prepares its digit planes once and walks several tiles with them
+    for samples in (1, 2, 3):
+        x = helpers.activations(samples, 896, seed=16 + samples, dtype=torch.float32)
+        y = run_matvec(layer, x, scale_dtype=torch.float16)
+        reference = oracle_matvec.reconstruct_then_matmul_f64(x.double().numpy(), layer["dense"], None)
+        np.testing.assert_allclose(y, reference, rtol=1e-4, atol=1e-5)
 
 
 CODECS = {
