@@ -440,14 +440,18 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const S
 // t's activations for chunk b in their natural order.  A wavefront owns 2048 codes of K as
 // four sub-slices of sixteen chunks; the four row sums of a result lane take their scales
 // from the four lanes of its quad.
-template <int BITS, int SETS, bool HAS_ZERO, int XT, int LOOKUP, int SLICES>
+// SHIFTED (uniform 8-bit grids, fp16 activations): no table; a word and the word shifted by 8, each masked with
+// 0x00ff00ff, are the four codes of one instruction as fp16 subnormals (in the order 0, 2, 1, 3, which the
+// activations are permuted to once per tile), and the grid's affine map applies to the block's sums.
+template <int BITS, int SETS, bool HAS_ZERO, int XT, int LOOKUP, int SLICES, bool SHIFTED = false>
 __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, const Stream4Group members) {
+    static_assert(!SHIFTED || (BITS == 8 && XT == MK_F16), "shifted decoding on the matrix cores: 8 bits, fp16 activations");
     constexpr int kQuads = kPairRows / 4;
     constexpr int kSlices = SLICES;  // sub-slices of sixteen chunks per wavefront (rows of up to 512 / 1024 codes: 1 / 2)
     constexpr int kSteps = kQuads * kSlices;
     constexpr int kAhead = rows_in_flight<BITS>() < kSteps ? rows_in_flight<BITS>() : kSteps;
     constexpr int kEntries = 1 << (LOOKUP * BITS);
-    constexpr int kTableWords = kEntries * LOOKUP / 2;
+    constexpr int kTableWords = SHIFTED ? 2 : kEntries * LOOKUP / 2;
     __shared__ __attribute__((aligned(8))) uint32_t table[kTableWords];
     __shared__ float partials[SETS * kPairRows * 4 * 8];  // [set][row][sample in set][wavefront]
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
@@ -469,7 +473,7 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
     const uint8_t *scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
     const uint8_t *zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
 
-    fill_table<BITS, LOOKUP, XT>(table, a);
+    if constexpr (!SHIFTED) fill_table<BITS, LOOKUP, XT>(table, a);
 
     // Chunks past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
     // activations: they add nothing.
@@ -539,9 +543,18 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
 #pragma unroll
                 for (int i = 0; i < 16; ++i) x[set][s].r[i] &= keep;
             }
-            x_sum[set][s] = HAS_ZERO ? chunk_sum<XT>(x[set][s]) : 0.0f;
+            x_sum[set][s] = HAS_ZERO || SHIFTED ? chunk_sum<XT>(x[set][s]) : 0.0f;
+            if constexpr (SHIFTED) {   // (x0,x1)(x2,x3) -> (x0,x2)(x1,x3) for every four values
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t p0 = x[set][s].r[2 * i], p1 = x[set][s].r[2 * i + 1];
+                    x[set][s].r[2 * i] = __builtin_amdgcn_perm(p1, p0, 0x05040100u);
+                    x[set][s].r[2 * i + 1] = __builtin_amdgcn_perm(p1, p0, 0x07060302u);
+                }
+            }
         }
     }
+    const float shifted_step = a.grid_step * 16777216.0f;   // the subnormal codes are c * 2^-24
 
     float sums[SETS][kPairRows];
 #pragma unroll
@@ -578,13 +591,28 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
             }
         }
     };
-    look_up(0, looked_up_next);
+    if constexpr (!SHIFTED) look_up(0, looked_up_next);
 #pragma unroll
     for (int step = 0; step < kSteps; ++step) {
         const int q = step / kSlices, s = step % kSlices;
         mk_f4 dot[SETS];
 #pragma unroll
         for (int set = 0; set < SETS; ++set) dot[set] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (SHIFTED) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t word = codes[step].w[i];
+                const uint32_t low = word & 0x00ff00ffu, high = (word >> 8) & 0x00ff00ffu;
+#pragma unroll
+                for (int set = 0; set < SETS; ++set)
+                    dot[set] = blocks(low, high, x[set][s].r[2 * i], x[set][s].r[2 * i + 1], dot[set]);
+            }
+#pragma unroll
+            for (int set = 0; set < SETS; ++set)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    dot[set][r] = __builtin_fmaf(shifted_step, dot[set][r], a.grid_min * x_sum[set][s]);
+        } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) looked_up[i][0] = looked_up_next[i][0], looked_up[i][1] = looked_up_next[i][1];
         if (step + 1 < kSteps) look_up(step + 1, looked_up_next);
@@ -594,6 +622,7 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
 #pragma unroll
             for (int set = 0; set < SETS; ++set)
                 dot[set] = blocks(looked_up[i][0], looked_up[i][1], x[set][s].r[2 * i], x[set][s].r[2 * i + 1], dot[set]);
+        }
         if (step + kAhead < kSteps)
             load_codes<BITS>(codes[step + kAhead], codes_base + static_cast<size_t>(4 * ((step + kAhead) / kSlices)) * row_bytes +
                                                        code_offset[(step + kAhead) % kSlices]);
@@ -653,6 +682,13 @@ void launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int
         }
         hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
     };
+    if constexpr (BITS == 8 && XT == MK_F16) {
+        if (a.uniform) {   // no table: the bytes as fp16 subnormals
+            if (a.zeros) launch(pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP, SLICES, true>);
+            else launch(pairs_blocks_kernel<BITS, SETS, false, XT, LOOKUP, SLICES, true>);
+            return;
+        }
+    }
     if (a.zeros) launch(pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP, SLICES>);
     else launch(pairs_blocks_kernel<BITS, SETS, false, XT, LOOKUP, SLICES>);
 }
