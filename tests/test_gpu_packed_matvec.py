@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import matvec as oracle_matvec, scaling
+from oracle import bitstream as oracle_bitstream, matvec as oracle_matvec, scaling
 
 import helpers
 
@@ -685,3 +685,19 @@ def test_fp32_activations_that_are_not_finite_stay_so():
             y = run_matvec(layer, x, None, scale_dtype=torch.float16)
             assert not np.isfinite(y[0]).any()
             np.testing.assert_array_equal(y[1:], clean[1:])
+
+
+def test_fp32_activations_with_bf16_scales():
+    """fp32 activations against bf16 scales and offsets (the digit-plane kernel converts the sides itself): against
+    the float64 product of the weights that those rounded scales and offsets give."""
+    rows, width, group = 80, 4096, 128
+    weight = helpers.normal_weight(rows, width, seed=21)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=group, integer=True, asym=True)
+    scales = torch.from_numpy(layer["scales"]).bfloat16().double().numpy()
+    zeros = torch.from_numpy(layer["zero"]).bfloat16().double().numpy()
+    codes = oracle_bitstream.unpack(layer["packed"], 4, layer["shape"]).astype(np.float64)
+    dense = (codes + float(layer["values"][0])) * np.repeat(scales, group, axis=1) + np.repeat(zeros, group, axis=1)
+    for samples in (1, 2, 4):
+        x = helpers.activations(samples, width, seed=22 + samples, dtype=torch.float32)
+        y = run_matvec(layer, x, scale_dtype=torch.bfloat16)
+        np.testing.assert_allclose(y, x.double().numpy() @ dense.T, rtol=1e-4, atol=1e-5)
