@@ -701,3 +701,38 @@ def test_fp32_activations_with_bf16_scales():
         x = helpers.activations(samples, width, seed=22 + samples, dtype=torch.float32)
         y = run_matvec(layer, x, scale_dtype=torch.bfloat16)
         np.testing.assert_allclose(y, x.double().numpy() @ dense.T, rtol=1e-4, atol=1e-5)
+
+
+SWEEP_CODECS = [
+    (scaling.int_values(4), 4, True), (scaling.int_values(2), 2, True), (scaling.int_values(3), 3, True),
+    (scaling.int_values(8), 8, True), (scaling.NF4_VALUES, 4, False),
+    (np.array([-1, -.5, -.25, 0, .25, .5, 1], dtype=np.float32), 3, False), (scaling.int_values(5), 5, True),
+    (scaling.int_values(6), 6, True),
+]
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_layouts_against_the_oracle(seed):
+    """Forty layers per seed drawn over the codecs, row lengths (32 ... 16384), scale groups, row counts (ragged
+    tiles, short and tall matrices), offsets, bias, the three activation types and one to nine samples: every kernel
+    the dispatch can choose, against the float64 product at the tolerance of the activation type."""
+    rng = np.random.default_rng(seed)
+    for trial in range(40):
+        values, bits, integer = SWEEP_CODECS[rng.integers(len(SWEEP_CODECS))]
+        width = int(rng.choice([32, 64, 96, 256, 512, 896, 1024, 1536, 2048, 2080, 3072, 4096, 4864, 6144, 8192, 11008, 14336, 16384]))
+        group = int(rng.choice([g for g in (32, 64, 128, 256) if width % g == 0] + [width]))
+        tall = [1, 3, 16, 37, 64, 130, 260, 1024, 4096 + 5, 4100, 6144, 9000]
+        rows = int(rng.choice(tall)) if width <= 4096 else int(rng.choice([3, 16, 40, 4096 + 7]))
+        asym, with_bias = bool(rng.integers(2)), bool(rng.integers(2))
+        dtype = [torch.float16, torch.bfloat16, torch.float32][rng.integers(3)]
+        samples = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9]))
+        weight = helpers.normal_weight(rows, width, seed=100 * seed + trial)
+        layer = helpers.quantised_layer(weight, values, bits=bits, group=group, integer=integer, asym=asym)
+        x = helpers.activations(samples, width, seed=1000 + trial, dtype=dtype)
+        bias = helpers.activations(1, rows, seed=5, dtype=dtype)[0] if with_bias else None
+        y = run_matvec(layer, x, bias)
+        reference = oracle_matvec.reconstruct_then_matmul_f64(
+            x.double().numpy(), layer["dense"], None if bias is None else bias.double().numpy())
+        tolerance = {torch.float16: 1e-3, torch.bfloat16: 8e-3, torch.float32: 2e-5}[dtype]
+        error = np.abs(y - reference).max() / max(np.abs(reference).max(), 1e-30)
+        assert error <= tolerance, (trial, bits, integer, rows, width, group, asym, with_bias, dtype, samples, error)
