@@ -1006,3 +1006,42 @@ def test_forward_of_packed_layers_captured_in_a_hip_graph(group_siblings, rows):
             eager = block(fresh.clone())     # eager work between the replays
             torch.cuda.synchronize()
             assert torch.equal(result, eager), (group_siblings, rows, trial)
+
+
+SWEEP_TABLES = [
+    (scaling.int_values(4), True), (scaling.int_values(3), True), (scaling.int_values(8), True), (scaling.NF4_VALUES, False),
+    (np.array([-1, -.5, -.25, 0, .25, .5, 1], dtype=np.float32), False), ((np.linspace(-1, 1, 40) ** 3).astype(np.float32), False),
+    (np.sinh(np.linspace(-3, 3, 256)).astype(np.float32), False), (np.linspace(-1, 1, 17).astype(np.float32), False),
+    (np.tanh(np.linspace(-2, 2, 100)).astype(np.float32), False),
+]
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_gptq_configurations_match_the_oracle_sweep(seed):
+    """Twenty-five configurations per seed drawn over grids and tables (7 to 256 values), scale groups, block and
+    refit widths (regions that are and are not whole 128-column tiles), offsets, row counts and widths: every sweep
+    kernel the dispatch can choose; codes, scales and reconstruction equal the oracle's bit for bit."""
+    rng = np.random.default_rng(seed)
+    for trial in range(25):
+        values, integer = SWEEP_TABLES[rng.integers(len(SWEEP_TABLES))]
+        width = int(rng.choice([256, 384, 512, 640, 1024]))
+        rows = int(rng.choice([5, 64, 80, 130]))
+        group = int(rng.choice([g for g in (16, 32, 64, 128) if width % g == 0]))
+        block = int(rng.choice([64, 96, 128, 256]))
+        refit = [None, block, 2 * block, 128][rng.integers(4)]
+        asym = bool(rng.integers(2))
+        weight = helpers.normal_weight(rows, width, seed=100 * seed + trial)
+        inputs = rng.standard_normal((3 * width, width)).astype(F32)
+        inputs[:, ::9] *= 5
+        hessian = (inputs.T @ inputs / (3 * width)).astype(F32)
+        bits = int(np.log2(len(values))) if integer else max(4, int(np.ceil(np.log2(len(values)))))
+        grid = mk.grid.int(bits) if integer else mk.grid.values(values, bits=bits)
+        quantizer = mk.gptq(mk.scaled(grid, group=group, asym=asym), refit=refit, block_size=block)
+        result = quantizer(dev(weight), Ctx("layer", H=dev(hessian)))
+        coeff = host(mk.feedback_coefficients(dev(hessian).clone(), 1)[0])
+        expected = oracle_feedback.sweep(weight, coeff, values, group=group, integer=integer, refit=refit, block=block,
+                                         asym=asym, dead=np.diag(hessian) == 0, update_mode=0)
+        case = (trial, len(values), integer, rows, width, group, block, refit, asym)
+        np.testing.assert_array_equal(host(result.params["scales"]), expected["scales"], err_msg=str(case))
+        np.testing.assert_array_equal(host(result.codes), expected["codes"], err_msg=str(case))
+        np.testing.assert_array_equal(host(result.w), expected["w"], err_msg=str(case))
