@@ -21,6 +21,8 @@
 #pragma once
 #include <cstddef>
 
+#include <atomic>
+
 #include "mk_common.h"
 
 namespace mk_matvec {
@@ -133,6 +135,23 @@ __device__ __forceinline__ TileSource tile_source(const Stream4Args &a, const St
     return s;
 }
 
+// The number of workgroups of `kernel` the GPU holds at once, asked of the runtime the first
+// time and remembered per kernel (`known`).
+template <typename Kernel>
+inline int resident_workgroups(Kernel kernel, int threads, size_t dynamic_lds, std::atomic<int> &known) {
+    int value = known.load(std::memory_order_relaxed);
+    if (value == 0) {  // two threads asking at once both get the same answer
+        int per_cu = 0, device = 0, units = 256;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess || per_cu < 1)
+            per_cu = 4;
+        if (hipGetDevice(&device) == hipSuccess)
+            (void)hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device);
+        value = per_cu * units;
+        known.store(value, std::memory_order_relaxed);
+    }
+    return value;
+}
+
 // Pair-table kernel (packed_matvec_pairs.hip): 2-, 3- and 4-bit codes of any scalar grid.
 bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype);
 int pairs_launch(const Stream4Args &a, hipStream_t stream);
@@ -140,6 +159,10 @@ int pairs_launch_group(const Stream4Args &shared, Stream4Group &group, const int
                        hipStream_t stream);
 bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
+// Three to eight samples of fp32 activations against 4-bit uniform-grid codes as integer matrix-core blocks
+// (packed_matvec_digits.hip): `tiles` tiles of `rows_per_tile` rows of the single matrix or of every member.
+bool digits_accepts(const Stream4Args &a, int rows_per_tile);
+int digits_launch(const Stream4Args &a, const Stream4Group &members, int tiles, int rows_per_tile, hipStream_t stream);
 // One sample of fp16 activations, a row of whole 2048-code slices made of power-of-two blocks
 // (one block: a power-of-two row) and whole tiles of rows only: the kernel rotates the
 // activations itself (see Stream4Args).  Returns 0 when

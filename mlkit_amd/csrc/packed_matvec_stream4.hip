@@ -674,23 +674,6 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
     } while (true);
 }
 
-// The number of workgroups of `kernel` the GPU holds at once, asked of the runtime the first
-// time and remembered per kernel (`known`).
-template <typename Kernel>
-int resident_workgroups(Kernel kernel, int threads, size_t dynamic_lds, std::atomic<int> &known) {
-    int value = known.load(std::memory_order_relaxed);
-    if (value == 0) {  // two threads asking at once both get the same answer
-        int per_cu = 0, device = 0, units = 256;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess || per_cu < 1)
-            per_cu = 4;
-        if (hipGetDevice(&device) == hipSuccess)
-            (void)hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device);
-        value = per_cu * units;
-        known.store(value, std::memory_order_relaxed);
-    }
-    return value;
-}
-
 template <int SETS, int ROWS, int SLICES>
 int launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
@@ -798,8 +781,12 @@ int launch_rows(const Stream4Args &a, const Stream4Group &members, int tiles, hi
     // One or two samples: v_dot2 kernel.  Three and more: matrix-core blocks (measured at
     // 4096 x 14336: 9.5 against 10.8 us for four samples, 13.3 against 17.6 us for eight).
     if (a.samples >= 3) {
-        // fp32 activations: four samples' digit planes per lane, samples 5 - 8 in a second pass over the codes
-        if (a.x_dtype == MK_F32) return launch_tile<4, ROWS>(a, members, tiles, stream);
+        // fp32 activations: four samples' planes per lane, samples 5 - 8 in a second pass over the codes; rows of
+        // more than 1024 codes as byte planes on the matrix cores, shorter ones as 4-bit planes against v_dot8
+        if (a.x_dtype == MK_F32) {
+            if (digits_accepts(a, ROWS)) return digits_launch(a, members, tiles, ROWS, stream);
+            return launch_tile<4, ROWS>(a, members, tiles, stream);
+        }
         if (a.samples <= 4) return launch_blocks<1, ROWS>(a, members, tiles, stream);
         return launch_blocks<2, ROWS>(a, members, tiles, stream);
     }

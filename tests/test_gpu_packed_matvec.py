@@ -641,7 +641,8 @@ def test_small_and_large_activations_keep_the_tolerance():
 def test_fp32_activations_on_the_streaming_kernel(rows, width, group, asym, with_bias, scale_format):
     """INT4 with fp32 activations, one to eight samples (what the reference's own matvec tests run,
     tests/inference/test_packed_linear.py:91-98): chunks of 32 activations are scaled by a power of two, rounded
-    to 22-bit integers and multiplied with the codes exactly, as planes of 4-bit digits.  Against the float64
+    to 22-bit integers and multiplied with the codes exactly, as planes of 4-bit digits (v_dot8_i32_i4) or, from
+    three samples and 1025 codes a row on, of bytes (integer matrix-core blocks).  Against the float64
     product within 1.5e-7 of sum |w| |x| (an fp32 dot product of these lengths measures 2e-8 to 4.5e-8 of it on the
     CPU, this path 1.5e-8 to 8.5e-8), and against the oracle's fp32 reconstruct-then-matmul at the reference's own
     bound (rtol 1e-4, atol 1e-5); with fp32 and with fp16 scales; activations spanning sixty
@@ -670,6 +671,24 @@ def test_fp32_activations_on_the_streaming_kernel(rows, width, group, asym, with
                     x.numpy(), layer["packed"], 4, layer["shape"], layer["scales"], layer["values"], group, layer["zero"],
                     None if bias is None else bias.numpy())
                 np.testing.assert_allclose(y, fp32_reference, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("scale_format", ["fp32", "fp16"])
+def test_fp32_activations_on_layers_taller_than_the_gpu_holds_workgroups(scale_format):
+    """Five to eight fp32 samples of a layer with more tiles of sixteen rows, times two passes of four samples, than
+    the GPU holds workgroups at once: every workgroup of the matrix-core kernel prepares its activations once and
+    walks several tiles.  With offsets and bias, against the float64 product at the bound of the test above."""
+    rows, width, group = 8192 + 16 + 3, 8192, 128
+    weight = helpers.normal_weight(rows, width, seed=31)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=group, integer=True, asym=True, fmt=scale_format)
+    bias = helpers.activations(1, rows, seed=9, dtype=torch.float32)[0]
+    for samples in (5, 8):
+        x = helpers.activations(samples, width, seed=80 + samples, dtype=torch.float32)
+        y = run_matvec(layer, x, bias, scale_dtype=torch.float32 if scale_format == "fp32" else torch.float16)
+        reference = oracle_matvec.reconstruct_then_matmul_f64(x.double().numpy(), layer["dense"], bias.double().numpy())
+        budget = 1.5e-7 * (np.abs(x.double().numpy()) @ np.abs(layer["dense"]).T.astype(np.float64)) + 1e-7 * np.abs(reference) + 1e-30
+        worst = float((np.abs(y - reference) / budget).max())
+        assert worst <= 1.0, (samples, worst)
 
 
 def test_fp32_activations_that_are_not_finite_stay_so():
