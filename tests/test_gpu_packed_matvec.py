@@ -445,6 +445,23 @@ def test_grouped_launch_with_fp32_activations():
             np.testing.assert_allclose(grouped[0].cpu().numpy(), reference, rtol=1e-4, atol=1e-5)
 
 
+def test_grouped_launch_of_tall_members_with_fp32_activations():
+    """Four tall members and eight fp32 samples: more (tile, pass, member) units than the GPU holds workgroups, so
+    the workgroups of the matrix-core kernel walk their member's tiles; members of different heights (one ends
+    inside a tile), offsets and bias.  Equal to the separate launches bit for bit."""
+    width, group = 2048, 128
+    heights = (8192, 4096 + 16 + 5, 6144, 8192 + 16)
+    layers = [helpers.quantised_layer(helpers.normal_weight(n, width, seed=91 + i), INT4, bits=4, group=group,
+                                      integer=True, asym=True, fmt="fp32") for i, n in enumerate(heights)]
+    for samples in (4, 8):
+        x = helpers.activations(samples, width, seed=92 + samples, dtype=torch.float32)
+        grouped = run_group(layers, x, scale_dtype=torch.float32)
+        for index, layer in enumerate(layers):
+            assert np.array_equal(grouped[index].cpu().numpy(), run_matvec(layer, x, scale_dtype=torch.float32)), (samples, index)
+        reference = oracle_matvec.reconstruct_then_matmul_f64(x.double().numpy(), layers[1]["dense"], None)
+        np.testing.assert_allclose(grouped[1].cpu().numpy(), reference, rtol=1e-4, atol=1e-5)
+
+
 def test_grouped_launch_validation():
     from mlkit_amd import native
 
