@@ -176,10 +176,7 @@ __global__ void __launch_bounds__(512) digits_blocks_kernel(const Stream4Args a,
             wave_exchange_fence();
             if (t == j) {
 #pragma unroll
-                for (int s = 0; s < kSlices; ++s) {
-                    const uint32_t keep = in_row[s] && sample_base + j < a.samples ? 0xffffffffu : 0u;
-                    planes_from_slice(planes[s], unscale[s], x_sum[s], x_slice, s * 16 + block, keep);
-                }
+                for (int s = 0; s < kSlices; ++s) planes_from_slice(planes[s], unscale[s], x_sum[s], x_slice, s * 16 + block, 0xffffffffu);
             }
             wave_exchange_fence();   // the next sample's planes go to the same buffer
         };
@@ -193,8 +190,19 @@ __global__ void __launch_bounds__(512) digits_blocks_kernel(const Stream4Args a,
         place_sample(2, even_pieces);
         place_sample(3, odd_pieces);
     }
+    // Chunks past the end of the row and samples past the last add nothing.
+    const bool sample_present = static_cast<int>(blockIdx.y) * 4 + t < a.samples;
 #pragma unroll
-    for (int s = 0; s < kSlices; ++s) grid_term[s] = a.grid_min * x_sum[s];
+    for (int s = 0; s < kSlices; ++s) {
+        const bool kept = in_row[s] && sample_present;
+        if (__builtin_amdgcn_ballot_w64(!kept) != 0) {  // uniform; rarely taken
+            const uint32_t keep = kept ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int i = 0; i < 4 * kBytePlanes; ++i) planes[s][i] &= keep;
+            x_sum[s] = kept ? x_sum[s] : 0.0f;
+        }
+        grid_term[s] = a.grid_min * x_sum[s];
+    }
 
     while (true) {
     float sums[kSums];
