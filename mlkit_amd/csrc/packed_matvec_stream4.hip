@@ -819,6 +819,20 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream) {
             const int tiles = a.rows / kMidRows;
             return launch_rows<kMidRows>(a, none, tiles, stream) ? -1 : tiles * kMidRows;
         }
+        // One and two samples: with at most two sixteen-row tiles per compute unit the SIMDs hold one wavefront or
+        // none; tiles of eight rows double the wavefronts in flight (8192 x 4096: 6.2 -> 5.2 us at one sample, 7.3 ->
+        // 5.8 at two; 5120 x 5120: 5.8 -> 5.3, 7.4 -> 6.5; 8192 x 2048: 4.3 -> 4.0, 5.1 -> 4.4).  Measured no faster
+        // or slower: exactly one tile per compute unit of rows over 2048 codes (4096 x 4096: 4.3 -> 4.4), rows of
+        // four and more wavefronts (8192 x 8192: 7.5 -> 8.0), more than 512 tiles (12288 x 4096: 6.7 -> 6.9).
+        {
+            const int wide_tiles = a.rows / kWideRows, row_waves = mk_cdiv(a.width, 2048);
+            const bool few_waves = row_waves == 1 ? wide_tiles <= 2 * kComputeUnits
+                                                  : row_waves <= 3 && wide_tiles > kComputeUnits && wide_tiles <= 2 * kComputeUnits;
+            if (a.samples <= 2 && a.x_dtype != MK_F32 && few_waves) {
+                const int tiles = a.rows / kMidRows;
+                return launch_rows<kMidRows>(a, none, tiles, stream) ? -1 : tiles * kMidRows;
+            }
+        }
         const int tiles = a.rows / kWideRows;
         return launch_rows<kWideRows>(a, none, tiles, stream) ? -1 : tiles * kWideRows;
     }
