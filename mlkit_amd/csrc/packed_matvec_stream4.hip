@@ -432,7 +432,8 @@ __global__ void __launch_bounds__(512) stream4_rotating_kernel(const Stream4Args
 // sit in the four lanes of its quad (each loaded by the lane that loads that row's codes)
 // and reach the multiply as DPP quad broadcasts.
 
-template <int SETS, bool HAS_ZERO, int ROWS, int XT, int SLICES>
+// WALK: long rows too take every gridDim.x-th tile (launched with as many workgroups as the GPU holds at once).
+template <int SETS, bool HAS_ZERO, int ROWS, int XT, int SLICES, bool WALK = false>
 __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a, const Stream4Group members) {
     // Short rows (one or two sub-slices per wavefront) leave registers for the tile loop below.
     constexpr bool kStrided = SLICES <= 2;
@@ -667,14 +668,15 @@ __global__ void __launch_bounds__(512) stream4_blocks_kernel(const Stream4Args a
             store_output<XT>(source.y, static_cast<size_t>(sample) * source.rows + row, total);
         }
     }
-    if constexpr (!kStrided) break;
+    if constexpr (!kStrided && !WALK) break;
     tile += gridDim.x;
     if (tile >= source.tiles) break;
     __syncthreads();  // `partials` is reused by the next tile
+    if constexpr (!kStrided) request_tile(tile);
     } while (true);
 }
 
-template <int SETS, int ROWS, int SLICES>
+template <int SETS, int ROWS, int SLICES, bool WALK = false>
 int launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
     // at most 8 wavefronts x 4 samples x 4112 bytes = 129 KB of the CU's 160 KB
@@ -690,22 +692,28 @@ int launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int 
                 return -1;
             allowed.store(slices, std::memory_order_relaxed);
         }
-        if constexpr (SLICES <= 2) {
+        if constexpr (SLICES <= 2 || WALK) {
             // Short rows: as many workgroups as the GPU holds at once; each walks the tiles
             // with that stride.  (Asked of the runtime once per kernel and workgroup size.)
-            static std::atomic<int> resident[3];
+            static std::atomic<int> resident[9];
             const int known = resident_workgroups(kernel, static_cast<int>(block.x), slices, resident[block.x / 64]);
             if (grid.x * grid.z > static_cast<unsigned>(known)) grid.x = mk_cdiv(known, static_cast<int>(grid.z));
         }
         hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
         return 0;
     };
-    if (a.x_dtype == MK_F16) {
-        if (a.zeros) return launch(stream4_blocks_kernel<SETS, true, ROWS, MK_F16, SLICES>);
-        return launch(stream4_blocks_kernel<SETS, false, ROWS, MK_F16, SLICES>);
+    // (eight samples with offsets do not walk long rows: that variant has no registers left for the loop)
+    constexpr bool kWithOffsets = !(WALK && SLICES == 4 && SETS == 2);
+    if (a.zeros) {
+        if constexpr (kWithOffsets) {
+            if (a.x_dtype == MK_F16) return launch(stream4_blocks_kernel<SETS, true, ROWS, MK_F16, SLICES, WALK>);
+            return launch(stream4_blocks_kernel<SETS, true, ROWS, MK_BF16, SLICES, WALK>);
+        } else {
+            return -1;
+        }
     }
-    if (a.zeros) return launch(stream4_blocks_kernel<SETS, true, ROWS, MK_BF16, SLICES>);
-    return launch(stream4_blocks_kernel<SETS, false, ROWS, MK_BF16, SLICES>);
+    if (a.x_dtype == MK_F16) return launch(stream4_blocks_kernel<SETS, false, ROWS, MK_F16, SLICES, WALK>);
+    return launch(stream4_blocks_kernel<SETS, false, ROWS, MK_BF16, SLICES, WALK>);
 }
 
 // A wavefront covers 512 codes per sub-slice: short rows get fewer sub-slices, so that no
@@ -720,6 +728,11 @@ int launch_blocks(const Stream4Args &a, const Stream4Group &members, int tiles, 
     // tile per compute unit and at most four samples it measures 4 % slower (4.8 -> 5.0 us), and so do longer rows.
     if (a.width <= 4096 && (tiles > kComputeUnits || a.samples > 4))
         return launch_blocks_sliced<SETS, ROWS, 2>(a, members, tiles, stream);
+    // More tiles of eight long rows than compute units (stream4_launch chooses that height for them): walked.
+    if constexpr (ROWS == kMidRows) {
+        const int units = tiles * (members.count > 0 ? members.count : 1);
+        if (units > kComputeUnits && !(SETS == 2 && a.zeros)) return launch_blocks_sliced<SETS, ROWS, 4, true>(a, members, tiles, stream);
+    }
     return launch_blocks_sliced<SETS, ROWS, 4>(a, members, tiles, stream);
 }
 
@@ -815,6 +828,16 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream) {
         // fewer than 512 tiles of sixteen rows leave SIMDs without a wavefront: tiles of eight rows fill them
         // (4096 x 2048 at eight samples: 6.2 -> 5.2 us; with two and more wavefronts per row the activation
         // preparation repeated per tile costs more than the idle SIMDs: 4096 x 4096 6.4 -> 7.0 us).
+        // Three and more samples of rows over 4096 codes (one workgroup per compute unit at a time) whose second
+        // round of sixteen-row tiles would be at most half full: as many workgroups as the GPU holds walk tiles of
+        // eight rows on one preparation of their activations (5120 x 13824 at M = 4 / 8: 15.2 -> 12.9 / 21.6 -> 16.4 us;
+        // 6144 x 8192: 9.0 -> 8.0 / 11.9 -> 10.9; a second round three quarters full, 7168 x 8192: 9.1 -> 9.3 / 12.1 ->
+        // 12.8).  Eight samples with offsets keep sixteen rows: that variant of the walking kernel spills registers.
+        if (a.samples >= 3 && a.x_dtype != MK_F32 && a.width > 4096 && a.rows / kWideRows > kComputeUnits &&
+            a.rows / kWideRows <= kComputeUnits + kComputeUnits / 2 && !(a.zeros && a.samples > 4)) {
+            const int tiles = a.rows / kMidRows;
+            return launch_rows<kMidRows>(a, none, tiles, stream) ? -1 : tiles * kMidRows;
+        }
         if (a.samples >= 3 && a.x_dtype != MK_F32 && a.width <= 2048 && a.rows / kWideRows < 2 * kComputeUnits) {
             const int tiles = a.rows / kMidRows;
             return launch_rows<kMidRows>(a, none, tiles, stream) ? -1 : tiles * kMidRows;
@@ -823,11 +846,14 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream) {
         // none; tiles of eight rows double the wavefronts in flight (8192 x 4096: 6.2 -> 5.2 us at one sample, 7.3 ->
         // 5.8 at two; 5120 x 5120: 5.8 -> 5.3, 7.4 -> 6.5; 8192 x 2048: 4.3 -> 4.0, 5.1 -> 4.4).  Measured no faster
         // or slower: exactly one tile per compute unit of rows over 2048 codes (4096 x 4096: 4.3 -> 4.4), rows of
-        // four and more wavefronts (8192 x 8192: 7.5 -> 8.0), more than 512 tiles (12288 x 4096: 6.7 -> 6.9).
+        // four and more wavefronts in two full rounds (8192 x 8192: 7.5 -> 8.0), more than 512 tiles (12288 x 4096: 6.7 -> 6.9).
         {
             const int wide_tiles = a.rows / kWideRows, row_waves = mk_cdiv(a.width, 2048);
-            const bool few_waves = row_waves == 1 ? wide_tiles <= 2 * kComputeUnits
-                                                  : row_waves <= 3 && wide_tiles > kComputeUnits && wide_tiles <= 2 * kComputeUnits;
+            // (longer rows, one workgroup per compute unit at a time: only where a last round of at most half the
+            // compute units becomes a shorter one, 5120 x 13824: 10.4 -> 9.0 / 13.1 -> 11.2 us, 6144 x 8192: 6.9 -> 6.4 /
+            // 8.1 -> 7.7; 7168 x 8192, whose second round is three quarters full: 7.0 -> 7.3)
+            const int most_tiles = row_waves <= 3 ? 2 * kComputeUnits : kComputeUnits + kComputeUnits / 2;
+            const bool few_waves = wide_tiles <= most_tiles && (row_waves == 1 || wide_tiles > kComputeUnits);
             if (a.samples <= 2 && a.x_dtype != MK_F32 && few_waves) {
                 const int tiles = a.rows / kMidRows;
                 return launch_rows<kMidRows>(a, none, tiles, stream) ? -1 : tiles * kMidRows;
@@ -835,6 +861,21 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream) {
         }
         const int tiles = a.rows / kWideRows;
         return launch_rows<kWideRows>(a, none, tiles, stream) ? -1 : tiles * kWideRows;
+    }
+    // Fewer than 256 tiles of sixteen rows: tiles of four rows spread them over the compute units.  From three
+    // samples on every tile repeats a longer preparation of the activations, and taller tiles win again on the
+    // larger of these layers (M = 4 / 8: 3072 x 8192 7.4 / 10.6 -> 5.8 / 7.7 us with sixteen rows; 3584 x 3584 5.0 /
+    // 7.2 -> 4.7 / 5.8 and 2048 x 4096 4.2 / 5.2 -> 4.0 / 4.9 with eight; 3072 x 3072 4.25 -> 4.4 / 6.0 -> 5.3;
+    // layers of 1024 rows and one or two samples are fastest on four rows throughout).
+    if (a.samples >= 3 && a.x_dtype != MK_F32 && a.rows >= 2048) {
+        if (a.rows >= 3072 && a.width >= 8192) {
+            const int tiles = a.rows / kWideRows;
+            return launch_rows<kWideRows>(a, none, tiles, stream) ? -1 : tiles * kWideRows;
+        }
+        if (a.samples >= 5 || a.width >= 3584) {
+            const int tiles = a.rows / kMidRows;
+            return launch_rows<kMidRows>(a, none, tiles, stream) ? -1 : tiles * kMidRows;
+        }
     }
     const int tiles = a.rows / kNarrowRows;
     return launch_rows<kNarrowRows>(a, none, tiles, stream) ? -1 : tiles * kNarrowRows;

@@ -68,6 +68,36 @@ def test_config2_decoder_shapes_int4_g128(shape, samples):
     check(run_matvec(layer, x), layer, x)
 
 
+@pytest.mark.parametrize("rows,width", [
+    (5120 + 5, 8192),    # 320 tiles of sixteen long rows: a last round a quarter full
+    (6144 + 11, 4096),   # 384 tiles of two wavefronts
+    (8192 + 3, 2048),    # 512 tiles of one wavefront
+    (3584 + 2, 3584),    # fewer tiles than compute units: tall tiles from three samples on
+    (3072 + 7, 8192),
+])
+@pytest.mark.parametrize("asym", [False, True])
+def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
+    """Layers for which the launcher leaves its default tile of sixteen (or four) rows: tiles of eight rows where
+    sixteen would leave SIMDs idle or the last round sparse, walked by as many workgroups as the GPU holds from
+    three samples on, and tall tiles on small layers with several samples.  Every sample count, fp16 and bf16,
+    ragged row counts, with bias; with one and two samples every row equals the same row of a launch on a
+    sub-matrix that takes the default tiles, bit for bit, since a row's sums do not depend on its tile."""
+    weight = helpers.normal_weight(rows, width, seed=rows % 97)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True, asym=asym)
+    bias = helpers.activations(1, rows, seed=3)[0]
+    part = 2048 if rows < 4096 else 4096
+    head = dict(layer, packed=layer["packed"][: part * width // 2], scales=layer["scales"][:part],
+                zero=None if layer["zero"] is None else layer["zero"][:part], dense=layer["dense"][:part],
+                shape=(part, width))
+    for dtype in (torch.float16, torch.bfloat16):
+        for samples in (1, 2, 3, 4, 5, 8):
+            x = helpers.activations(samples, width, seed=40 + samples, dtype=dtype)
+            y = run_matvec(layer, x, bias.to(dtype))
+            check(y, layer, x.float(), bias.to(dtype).float(), relative=1e-3 if dtype == torch.float16 else 8e-3)
+            if samples <= 2:   # (from three samples on the split of a row over wavefronts depends on the shape too)
+                np.testing.assert_array_equal(y[:, :part], run_matvec(head, x, bias[:part].to(dtype)))
+
+
 def test_config2_tied_output_head():
     weight = helpers.normal_weight(151936, 896, seed=5, outlier_fraction=0.001)
     layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
