@@ -159,6 +159,10 @@ int pairs_launch_group(const Stream4Args &shared, Stream4Group &group, const int
                        hipStream_t stream);
 bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
+// 4-bit uniform-grid codes in rows of 16416 to 32768 codes, fp16 or bf16 activations (packed_matvec_long.hip):
+// multiplies the leading whole tiles of rows and returns the number of rows covered, or -1.
+bool long_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
+int long_launch(const Stream4Args &a, hipStream_t stream);
 // Three to eight samples of fp32 activations against 4-bit uniform-grid codes as integer matrix-core blocks
 // (packed_matvec_digits.hip): `tiles` tiles of `rows_per_tile` rows of the single matrix or of every member.
 bool digits_accepts(const Stream4Args &a, int rows_per_tile);
@@ -606,6 +610,58 @@ __device__ __forceinline__ void chunk_dot_subnormal(const CodeChunk<4> &codes, c
     }
 #pragma unroll
     for (int m = 0; m < MT; ++m) dot[m] = __builtin_fmaf(upper[m], 0.0625f, lower[m]);
+}
+
+// ---- bf16 activations ----------------------------------------------------------------------
+//
+// bf16 has seven mantissa bits, so only the low nibble of each half fits the magic-number
+// insertion (128 + c); every pair of codes needs its own shift: 3 shifts, 4 v_bfi and 4
+// v_dot2_f32_bf16 per eight codes, against 1 + 4 + 4 for fp16.  Pairs are (x0,x4) (x1,x5)
+// (x2,x6) (x3,x7) of every eight codes, unscaled.
+
+// Re-pairs a chunk in place; returns the sum of its activations.
+__device__ __forceinline__ float pair_for_nibbles_bf16(XChunk<MK_BF16> &x) {
+    const uint32_t ones = 0x3f803f80u;
+    float total = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const uint32_t p0 = x.r[4 * g + 0], p1 = x.r[4 * g + 1];
+        const uint32_t p2 = x.r[4 * g + 2], p3 = x.r[4 * g + 3];
+        x.r[4 * g + 0] = __builtin_amdgcn_perm(p2, p0, 0x05040100u);
+        x.r[4 * g + 1] = __builtin_amdgcn_perm(p2, p0, 0x07060302u);
+        x.r[4 * g + 2] = __builtin_amdgcn_perm(p3, p1, 0x05040100u);
+        x.r[4 * g + 3] = __builtin_amdgcn_perm(p3, p1, 0x07060302u);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            total = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mk_bf2, ones), __builtin_bit_cast(mk_bf2, x.r[4 * g + i]), total, false);
+    }
+    return total;
+}
+
+// sum over the chunk of (128 + code_k) x_k for MT samples.
+template <int MT>
+__device__ __forceinline__ void chunk_dot_bf16(const CodeChunk<4> &codes, const XChunk<MK_BF16> (&x)[MT], float (&dot)[MT]) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) dot[m] = 0.0f;
+    uint32_t magic = 0x43004300u;
+    asm volatile("" : "+v"(magic));
+    auto insert = [&](uint32_t word) __attribute__((always_inline)) {
+        return __builtin_bit_cast(mk_bf2, (word & 0x000f000fu) | (magic & ~0x000f000fu));
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w = codes.w[i];
+        const mk_bf2 h0 = insert(w), h1 = insert(w >> 4), h2 = insert(w >> 8), h3 = insert(w >> 12);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            float d = dot[m];
+            d = __builtin_amdgcn_fdot2_f32_bf16(h0, __builtin_bit_cast(mk_bf2, x[m].r[4 * i + 0]), d, false);
+            d = __builtin_amdgcn_fdot2_f32_bf16(h1, __builtin_bit_cast(mk_bf2, x[m].r[4 * i + 1]), d, false);
+            d = __builtin_amdgcn_fdot2_f32_bf16(h2, __builtin_bit_cast(mk_bf2, x[m].r[4 * i + 2]), d, false);
+            d = __builtin_amdgcn_fdot2_f32_bf16(h3, __builtin_bit_cast(mk_bf2, x[m].r[4 * i + 3]), d, false);
+            dot[m] = d;
+        }
+    }
 }
 
 // A chunk of 32 codes against the digit planes of MT fp32 samples (planes_of_piece): sum_k (c_k - 8) X_k, exact

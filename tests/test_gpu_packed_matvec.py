@@ -98,6 +98,30 @@ def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
                 np.testing.assert_array_equal(y[:, :part], run_matvec(head, x, bias[:part].to(dtype)))
 
 
+@pytest.mark.parametrize("rows,width,group,asym", [
+    (4096 + 5, 18944, 128, False),   # sixteen-row tiles, five wavefronts of two spans, the second span partly past the row
+    (260, 28672, 128, True),         # four-row tiles, seven wavefronts
+    (70, 32768, 64, True),           # the longest row
+    (48, 16384 + 32, 32, False),     # one chunk in the second span
+])
+def test_rows_of_more_than_16384_codes(rows, width, group, asym):
+    """Down projections of the larger decoders (K = 18944, 28672): every wavefront owns two spans of 2048 codes.
+    One to eight samples, fp16 and bf16 activations, 16-bit and fp32 scales, offsets and bias, against the float64
+    product."""
+    weight = helpers.normal_weight(rows, width, seed=width % 89)
+    layer = helpers.quantised_layer(weight, INT4, bits=4, group=group, integer=True, asym=asym)
+    bias = helpers.activations(1, rows, seed=3)[0]
+    for dtype, scale_dtype in ((torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32)):
+        for samples in (1, 2, 3, 4, 5, 8):
+            x = helpers.activations(samples, width, seed=50 + samples, dtype=dtype)
+            y = run_matvec(layer, x, bias.to(dtype), scale_dtype=scale_dtype)
+            sides = {key: None if layer[key] is None else torch.from_numpy(layer[key]).to(scale_dtype).float().numpy()
+                     for key in ("scales", "zero")}
+            check(y, layer if scale_dtype != torch.bfloat16 else dict(layer, dense=scaling.decode_grouped(
+                layer["codes"], sides["scales"], layer["values"], layer["group"], sides["zero"])),
+                x.float(), bias.to(dtype).float(), relative=1e-3 if dtype == torch.float16 else 8e-3)
+
+
 def test_config2_tied_output_head():
     weight = helpers.normal_weight(151936, 896, seed=5, outlier_fraction=0.001)
     layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
