@@ -193,6 +193,260 @@ int launch_rows_of(const Stream4Args &a, int tiles, hipStream_t stream) {
     return of(std::false_type{}, std::false_type{});
 }
 
+// ---- three to eight samples: 4 x 4 x 4 matrix-core blocks -----------------------------------
+//
+// As in the streaming kernel's matrix-core variant, lane 4 b + t of a wavefront holds the codes of row t and the
+// activations of sample t for chunk b of a sub-slice of sixteen chunks; here a wavefront owns 4096 adjacent codes
+// of K as eight sub-slices (128 registers of activations), so one pass takes four samples and samples 5 - 8 are a
+// second pass over the codes (blockIdx.y).  A sample's slice goes through the wavefront's LDS buffer by itself
+// (8 KB), and with more (tile, pass) units than the GPU holds workgroups each workgroup walks its share of the
+// tiles on one preparation of its activations.
+template <bool HAS_ZERO, int ROWS, int XT, bool WALK>
+__global__ void __launch_bounds__(512) long_blocks_kernel(const Stream4Args a, const Stream4Group members) {
+    constexpr int kQuads = ROWS / 4;
+    constexpr int kSlices = 8;                       // sub-slices of sixteen chunks per wavefront
+    constexpr int kSteps = kQuads * kSlices;
+    constexpr int kMostAhead = 4;
+    constexpr int kAhead = kSteps < kMostAhead ? kSteps : kMostAhead;
+    constexpr int kSums = ROWS;
+    constexpr int kSampleWords = kSlices * 16 * 16;  // one sample's 4096 values of a wavefront, 16-bit
+    __shared__ float partials[ROWS * 4 * 8];  // [row][sample][wavefront]
+    extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
+    uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSampleWords;
+
+    const TileSource source = tile_source<ROWS>(a, members, blockIdx.z);
+    if (static_cast<int>(blockIdx.x) >= source.tiles) return;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int waves = blockDim.x >> 6;
+    const int block = lane >> 2, t = lane & 3;
+    const uint32_t row_bytes = static_cast<uint32_t>(a.width) >> 1;
+    const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * 2u;
+
+    // Sub-slice s of this lane is chunk `first_chunk + 16 s`; those past the end of the row read chunk 0 with zeroed
+    // activations.  Offsets are worked out where they are used (sixteen of them would not fit beside 128 registers
+    // of activations): scale groups are powers of two, or one group spans the row (`group_shift` 31).
+    const int first_chunk = wave * (16 * kSlices) + block;
+    const int chunks = a.width / kChunkCodes;
+    const uint32_t own_row_codes = static_cast<uint32_t>(t) * row_bytes, own_row_sides = static_cast<uint32_t>(t) * scale_row_bytes;
+    const int group_shift = a.group >= a.width ? 31 : 31 - __builtin_clz(static_cast<unsigned>(a.group) / kChunkCodes);
+    auto in_row = [&](int s) __attribute__((always_inline)) { return first_chunk + 16 * s < chunks; };
+    // (`chunk` is first_chunk behind an empty asm: the compiler must not keep every step's offsets in registers)
+    auto code_offset = [&](int s, int chunk) __attribute__((always_inline)) {
+        return own_row_codes + (chunk + 16 * s < chunks ? static_cast<uint32_t>(chunk + 16 * s) * 16u : 0u);
+    };
+    auto group_offset = [&](int s, int chunk) __attribute__((always_inline)) {
+        return own_row_sides + (chunk + 16 * s < chunks ? (static_cast<uint32_t>(chunk + 16 * s) >> group_shift) * 2u : 0u);
+    };
+
+    __syncthreads();  // aligns the workgroup's wavefronts before their first loads
+
+    int tile = blockIdx.x;
+    int row_base = tile * ROWS;
+    const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
+    uint16_t scale_raw[kSteps], zero_raw[HAS_ZERO ? kSteps : 1];
+    CodeChunk<4> codes[kSteps];
+    // Step `step` of a tile is rows 4 q ... 4 q + 3 at sub-slice s: its codes, and the scale (and offset) of row
+    // 4 q + t there, are requested kAhead steps before they are used.
+    auto request_step = [&](int step) __attribute__((always_inline)) {
+        const int q = step / kSlices, s = step % kSlices;
+        int chunk = first_chunk;
+        asm volatile("" : "+v"(chunk));
+        const size_t quad_offset = static_cast<size_t>(row_base + 4 * q) * scale_row_bytes;
+        const uint32_t sides_at = group_offset(s, chunk);
+        scale_raw[step] = *reinterpret_cast<const uint16_t *>(source.scales + quad_offset + sides_at);
+        if constexpr (HAS_ZERO) zero_raw[step] = *reinterpret_cast<const uint16_t *>(source.zeros + quad_offset + sides_at);
+        load_codes<4>(codes[step], codes_base + static_cast<size_t>(4 * q) * row_bytes + code_offset(s, chunk));
+    };
+    auto request_tile = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int step = 0; step < kAhead; ++step) {
+            request_step(step);
+            __builtin_amdgcn_sched_barrier(0);  // in order
+        }
+    };
+
+    // Activations of sample t for this lane's eight chunks: the wavefront reads one sample's slice coalesced, parks
+    // it in its LDS buffer, and the sixteen lanes of that sample pick their chunks; then the next sample.
+    XChunk<XT> x[kSlices];
+    {
+        const int sample_base = blockIdx.y * 4;
+        mk_u32x4 even_pieces[kSlices], odd_pieces[kSlices];   // of samples 0 and 2, of samples 1 and 3
+        auto request_sample = [&](int j, mk_u32x4 (&pieces)[kSlices]) __attribute__((always_inline)) {
+            const int sample = sample_base + j < a.samples ? sample_base + j : a.samples - 1;
+#pragma unroll
+            for (int i = 0; i < kSlices; ++i) pieces[i] = request_piece(source.x, a.width, sample, wave * (512 * kSlices), i, lane);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto place_sample = [&](int j, const mk_u32x4 (&pieces)[kSlices]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < kSlices; ++i) park_piece_swizzled(x_slice, i, lane, pieces[i]);
+            wave_exchange_fence();
+            if (t == j) {
+#pragma unroll
+                for (int s = 0; s < kSlices; ++s) chunk_from_swizzled_slice(x[s], x_slice, s * 16 + block);
+            }
+            wave_exchange_fence();   // the next sample goes to the same buffer
+        };
+        if constexpr (WALK) {
+            // (a walking workgroup prepares once for several tiles and has no registers for loads in flight beside
+            // the activations: one sample at a time, the first tile behind them)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                request_sample(j, even_pieces);
+                place_sample(j, even_pieces);
+            }
+            request_tile();
+        } else {
+            request_sample(0, even_pieces);
+            request_sample(1, odd_pieces);
+            place_sample(0, even_pieces);
+            request_sample(2, even_pieces);
+            place_sample(1, odd_pieces);
+            request_sample(3, odd_pieces);
+            request_tile();
+            place_sample(2, even_pieces);
+            place_sample(3, odd_pieces);
+        }
+    }
+    float x_sum[kSlices], grid_term[kSlices];
+    {
+        const bool sample_present = static_cast<int>(blockIdx.y) * 4 + t < a.samples;
+#pragma unroll
+        for (int s = 0; s < kSlices; ++s) {
+            const bool kept = in_row(s) && sample_present;
+            if (__builtin_amdgcn_ballot_w64(!kept) != 0) {  // uniform; rarely taken
+                const uint32_t keep = kept ? 0xffffffffu : 0u;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) x[s].r[i] &= keep;
+            }
+            float code_free;
+            if constexpr (XT == MK_F16) {
+                code_free = pair_for_nibbles(x[s], &x_sum[s]);
+            } else {
+                x_sum[s] = pair_for_nibbles_bf16(x[s]);
+                code_free = 128.0f * x_sum[s];
+            }
+            grid_term[s] = a.grid_min * x_sum[s] - a.grid_step * code_free;
+        }
+    }
+
+    while (true) {
+    float sums[kSums];
+#pragma unroll
+    for (int j = 0; j < kSums; ++j) sums[j] = 0.0f;
+
+    uint32_t magic = XT == MK_F16 ? 0x64006400u : 0x43004300u;
+    asm volatile("" : "+v"(magic));
+    auto insert = [&](uint32_t mask, uint32_t word) __attribute__((always_inline)) {
+        return (word & mask) | (magic & ~mask);
+    };
+    auto blocks = [](uint32_t a_low, uint32_t a_high, uint32_t b_low, uint32_t b_high, mk_f4 sum) __attribute__((always_inline)) {
+        const mk_u32x2 left = {a_low, a_high}, right = {b_low, b_high};
+        if constexpr (XT == MK_F16)
+            return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(mk_h4, left), __builtin_bit_cast(mk_h4, right), sum, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(mk_s4, left), __builtin_bit_cast(mk_s4, right), sum, 0, 0, 0);
+    };
+
+#pragma unroll
+    for (int step = 0; step < kSteps; ++step) {
+        const int q = step / kSlices, s = step % kSlices;
+        mk_f4 dot = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w = codes[step].w[i];
+            uint32_t pair[4];  // codes (0, 4), (1, 5), (2, 6), (3, 7) as 16-bit floats
+            if constexpr (XT == MK_F16) {
+                const uint32_t w8 = w >> 8;
+                pair[0] = insert(0x000f000fu, w), pair[1] = insert(0x00f000f0u, w);
+                pair[2] = insert(0x000f000fu, w8), pair[3] = insert(0x00f000f0u, w8);
+            } else {
+                pair[0] = insert(0x000f000fu, w), pair[1] = insert(0x000f000fu, w >> 4);
+                pair[2] = insert(0x000f000fu, w >> 8), pair[3] = insert(0x000f000fu, w >> 12);
+            }
+            dot = blocks(pair[0], pair[1], x[s].r[4 * i + 0], x[s].r[4 * i + 1], dot);
+            dot = blocks(pair[2], pair[3], x[s].r[4 * i + 2], x[s].r[4 * i + 3], dot);
+        }
+        if (step + kAhead < kSteps) request_step(step + kAhead);
+        // Row 4 q + r of the block: scale (and offset) come from lane r of the quad.
+        const float scale = side_as_float(scale_raw[step], a.scale_dtype);
+        float zero = 0.0f;
+        if constexpr (HAS_ZERO) zero = side_as_float(zero_raw[step], a.scale_dtype);
+        auto add_row = [&](auto r) __attribute__((always_inline)) {
+            constexpr int R = decltype(r)::value;
+            float total = sums[4 * q + R];
+            total = __builtin_fmaf(quad_value<R>(scale), __builtin_fmaf(a.grid_step, dot[R], grid_term[s]), total);
+            if constexpr (HAS_ZERO) total = __builtin_fmaf(quad_value<R>(zero), x_sum[s], total);
+            sums[4 * q + R] = total;
+        };
+        add_row(std::integral_constant<int, 0>{});
+        add_row(std::integral_constant<int, 1>{});
+        add_row(std::integral_constant<int, 2>{});
+        add_row(std::integral_constant<int, 3>{});
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // Over the sixteen blocks of the wavefront (lane bits 2 - 5), then over the wavefronts.
+    transposed_wave_sum<kSums, 2>(sums, lane);
+    static_assert(kSums == 16 || kSums == 8 || kSums == 4, "one, two or four lanes per total");
+    const bool writer = ((lane >> 2) >> (kSums == 16 ? 4 : kSums == 8 ? 3 : 2)) == 0;
+    if (writer) partials[(transposed_value_of_lane<kSums>(lane >> 2) * 4 + t) * 8 + wave] = sums[0];
+    __syncthreads();
+    for (int index = tid; index < ROWS * 4; index += blockDim.x) {
+        float total = partials[index * 8];
+#pragma unroll
+        for (int w = 1; w < 8; ++w) total += w < waves ? partials[index * 8 + w] : 0.0f;
+        const int row = row_base + index / 4;
+        const int sample = blockIdx.y * 4 + (index & 3);
+        if (sample < a.samples) {
+            if (source.bias) total += mk_load_as_float(source.bias, row, a.bias_dtype);
+            store_output<XT>(source.y, static_cast<size_t>(sample) * source.rows + row, total);
+        }
+    }
+    if constexpr (!WALK) break;
+    tile += gridDim.x;
+    if (tile >= source.tiles) break;
+    __syncthreads();  // `partials` is reused by the next tile
+    row_base = tile * ROWS;
+    codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
+    request_tile();
+    }
+}
+
+template <int ROWS>
+int launch_blocks_of(const Stream4Args &a, hipStream_t stream) {
+    const int tiles = a.rows / ROWS;
+    if (tiles == 0) return 0;
+    Stream4Group none;
+    none.count = 0;
+    none.widest_tiles = 0;
+    const dim3 block(mk_cdiv(a.width, 4096) * 64);
+    const size_t slices = static_cast<size_t>(block.x / 64) * 8 * 16 * 16 * sizeof(uint32_t);   // 8 KB per wavefront
+    dim3 grid(tiles, mk_cdiv(a.samples, 4), 1);
+    auto launch = [&](auto walking, auto plain) -> int {
+        // the launch asks for 64 KB of dynamic LDS at eight wavefronts: within the default limit
+        static std::atomic<int> resident[9];
+        const int known = resident_workgroups(walking, static_cast<int>(block.x), slices, resident[block.x / 64]);
+        const int passes = static_cast<int>(grid.y);
+        if (static_cast<int>(grid.x) * passes > known) {
+            grid.x = known / passes > 0 ? known / passes : 1;
+            hipLaunchKernelGGL(walking, grid, block, slices, stream, a, none);
+        } else {
+            hipLaunchKernelGGL(plain, grid, block, slices, stream, a, none);
+        }
+        return 0;
+    };
+    auto of = [&](auto has_zero) -> int {
+        constexpr bool Z = decltype(has_zero)::value;
+        if (a.x_dtype == MK_F16) return launch(long_blocks_kernel<Z, ROWS, MK_F16, true>, long_blocks_kernel<Z, ROWS, MK_F16, false>);
+        return launch(long_blocks_kernel<Z, ROWS, MK_BF16, true>, long_blocks_kernel<Z, ROWS, MK_BF16, false>);
+    };
+    const int status = a.zeros ? of(std::true_type{}) : of(std::false_type{});
+    return status ? -1 : tiles * ROWS;
+}
+
 template <int ROWS>
 int launch_tiles(const Stream4Args &a, hipStream_t stream) {
     const int tiles = a.rows / ROWS;
@@ -203,9 +457,11 @@ int launch_tiles(const Stream4Args &a, hipStream_t stream) {
 }  // namespace
 
 bool long_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform) {
-    (void)scale_dtype;   // 16-bit and fp32 scales both
-    return bits == 4 && uniform && samples <= 2 && (x_dtype == MK_F16 || x_dtype == MK_BF16) && width > 16384 && width <= 32768 &&
-           width % kChunkCodes == 0 && (group % kChunkCodes == 0 || group >= width);
+    // one and two samples with 16-bit or fp32 scales, more samples with 16-bit scales (as for shorter rows)
+    const bool whole_chunks = group % kChunkCodes == 0 || group >= width;
+    const bool power_of_two = (group & (group - 1)) == 0 || group >= width;   // the matrix-core kernel shifts instead of dividing
+    return bits == 4 && uniform && (samples <= 2 || (scale_dtype != MK_F32 && power_of_two)) &&
+           (x_dtype == MK_F16 || x_dtype == MK_BF16) && width > 16384 && width <= 32768 && width % kChunkCodes == 0 && whole_chunks;
 }
 
 // Multiplies the leading whole tiles of rows; returns the number of rows covered.
@@ -214,6 +470,15 @@ int long_launch(const Stream4Args &a, hipStream_t stream) {
     // workgroup while that leaves half the compute units one each, eight rows where the second round of sixteen-row
     // tiles would be at most half full, fewer rows only for small layers.
     const int wide_tiles = a.rows / 16;
+    if (a.samples >= 3) {
+        // Every workgroup prepares four samples of all of x, so a launch takes that preparation plus the rows of its
+        // tallest share: the lowest tiles that still give every (tile, pass) a compute unit of its own, else sixteen
+        // rows, walked.
+        const int passes = mk_cdiv(a.samples, 4);
+        if ((a.rows / 4) * passes <= kComputeUnits) return launch_blocks_of<4>(a, stream);
+        if ((a.rows / 8) * passes <= kComputeUnits) return launch_blocks_of<8>(a, stream);
+        return launch_blocks_of<16>(a, stream);
+    }
     if (wide_tiles > kComputeUnits && wide_tiles <= kComputeUnits + kComputeUnits / 2) return launch_tiles<8>(a, stream);
     if (wide_tiles >= kComputeUnits / 2) return launch_tiles<16>(a, stream);
     if (a.rows / 8 >= kComputeUnits / 2) return launch_tiles<8>(a, stream);
