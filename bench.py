@@ -575,6 +575,9 @@ def other_kernels(device: torch.device, full: bool) -> dict:
     if full:
         matvec(ROWS, WIDTH, 128, 4, values, True, False, "int4 g128, bf16 activations", dtype=torch.bfloat16)
         matvec(151936, 896, 128, 4, values, True, False, "int4 g128 (tied head)")
+        # down projections of larger decoders: rows of more than 16384 codes (two spans of 2048 codes per wavefront)
+        matvec(3584, 18944, 128, 4, values, True, False, "int4 g128 (K = 18944)")
+        matvec(8192, 28672, 128, 4, values, True, False, "int4 g128 (K = 28672)")
         matvec(ROWS, WIDTH, 128, 8, torch.arange(-128, 128, dtype=torch.float32, device=device), True, False, "int8 g128")
         for rows, width in ((896, 896), (128, 896), (4864, 896), (896, 4864)):
             matvec(rows, width, 128, 4, values, True, False, "int4 g128 (decoder layer)")
