@@ -811,16 +811,21 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream) {
         return launch_rows<kWideRows>(a, none, tiles, stream) ? -1 : tiles * kWideRows;
     }
     // Fewer than 256 tiles of sixteen rows: tiles of four rows spread them over the compute units.  From three
-    // samples on every tile repeats a longer preparation of the activations, and taller tiles win again on the
-    // larger of these layers (M = 4 / 8: 3072 x 8192 7.4 / 10.6 -> 5.8 / 7.7 us with sixteen rows; 3584 x 3584 5.0 /
-    // 7.2 -> 4.7 / 5.8 and 2048 x 4096 4.2 / 5.2 -> 4.0 / 4.9 with eight; 3072 x 3072 4.25 -> 4.4 / 6.0 -> 5.3;
-    // layers of 1024 rows and one or two samples are fastest on four rows throughout).
-    if (a.samples >= 3 && a.x_dtype != MK_F32 && a.rows >= 2048) {
-        if (a.rows >= 3072 && a.width >= 8192) {
+    // samples on every tile repeats a longer preparation of the activations.  Rows over 4096 codes (one workgroup per
+    // compute unit at a time): the lowest tiles that still give every tile a compute unit of its own (M = 4 / 8:
+    // 1536 x 8960 8.4 / 11.9 -> 5.8 / 7.9 us with eight rows, 3072 x 8192 7.4 / 10.6 -> 5.8 / 7.7 and 2560 x 10240
+    // 8.6 / 11.1 -> 7.4 / 10.2 with sixteen; 1024 x 14336 stays on four).  Shorter rows (several workgroups per
+    // compute unit): eight rows on the larger layers (3584 x 3584 5.0 / 7.2 -> 4.7 / 5.8, 2048 x 4096 4.2 / 5.2 ->
+    // 4.0 / 4.9; 3072 x 3072 4.25 -> 4.4 / 6.0 -> 5.3).  One and two samples are fastest on four rows throughout.
+    if (a.samples >= 3 && a.x_dtype != MK_F32) {
+        int rows_per_tile = kNarrowRows;
+        if (a.width > 4096) rows_per_tile = a.rows / kNarrowRows <= kComputeUnits ? kNarrowRows : a.rows / kMidRows <= kComputeUnits ? kMidRows : kWideRows;
+        else if (a.rows >= 2048 && (a.samples >= 5 || a.width >= 3584)) rows_per_tile = kMidRows;
+        if (rows_per_tile == kWideRows) {
             const int tiles = a.rows / kWideRows;
             return launch_rows<kWideRows>(a, none, tiles, stream) ? -1 : tiles * kWideRows;
         }
-        if (a.samples >= 5 || a.width >= 3584) {
+        if (rows_per_tile == kMidRows) {
             const int tiles = a.rows / kMidRows;
             return launch_rows<kMidRows>(a, none, tiles, stream) ? -1 : tiles * kMidRows;
         }
