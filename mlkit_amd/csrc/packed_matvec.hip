@@ -316,6 +316,7 @@ extern "C" int mk_packed_matvec_group(const void *const *x, int x_dtype, int cou
                            mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0);
     const bool tables = dtypes_valid && !streaming && !tuning().no_pairs && (uniform || (values && n_values >= 1 && n_values <= (1 << bits))) &&
                         mk_packed_layout_supported(bits, input_width, group) &&
+                        input_width <= 16384 &&   // (longer rows: one launch per matrix)
                         mk_matvec::pairs_accepts(input_width, group, bits, x_dtype, scale_dtype);
     bool one_launch = (streaming || tables) && (static_cast<size_t>(input_width) * mk_dtype_bytes(x_dtype)) % 16 == 0;
     for (int i = 0; i < count; ++i) {

@@ -1,5 +1,5 @@
 // Packed matvec for 2- to 8-bit codes of any scalar grid (integer grids, NF4, small
-// codebooks) with fp16 or bf16 activations and 16-bit scales, rows of K = 32 ... 16384 codes (K % 32 == 0).
+// codebooks) with fp16 or bf16 activations and 16-bit scales, rows of K = 32 ... 32768 codes (K % 32 == 0).
 //
 // Adjacent codes (one, two or four, by code width) index a table of 16-bit values held in
 // LDS, so one LDS read decodes up to four weights and one v_dot2_f32_f16 (v_dot2_f32_bf16)
@@ -43,15 +43,18 @@ __device__ __forceinline__ float side_value(uint16_t raw, int dtype) {
 // (two per CU at 4096 rows); short rows keep sixteen rows per table fill.
 constexpr int kShortTileRows = 8;
 constexpr int kShortTileWidth = 4096;
+// A workgroup of eight wavefronts covers 16384 codes of a row at once; longer rows (up to twice that) take two
+// turns (the LONG kernels), with sixteen rows per workgroup and table decoding.
+constexpr int kMostRowCodes = 16384;
 // Uniform 2-, 3- and 8-bit grids with fp16 activations, one or two samples: decoded by shifts and masks.
 inline bool shifted_decoding(const Stream4Args &a) {
-    return a.uniform && a.x_dtype == MK_F16 && (a.bits == 2 || a.bits == 3 || a.bits == 8) && a.samples <= 2;
+    return a.uniform && a.x_dtype == MK_F16 && (a.bits == 2 || a.bits == 3 || a.bits == 8) && a.samples <= 2 && a.width <= kMostRowCodes;
 }
 
 // (Without lookups to wait on, sixteen rows per workgroup measure faster: 5.8 against 6.0 us for two bits, 6.5
 // against 6.8 us for three bits at 4096 x 14336.)
 inline int tile_rows(const Stream4Args &a) {
-    return a.samples == 1 && a.width >= kShortTileWidth && !shifted_decoding(a) ? kShortTileRows : kPairRows;
+    return a.samples == 1 && a.width >= kShortTileWidth && a.width <= kMostRowCodes && !shifted_decoding(a) ? kShortTileRows : kPairRows;
 }
 
 template <int MT, int ROWS>
@@ -257,9 +260,12 @@ __device__ __forceinline__ void shifted_chunk_dot(const CodeChunk<BITS> &codes, 
 }
 
 // SHIFTED: a uniform 2- or 3-bit grid with fp16 activations, decoded by shifts and masks (no table).
-template <int BITS, int MT, bool HAS_ZERO, int XT, int LOOKUP, int ROWS, bool SHIFTED = false>
+// LONG: rows of more than 16384 codes.  The workgroup covers the row in `phases` turns of blockDim.x chunks, each
+// with its own activations, scales and stream of codes, and adds the turns' row sums before the reduction.
+template <int BITS, int MT, bool HAS_ZERO, int XT, int LOOKUP, int ROWS, bool SHIFTED = false, bool LONG = false>
 __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const Stream4Group members) {
     static_assert(!SHIFTED || ((BITS == 2 || BITS == 3 || BITS == 8) && XT == MK_F16), "shifted decoding: 2, 3 or 8 bits, fp16 activations");
+    static_assert(!LONG || (ROWS * MT <= 64 && !SHIFTED), "long rows: one reduction for all rows of the tile, table decoding");
     constexpr int kLookup = LOOKUP;
     constexpr int kPairRows = ROWS;
     constexpr int kPairAhead = rows_in_flight<BITS>();
@@ -282,15 +288,20 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const S
     const int sample_base = blockIdx.y * MT;
     const uint32_t row_bytes = (static_cast<uint32_t>(a.width) * BITS) >> 3;
     const uint8_t *codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;  // uniform
-    // Lanes past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
-    // activations: they add nothing.
-    const bool in_row = tid * kChunkCodes < a.width;
-    const int chunk = in_row ? tid : 0;
-    const uint32_t code_offset = static_cast<uint32_t>(chunk) * (4u * BITS);
-
     if constexpr (!SHIFTED) fill_table<BITS, LOOKUP, XT>(table, a);
     // Also aligns the wavefronts, so that nobody's small loads queue behind another's codes.
     __syncthreads();
+
+    const int turn_codes = static_cast<int>(blockDim.x) * kChunkCodes;
+    const int phases = LONG ? (a.width + turn_codes - 1) / turn_codes : 1;   // uniform
+    float long_sums[LONG ? kSums : 1];
+    for (int phase = 0; phase < phases; ++phase) {
+    // Lanes past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
+    // activations: they add nothing.
+    const int wanted_chunk = LONG ? phase * static_cast<int>(blockDim.x) + tid : tid;
+    const bool in_row = wanted_chunk * kChunkCodes < a.width;
+    const int chunk = in_row ? wanted_chunk : 0;
+    const uint32_t code_offset = static_cast<uint32_t>(chunk) * (4u * BITS);
 
     XChunk<XT> x[MT];
 #pragma unroll
@@ -412,6 +423,13 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const S
             __builtin_amdgcn_sched_barrier(0);
         }
 
+        if constexpr (LONG) {   // (one pass holds all rows of the tile)
+#pragma unroll
+            for (int k = 0; k < kSums; ++k) long_sums[k] = phase == 0 ? sums[k] : long_sums[k] + sums[k];
+            if (phase + 1 < phases) break;   // the next turn of the row
+#pragma unroll
+            for (int k = 0; k < kSums; ++k) sums[k] = long_sums[k];
+        }
         transposed_wave_sum<kSums>(sums, lane);
         if (pass > 0) __syncthreads();
         if (lane < kSums) partials[transposed_value_of_lane<kSums>(lane) * 8 + wave] = sums[0];
@@ -429,6 +447,7 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const S
             }
         }
     }
+    }
 }
 
 // ---- three to eight samples: the dot products on the matrix cores -------------------------
@@ -443,7 +462,8 @@ __global__ void __launch_bounds__(512) pairs_kernel(const Stream4Args a, const S
 // SHIFTED (uniform 8-bit grids, fp16 activations): no table; a word and the word shifted by 8, each masked with
 // 0x00ff00ff, are the four codes of one instruction as fp16 subnormals (in the order 0, 2, 1, 3, which the
 // activations are permuted to once per tile), and the grid's affine map applies to the block's sums.
-template <int BITS, int SETS, bool HAS_ZERO, int XT, int LOOKUP, int SLICES, bool SHIFTED = false>
+// LONG: rows of more than 16384 codes, covered in `phases` turns of the workgroup's width (see pairs_kernel).
+template <int BITS, int SETS, bool HAS_ZERO, int XT, int LOOKUP, int SLICES, bool SHIFTED = false, bool LONG = false>
 __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, const Stream4Group members) {
     static_assert(!SHIFTED || (BITS == 8 && XT == MK_F16), "shifted decoding on the matrix cores: 8 bits, fp16 activations");
     constexpr int kQuads = kPairRows / 4;
@@ -475,20 +495,30 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
 
     if constexpr (!SHIFTED) fill_table<BITS, LOOKUP, XT>(table, a);
 
+    float sums[SETS][kPairRows];
+#pragma unroll
+    for (int set = 0; set < SETS; ++set)
+#pragma unroll
+        for (int j = 0; j < kPairRows; ++j) sums[set][j] = 0.0f;
+
+    const int turn_codes = waves * (512 * kSlices);
+    const int phases = LONG ? (a.width + turn_codes - 1) / turn_codes : 1;   // uniform
+    for (int phase = 0; phase < phases; ++phase) {
+    const int phase_wave = LONG ? phase * waves + wave : wave;
     // Chunks past the end of a row (K is not a multiple of 2048) read chunk 0 with zeroed
     // activations: they add nothing.
     bool in_row[kSlices];
     uint32_t code_offset[kSlices], group_offset[kSlices];
 #pragma unroll
     for (int s = 0; s < kSlices; ++s) {
-        const int wanted = wave * (16 * kSlices) + s * 16 + block;
+        const int wanted = phase_wave * (16 * kSlices) + s * 16 + block;
         in_row[s] = wanted * kChunkCodes < a.width;
         const int chunk = in_row[s] ? wanted : 0;
         code_offset[s] = static_cast<uint32_t>(t) * row_bytes + static_cast<uint32_t>(chunk) * (4u * BITS);
         group_offset[s] = static_cast<uint32_t>(t) * scale_row_bytes +
                           ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * 2u;
     }
-    __syncthreads();  // the table is complete; also aligns the wavefronts before their loads
+    if (!LONG || phase == 0) __syncthreads();  // the table is complete; also aligns the wavefronts before their loads
 
     // Activations of sample t (and t + 4) for this lane's four chunks: the slices of a set's
     // four samples are read coalesced and parked side by side; every lane picks its sample's chunks.
@@ -501,7 +531,7 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
             const int wanted_sample = blockIdx.y * 4 * SETS + 4 * set + j;
             const int sample = wanted_sample < a.samples ? wanted_sample : a.samples - 1;
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(source.x, a.width, sample, wave * (512 * kSlices), i, lane);
+            for (int i = 0; i < kSlices; ++i) pieces[j][i] = request_piece(source.x, a.width, sample, phase_wave * (512 * kSlices), i, lane);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -555,12 +585,6 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
         }
     }
     const float shifted_step = a.grid_step * 16777216.0f;   // the subnormal codes are c * 2^-24
-
-    float sums[SETS][kPairRows];
-#pragma unroll
-    for (int set = 0; set < SETS; ++set)
-#pragma unroll
-        for (int j = 0; j < kPairRows; ++j) sums[set][j] = 0.0f;
 
     auto blocks = [](uint32_t a_low, uint32_t a_high, uint32_t b_low, uint32_t b_high, mk_f4 sum) __attribute__((always_inline)) {
         const mk_u32x2 left = {a_low, a_high}, right = {b_low, b_high};
@@ -645,6 +669,8 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
         add_row(std::integral_constant<int, 3>{});
         __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (LONG) wave_exchange_fence();   // the next turn's activations go to the same LDS buffers
+    }
 
     // Over the sixteen blocks of the wavefront (lane bits 2 - 5), then over the wavefronts.
 #pragma unroll
@@ -669,7 +695,8 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
 template <int BITS, int SETS, int XT, int LOOKUP, int SLICES>
 void launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS), members.count > 0 ? members.count : 1);
-    const dim3 block(mk_cdiv(a.width, 512 * SLICES) * 64);
+    const bool long_rows = a.width > kMostRowCodes;   // two turns of half the row (rounded up to whole wavefronts)
+    const dim3 block(mk_cdiv(long_rows ? mk_cdiv(a.width, 2) : a.width, 512 * SLICES) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * 4 * blocks_sample_words(SLICES) * sizeof(uint32_t);
     // More than 64 KB of dynamic LDS has to be allowed per kernel (static LDS counts against
     // the CU's 160 KB too, so only what this launch needs is asked for).
@@ -682,6 +709,13 @@ void launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int
         }
         hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
     };
+    if constexpr (SLICES == 4 && SETS == 1) {   // (long rows take four samples per pass: launch_bits)
+        if (long_rows) {
+            if (a.zeros) launch(pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP, SLICES, false, true>);
+            else launch(pairs_blocks_kernel<BITS, SETS, false, XT, LOOKUP, SLICES, false, true>);
+            return;
+        }
+    }
     if constexpr (BITS == 8 && XT == MK_F16) {
         if (a.uniform) {   // no table: the bytes as fp16 subnormals
             if (a.zeros) launch(pairs_blocks_kernel<BITS, SETS, true, XT, LOOKUP, SLICES, true>);
@@ -703,6 +737,14 @@ void launch_blocks_with(const Stream4Args &a, const Stream4Group &members, int t
 template <int BITS, int MT, int XT, int LOOKUP>
 void launch_tile_with(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1);
+    if (a.width > kMostRowCodes) {   // two turns of half the row (rounded up to whole wavefronts)
+        const dim3 half(mk_cdiv(mk_cdiv(a.width, 2), 2048) * 64);
+        if (a.zeros)
+            hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP, kPairRows, false, true>), grid, half, 0, stream, a, members);
+        else
+            hipLaunchKernelGGL((pairs_kernel<BITS, MT, false, XT, LOOKUP, kPairRows, false, true>), grid, half, 0, stream, a, members);
+        return;
+    }
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
     if constexpr ((BITS == 2 || BITS == 3 || BITS == 8) && XT == MK_F16 && MT <= 2) {
         if (shifted_decoding(a)) {
@@ -781,7 +823,8 @@ void launch_blocks(const Stream4Args &a, const Stream4Group &members, int tiles,
 template <int BITS>
 void launch_bits(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     if (a.samples >= 3) {  // measured against the v_dot2 kernel at 4096 x 14336
-        if (a.samples <= 4) launch_blocks<BITS, 1>(a, members, tiles, stream);
+        // (two sets of four samples and a sum carried over the turns of a long row do not fit the registers)
+        if (a.samples <= 4 || a.width > kMostRowCodes) launch_blocks<BITS, 1>(a, members, tiles, stream);
         else launch_blocks<BITS, 2>(a, members, tiles, stream);
         return;
     }
@@ -793,7 +836,7 @@ void launch_bits(const Stream4Args &a, const Stream4Group &members, int tiles, h
 
 bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype) {
     return bits >= 2 && bits <= 8 && x_dtype != MK_F32 && scale_dtype != MK_F32 && width % kChunkCodes == 0 &&
-           width <= 16384 && (group % kChunkCodes == 0 || group >= width);
+           width <= 2 * kMostRowCodes && (group % kChunkCodes == 0 || group >= width);
 }
 
 namespace {

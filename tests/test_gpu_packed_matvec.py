@@ -170,6 +170,34 @@ def test_config3_sub_byte_and_codebook_codecs(name, shape):
         np.testing.assert_allclose(y, fp32_reference, rtol=2e-3, atol=2e-3)
 
 
+LONG_ROW_CODECS = dict(CODECS, **{
+    "int8-g128": dict(values=scaling.int_values(8), bits=8, group=128, integer=True),
+    "int5-g32": dict(values=scaling.int_values(5), bits=5, group=32, integer=True),
+    "int6-g64-asym": dict(values=scaling.int_values(6), bits=6, group=64, integer=True, asym=True),
+    "int2-g64-asym": dict(values=scaling.int_values(2), bits=2, group=64, integer=True, asym=True),
+})
+
+
+@pytest.mark.parametrize("name", LONG_ROW_CODECS)
+@pytest.mark.parametrize("rows,width", [(1040 + 3, 18944), (100, 28672), (48, 16384 + 64), (40, 32768)])
+def test_rows_of_more_than_16384_codes_of_every_codec(name, rows, width):
+    """The table kernels cover rows of 16416 to 32768 codes in two turns of the workgroup's width, adding the
+    turns' row sums before the reduction.  Every codec, one to eight samples, fp16 and bf16, with bias, ragged
+    row counts (rows past the last whole tile), against the float64 product."""
+    options = dict(LONG_ROW_CODECS[name])
+    values = options.pop("values")
+    layer = helpers.quantised_layer(helpers.normal_weight(rows, width, seed=width % 83, student_t=True), values, **options)
+    bias = helpers.activations(1, rows, seed=4)[0]
+    for dtype in (torch.float16, torch.bfloat16):
+        for samples in (1, 2, 3, 4, 5, 8):
+            x = helpers.activations(samples, width, seed=70 + samples, dtype=dtype)
+            y = run_matvec(layer, x, bias.to(dtype), scale_dtype=dtype)
+            sides = {key: None if layer[key] is None else torch.from_numpy(layer[key]).to(dtype).float().numpy()
+                     for key in ("scales", "zero")}
+            rounded = dict(layer, dense=scaling.decode_grouped(layer["codes"], sides["scales"], layer["values"], layer["group"], sides["zero"]))
+            check(y, rounded, x.float(), bias.to(dtype).float(), relative=1e-3 if dtype == torch.float16 else 8e-3)
+
+
 def test_metric_shape_int4_g128_4096x14336_all_row_counts():
     weight = helpers.normal_weight(4096, 14336, seed=9)
     layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True)
