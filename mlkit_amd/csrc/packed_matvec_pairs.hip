@@ -1,5 +1,5 @@
 // Packed matvec for 2- to 8-bit codes of any scalar grid (integer grids, NF4, small
-// codebooks) with fp16 or bf16 activations and 16-bit scales, rows of K = 32 ... 32768 codes (K % 32 == 0).
+// codebooks) with fp16 or bf16 activations and 16-bit scales, rows of K = 32 ... 131072 codes (K % 32 == 0).
 //
 // Adjacent codes (one, two or four, by code width) index a table of 16-bit values held in
 // LDS, so one LDS read decodes up to four weights and one v_dot2_f32_f16 (v_dot2_f32_bf16)
@@ -43,9 +43,10 @@ __device__ __forceinline__ float side_value(uint16_t raw, int dtype) {
 // (two per CU at 4096 rows); short rows keep sixteen rows per table fill.
 constexpr int kShortTileRows = 8;
 constexpr int kShortTileWidth = 4096;
-// A workgroup of eight wavefronts covers 16384 codes of a row at once; longer rows (up to twice that) take two
-// turns (the LONG kernels), with sixteen rows per workgroup and table decoding.
+// A workgroup of eight wavefronts covers 16384 codes of a row at once; longer rows (up to eight times that) take
+// several turns (the LONG kernels), with sixteen rows per workgroup and table decoding.
 constexpr int kMostRowCodes = 16384;
+constexpr int kMostTurns = 8;
 // Uniform 2-, 3- and 8-bit grids with fp16 activations, one or two samples: decoded by shifts and masks.
 inline bool shifted_decoding(const Stream4Args &a) {
     return a.uniform && a.x_dtype == MK_F16 && (a.bits == 2 || a.bits == 3 || a.bits == 8) && a.samples <= 2 && a.width <= kMostRowCodes;
@@ -695,8 +696,8 @@ __global__ void __launch_bounds__(512) pairs_blocks_kernel(const Stream4Args a, 
 template <int BITS, int SETS, int XT, int LOOKUP, int SLICES>
 void launch_blocks_sliced(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, 4 * SETS), members.count > 0 ? members.count : 1);
-    const bool long_rows = a.width > kMostRowCodes;   // two turns of half the row (rounded up to whole wavefronts)
-    const dim3 block(mk_cdiv(long_rows ? mk_cdiv(a.width, 2) : a.width, 512 * SLICES) * 64);
+    const bool long_rows = a.width > kMostRowCodes;   // several turns of an equal share of the row (in whole wavefronts)
+    const dim3 block(mk_cdiv(long_rows ? mk_cdiv(a.width, mk_cdiv(a.width, kMostRowCodes)) : a.width, 512 * SLICES) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * 4 * blocks_sample_words(SLICES) * sizeof(uint32_t);
     // More than 64 KB of dynamic LDS has to be allowed per kernel (static LDS counts against
     // the CU's 160 KB too, so only what this launch needs is asked for).
@@ -737,8 +738,8 @@ void launch_blocks_with(const Stream4Args &a, const Stream4Group &members, int t
 template <int BITS, int MT, int XT, int LOOKUP>
 void launch_tile_with(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     const dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1);
-    if (a.width > kMostRowCodes) {   // two turns of half the row (rounded up to whole wavefronts)
-        const dim3 half(mk_cdiv(mk_cdiv(a.width, 2), 2048) * 64);
+    if (a.width > kMostRowCodes) {   // several turns of an equal share of the row (in whole wavefronts)
+        const dim3 half(mk_cdiv(mk_cdiv(a.width, mk_cdiv(a.width, kMostRowCodes)), 2048) * 64);
         if (a.zeros)
             hipLaunchKernelGGL((pairs_kernel<BITS, MT, true, XT, LOOKUP, kPairRows, false, true>), grid, half, 0, stream, a, members);
         else
@@ -836,7 +837,7 @@ void launch_bits(const Stream4Args &a, const Stream4Group &members, int tiles, h
 
 bool pairs_accepts(int width, int group, int bits, int x_dtype, int scale_dtype) {
     return bits >= 2 && bits <= 8 && x_dtype != MK_F32 && scale_dtype != MK_F32 && width % kChunkCodes == 0 &&
-           width <= 2 * kMostRowCodes && (group % kChunkCodes == 0 || group >= width);
+           width <= kMostTurns * kMostRowCodes && (group % kChunkCodes == 0 || group >= width);
 }
 
 namespace {

@@ -103,6 +103,7 @@ def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
     (260, 28672, 128, True),         # four-row tiles, seven wavefronts
     (70, 32768, 64, True),           # the longest row
     (48, 16384 + 32, 32, False),     # one chunk in the second span
+    (37, 53248, 128, True),          # beyond two spans: the table kernel's turns
 ])
 def test_rows_of_more_than_16384_codes(rows, width, group, asym):
     """Down projections of the larger decoders (K = 18944, 28672): every wavefront owns two spans of 2048 codes.
@@ -179,9 +180,9 @@ LONG_ROW_CODECS = dict(CODECS, **{
 
 
 @pytest.mark.parametrize("name", LONG_ROW_CODECS)
-@pytest.mark.parametrize("rows,width", [(1040 + 3, 18944), (100, 28672), (48, 16384 + 64), (40, 32768)])
+@pytest.mark.parametrize("rows,width", [(1040 + 3, 18944), (100, 28672), (48, 16384 + 64), (40, 32768), (35, 53248)])
 def test_rows_of_more_than_16384_codes_of_every_codec(name, rows, width):
-    """The table kernels cover rows of 16416 to 32768 codes in two turns of the workgroup's width, adding the
+    """The table kernels cover rows of more than 16384 codes in several turns of the workgroup's width, adding the
     turns' row sums before the reduction.  Every codec, one to eight samples, fp16 and bf16, with bias, ragged
     row counts (rows past the last whole tile), against the float64 product."""
     options = dict(LONG_ROW_CODECS[name])
