@@ -225,7 +225,19 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
     int done_rows = 0;  // rows [0, done_rows) are covered by a chunked kernel
     Plan plan;
     if (aligned && !tuning().no_stream4 &&
-        mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
+        mk_matvec::long_accepts(samples, output_width, input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
+        (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
+        mk_matvec::Stream4Args s4;
+        s4.x = x; s4.packed = packed; s4.scales = scales; s4.zeros = zeros; s4.bias = bias; s4.y = y;
+        s4.samples = samples; s4.rows = output_width; s4.width = input_width; s4.group = group;
+        s4.groups = groups; s4.bias_dtype = bias_dtype; s4.grid_min = grid_min; s4.grid_step = grid_step;
+        s4.values = values; s4.n_values = n_values; s4.uniform = uniform; s4.bits = bits;
+        s4.x_dtype = x_dtype; s4.scale_dtype = scale_dtype;
+        done_rows = mk_matvec::long_launch(s4, stream);
+        MK_REQUIRE(done_rows >= 0, MK_ERR_HIP, "mk_packed_matvec: the runtime refused the kernel's launch");
+        if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
+    } else if (aligned && !tuning().no_stream4 &&
+               mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
         (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
         mk_matvec::Stream4Args s4;
         s4.x = x; s4.packed = packed; s4.scales = scales; s4.zeros = zeros; s4.bias = bias; s4.y = y;
@@ -235,18 +247,6 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
         s4.x_dtype = x_dtype; s4.scale_dtype = scale_dtype;
         done_rows = mk_matvec::stream4_launch(s4, stream);
         MK_REQUIRE(done_rows >= 0, MK_ERR_HIP, "mk_packed_matvec: the runtime refused the kernel's LDS size");
-        if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
-    } else if (aligned && !tuning().no_stream4 &&
-               mk_matvec::long_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
-               (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
-        mk_matvec::Stream4Args s4;
-        s4.x = x; s4.packed = packed; s4.scales = scales; s4.zeros = zeros; s4.bias = bias; s4.y = y;
-        s4.samples = samples; s4.rows = output_width; s4.width = input_width; s4.group = group;
-        s4.groups = groups; s4.bias_dtype = bias_dtype; s4.grid_min = grid_min; s4.grid_step = grid_step;
-        s4.values = values; s4.n_values = n_values; s4.uniform = uniform; s4.bits = bits;
-        s4.x_dtype = x_dtype; s4.scale_dtype = scale_dtype;
-        done_rows = mk_matvec::long_launch(s4, stream);
-        MK_REQUIRE(done_rows >= 0, MK_ERR_HIP, "mk_packed_matvec: the runtime refused the kernel's launch");
         if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
     } else if (aligned && !tuning().no_pairs &&
                mk_matvec::pairs_accepts(input_width, group, bits, x_dtype, scale_dtype) &&

@@ -159,9 +159,10 @@ int pairs_launch_group(const Stream4Args &shared, Stream4Group &group, const int
                        hipStream_t stream);
 bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
-// 4-bit uniform-grid codes in rows of 16416 to 32768 codes, fp16 or bf16 activations (packed_matvec_long.hip):
+// 4-bit uniform-grid codes in rows of 16416 to 32768 codes, and one or two samples of some shorter rows, fp16 or bf16
+// activations (packed_matvec_long.hip: a wavefront owns two spans of 2048 codes):
 // multiplies the leading whole tiles of rows and returns the number of rows covered, or -1.
-bool long_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
+bool long_accepts(int samples, int rows, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int long_launch(const Stream4Args &a, hipStream_t stream);
 // Three to eight samples of fp32 activations against 4-bit uniform-grid codes as integer matrix-core blocks
 // (packed_matvec_digits.hip): `tiles` tiles of `rows_per_tile` rows of the single matrix or of every member.

@@ -38,9 +38,11 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
     // bf16: with the exponent of 128 inserted, taken out again through the sum of the activations.
     constexpr bool kSubnormalCodes = XT == MK_F16;
     const float code_step = kSubnormalCodes ? a.grid_step * 16777216.0f : a.grid_step;
-    constexpr int kAhead = ROWS < 4 ? ROWS : 4;   // rows of codes in flight: two pieces each
-    constexpr int kSums = ROWS * MT;
-    __shared__ float partials[64 * 8];  // [row sum][wavefront]
+    constexpr int kAhead = ROWS < 4 ? ROWS : 4;   // rows of codes in flight, two pieces each (six and eight rows measured slower)
+    constexpr int kSums = ROWS * MT;              // row sums of the tile; every span keeps its own until the end
+    constexpr int kSlots = 16;                    // spans of the workgroup: at most eight wavefronts of two
+    static_assert(kSpans * kSums <= 64, "one transposed reduction per workgroup");
+    __shared__ float partials[kSums * kSlots];  // [row sum][span of the row]
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
     uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
 
@@ -126,12 +128,11 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
             grid_term[s][m] = a.grid_min * x_sum[s][m] - a.grid_step * code_free;
         }
 
-    float sums[kSums];
+    // A span's sums stay apart from the other span's: span s of wavefront w is what wavefront s * waves + w of the
+    // streaming kernel sums, and the spans meet in that order, so a row's result equals that kernel's bit for bit.
+    float sums[kSpans * kSums];
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-        float value[MT];
-#pragma unroll
-        for (int m = 0; m < MT; ++m) value[m] = 0.0f;
 #pragma unroll
         for (int s = 0; s < kSpans; ++s) {
             float dot[MT];
@@ -140,24 +141,27 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
             const float scale = side_of(scale_raw[r][s]);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-                value[m] = __builtin_fmaf(scale, __builtin_fmaf(code_step, dot[m], grid_term[s][m]), value[m]);
-                if constexpr (HAS_ZERO) value[m] = __builtin_fmaf(side_of(zero_raw[r][s]), x_sum[s][m], value[m]);
+                float value = scale * __builtin_fmaf(code_step, dot[m], grid_term[s][m]);
+                if constexpr (HAS_ZERO) value = __builtin_fmaf(side_of(zero_raw[r][s]), x_sum[s][m], value);
+                sums[s * kSums + r * MT + m] = value;
             }
         }
         if (r + kAhead < ROWS) request_row(r + kAhead);
-#pragma unroll
-        for (int m = 0; m < MT; ++m) sums[r * MT + m] = value[m];
         __builtin_amdgcn_sched_barrier(0);  // rows in arrival order, temporaries short-lived
     }
 
-    // All row sums over the lanes at once, then over the wavefronts.
-    transposed_wave_sum<kSums, 0, 6>(sums, lane);
-    if (lane < kSums) partials[transposed_value_of_lane<kSums>(lane) * 8 + wave] = sums[0];
+    // All sums over the lanes at once, then over the spans of the row in ascending order.
+    transposed_wave_sum<kSpans * kSums, 0, 6>(sums, lane);
+    if (lane < kSpans * kSums) {
+        const int value = transposed_value_of_lane<kSpans * kSums>(lane);
+        const int span = value / kSums;
+        partials[(value - span * kSums) * kSlots + span * waves + wave] = sums[0];
+    }
     __syncthreads();
     if (tid < kSums) {
-        float total = partials[tid * 8];
+        float total = partials[tid * kSlots];
 #pragma unroll
-        for (int w = 1; w < 8; ++w) total += w < waves ? partials[tid * 8 + w] : 0.0f;
+        for (int w = 1; w < kSlots; ++w) total += w < kSpans * waves ? partials[tid * kSlots + w] : 0.0f;
         const int j = tid / MT, m = tid - j * MT;
         const int row = row_base + j;
         const int sample = sample_base + m;
@@ -456,12 +460,26 @@ int launch_tiles(const Stream4Args &a, hipStream_t stream) {
 
 }  // namespace
 
-bool long_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform) {
-    // one and two samples with 16-bit or fp32 scales, more samples with 16-bit scales (as for shorter rows)
+bool long_accepts(int samples, int rows, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform) {
     const bool whole_chunks = group % kChunkCodes == 0 || group >= width;
-    const bool power_of_two = (group & (group - 1)) == 0 || group >= width;   // the matrix-core kernel shifts instead of dividing
-    return bits == 4 && uniform && (samples <= 2 || (scale_dtype != MK_F32 && power_of_two)) &&
-           (x_dtype == MK_F16 || x_dtype == MK_BF16) && width > 16384 && width <= 32768 && width % kChunkCodes == 0 && whole_chunks;
+    if (!(bits == 4 && uniform && (x_dtype == MK_F16 || x_dtype == MK_BF16) && width % kChunkCodes == 0 && whole_chunks && width <= 32768))
+        return false;
+    if (width > 16384) {
+        // one and two samples with 16-bit or fp32 scales, more samples with 16-bit scales (as for shorter rows)
+        const bool power_of_two = (group & (group - 1)) == 0 || group >= width;   // the matrix-core kernel shifts instead of dividing
+        return samples <= 2 || (scale_dtype != MK_F32 && power_of_two);
+    }
+    // Shorter rows, one and two samples: rows of five to seven wavefronts leave one of a compute unit's four SIMDs
+    // with half the work of the others (seven wavefronts: 2, 2, 2, 1); as three or four wavefronts of two spans every
+    // SIMD holds one, and a wavefront's fixed costs are paid once for two spans.  Results are the streaming kernel's
+    // bit for bit.  Measured (M = 1 / 2): 4096 x 14336 7.1 -> 6.95 / 8.3 -> 7.85 us, 4096 x 11008 6.4 -> 6.05 / 7.8 -> 7.6,
+    // 8192 x 12288 10.9 -> 10.7 / 13.6 -> 12.85, 3584 x 14336 7.0 -> 6.45 / 9.3 -> 7.8, 4096 x 10240 6.25 -> 5.9 (7.4 -> 7.6
+    // with two samples: not taken); eight wavefronts (4096 x 16384: 7.6 -> 7.7), layers of fewer than 224 tiles
+    // (2048 x 11008: 4.7 -> 5.7) and those whose second round of tiles is at most half full (6144 x 14336: 9.85 ->
+    // 10.05; the streaming kernel takes eight-row tiles there) are slower and stay.
+    const int row_waves = mk_cdiv(width, 2048), wide_tiles = rows / 16;
+    const bool sparse_round = wide_tiles > kComputeUnits && wide_tiles <= kComputeUnits + kComputeUnits / 2;
+    return samples <= 2 && wide_tiles >= 224 && !sparse_round && (row_waves == 6 || row_waves == 7 || (row_waves == 5 && samples == 1));
 }
 
 // Multiplies the leading whole tiles of rows; returns the number of rows covered.
