@@ -42,8 +42,8 @@ RECORDED_TRAFFIC = {
     "single": {"bytes_per_launch": 30_736_800,
                "source": "profiles/packed_matvec_long_rows_int4_g128_4096x14336_m1.md (rocprofv3 --pmc FETCH_SIZE, then "
                          "WRITE_SIZE); recorded there, not measured in this run"},
-    "group_of_8": {"bytes_per_launch": 8 * 30_331_800,
-                   "source": "profiles/packed_matvec_stream4_int4_g128_4096x14336_m1_group8.md (rocprofv3 --pmc FETCH_SIZE, "
+    "group_of_8": {"bytes_per_launch": 243_530_736,
+                   "source": "profiles/packed_matvec_long_rows_int4_g128_4096x14336_m1_group8.md (rocprofv3 --pmc FETCH_SIZE, "
                              "then WRITE_SIZE of the 8-matrix launch); recorded there, not measured in this run"},
 }
 
@@ -784,7 +784,7 @@ def main() -> None:
         },
         "roofline": {
             "kernel": ("long_rows_kernel<1,false,16,f16> (one launch per step)" if members == 1 else
-                       f"stream4_kernel<1,false,16,f16,1> (one grouped launch of {members} matrices per step)"),
+                       f"long_rows_kernel<1,false,16,f16> (one grouped launch of {members} matrices per step)"),
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,

@@ -164,6 +164,8 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream);
 // multiplies the leading whole tiles of rows and returns the number of rows covered, or -1.
 bool long_accepts(int samples, int rows, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int long_launch(const Stream4Args &a, hipStream_t stream);
+bool long_group_accepts(const Stream4Args &shared, const Stream4Group &group, const int *member_rows);
+int long_launch_group(const Stream4Args &shared, Stream4Group &group, const int *member_rows, int *rows_per_tile, hipStream_t stream);
 // Three to eight samples of fp32 activations against 4-bit uniform-grid codes as integer matrix-core blocks
 // (packed_matvec_digits.hip): `tiles` tiles of `rows_per_tile` rows of the single matrix or of every member.
 bool digits_accepts(const Stream4Args &a, int rows_per_tile);

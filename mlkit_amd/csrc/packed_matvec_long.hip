@@ -173,15 +173,12 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
 }
 
 template <int MT, int ROWS>
-int launch_rows_of(const Stream4Args &a, int tiles, hipStream_t stream) {
+int launch_rows_of(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     if (tiles == 0) return 0;
-    Stream4Group none;
-    none.count = 0;
-    none.widest_tiles = 0;
-    const dim3 grid(tiles, mk_cdiv(a.samples, MT), 1), block(mk_cdiv(a.width, 2048 * kSpans) * 64);
+    const dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1), block(mk_cdiv(a.width, 2048 * kSpans) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
     auto launch = [&](auto kernel) -> int {
-        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, none);
+        hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
         return 0;
     };
     auto of = [&](auto has_zero, auto wide) -> int {
@@ -453,8 +450,11 @@ int launch_blocks_of(const Stream4Args &a, hipStream_t stream) {
 
 template <int ROWS>
 int launch_tiles(const Stream4Args &a, hipStream_t stream) {
+    Stream4Group none;
+    none.count = 0;
+    none.widest_tiles = 0;
     const int tiles = a.rows / ROWS;
-    const int status = a.samples == 1 ? launch_rows_of<1, ROWS>(a, tiles, stream) : launch_rows_of<2, ROWS>(a, tiles, stream);
+    const int status = a.samples == 1 ? launch_rows_of<1, ROWS>(a, none, tiles, stream) : launch_rows_of<2, ROWS>(a, none, tiles, stream);
     return status ? -1 : tiles * ROWS;
 }
 
@@ -480,6 +480,35 @@ bool long_accepts(int samples, int rows, int width, int group, int bits, int x_d
     const int row_waves = mk_cdiv(width, 2048), wide_tiles = rows / 16;
     const bool sparse_round = wide_tiles > kComputeUnits && wide_tiles <= kComputeUnits + kComputeUnits / 2;
     return samples <= 2 && wide_tiles >= 224 && !sparse_round && (row_waves == 6 || row_waves == 7 || (row_waves == 5 && samples == 1));
+}
+
+// Up to eight matrices of one input width in one launch of the two-span kernel: the members' whole tiles of
+// sixteen rows (`rows_per_tile` receives 16).  For one and two samples of rows of six and seven wavefronts (five
+// with one sample) when the members bring at least a tile per compute unit together; results equal the streaming
+// kernel's, and the single call's, bit for bit.
+bool long_group_accepts(const Stream4Args &shared, const Stream4Group &group, const int *member_rows) {
+    if (!(shared.bits == 4 && shared.uniform && (shared.x_dtype == MK_F16 || shared.x_dtype == MK_BF16) && shared.samples <= 2 &&
+          shared.width <= 16384))
+        return false;
+    const int row_waves = mk_cdiv(shared.width, 2048);
+    if (!(row_waves == 6 || row_waves == 7 || (row_waves == 5 && shared.samples == 1))) return false;
+    long long wide_tiles = 0;
+    for (int i = 0; i < group.count; ++i) wide_tiles += member_rows[i] / 16;
+    return wide_tiles >= kComputeUnits;
+}
+
+int long_launch_group(const Stream4Args &shared, Stream4Group &group, const int *member_rows, int *rows_per_tile, hipStream_t stream) {
+    int widest = 0;
+    for (int i = 0; i < group.count; ++i) {
+        group.member[i].rows = member_rows[i];
+        group.member[i].tiles = member_rows[i] / 16;
+        if (group.member[i].tiles > widest) widest = group.member[i].tiles;
+    }
+    group.widest_tiles = widest;
+    *rows_per_tile = 16;
+    Stream4Args a = shared;
+    a.zeros = group.member[0].zeros;  // selects the kernel variant; the members agree on it
+    return a.samples == 1 ? launch_rows_of<1, 16>(a, group, widest, stream) : launch_rows_of<2, 16>(a, group, widest, stream);
 }
 
 // Multiplies the leading whole tiles of rows; returns the number of rows covered.

@@ -874,6 +874,7 @@ int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream) {
 
 int stream4_launch_group(const Stream4Args &shared, Stream4Group &group, const int *member_rows, int *rows_per_tile,
                          hipStream_t stream) {
+    if (long_group_accepts(shared, group, member_rows)) return long_launch_group(shared, group, member_rows, rows_per_tile, stream);
     long long wide_tiles = 0;
     for (int i = 0; i < group.count; ++i) wide_tiles += member_rows[i] / kWideRows;
     const int rows = wide_tiles >= kComputeUnits ? kWideRows : kNarrowRows;
