@@ -39,10 +39,9 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
     constexpr bool kSubnormalCodes = XT == MK_F16;
     const float code_step = kSubnormalCodes ? a.grid_step * 16777216.0f : a.grid_step;
     constexpr int kAhead = ROWS < 4 ? ROWS : 4;   // rows of codes in flight, two pieces each (six and eight rows measured slower)
-    constexpr int kSums = ROWS * MT;              // row sums of the tile; every span keeps its own until the end
-    constexpr int kSlots = 16;                    // spans of the workgroup: at most eight wavefronts of two
-    static_assert(kSpans * kSums <= 64, "one transposed reduction per workgroup");
-    __shared__ float partials[kSums * kSlots];  // [row sum][span of the row]
+    constexpr int kSums = ROWS * MT;              // row sums of the tile
+    constexpr int kSlots = 8;                     // wavefronts of the workgroup
+    __shared__ float partials[kSums * kSlots];  // [row sum][wavefront]
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
     uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
 
@@ -128,9 +127,10 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
             grid_term[s][m] = a.grid_min * x_sum[s][m] - a.grid_step * code_free;
         }
 
-    // A span's sums stay apart from the other span's: span s of wavefront w is what wavefront s * waves + w of the
-    // streaming kernel sums, and the spans meet in that order, so a row's result equals that kernel's bit for bit.
-    float sums[kSpans * kSums];
+    // A lane adds its second span's term to its first span's, then the lanes of the wavefront meet, then the
+    // wavefronts in ascending order.  The streaming kernel sums rows of six and seven wavefronts in this order too
+    // (its wavefront w + waves hands its terms to wavefront w), so a row's result equals that kernel's bit for bit.
+    float sums[kSums];
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
 #pragma unroll
@@ -141,27 +141,25 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
             const float scale = side_of(scale_raw[r][s]);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
+#pragma clang fp contract(off)   // the span's term is rounded before it meets the other span's, as between wavefronts
                 float value = scale * __builtin_fmaf(code_step, dot[m], grid_term[s][m]);
                 if constexpr (HAS_ZERO) value = __builtin_fmaf(side_of(zero_raw[r][s]), x_sum[s][m], value);
-                sums[s * kSums + r * MT + m] = value;
+                if (s == 0) sums[r * MT + m] = value;
+                else sums[r * MT + m] += value;
             }
         }
         if (r + kAhead < ROWS) request_row(r + kAhead);
         __builtin_amdgcn_sched_barrier(0);  // rows in arrival order, temporaries short-lived
     }
 
-    // All sums over the lanes at once, then over the spans of the row in ascending order.
-    transposed_wave_sum<kSpans * kSums, 0, 6>(sums, lane);
-    if (lane < kSpans * kSums) {
-        const int value = transposed_value_of_lane<kSpans * kSums>(lane);
-        const int span = value / kSums;
-        partials[(value - span * kSums) * kSlots + span * waves + wave] = sums[0];
-    }
+    // All sums over the lanes at once, then over the wavefronts in ascending order.
+    transposed_wave_sum<kSums, 0, 6>(sums, lane);
+    if (lane < kSums) partials[transposed_value_of_lane<kSums>(lane) * kSlots + wave] = sums[0];
     __syncthreads();
     if (tid < kSums) {
         float total = partials[tid * kSlots];
 #pragma unroll
-        for (int w = 1; w < kSlots; ++w) total += w < kSpans * waves ? partials[tid * kSlots + w] : 0.0f;
+        for (int w = 1; w < kSlots; ++w) total += w < waves ? partials[tid * kSlots + w] : 0.0f;
         const int j = tid / MT, m = tid - j * MT;
         const int row = row_base + j;
         const int sample = sample_base + m;
@@ -458,6 +456,37 @@ int launch_tiles(const Stream4Args &a, hipStream_t stream) {
     return status ? -1 : tiles * ROWS;
 }
 
+// Rows of at most 16384 codes, one and two samples: rows of six and seven wavefronts leave a compute unit's four
+// SIMDs with unequal work (seven wavefronts: 2, 2, 2, 1); as three or four wavefronts of two spans
+// every SIMD holds one, and a wavefront's fixed costs are paid once for two spans.  Results are the streaming
+// kernel's bit for bit (it sums such rows in this kernel's order).  Returns the rows per tile, or 0 where the
+// streaming kernel is as fast or faster.
+//
+// A workgroup costs about four rows' worth of time before its first row (all of x read and prepared), and a launch
+// takes as many rounds as its tiles need on 256 compute units: the tile height with the lowest
+// rounds x (4 + height) wins.  Measured against the streaming kernel (M = 1 / 2, us): 4096 x 14336 6.98 -> 6.76 / 7.88 ->
+// 7.76 and 4096 x 11008 6.07 -> 5.82 / 7.73 -> 7.43 (sixteen rows), 2048 x 14336 5.33 -> 4.81 / 6.42 -> 5.61, 2048 x 11008
+// 4.92 -> 4.30 / 6.03 -> 5.36 and 6144 x 14336 9.89 -> 9.68 / 12.4 -> 12.1 (eight), 1024 x 14336 4.08 -> 3.83 (four, one
+// sample; two: 4.51 -> 4.63, not taken).  Not taken: fewer than 192 tiles (512 x 14336: 3.61 -> 3.61 / 4.21 -> 4.61), rows
+// of five wavefronts (three wavefronts of 2, 2 and 1 spans: 2560 x 10240 5.13 -> 5.65, 1536 x 8960 4.1 -> 4.2 / 5.0 -> 5.3;
+// only one sample of tall layers gained, 4096 x 10240 6.25 -> 5.9), eight wavefronts (4096 x 16384: 7.6 -> 7.7), layers
+// whose second round of sixteen-row tiles is at most half full (5120 x 12288: 8.0 -> 8.6 with eight-row tiles).
+int two_span_tile_rows(int samples, int rows, int width) {
+    const int row_waves = mk_cdiv(width, 2048);
+    if (samples > 2 || row_waves < 6 || row_waves > 7) return 0;
+    // a second round of sixteen-row tiles at most half full: the streaming kernel's eight-row tiles are as fast
+    if (rows / 16 > kComputeUnits && rows / 16 <= kComputeUnits + kComputeUnits / 2) return 0;
+    int best = 0, best_cost = 0;
+    for (int height = 16; height >= 4; height /= 2) {
+        const int tiles = rows / height;
+        if (tiles == 0) continue;
+        const int cost = mk_cdiv(tiles, kComputeUnits) * (4 + height);
+        if (best == 0 || cost < best_cost) best = height, best_cost = cost;
+    }
+    if (best == 0 || rows / best < 192 || (best == 4 && samples == 2)) return 0;
+    return best;
+}
+
 }  // namespace
 
 bool long_accepts(int samples, int rows, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform) {
@@ -469,29 +498,19 @@ bool long_accepts(int samples, int rows, int width, int group, int bits, int x_d
         const bool power_of_two = (group & (group - 1)) == 0 || group >= width;   // the matrix-core kernel shifts instead of dividing
         return samples <= 2 || (scale_dtype != MK_F32 && power_of_two);
     }
-    // Shorter rows, one and two samples: rows of five to seven wavefronts leave one of a compute unit's four SIMDs
-    // with half the work of the others (seven wavefronts: 2, 2, 2, 1); as three or four wavefronts of two spans every
-    // SIMD holds one, and a wavefront's fixed costs are paid once for two spans.  Results are the streaming kernel's
-    // bit for bit.  Measured (M = 1 / 2): 4096 x 14336 7.1 -> 6.95 / 8.3 -> 7.85 us, 4096 x 11008 6.4 -> 6.05 / 7.8 -> 7.6,
-    // 8192 x 12288 10.9 -> 10.7 / 13.6 -> 12.85, 3584 x 14336 7.0 -> 6.45 / 9.3 -> 7.8, 4096 x 10240 6.25 -> 5.9 (7.4 -> 7.6
-    // with two samples: not taken); eight wavefronts (4096 x 16384: 7.6 -> 7.7), layers of fewer than 224 tiles
-    // (2048 x 11008: 4.7 -> 5.7) and those whose second round of tiles is at most half full (6144 x 14336: 9.85 ->
-    // 10.05; the streaming kernel takes eight-row tiles there) are slower and stay.
-    const int row_waves = mk_cdiv(width, 2048), wide_tiles = rows / 16;
-    const bool sparse_round = wide_tiles > kComputeUnits && wide_tiles <= kComputeUnits + kComputeUnits / 2;
-    return samples <= 2 && wide_tiles >= 224 && !sparse_round && (row_waves == 6 || row_waves == 7 || (row_waves == 5 && samples == 1));
+    return two_span_tile_rows(samples, rows, width) != 0;
 }
 
 // Up to eight matrices of one input width in one launch of the two-span kernel: the members' whole tiles of
-// sixteen rows (`rows_per_tile` receives 16).  For one and two samples of rows of six and seven wavefronts (five
-// with one sample) when the members bring at least a tile per compute unit together; results equal the streaming
+// sixteen rows (`rows_per_tile` receives 16).  For one and two samples of rows of six and seven wavefronts
+// when the members bring at least a tile per compute unit together; results equal the streaming
 // kernel's, and the single call's, bit for bit.
 bool long_group_accepts(const Stream4Args &shared, const Stream4Group &group, const int *member_rows) {
     if (!(shared.bits == 4 && shared.uniform && (shared.x_dtype == MK_F16 || shared.x_dtype == MK_BF16) && shared.samples <= 2 &&
           shared.width <= 16384))
         return false;
     const int row_waves = mk_cdiv(shared.width, 2048);
-    if (!(row_waves == 6 || row_waves == 7 || (row_waves == 5 && shared.samples == 1))) return false;
+    if (!(row_waves == 6 || row_waves == 7)) return false;
     long long wide_tiles = 0;
     for (int i = 0; i < group.count; ++i) wide_tiles += member_rows[i] / 16;
     return wide_tiles >= kComputeUnits;
@@ -525,6 +544,10 @@ int long_launch(const Stream4Args &a, hipStream_t stream) {
         if ((a.rows / 4) * passes <= kComputeUnits) return launch_blocks_of<4>(a, stream);
         if ((a.rows / 8) * passes <= kComputeUnits) return launch_blocks_of<8>(a, stream);
         return launch_blocks_of<16>(a, stream);
+    }
+    if (a.width <= 16384) {
+        const int height = two_span_tile_rows(a.samples, a.rows, a.width);
+        return height == 4 ? launch_tiles<4>(a, stream) : height == 8 ? launch_tiles<8>(a, stream) : launch_tiles<16>(a, stream);
     }
     if (wide_tiles > kComputeUnits && wide_tiles <= kComputeUnits + kComputeUnits / 2) return launch_tiles<8>(a, stream);
     if (wide_tiles >= kComputeUnits / 2) return launch_tiles<16>(a, stream);

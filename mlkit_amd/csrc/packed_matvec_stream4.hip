@@ -162,6 +162,9 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
     constexpr int kStreamAhead = rows_ahead_of<kStreamRows>();  // (with ROTATE too: all 16 rows ahead measured slower)
     constexpr int kSums = kStreamRows * MT;
     constexpr int kRowLanes = 64 / PARTS;
+    constexpr bool kSpansMeet = !SPLIT && PARTS == 1 && MT <= 2;
+    // words of a wavefront's share of the dynamic LDS that precedes the handed-over terms
+    const uint32_t handed_after_words = ROTATE && a.rotate_log_block > 11 ? 64u * kChunkCodes : static_cast<uint32_t>(kSliceWords);
 
     const TileSource source = tile_source<ROWS>(a, members, blockIdx.z);
     if (static_cast<int>(blockIdx.x) >= source.tiles) return;  // a shorter member of a group: the whole workgroup leaves
@@ -327,16 +330,39 @@ __device__ __forceinline__ void stream4_body(const Stream4Args &a, const Stream4
         __builtin_amdgcn_sched_barrier(0);
     }
 
+    // One and two 16-bit samples of rows of six and seven wavefronts: the upper wavefronts hand their terms, lane by
+    // lane, to the wavefronts `meeting` below them, which add them to their own before the lanes meet.  That is the
+    // order in which the two-span kernel (a wavefront owns both spans, packed_matvec_long.hip) sums such a row, and
+    // the single call, the grouped launch and the rotating kernel promise each other's results bit for bit.
+    int meeting = waves;   // wavefronts whose sums reach `partials`
+    if constexpr (kSpansMeet) {
+        if (waves == 6 || waves == 7) {   // uniform
+            meeting = (waves + 1) >> 1;
+            float *const handed = reinterpret_cast<float *>(x_slices_storage + waves * handed_after_words);
+            if (wave >= meeting) {
+#pragma unroll
+                for (int j = 0; j < kSums; ++j) handed[((wave - meeting) * kSums + j) * 64 + lane] = sums[j];
+            }
+            __syncthreads();
+            if (wave + meeting < waves) {
+#pragma unroll
+                for (int j = 0; j < kSums; ++j) sums[j] += handed[(wave * kSums + j) * 64 + lane];
+            }
+        }
+    }
+
     // All row sums over the lanes of a row at once, then over the wavefronts.
-    transposed_wave_sum<kSums, 0, PARTS == 1 ? 6 : 5>(sums, lane);
-    const int lane_in_row = lane & (kRowLanes - 1);
-    if (lane_in_row < kSums)
-        partials[(transposed_value_of_lane<kSums>(lane_in_row) * PARTS + part) * 8 + wave] = sums[0];
+    if (wave < meeting) {   // uniform per wavefront
+        transposed_wave_sum<kSums, 0, PARTS == 1 ? 6 : 5>(sums, lane);
+        const int lane_in_row = lane & (kRowLanes - 1);
+        if (lane_in_row < kSums)
+            partials[(transposed_value_of_lane<kSums>(lane_in_row) * PARTS + part) * 8 + wave] = sums[0];
+    }
     __syncthreads();
     if (tid < kSums * PARTS) {
         float total = partials[tid * 8];
 #pragma unroll
-        for (int w = 1; w < 8; ++w) total += w < waves ? partials[tid * 8 + w] : 0.0f;
+        for (int w = 1; w < 8; ++w) total += w < meeting ? partials[tid * 8 + w] : 0.0f;
         const int value = tid / PARTS, j = value / MT, m = value - j * MT;
         const int row = row_base + PARTS * j + (tid - value * PARTS);
         const int sample = sample_base + m;
@@ -684,12 +710,29 @@ int launch_blocks(const Stream4Args &a, const Stream4Group &members, int tiles, 
     return launch_blocks_sliced<SETS, ROWS, 4>(a, members, tiles, stream);
 }
 
+// LDS for the terms that the upper wavefronts of a row of six or seven hand to the lower ones (stream4_body).
+size_t handed_terms_bytes(int row_waves, int sums) {
+    if (row_waves != 6 && row_waves != 7) return 0;
+    return static_cast<size_t>(row_waves - ((row_waves + 1) >> 1)) * sums * 64 * sizeof(float);
+}
+
 template <int MT, int ROWS, int PARTS>
 int launch_tile_parts(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1);
     const dim3 block(mk_cdiv(a.width, 2048) * 64);
-    const size_t slices = static_cast<size_t>(block.x / 64) * (a.x_dtype == MK_F32 ? kPlaneSliceWords : kSliceWords) * sizeof(uint32_t);
+    const int row_waves = static_cast<int>(block.x / 64);
+    size_t slices = static_cast<size_t>(row_waves) * (a.x_dtype == MK_F32 ? kPlaneSliceWords : kSliceWords) * sizeof(uint32_t);
+    if (a.x_dtype != MK_F32 && PARTS == 1 && MT <= 2) slices += handed_terms_bytes(row_waves, (ROWS / PARTS) * MT);
     auto launch = [&](auto kernel) -> int {
+        if (slices > 48 * 1024) {
+            static std::atomic<bool> raised{false};
+            if (!raised.load(std::memory_order_relaxed)) {
+                if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        64 * 1024) != hipSuccess)
+                    return -1;
+                raised.store(true, std::memory_order_relaxed);
+            }
+        }
         if constexpr (PARTS == 2) {  // short rows: one wavefront per workgroup, which walks the tiles
             static std::atomic<int> known{0};
             const int resident = resident_workgroups(kernel, static_cast<int>(block.x), slices, known);
@@ -851,7 +894,8 @@ int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream) {
     const dim3 grid(a.rows / tile_rows, 1, 1), block(waves * 64);
     // the exchange between the wavefronts of a block (8 KB each) overlays the activation buffers (5 KB each)
     const size_t lds = static_cast<size_t>(waves) * (a.rotate_log_block > 11 ? 64 * kChunkCodes * sizeof(float)
-                                                                                : kSliceWords * sizeof(uint32_t));
+                                                                                : kSliceWords * sizeof(uint32_t)) +
+                       handed_terms_bytes(waves, tile_rows);
     auto launch = [&](auto kernel) -> int {
         static std::atomic<bool> raised{false};
         if (lds > 48 * 1024 && !raised.load(std::memory_order_relaxed)) {

@@ -74,6 +74,9 @@ def test_config2_decoder_shapes_int4_g128(shape, samples):
     (8192 + 3, 2048),    # 512 tiles of one wavefront
     (3584 + 2, 3584),    # fewer tiles than compute units: tall tiles from three samples on
     (3072 + 7, 8192),
+    (3072 + 7, 11008),   # six wavefronts: sixteen-row tiles of two spans (the sub-matrix: eight-row tiles)
+    (2560 + 9, 12288),   # too few tiles for two spans: the streaming kernel's wavefronts hand over their terms
+    (6144 + 3, 14336),   # seven wavefronts, a sparse second round: eight-row tiles of the streaming kernel
 ])
 @pytest.mark.parametrize("asym", [False, True])
 def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
@@ -81,7 +84,8 @@ def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
     sixteen would leave SIMDs idle or the last round sparse, walked by as many workgroups as the GPU holds from
     three samples on, and tall tiles on small layers with several samples.  Every sample count, fp16 and bf16,
     ragged row counts, with bias; with one and two samples every row equals the same row of a launch on a
-    sub-matrix that takes the default tiles, bit for bit, since a row's sums do not depend on its tile."""
+    sub-matrix that takes the default tiles, bit for bit, since a row's sums do not depend on its tile (nor, for
+    rows of six and seven wavefronts, on whether the two-span kernel or the streaming kernel sums them)."""
     weight = helpers.normal_weight(rows, width, seed=rows % 97)
     layer = helpers.quantised_layer(weight, INT4, bits=4, group=128, integer=True, asym=asym)
     bias = helpers.activations(1, rows, seed=3)[0]
