@@ -40,8 +40,9 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
     const float code_step = kSubnormalCodes ? a.grid_step * 16777216.0f : a.grid_step;
     constexpr int kAhead = ROWS < 4 ? ROWS : 4;   // rows of codes in flight, two pieces each (six and eight rows measured slower)
     constexpr int kSums = ROWS * MT;              // row sums of the tile
+    constexpr int kMeeting = kSums <= 4 ? 4 : kSums <= 8 ? 8 : kSums <= 16 ? 16 : kSums <= 32 ? 32 : 64;  // the reduction halves
     constexpr int kSlots = 8;                     // wavefronts of the workgroup
-    __shared__ float partials[kSums * kSlots];  // [row sum][wavefront]
+    __shared__ float partials[kMeeting * kSlots];  // [row sum][wavefront]
     extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
     uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
 
@@ -130,7 +131,9 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
     // A lane adds its second span's term to its first span's, then the lanes of the wavefront meet, then the
     // wavefronts in ascending order.  The streaming kernel sums rows of six and seven wavefronts in this order too
     // (its wavefront w + waves hands its terms to wavefront w), so a row's result equals that kernel's bit for bit.
-    float sums[kSums];
+    float sums[kMeeting];
+#pragma unroll
+    for (int j = kSums; j < kMeeting; ++j) sums[j] = 0.0f;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
 #pragma unroll
@@ -153,8 +156,8 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
     }
 
     // All sums over the lanes at once, then over the wavefronts in ascending order.
-    transposed_wave_sum<kSums, 0, 6>(sums, lane);
-    if (lane < kSums) partials[transposed_value_of_lane<kSums>(lane) * kSlots + wave] = sums[0];
+    transposed_wave_sum<kMeeting, 0, 6>(sums, lane);
+    if (lane < kMeeting) partials[transposed_value_of_lane<kMeeting>(lane) * kSlots + wave] = sums[0];
     __syncthreads();
     if (tid < kSums) {
         float total = partials[tid * kSlots];
@@ -185,8 +188,12 @@ int launch_rows_of(const Stream4Args &a, const Stream4Group &members, int tiles,
         return launch(long_rows_kernel<MT, Z, ROWS, MK_BF16, W>);
     };
     if (a.scale_dtype == MK_F32) {
-        if (a.zeros) return of(std::true_type{}, std::true_type{});
-        return of(std::false_type{}, std::true_type{});
+        if constexpr (ROWS <= 16) {   // (tiles taller than sixteen rows are built for 16-bit scales only)
+            if (a.zeros) return of(std::true_type{}, std::true_type{});
+            return of(std::false_type{}, std::true_type{});
+        } else {
+            return -1;
+        }
     }
     if (a.zeros) return of(std::true_type{}, std::false_type{});
     return of(std::false_type{}, std::false_type{});
@@ -446,6 +453,22 @@ int launch_blocks_of(const Stream4Args &a, hipStream_t stream) {
     return status ? -1 : tiles * ROWS;
 }
 
+// The tile height with the lowest rounds x (4 + height): a launch takes as many rounds as its tiles need on 256
+// compute units, and a workgroup costs about four rows' worth of time before its first row (all of x read and
+// prepared).  Tiles of 20 to 32 rows give layers of 4097 to 8192 rows one round (5120 rows: 256 tiles of 20).
+int tile_rows_by_rounds(int rows, bool tall) {
+    constexpr int heights[] = {16, 8, 4, 20, 24, 28, 32};   // earlier wins a tie
+    int best = 0, best_cost = 0;
+    for (int height : heights) {
+        const int tiles = rows / height;
+        if (tiles == 0 || (height > 16 && !tall)) continue;
+        // (rows past the last whole tile take a launch of the word kernel: about eight rows' worth)
+        const int cost = mk_cdiv(tiles, kComputeUnits) * (4 + height) + (rows % height ? 8 : 0);
+        if (best == 0 || cost < best_cost) best = height, best_cost = cost;
+    }
+    return best;
+}
+
 template <int ROWS>
 int launch_tiles(const Stream4Args &a, hipStream_t stream) {
     Stream4Group none;
@@ -467,24 +490,33 @@ int launch_tiles(const Stream4Args &a, hipStream_t stream) {
 // rounds x (4 + height) wins.  Measured against the streaming kernel (M = 1 / 2, us): 4096 x 14336 6.98 -> 6.76 / 7.88 ->
 // 7.76 and 4096 x 11008 6.07 -> 5.82 / 7.73 -> 7.43 (sixteen rows), 2048 x 14336 5.33 -> 4.81 / 6.42 -> 5.61, 2048 x 11008
 // 4.92 -> 4.30 / 6.03 -> 5.36 and 6144 x 14336 9.89 -> 9.68 / 12.4 -> 12.1 (eight), 1024 x 14336 4.08 -> 3.83 (four, one
-// sample; two: 4.51 -> 4.63, not taken).  Not taken: fewer than 192 tiles (512 x 14336: 3.61 -> 3.61 / 4.21 -> 4.61), rows
+// sample; two: 4.51 -> 4.63, not taken), 5120 x 13824 9.0 -> 7.7 / 11.5 -> 9.1 (256 tiles of twenty rows), 6144 x 14336
+// 9.9 -> 9.05 / 12.1 -> 10.4 (24 rows), 8192 x 12288 10.45 -> 9.95 / 12.3 -> 11.85 (32 rows).  Not taken: fewer than 192 tiles (512 x 14336: 3.61 -> 3.61 / 4.21 -> 4.61), rows
 // of five wavefronts (three wavefronts of 2, 2 and 1 spans: 2560 x 10240 5.13 -> 5.65, 1536 x 8960 4.1 -> 4.2 / 5.0 -> 5.3;
 // only one sample of tall layers gained, 4096 x 10240 6.25 -> 5.9), eight wavefronts (4096 x 16384: 7.6 -> 7.7), layers
-// whose second round of sixteen-row tiles is at most half full (5120 x 12288: 8.0 -> 8.6 with eight-row tiles).
-int two_span_tile_rows(int samples, int rows, int width) {
+// with fp32 scales (no tiles over sixteen rows are built for them) whose second round of sixteen-row tiles is at
+// most half full (5120 x 12288: 8.0 -> 8.6 with eight-row tiles).
+int two_span_tile_rows(int samples, int rows, int width, bool wide_sides) {
     const int row_waves = mk_cdiv(width, 2048);
     if (samples > 2 || row_waves < 6 || row_waves > 7) return 0;
-    // a second round of sixteen-row tiles at most half full: the streaming kernel's eight-row tiles are as fast
-    if (rows / 16 > kComputeUnits && rows / 16 <= kComputeUnits + kComputeUnits / 2) return 0;
-    int best = 0, best_cost = 0;
-    for (int height = 16; height >= 4; height /= 2) {
-        const int tiles = rows / height;
-        if (tiles == 0) continue;
-        const int cost = mk_cdiv(tiles, kComputeUnits) * (4 + height);
-        if (best == 0 || cost < best_cost) best = height, best_cost = cost;
-    }
+    const int best = tile_rows_by_rounds(rows, !wide_sides);
     if (best == 0 || rows / best < 192 || (best == 4 && samples == 2)) return 0;
+    // a second round of sixteen-row tiles at most half full (fp32 scales, which have no taller tiles): the streaming
+    // kernel's eight-row tiles are as fast
+    if (best <= 16 && rows / 16 > kComputeUnits && rows / 16 <= kComputeUnits + kComputeUnits / 2) return 0;
     return best;
+}
+
+int launch_tiles_of(int height, const Stream4Args &a, hipStream_t stream) {
+    switch (height) {
+        case 4: return launch_tiles<4>(a, stream);
+        case 8: return launch_tiles<8>(a, stream);
+        case 20: return launch_tiles<20>(a, stream);
+        case 24: return launch_tiles<24>(a, stream);
+        case 28: return launch_tiles<28>(a, stream);
+        case 32: return launch_tiles<32>(a, stream);
+        default: return launch_tiles<16>(a, stream);
+    }
 }
 
 }  // namespace
@@ -498,7 +530,7 @@ bool long_accepts(int samples, int rows, int width, int group, int bits, int x_d
         const bool power_of_two = (group & (group - 1)) == 0 || group >= width;   // the matrix-core kernel shifts instead of dividing
         return samples <= 2 || (scale_dtype != MK_F32 && power_of_two);
     }
-    return two_span_tile_rows(samples, rows, width) != 0;
+    return two_span_tile_rows(samples, rows, width, scale_dtype == MK_F32) != 0;
 }
 
 // Up to eight matrices of one input width in one launch of the two-span kernel: the members' whole tiles of
@@ -545,11 +577,10 @@ int long_launch(const Stream4Args &a, hipStream_t stream) {
         if ((a.rows / 8) * passes <= kComputeUnits) return launch_blocks_of<8>(a, stream);
         return launch_blocks_of<16>(a, stream);
     }
-    if (a.width <= 16384) {
-        const int height = two_span_tile_rows(a.samples, a.rows, a.width);
-        return height == 4 ? launch_tiles<4>(a, stream) : height == 8 ? launch_tiles<8>(a, stream) : launch_tiles<16>(a, stream);
-    }
-    if (wide_tiles > kComputeUnits && wide_tiles <= kComputeUnits + kComputeUnits / 2) return launch_tiles<8>(a, stream);
+    if (a.width <= 16384) return launch_tiles_of(two_span_tile_rows(a.samples, a.rows, a.width, a.scale_dtype == MK_F32), a, stream);
+    // (5120 x 27648 at M = 1 / 2: 15.6 -> 13.75 / 22.2 -> 16.6 us with 256 tiles of twenty rows, 8192 x 28672: 20.6 -> 20.1 /
+    // 26.3 -> 23.2 with tiles of 32)
+    if (wide_tiles >= kComputeUnits) return launch_tiles_of(tile_rows_by_rounds(a.rows, a.scale_dtype != MK_F32), a, stream);
     if (wide_tiles >= kComputeUnits / 2) return launch_tiles<16>(a, stream);
     if (a.rows / 8 >= kComputeUnits / 2) return launch_tiles<8>(a, stream);
     return launch_tiles<4>(a, stream);

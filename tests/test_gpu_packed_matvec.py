@@ -76,7 +76,9 @@ def test_config2_decoder_shapes_int4_g128(shape, samples):
     (3072 + 7, 8192),
     (3072 + 7, 11008),   # six wavefronts: sixteen-row tiles of two spans (the sub-matrix: eight-row tiles)
     (2560 + 9, 12288),   # too few tiles for two spans: the streaming kernel's wavefronts hand over their terms
-    (6144 + 3, 14336),   # seven wavefronts, a sparse second round: eight-row tiles of the streaming kernel
+    (6144 + 3, 14336),   # seven wavefronts: 256 tiles of 24 rows of two spans
+    (5120 + 5, 13824),   # 256 tiles of twenty rows
+    (7168 + 3, 12288),   # 256 tiles of 28 rows
 ])
 @pytest.mark.parametrize("asym", [False, True])
 def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
@@ -105,6 +107,7 @@ def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
 @pytest.mark.parametrize("rows,width,group,asym", [
     (4096 + 5, 18944, 128, False),   # sixteen-row tiles, five wavefronts of two spans, the second span partly past the row
     (260, 28672, 128, True),         # four-row tiles, seven wavefronts
+    (5120 + 9, 18944, 128, True),    # 256 tiles of twenty rows
     (70, 32768, 64, True),           # the longest row
     (48, 16384 + 32, 32, False),     # one chunk in the second span
     (37, 53248, 128, True),          # beyond two spans: the table kernel's turns
