@@ -38,7 +38,7 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
     // bf16: with the exponent of 128 inserted, taken out again through the sum of the activations.
     constexpr bool kSubnormalCodes = XT == MK_F16;
     const float code_step = kSubnormalCodes ? a.grid_step * 16777216.0f : a.grid_step;
-    constexpr int kAhead = ROWS < 4 ? ROWS : 4;   // rows of codes in flight, two pieces each (six and eight rows measured slower)
+    constexpr int kAhead = ROWS < 4 ? ROWS : 4;   // rows of codes in flight, two pieces each (4096 x 14336 at M = 1 / 2: three rows 6.7 / 7.85 us, four 6.7 / 7.7, six 6.8 / 8.25; 4096 x 11008: 6.1, 5.8, 5.9)
     constexpr int kSums = ROWS * MT;              // row sums of the tile
     constexpr int kMeeting = kSums <= 4 ? 4 : kSums <= 8 ? 8 : kSums <= 16 ? 16 : kSums <= 32 ? 32 : 64;  // the reduction halves
     constexpr int kSlots = 8;                     // wavefronts of the workgroup

@@ -39,7 +39,8 @@ struct RowsArgs {
 // of s = 0 then run the Walsh-Hadamard stages.
 template <int SOURCE>
 __global__ void __launch_bounds__(1024) rotate_rows_kernel(const RowsArgs a) {
-    __shared__ float exchange[1024];
+    __shared__ float exchange[1024];   // the partial sums of a point's splits
+    __shared__ float across[1024];     // the block between its wavefronts
     constexpr int kBatch = 16;
     const int p = threadIdx.x % a.power;
     const int split = threadIdx.x / a.power;
@@ -78,22 +79,35 @@ __global__ void __launch_bounds__(1024) rotate_rows_kernel(const RowsArgs a) {
         __syncthreads();
         if (split == 0)
             for (int s = 1; s < a.splits; ++s) mixed += exchange[s * a.power + p];
-        __syncthreads();
     }
-    // Walsh-Hadamard over the block's `power` values: strides below 64 inside the wavefront,
-    // the rest through LDS (every thread of the workgroup reaches the barriers).
-    for (int stage = 0; stage < a.log_power; ++stage) {
+    // Walsh-Hadamard over the block's `power` values, strides ascending: those below 64 inside the wavefront;
+    // for the rest every thread reads the value of its lane in each of the block's wavefronts (at most sixteen)
+    // after ONE barrier and runs their stages in registers, the same additions as stage by stage through LDS.
+    for (int stage = 0; stage < a.log_power && stage < 6; ++stage) {
         const int stride = 1 << stage;
-        float partner;
-        if (stride < 64) {
-            partner = __shfl_xor(mixed, stride, 64);
-        } else {
-            if (split == 0) exchange[p] = mixed;
-            __syncthreads();
-            partner = exchange[p ^ stride];
-            __syncthreads();
-        }
+        const float partner = __shfl_xor(mixed, stride, 64);
         mixed = (p & stride) ? partner - mixed : mixed + partner;
+    }
+    if (a.log_power > 6) {  // uniform
+        if (split == 0) across[p] = mixed;
+        __syncthreads();
+        const int slices = a.power >> 6, own = p >> 6, lane = p & 63;
+        float v[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v[j] = across[(j < slices ? j : 0) * 64 + lane];
+#pragma unroll
+        for (int bit = 1; bit < 16; bit <<= 1) {
+            if (bit < slices) {  // uniform
+                float next[16];
+#pragma unroll
+                for (int j = 0; j < 16; ++j) next[j] = (j & bit) ? v[j ^ bit] - v[j] : v[j] + v[j ^ bit];
+#pragma unroll
+                for (int j = 0; j < 16; ++j) v[j] = next[j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            if (j == own) mixed = v[j];
     }
     if (split == 0)
         mk_store_from_float(a.target, row_start + static_cast<size_t>(block) * a.power + p, a.target_dtype, mixed * a.scale);
