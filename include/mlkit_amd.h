@@ -73,11 +73,10 @@ int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packed, const vo
  * activations and scales, or 4-bit codes of a uniform grid with fp32 activations and scales of
  * any type; input_width a multiple of 32 up to 16384, scale groups of whole multiples of 32
  * codes) run as ONE launch whose grid covers all the matrices; every other layout runs as
- * `count` launches of mk_packed_matvec.  Results equal
- * those of `count` separate calls bit for bit for every row inside a member's whole tiles of
- * sixteen rows; the up to fifteen rows past them are multiplied by the word-at-a-time kernel,
- * which sums a row in another order than the tile kernels a separate call of a small member
- * may still use for them (equal to fp32 rounding).
+ * `count` launches of mk_packed_matvec.  With one and two samples the results equal those of
+ * `count` separate calls bit for bit; from three samples on the kernels split a row's sum by
+ * the size of the launch, and a few outputs in a thousand differ from the separate call's by
+ * one rounding of the output type.
  * Replaces: the consecutive launches of kernels/packed_linear.py:181-226 that a model makes
  * for such layers (it calls PackedLinear.forward, inference/packed_linear.py:148-245, once
  * per layer). */

@@ -235,6 +235,11 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
         s4.x_dtype = x_dtype; s4.scale_dtype = scale_dtype;
         done_rows = mk_matvec::long_launch(s4, stream);
         MK_REQUIRE(done_rows >= 0, MK_ERR_HIP, "mk_packed_matvec: the runtime refused the kernel's launch");
+        if (input_width <= 16384 && output_width - done_rows >= 4) {   // (the grouped launch leaves the same rows % 4 to the word kernel)
+            const int more = mk_matvec::stream4_launch_remainder(s4, done_rows, stream);
+            MK_REQUIRE(more >= 0, MK_ERR_HIP, "mk_packed_matvec: the runtime refused the kernel's LDS size");
+            done_rows += more;
+        }
         if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
     } else if (aligned && !tuning().no_stream4 &&
                mk_matvec::stream4_accepts(samples, input_width, group, bits, x_dtype, scale_dtype, uniform != 0) &&
@@ -247,6 +252,11 @@ extern "C" int mk_packed_matvec(const void *x, int x_dtype, const uint8_t *packe
         s4.x_dtype = x_dtype; s4.scale_dtype = scale_dtype;
         done_rows = mk_matvec::stream4_launch(s4, stream);
         MK_REQUIRE(done_rows >= 0, MK_ERR_HIP, "mk_packed_matvec: the runtime refused the kernel's LDS size");
+        if (output_width - done_rows >= 4) {
+            const int more = mk_matvec::stream4_launch_remainder(s4, done_rows, stream);
+            MK_REQUIRE(more >= 0, MK_ERR_HIP, "mk_packed_matvec: the runtime refused the kernel's LDS size");
+            done_rows += more;
+        }
         if (done_rows > 0) MK_LAUNCH_CHECK("mk_packed_matvec");
     } else if (aligned && !tuning().no_pairs &&
                mk_matvec::pairs_accepts(input_width, group, bits, x_dtype, scale_dtype) &&
@@ -363,7 +373,16 @@ extern "C" int mk_packed_matvec_group(const void *const *x, int x_dtype, int cou
         mk_matvec::pairs_launch_group(shared, members, output_widths, &rows_per_tile, stream);
     MK_LAUNCH_CHECK("mk_packed_matvec_group");
     for (int i = 0; i < count; ++i) {  // rows past a member's last whole tile
-        const int covered = output_widths[i] / rows_per_tile * rows_per_tile;
+        int covered = output_widths[i] / rows_per_tile * rows_per_tile;
+        if (streaming && output_widths[i] - covered >= 4) {   // their whole four-row tiles, as in the single call
+            mk_matvec::Stream4Args own = shared;
+            own.x = x[i]; own.packed = packed[i]; own.scales = scales[i]; own.zeros = members.member[i].zeros;
+            own.bias = members.member[i].bias; own.y = y[i]; own.rows = output_widths[i];
+            const int more = mk_matvec::stream4_launch_remainder(own, covered, stream);
+            MK_REQUIRE(more >= 0, MK_ERR_HIP, "mk_packed_matvec_group: the runtime refused the kernel's LDS size");
+            MK_LAUNCH_CHECK("mk_packed_matvec_group");
+            covered += more;
+        }
         if (covered < output_widths[i])
             if (int status = launch_words(x[i], x_dtype, packed[i], scales[i], scale_dtype, values, members.member[i].zeros,
                                           members.member[i].bias, bias_dtype, y[i], samples, output_widths[i],

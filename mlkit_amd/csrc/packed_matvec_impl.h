@@ -159,6 +159,8 @@ int pairs_launch_group(const Stream4Args &shared, Stream4Group &group, const int
                        hipStream_t stream);
 bool stream4_accepts(int samples, int width, int group, int bits, int x_dtype, int scale_dtype, bool uniform);
 int stream4_launch(const Stream4Args &a, hipStream_t stream);
+// The whole four-row tiles of rows [first_row, rows) after a launch of taller tiles; returns the rows covered, or -1.
+int stream4_launch_remainder(const Stream4Args &a, int first_row, hipStream_t stream);
 // 4-bit uniform-grid codes in rows of 16416 to 32768 codes, and one or two samples of some shorter rows, fp16 or bf16
 // activations (packed_matvec_long.hip: a wavefront owns two spans of 2048 codes):
 // multiplies the leading whole tiles of rows and returns the number of rows covered, or -1.

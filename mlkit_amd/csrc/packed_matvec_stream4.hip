@@ -877,6 +877,30 @@ int stream4_launch(const Stream4Args &a, hipStream_t stream) {
     return launch_rows<kNarrowRows>(a, none, tiles, stream) ? -1 : tiles * kNarrowRows;
 }
 
+// The whole four-row tiles of rows [first_row, a.rows), which a launch of taller tiles left over (first_row is a
+// multiple of four): one member of a group whose pointers start at that row.  A row's sums do not depend on its
+// tile, so the single call and the grouped launch, which may tile a matrix differently, leave the same rows (the
+// last rows % 4) to the word kernel.  Returns the rows covered, or -1.
+int stream4_launch_remainder(const Stream4Args &a, int first_row, hipStream_t stream) {
+    const int tiles = (a.rows - first_row) / kNarrowRows;
+    if (tiles <= 0) return 0;
+    Stream4Group one{};
+    one.count = 1;
+    one.widest_tiles = tiles;
+    Stream4Member &member = one.member[0];
+    const size_t row = static_cast<size_t>(first_row);
+    const size_t side_bytes = static_cast<size_t>(a.groups) * (a.scale_dtype == MK_F32 ? 4 : 2);
+    member.x = a.x;
+    member.packed = a.packed + row * (static_cast<size_t>(a.width) >> 1);
+    member.scales = static_cast<const uint8_t *>(a.scales) + row * side_bytes;
+    member.zeros = a.zeros ? static_cast<const uint8_t *>(a.zeros) + row * side_bytes : nullptr;
+    member.bias = a.bias ? static_cast<const uint8_t *>(a.bias) + row * mk_dtype_bytes(a.bias_dtype) : nullptr;
+    member.y = static_cast<uint8_t *>(a.y) + row * mk_dtype_bytes(a.x_dtype);   // outputs have the activations' type
+    member.rows = a.rows;
+    member.tiles = tiles;
+    return launch_rows<kNarrowRows>(a, one, tiles, stream) ? -1 : tiles * kNarrowRows;
+}
+
 int stream4_launch_rotating(const Stream4Args &a, hipStream_t stream) {
     const bool wide = a.rows / kWideRows >= kComputeUnits;
     const int tile_rows = wide ? kWideRows : kNarrowRows;
