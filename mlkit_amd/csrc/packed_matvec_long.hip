@@ -21,13 +21,12 @@ namespace mk_matvec {
 
 namespace {
 
-constexpr int kSpans = 2;
 constexpr int kComputeUnits = 256;
 
-// One or two samples.  ROWS rows per workgroup, cdiv(K, 4096) wavefronts.
-template <int MT, bool HAS_ZERO, int ROWS, int XT, bool WIDE_SIDES>
-__global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, const Stream4Group members) {
-    static_assert(ROWS * MT <= 64, "one transposed reduction per workgroup");
+// The sums of a tile's rows over this lane's chunks of N spans of 2048 codes (span s of wavefront w of `waves` is span
+// s * waves + w of the row): sums[r * MT + m] for row r and sample m, the rest of `sums` zero.
+template <int N, int MT, bool HAS_ZERO, int ROWS, int XT, bool WIDE_SIDES, int SUMS>
+__device__ __forceinline__ void long_rows_sums(const Stream4Args &a, const TileSource &source, uint32_t *x_slice, float (&sums)[SUMS]) {
     using SideRaw = std::conditional_t<WIDE_SIDES, uint32_t, uint16_t>;
     constexpr uint32_t kSideBytes = WIDE_SIDES ? 4u : 2u;
     auto side_of = [&](SideRaw raw) __attribute__((always_inline)) {
@@ -38,28 +37,20 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
     // bf16: with the exponent of 128 inserted, taken out again through the sum of the activations.
     constexpr bool kSubnormalCodes = XT == MK_F16;
     const float code_step = kSubnormalCodes ? a.grid_step * 16777216.0f : a.grid_step;
-    constexpr int kAhead = ROWS < 4 ? ROWS : 4;   // rows of codes in flight, two pieces each (4096 x 14336 at M = 1 / 2: three rows 6.7 / 7.85 us, four 6.7 / 7.7, six 6.8 / 8.25; 4096 x 11008: 6.1, 5.8, 5.9)
-    constexpr int kSums = ROWS * MT;              // row sums of the tile
-    constexpr int kMeeting = kSums <= 4 ? 4 : kSums <= 8 ? 8 : kSums <= 16 ? 16 : kSums <= 32 ? 32 : 64;  // the reduction halves
-    constexpr int kSlots = 8;                     // wavefronts of the workgroup
-    __shared__ float partials[kMeeting * kSlots];  // [row sum][wavefront]
-    extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
-    uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
-
-    const TileSource source = tile_source<ROWS>(a, members, blockIdx.z);
-    if (static_cast<int>(blockIdx.x) >= source.tiles) return;
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
+    // rows of codes in flight, N pieces each (two spans, 4096 x 14336 at M = 1 / 2: three rows 6.7 / 7.85 us, four 6.7 / 7.7, six 6.8 / 8.25; 4096 x 11008: 6.1, 5.8, 5.9)
+    constexpr int kMost = N == 2 ? 4 : 3;
+    constexpr int kAhead = ROWS < kMost ? ROWS : kMost;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
     const int waves = blockDim.x >> 6;
     const int sample_base = blockIdx.y * MT;
     const uint32_t row_bytes = static_cast<uint32_t>(a.width) >> 1;
     const uint32_t scale_row_bytes = static_cast<uint32_t>(a.groups) * kSideBytes;
     // Lanes past the end of a row read chunk 0 with zeroed activations: they add nothing.
-    bool in_row[kSpans];
-    uint32_t code_offset[kSpans], group_offset[kSpans];
+    bool in_row[N];
+    uint32_t code_offset[N], group_offset[N];
 #pragma unroll
-    for (int s = 0; s < kSpans; ++s) {
+    for (int s = 0; s < N; ++s) {
         const int wanted = (s * waves + wave) * 64 + lane;
         in_row[s] = wanted * kChunkCodes < a.width;
         const int chunk = in_row[s] ? wanted : 0;
@@ -67,11 +58,9 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
         group_offset[s] = ((static_cast<uint32_t>(chunk) * kChunkCodes) / static_cast<uint32_t>(a.group)) * kSideBytes;
     }
 
-    __syncthreads();  // aligns the workgroup's wavefronts before their first loads
-
-    mk_u32x4 pieces[kSpans][MT][4];
+    mk_u32x4 pieces[N][MT][4];
 #pragma unroll
-    for (int s = 0; s < kSpans; ++s)
+    for (int s = 0; s < N; ++s)
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             const int sample = sample_base + m < a.samples ? sample_base + m : a.samples - 1;
@@ -84,12 +73,12 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
     const uint8_t *const codes_base = source.packed + static_cast<size_t>(row_base) * row_bytes;
     const uint8_t *const scale_base = source.scales + static_cast<size_t>(row_base) * scale_row_bytes;
     const uint8_t *const zero_base = HAS_ZERO ? source.zeros + static_cast<size_t>(row_base) * scale_row_bytes : nullptr;
-    SideRaw scale_raw[ROWS][kSpans], zero_raw[HAS_ZERO ? ROWS : 1][kSpans];
-    CodeChunk<4> codes[ROWS][kSpans];
-    // A row's two pieces of codes and the two scales (and offsets) that go with them.
+    SideRaw scale_raw[ROWS][N], zero_raw[HAS_ZERO ? ROWS : 1][N];
+    CodeChunk<4> codes[ROWS][N];
+    // A row's pieces of codes and the scales (and offsets) that go with them.
     auto request_row = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
-        for (int s = 0; s < kSpans; ++s) {
+        for (int s = 0; s < N; ++s) {
             scale_raw[r][s] = *reinterpret_cast<const SideRaw *>(scale_base + static_cast<size_t>(r) * scale_row_bytes + group_offset[s]);
             if constexpr (HAS_ZERO)
                 zero_raw[r][s] = *reinterpret_cast<const SideRaw *>(zero_base + static_cast<size_t>(r) * scale_row_bytes + group_offset[s]);
@@ -102,11 +91,11 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
         __builtin_amdgcn_sched_barrier(0);  // in row order
     }
 
-    // Each lane's two chunks of every sample, through the wavefront's own LDS buffer.
-    XChunk<XT> x[kSpans][MT];
-    float x_sum[kSpans][MT], grid_term[kSpans][MT];
+    // Each lane's chunks of every sample, through the wavefront's own LDS buffer.
+    XChunk<XT> x[N][MT];
+    float x_sum[N][MT], grid_term[N][MT];
 #pragma unroll
-    for (int s = 0; s < kSpans; ++s)
+    for (int s = 0; s < N; ++s)
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             if (s + m > 0) wave_exchange_fence();   // the last readers before these pieces
@@ -128,23 +117,22 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
             grid_term[s][m] = a.grid_min * x_sum[s][m] - a.grid_step * code_free;
         }
 
-    // A lane adds its second span's term to its first span's, then the lanes of the wavefront meet, then the
-    // wavefronts in ascending order.  The streaming kernel sums rows of six and seven wavefronts in this order too
-    // (its wavefront w + waves hands its terms to wavefront w), so a row's result equals that kernel's bit for bit.
-    float sums[kMeeting];
+    // A lane adds its spans' terms, each rounded first; then the lanes of the wavefront meet, then the wavefronts
+    // in ascending order.  The streaming kernel sums rows of six and seven wavefronts in this order too (its
+    // wavefront w + waves hands its terms to wavefront w), so a row's result equals that kernel's bit for bit.
 #pragma unroll
-    for (int j = kSums; j < kMeeting; ++j) sums[j] = 0.0f;
+    for (int j = ROWS * MT; j < SUMS; ++j) sums[j] = 0.0f;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
 #pragma unroll
-        for (int s = 0; s < kSpans; ++s) {
+        for (int s = 0; s < N; ++s) {
             float dot[MT];
             if constexpr (kSubnormalCodes) chunk_dot_subnormal<MT>(codes[r][s], x[s], dot);
             else chunk_dot_bf16<MT>(codes[r][s], x[s], dot);
             const float scale = side_of(scale_raw[r][s]);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-#pragma clang fp contract(off)   // the span's term is rounded before it meets the other span's, as between wavefronts
+#pragma clang fp contract(off)   // the span's term is rounded before it meets the other spans', as between wavefronts
                 float value = scale * __builtin_fmaf(code_step, dot[m], grid_term[s][m]);
                 if constexpr (HAS_ZERO) value = __builtin_fmaf(side_of(zero_raw[r][s]), x_sum[s][m], value);
                 if (s == 0) sums[r * MT + m] = value;
@@ -153,6 +141,39 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
         }
         if (r + kAhead < ROWS) request_row(r + kAhead);
         __builtin_amdgcn_sched_barrier(0);  // rows in arrival order, temporaries short-lived
+    }
+}
+
+// One or two samples.  ROWS rows per workgroup; a wavefront owns up to SPANS spans of 2048 codes, cdiv(K, 2048 SPANS)
+// wavefronts.  SPANS = 3 (rows of 16416 to 24576 codes: four wavefronts, one per SIMD, where five or six wavefronts of
+// two spans put two on one SIMD): a wavefront whose third span lies past the row runs the two-span body.
+template <int MT, bool HAS_ZERO, int ROWS, int XT, bool WIDE_SIDES, int SPANS = 2>
+__global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, const Stream4Group members) {
+    static_assert(ROWS * MT <= 64, "one transposed reduction per workgroup");
+    constexpr int kSums = ROWS * MT;              // row sums of the tile
+    constexpr int kMeeting = kSums <= 4 ? 4 : kSums <= 8 ? 8 : kSums <= 16 ? 16 : kSums <= 32 ? 32 : 64;  // the reduction halves
+    constexpr int kSlots = 8;                     // wavefronts of the workgroup
+    __shared__ float partials[kMeeting * kSlots];  // [row sum][wavefront]
+    extern __shared__ __attribute__((aligned(16))) uint32_t x_slices_storage[];
+    uint32_t *const x_slice = x_slices_storage + (threadIdx.x >> 6) * kSliceWords;
+
+    const TileSource source = tile_source<ROWS>(a, members, blockIdx.z);
+    if (static_cast<int>(blockIdx.x) >= source.tiles) return;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int waves = blockDim.x >> 6;
+
+    __syncthreads();  // aligns the workgroup's wavefronts before their first loads
+
+    float sums[kMeeting];
+    if constexpr (SPANS == 3) {
+        if (((2 * waves + wave) * 2048) < a.width)   // uniform per wavefront
+            long_rows_sums<3, MT, HAS_ZERO, ROWS, XT, WIDE_SIDES>(a, source, x_slice, sums);
+        else
+            long_rows_sums<2, MT, HAS_ZERO, ROWS, XT, WIDE_SIDES>(a, source, x_slice, sums);
+    } else {
+        long_rows_sums<2, MT, HAS_ZERO, ROWS, XT, WIDE_SIDES>(a, source, x_slice, sums);
     }
 
     // All sums over the lanes at once, then over the wavefronts in ascending order.
@@ -164,8 +185,8 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
 #pragma unroll
         for (int w = 1; w < kSlots; ++w) total += w < waves ? partials[tid * kSlots + w] : 0.0f;
         const int j = tid / MT, m = tid - j * MT;
-        const int row = row_base + j;
-        const int sample = sample_base + m;
+        const int row = blockIdx.x * ROWS + j;
+        const int sample = blockIdx.y * MT + m;
         if (sample < a.samples) {
             if (source.bias) total += mk_load_as_float(source.bias, row, a.bias_dtype);
             store_output<XT>(source.y, static_cast<size_t>(sample) * source.rows + row, total);
@@ -173,10 +194,14 @@ __global__ void __launch_bounds__(512) long_rows_kernel(const Stream4Args a, con
     }
 }
 
+// Rows of 16416 to 24576 codes take three spans per wavefront (3584 x 18944 at M = 1 / 2: see long_launch).
+inline int spans_per_wavefront(int width) { return width > 16384 && width <= 24576 ? 3 : 2; }
+
 template <int MT, int ROWS>
 int launch_rows_of(const Stream4Args &a, const Stream4Group &members, int tiles, hipStream_t stream) {
     if (tiles == 0) return 0;
-    const dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1), block(mk_cdiv(a.width, 2048 * kSpans) * 64);
+    const int spans = spans_per_wavefront(a.width);
+    const dim3 grid(tiles, mk_cdiv(a.samples, MT), members.count > 0 ? members.count : 1), block(mk_cdiv(a.width, 2048 * spans) * 64);
     const size_t slices = static_cast<size_t>(block.x / 64) * kSliceWords * sizeof(uint32_t);
     auto launch = [&](auto kernel) -> int {
         hipLaunchKernelGGL(kernel, grid, block, slices, stream, a, members);
@@ -184,6 +209,10 @@ int launch_rows_of(const Stream4Args &a, const Stream4Group &members, int tiles,
     };
     auto of = [&](auto has_zero, auto wide) -> int {
         constexpr bool Z = decltype(has_zero)::value, W = decltype(wide)::value;
+        if (spans == 3) {
+            if (a.x_dtype == MK_F16) return launch(long_rows_kernel<MT, Z, ROWS, MK_F16, W, 3>);
+            return launch(long_rows_kernel<MT, Z, ROWS, MK_BF16, W, 3>);
+        }
         if (a.x_dtype == MK_F16) return launch(long_rows_kernel<MT, Z, ROWS, MK_F16, W>);
         return launch(long_rows_kernel<MT, Z, ROWS, MK_BF16, W>);
     };

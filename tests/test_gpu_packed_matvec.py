@@ -105,7 +105,9 @@ def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
 
 
 @pytest.mark.parametrize("rows,width,group,asym", [
-    (4096 + 5, 18944, 128, False),   # sixteen-row tiles, five wavefronts of two spans, the second span partly past the row
+    (4096 + 5, 18944, 128, False),   # sixteen-row tiles, four wavefronts of three spans: two of them have a third span, one partly past the row
+    (300, 22016, 64, True),          # eleven spans: three wavefronts of three, one of two
+    (67, 24576, 128, False),         # twelve spans, the longest row of three spans per wavefront
     (260, 28672, 128, True),         # four-row tiles, seven wavefronts
     (5120 + 9, 18944, 128, True),    # 256 tiles of twenty rows
     (70, 32768, 64, True),           # the longest row
@@ -113,7 +115,7 @@ def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
     (37, 53248, 128, True),          # beyond two spans: the table kernel's turns
 ])
 def test_rows_of_more_than_16384_codes(rows, width, group, asym):
-    """Down projections of the larger decoders (K = 18944, 28672): every wavefront owns two spans of 2048 codes.
+    """Down projections of the larger decoders (K = 18944, 28672): every wavefront owns two or three spans of 2048 codes.
     One to eight samples, fp16 and bf16 activations, 16-bit and fp32 scales, offsets and bias, against the float64
     product."""
     weight = helpers.normal_weight(rows, width, seed=width % 89)
