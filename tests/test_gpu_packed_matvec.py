@@ -869,3 +869,37 @@ def test_random_layouts_against_the_oracle(seed):
         tolerance = {torch.float16: 1e-3, torch.bfloat16: 8e-3, torch.float32: 2e-5}[dtype]
         error = np.abs(y - reference).max() / max(np.abs(reference).max(), 1e-30)
         assert error <= tolerance, (trial, bits, integer, rows, width, group, asym, with_bias, dtype, samples, error)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_shapes_alone_and_grouped(seed):
+    """Seeded random layers (any width that is a multiple of 32 up to 14336 and some up to 32768, ragged row counts,
+    fp16 / bf16, offsets, bias, one to eight samples): every output within the tolerance of the float64 product; with
+    one and two samples a sub-matrix of whole tiles (which takes other tiles or another kernel) and a grouped launch
+    over the layer and that sub-matrix return the same bits as the layer alone."""
+    rng = np.random.default_rng(1000 + seed)
+    width = int(rng.integers(1, 14336 // 32 + 1)) * 32 if seed % 4 else int(rng.integers(16384 // 32 + 1, 32768 // 32 + 1)) * 32
+    group = int(rng.choice([32, 64, 128, width]))
+    if width % group:
+        group = 32
+    rows = int(rng.integers(40, max(41, min(2600, 24_000_000 // width))))
+    asym = bool(rng.integers(2))
+    dtype = (torch.float16, torch.bfloat16)[int(rng.integers(2))]
+    layer = helpers.quantised_layer(helpers.normal_weight(rows, width, seed=seed), INT4, bits=4, group=group, integer=True, asym=asym)
+    if dtype == torch.bfloat16:   # the layer as the kernel sees it: scales and offsets rounded to bf16
+        sides = {key: None if layer[key] is None else torch.from_numpy(layer[key]).to(dtype).float().numpy() for key in ("scales", "zero")}
+        layer = dict(layer, dense=scaling.decode_grouped(layer["codes"], sides["scales"], layer["values"], group, sides["zero"]))
+    part = (rows // 3) // 16 * 16
+    head = dict(layer, packed=layer["packed"][: part * width // 2], scales=layer["scales"][:part],
+                zero=None if layer["zero"] is None else layer["zero"][:part], dense=layer["dense"][:part], shape=(part, width))
+    bias = helpers.activations(1, rows, seed=3, dtype=dtype)[0]
+    for samples in (1, 2, int(rng.choice([3, 4, 5, 8]))):
+        x = helpers.activations(samples, width, seed=20 + samples, dtype=dtype)
+        y = run_matvec(layer, x, bias, scale_dtype=dtype)
+        check(y, layer, x.float(), bias.float(), relative=1e-3 if dtype == torch.float16 else 8e-3)
+        if samples <= 2 and part >= 16:
+            alone = run_matvec(head, x, bias[:part], scale_dtype=dtype)
+            np.testing.assert_array_equal(y[:, :part], alone)
+            grouped = run_group([layer, head], x, [bias, bias[:part]], scale_dtype=dtype)
+            np.testing.assert_array_equal(grouped[0].float().cpu().numpy(), y)
+            np.testing.assert_array_equal(grouped[1].float().cpu().numpy(), alone)
