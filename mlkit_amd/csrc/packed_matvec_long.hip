@@ -217,7 +217,7 @@ int launch_rows_of(const Stream4Args &a, const Stream4Group &members, int tiles,
         return launch(long_rows_kernel<MT, Z, ROWS, MK_BF16, W>);
     };
     if (a.scale_dtype == MK_F32) {
-        if constexpr (ROWS <= 16) {   // (tiles taller than sixteen rows are built for 16-bit scales only)
+        if constexpr (ROWS == 4 || ROWS == 8 || ROWS == 16) {   // (the other heights are built for 16-bit scales only)
             if (a.zeros) return of(std::true_type{}, std::true_type{});
             return of(std::false_type{}, std::true_type{});
         } else {
@@ -484,13 +484,15 @@ int launch_blocks_of(const Stream4Args &a, hipStream_t stream) {
 
 // The tile height with the lowest rounds x (4 + height): a launch takes as many rounds as its tiles need on 256
 // compute units, and a workgroup costs about four rows' worth of time before its first row (all of x read and
-// prepared).  Tiles of 20 to 32 rows give layers of 4097 to 8192 rows one round (5120 rows: 256 tiles of 20).
-int tile_rows_by_rounds(int rows, bool tall) {
-    constexpr int heights[] = {16, 8, 4, 20, 24, 28, 32};   // earlier wins a tie
+// prepared).  Tiles of 20 to 32 rows give layers of 4097 to 8192 rows one round (5120 rows: 256 tiles of 20), tiles
+// of 12 and 14 rows give layers of 3072 and 3584 rows a tile per compute unit (sixteen rows: 192 and 224 tiles).
+// `more`: the heights other than 4, 8 and 16 (built for 16-bit scales only).
+int tile_rows_by_rounds(int rows, bool more) {
+    constexpr int heights[] = {16, 8, 4, 12, 14, 20, 24, 28, 32};   // earlier wins a tie
     int best = 0, best_cost = 0;
     for (int height : heights) {
         const int tiles = rows / height;
-        if (tiles == 0 || (height > 16 && !tall)) continue;
+        if (tiles == 0 || (height != 16 && height != 8 && height != 4 && !more)) continue;
         // (rows past the last whole tile take a launch of the word kernel: about eight rows' worth)
         const int cost = mk_cdiv(tiles, kComputeUnits) * (4 + height) + (rows % height ? 8 : 0);
         if (best == 0 || cost < best_cost) best = height, best_cost = cost;
@@ -540,6 +542,8 @@ int launch_tiles_of(int height, const Stream4Args &a, hipStream_t stream) {
     switch (height) {
         case 4: return launch_tiles<4>(a, stream);
         case 8: return launch_tiles<8>(a, stream);
+        case 12: return launch_tiles<12>(a, stream);
+        case 14: return launch_tiles<14>(a, stream);
         case 20: return launch_tiles<20>(a, stream);
         case 24: return launch_tiles<24>(a, stream);
         case 28: return launch_tiles<28>(a, stream);
@@ -609,7 +613,7 @@ int long_launch(const Stream4Args &a, hipStream_t stream) {
     if (a.width <= 16384) return launch_tiles_of(two_span_tile_rows(a.samples, a.rows, a.width, a.scale_dtype == MK_F32), a, stream);
     // (5120 x 27648 at M = 1 / 2: 15.6 -> 13.75 / 22.2 -> 16.6 us with 256 tiles of twenty rows, 8192 x 28672: 20.6 -> 20.1 /
     // 26.3 -> 23.2 with tiles of 32)
-    if (wide_tiles >= kComputeUnits) return launch_tiles_of(tile_rows_by_rounds(a.rows, a.scale_dtype != MK_F32), a, stream);
+    if (a.rows >= 12 * kComputeUnits) return launch_tiles_of(tile_rows_by_rounds(a.rows, a.scale_dtype != MK_F32), a, stream);
     if (wide_tiles >= kComputeUnits / 2) return launch_tiles<16>(a, stream);
     if (a.rows / 8 >= kComputeUnits / 2) return launch_tiles<8>(a, stream);
     return launch_tiles<4>(a, stream);

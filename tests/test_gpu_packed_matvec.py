@@ -79,6 +79,7 @@ def test_config2_decoder_shapes_int4_g128(shape, samples):
     (6144 + 3, 14336),   # seven wavefronts: 256 tiles of 24 rows of two spans
     (5120 + 5, 13824),   # 256 tiles of twenty rows
     (7168 + 3, 12288),   # 256 tiles of 28 rows
+    (3584 + 5, 11008),   # 256 tiles of fourteen rows
 ])
 @pytest.mark.parametrize("asym", [False, True])
 def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
@@ -110,6 +111,7 @@ def test_tile_heights_chosen_by_layer_shape(rows, width, asym):
     (67, 24576, 128, False),         # twelve spans, the longest row of three spans per wavefront
     (260, 28672, 128, True),         # four-row tiles, seven wavefronts
     (5120 + 9, 18944, 128, True),    # 256 tiles of twenty rows
+    (3072 + 3, 18944, 128, False),   # 256 tiles of twelve rows
     (70, 32768, 64, True),           # the longest row
     (48, 16384 + 32, 32, False),     # one chunk in the second span
     (37, 53248, 128, True),          # beyond two spans: the table kernel's turns
